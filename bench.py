@@ -1,0 +1,174 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-gradient encode + decode path on one MI355X.
+
+One step = exact top-k threshold + fused select/hash-partition/compaction of
+the rank's own gradient + merge of the P peer payloads addressed to rank 0,
+all inputs resident in HBM.  Prints one JSON line (see README / DESIGN).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--shrink S]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--shrink", type=int, default=1, help="divide the workload size (debugging)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-div", type=int, default=2,
+                    help="the CPU baseline runs on 1/div of the workload")
+    ap.add_argument("--no-kernel-timing", action="store_true",
+                    help="leave the HIP-event kernel timers off during the timed region")
+    return ap.parse_args()
+
+
+def cpu_baseline(cfg, grad_dev, div):
+    """The reference's torch-op sequence (insert: sequential C oracle) on this
+    box's host cores, on the first 1/div of the gradient."""
+    import torch
+
+    from oracle import torch_path
+    from zen_repro_amd import workloads
+
+    n_s = cfg.n // div // (16 * cfg.partitions) * (16 * cfg.partitions)
+    sub = workloads.Config(cfg.name, n_s, cfg.dtype, cfg.partitions, cfg.peers, cfg.overlap,
+                           k=int(cfg.k * n_s / cfg.n) if cfg.k else 0)
+    g = grad_dev[:n_s].cpu()
+    nnz_est = sub.k if sub.k else int(torch.count_nonzero(g))
+    per_peer = max(1, nnz_est // cfg.partitions)
+    idx_l, val_l, _, _ = workloads.peer_payloads(sub, per_peer, device="cpu", seed=1)
+    times, _ = torch_path.timed_pass(g, sub.k, cfg.partitions, idx_l, val_l)
+    total = sum(times.values())
+    return {
+        "value": n_s * g.element_size() / total / 1e9,
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"first {n_s} of {cfg.n} elements (1/{div}), k={sub.k}, {cfg.peers} peer payloads of {per_peer}; "
+                  f"select {times['select']:.2f}s partition {times['partition']:.2f}s merge {times['merge']:.2f}s; "
+                  f"torch ops use {torch.get_num_threads()} threads, the sequential insert 1",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU's share of the path; --gpus must be 1 "
+              "(the exchange between ranks is not part of it)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from zen_repro_amd import LoadBalanceAllreduce, LocalGroup, TensorPartition, _lib, topk_threshold, workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    _lib.lib()
+
+    cfg, grad = workloads.make(args.config, device=dev, seed=0, shrink=args.shrink)
+    n, esize, P = cfg.n, grad.element_size(), cfg.partitions
+    tp = TensorPartition(P, 1, 3)
+    lba = LoadBalanceAllreduce(LocalGroup(P), None, None)
+
+    if cfg.k:
+        nnz_guess = cfg.k
+        capacity = int(cfg.k * 1.25) + 4096  # room for ties at the threshold
+    else:
+        nnz_guess = int(torch.count_nonzero(grad))
+        capacity = nnz_guess + 16
+    per_peer = max(1, nnz_guess // P)
+    idx_l, val_l, flat_idx, flat_val = workloads.peer_payloads(cfg, per_peer, device=dev, seed=1)
+    received = flat_idx.numel()
+
+    def step():
+        thr = topk_threshold(grad, cfg.k) if cfg.k else None
+        enc = tp.load_balance_flat(grad, thr, capacity)
+        mrg = lba.merge_sparse_flat(flat_idx, flat_val, n, capacity=received)
+        return thr, enc, mrg
+
+    for _ in range(args.warmup):
+        out = step()
+    torch.cuda.synchronize()
+    if not args.no_kernel_timing:
+        _lib.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    kernels = {} if args.no_kernel_timing else _lib.profile_read()
+    _lib.profile_enable(False)
+
+    thr, (o_idx, o_val, splits, st_enc), (m_idx, m_val, m_count, st_mrg) = out
+    nnz = int(splits.sum())
+    merged = int(m_count)
+    flags = int(st_enc) | int(st_mrg)
+    if flags:
+        print("bench.py: device status " + _lib.describe_status(flags), file=sys.stderr)
+        sys.exit(1)
+
+    ms = (t1 - t0) * 1e3 / args.steps
+    value = n * esize / (ms * 1e-3) / 1e9
+    b_alg = workloads.algorithmic_bytes(n, esize, nnz, received, merged)
+
+    # dominant kernel: the one with the largest summed duration among the
+    # kernels that stream the dense gradient; its algorithmic bytes per launch
+    per_launch = {
+        "k_select_compact": n * esize + nnz * (4 + esize),
+        "k_topk_hist": n * esize,
+    }
+    roofline = None
+    stage_ms = {name: round(total / args.steps, 4) for name, (total, _) in kernels.items()}
+    cands = [(kernels[name][0], name) for name in per_launch if name in kernels]
+    if cands:
+        _, dom = max(cands)
+        total_ms, launches = kernels[dom]
+        avg_ms = total_ms / launches
+        achieved = per_launch[dom] / (avg_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "avg_launch_ms": round(avg_ms, 4), "launches_per_step": launches // args.steps,
+                    "algorithmic_bytes_per_launch": per_launch[dom]}
+
+    line = {
+        "metric": "encode+decode dense-gradient GB/s on 1 GPU; % of HBM roofline",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if grad.dtype == torch.bfloat16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: {cfg.note}", "elements": n, "partitions": P, "k": cfg.k,
+                   "selected": nnz, "received": received, "merged": merged, "peers": cfg.peers,
+                   "overlap": cfg.overlap, "shrink": args.shrink},
+        "path_algorithmic_GBps": round(b_alg / (ms * 1e-3) / 1e9, 2),
+        "path_frac_of_hbm_peak": round(b_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "stage_ms_per_step": stage_ms,
+        "roofline": roofline,
+        "cpu_baseline": None,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(cfg, grad, args.cpu_sample_div)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,209 @@
+/*
+ * libzen_hip: MI355X (gfx950) implementation of ZEN's sparse-gradient
+ * select / hash-partition / merge path.  Plain C ABI: device pointers, sizes
+ * and a HIP stream.  No torch types, no hidden allocation, no host
+ * synchronisation: every call only enqueues kernels on `stream`.
+ *
+ * Conventions
+ *   - every pointer is DEVICE memory unless a comment says "host";
+ *   - `dtype` is ZEN_F32 or ZEN_BF16 (bf16 as 16-bit patterns);
+ *   - `stream` is a hipStream_t (NULL = the null stream);
+ *   - the return value is a host-side code (ZEN_OK, ZEN_E...); conditions only
+ *     the device can see are OR-ed into `*status` (device int32, written by
+ *     kernels with atomic-or; the caller zeroes it and reads it after a sync);
+ *   - `workspace` is caller-provided scratch of at least the size the matching
+ *     `*_workspace` function returns; contents are undefined on return;
+ *   - indices are int32 (N < 2^31) as in the reference (functions_cuda.cpp:25-26
+ *     narrows numel() to int).
+ *
+ * Citations are file:line in the reference (Jabir0/ZEN_repro).
+ */
+#ifndef ZEN_HIP_H
+#define ZEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ZEN_ABI_VERSION 1
+
+#define ZEN_F32 0
+#define ZEN_BF16 1
+
+/* host return codes */
+#define ZEN_OK 0
+#define ZEN_EINVAL (-1)     /* bad argument (null, size, dtype, alignment) */
+#define ZEN_EHIP (-2)       /* a HIP runtime call failed, see zen_last_error() */
+#define ZEN_EWORKSPACE (-3) /* workspace too small */
+
+/* device status bits */
+#define ZEN_STAT_SERIAL_OVERFLOW 1 /* a partition had more overflow entries than serial slots */
+#define ZEN_STAT_CAPACITY 2        /* more output entries than `capacity`; the excess was dropped */
+#define ZEN_STAT_INTERNAL 4        /* a bounded in-kernel wait expired; outputs are invalid */
+#define ZEN_STAT_BAD_INDEX 8       /* merge/decode saw an index outside [0, dense_n); it was skipped */
+
+int zen_abi_version(void);
+
+/* host string describing the last ZEN_EHIP / ZEN_EINVAL on this thread */
+const char *zen_last_error(void);
+
+/* ------------------------------------------------------------------ hash */
+
+/*
+ * out[t] = (h1(t) % n) / (n / partitions) for t in [0, n).
+ * Replaces hash_index (extensions/cuda/functions_cuda.cpp:30-36) and
+ * hash_index_cuda (functions_cuda_kernel.cu:169-177, 201-205).
+ * n % partitions != 0 is allowed and can yield `partitions` as in the
+ * reference; n < partitions is ZEN_EINVAL (the reference divides by zero).
+ */
+int zen_hash_index(int32_t *out, int64_t n, int partitions, void *stream);
+
+/*
+ * Ascending list of t in [0,n) per partition, concatenated into out[n]
+ * (int64), counts[p] = length of list p.  Replaces calculate_mapping
+ * (comm.py:52-56).  Indices whose partition id equals `partitions`
+ * (n % partitions != 0) are left out, as in the reference.
+ */
+size_t zen_mapping_workspace(int64_t n, int partitions);
+int zen_mapping(int64_t n, int partitions, int64_t *out, int64_t *counts,
+                void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------- insert */
+
+/*
+ * In-place hash-table insert of every nonzero index of `input`.
+ * Replaces sparse_balance (functions_cuda.cpp:15-28) and sparse_balance_cuda
+ * with its three kernels (functions_cuda_kernel.cu:97-167, 180-199).
+ * memory[m] and serial[serial_n] must be zero on entry; offset[partitions]
+ * must hold the serial base offsets (extensions/cuda/functions.py:8-11) and
+ * ends as base + number of tickets.  The result is the one the reference
+ * kernel gives when its threads run in ascending order: a slot belongs to
+ * the smallest index that probes it, serial entries are ascending per
+ * partition.  Tickets beyond a partition's serial region are dropped and
+ * flagged (ZEN_STAT_SERIAL_OVERFLOW) instead of written out of bounds.
+ * m % partitions != 0 is ZEN_EINVAL.
+ */
+int zen_sparse_balance(const void *input, int dtype, int64_t n,
+                       int32_t *memory, int64_t m,
+                       int32_t *serial, int64_t serial_n,
+                       int32_t *offset, int partitions, int rehash,
+                       int32_t *status, void *stream);
+
+/* ---------------------------------------------------------------- select */
+
+/*
+ * thr[0] = magnitude key (bit pattern with the sign cleared) of the k-th
+ * largest |input|, thr[1] = number of elements whose key >= thr[0].
+ * Replaces topk(...)[0].min() in compress (train.py:81-82) with the whole
+ * tensor (or a caller-gathered sample) as the multiset.  1 <= k <= n.
+ */
+size_t zen_topk_threshold_workspace(void);
+int zen_topk_threshold(const void *input, int dtype, int64_t n, int64_t k,
+                       uint32_t *thr, void *workspace, size_t workspace_bytes,
+                       void *stream);
+
+/*
+ * out[i] = key(input[i]) >= thr[0] ? input[i] : 0.  Replaces
+ * torch.where(tensor_abs >= threshold, tensor, 0) (train.py:83).
+ */
+int zen_compress(const void *input, int dtype, int64_t n, const uint32_t *thr,
+                 void *out, void *stream);
+
+/*
+ * Ordered compaction: ascending indices i with key(i) >= max(thr[0], 1) and
+ * their values.  thr == NULL selects the nonzero elements, which is
+ * encode_sparse_tensor (comm.py:47-50).  out_idx is int64 when idx64 != 0,
+ * else int32.  *out_count (int64) receives the number found, which may
+ * exceed `capacity` (then ZEN_STAT_CAPACITY is set and the excess dropped).
+ */
+size_t zen_select_workspace(int64_t n, int dtype);
+int zen_select(const void *input, int dtype, int64_t n, const uint32_t *thr,
+               void *out_idx, int idx64, void *out_val, int64_t capacity,
+               int64_t *out_count, void *workspace, size_t workspace_bytes,
+               int32_t *status, void *stream);
+
+/* ---------------------------------------------------------- load balance */
+
+/*
+ * Fused select + insert + slot-order compaction.  Replaces
+ * TensorPartition.load_balance (tensor_load_balance.py:13-51) and, with
+ * thr != NULL, the masked copy of compress (train.py:83) in front of it.
+ * Output: out_idx / out_val hold partition 0's entries, then partition 1's,
+ * ...; inside a partition, table entries in ascending slot order followed by
+ * that partition's serial entries in ascending index order; splits[p] (int64)
+ * is partition p's length.  m is the table size of
+ * tensor_load_balance.py:15-16; the serial capacity is n / partitions / 10
+ * per partition (tensor_load_balance.py:18).
+ * `table` is int32[m] scratch that must be all zero on entry and is all zero
+ * again on return (so one allocation serves every call).
+ */
+size_t zen_load_balance_workspace(int64_t n, int dtype, int64_t capacity, int partitions);
+int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m,
+                     int partitions, int rehash, const uint32_t *thr,
+                     int32_t *out_idx, void *out_val, int64_t capacity,
+                     int64_t *splits, int32_t *table,
+                     void *workspace, size_t workspace_bytes,
+                     int32_t *status, void *stream);
+
+/* ----------------------------------------------------------------- merge */
+
+/*
+ * Merge r received (index, value) entries: sum values of equal indices in
+ * fp32, in the order the entries appear, drop sums equal to zero, return the
+ * rest in ascending index order.  Replaces decode_sparse_tensors +
+ * encode_sparse_tensor of the first exchange (comm.py:32-50, 125-127) without
+ * the dense intermediate.  idx is int32 (idx64_in == 0) or int64.  out_idx is
+ * int64 when idx64_out != 0.  out_val is fp32.  *out_count is int64.
+ */
+size_t zen_merge_workspace(int64_t r);
+int zen_merge(const void *idx, int idx64_in, const void *val, int dtype,
+              int64_t r, int64_t dense_n,
+              void *out_idx, int idx64_out, float *out_val, int64_t capacity,
+              int64_t *out_count, void *workspace, size_t workspace_bytes,
+              int32_t *status, void *stream);
+
+/*
+ * dense[0..dense_n) = 0, then dense[idx[j]] += val[j] with fp32 accumulation
+ * in entry order, rounded once to `dtype`.  Replaces decode_sparse_tensors
+ * (comm.py:32-44), whose result is a dense tensor in the value dtype.
+ */
+size_t zen_decode_dense_workspace(int64_t r);
+int zen_decode_dense(const void *idx, int idx64_in, const void *val, int dtype,
+                     int64_t r, void *dense, int64_t dense_n,
+                     void *workspace, size_t workspace_bytes,
+                     int32_t *status, void *stream);
+
+/* --------------------------------------------------------------- utility */
+
+/*
+ * Stable ascending sort of (key, value) pairs on the low `bits` bits of the
+ * key; count is read from *count_dev if that is not NULL, else `count`.
+ * No counterpart in the reference (torch ops sort internally); exposed
+ * because both fused paths are built on it and tests exercise it directly.
+ * keys/vals are sorted in place.
+ */
+size_t zen_sort_pairs_workspace(int64_t max_count);
+int zen_sort_pairs(uint32_t *keys, uint32_t *vals, int64_t max_count,
+                   const uint32_t *count_dev, int bits,
+                   void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Per-kernel timing with HIP events recorded on the launch stream, for
+ * benchmarks.  The reference's counterpart is its nvtx ranges
+ * (tensor_load_balance.py:25-38, comm.py:66-144).  zen_profile_enable(1)
+ * clears earlier samples and starts recording; zen_profile_read synchronises
+ * on the recorded events of one tag and returns their summed duration and the
+ * number of launches.  Process-wide, serialised by a mutex.
+ */
+int zen_profile_enable(int on);
+int zen_profile_tags(void);
+const char *zen_profile_name(int tag);
+int zen_profile_read(int tag, double *total_ms, int64_t *launches);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

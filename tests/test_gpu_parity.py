@@ -1,0 +1,421 @@
+"""Parity of the HIP library against the CPU oracle on seeded inputs.  Every
+test goes through libzen_hip.so's C ABI (directly or via the package's thin
+wrappers).  Bar: bit-exact for indices, slots, order and bit-copied values;
+merged sums bit-exact against the fp32 sequential oracle (same order of adds)
+and within 1e-6 relative of the fp64 truth."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import make_grad, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def zen():
+    import zen_repro_amd
+    from zen_repro_amd import _lib
+
+    _lib.lib()
+    assert torch.cuda.is_available()
+    return zen_repro_amd
+
+
+# ------------------------------------------------------------------ sort
+
+
+@pytest.mark.parametrize("count", [1, 63, 64, 65, 1000, 4095, 4096, 4097, 70001, 1 << 20])
+@pytest.mark.parametrize("bits", [1, 8, 9, 17, 30, 32])
+def test_sort_pairs_is_stable_sort(zen, count, bits):
+    from zen_repro_amd import _lib
+
+    rng = np.random.default_rng(count * 131 + bits)
+    hi = (1 << bits) - 1
+    # few distinct keys on purpose: stability must show
+    keys = rng.integers(0, min(hi, 500) + 1, count, dtype=np.uint64).astype(np.uint32)
+    if bits >= 9:
+        keys = (keys * np.uint32(max(1, hi // 501))).astype(np.uint32)
+    vals = np.arange(count, dtype=np.uint32)
+    dk = to_dev(keys.view(np.int32))
+    dv = to_dev(vals.view(np.int32))
+    L = _lib.lib()
+    ws = torch.empty(L.zen_sort_pairs_workspace(count), dtype=torch.uint8, device="cuda")
+    rc = L.zen_sort_pairs(_lib.ptr(dk), _lib.ptr(dv), count, None, bits, _lib.ptr(ws), ws.numel(),
+                          _lib.stream_of(dk.device))
+    assert rc == 0
+    order = np.argsort(keys, kind="stable")
+    assert np.array_equal(to_np(dk).view(np.uint32), keys[order])
+    assert np.array_equal(to_np(dv).view(np.uint32), vals[order])
+
+
+def test_sort_pairs_device_count(zen):
+    from zen_repro_amd import _lib
+
+    cap, live = 50000, 12345
+    rng = np.random.default_rng(9)
+    keys = rng.integers(0, 1 << 20, cap, dtype=np.uint64).astype(np.uint32)
+    vals = np.arange(cap, dtype=np.uint32)
+    dk, dv = to_dev(keys.view(np.int32)), to_dev(vals.view(np.int32))
+    cnt = torch.tensor([live], dtype=torch.int32, device="cuda")
+    L = _lib.lib()
+    ws = torch.empty(L.zen_sort_pairs_workspace(cap), dtype=torch.uint8, device="cuda")
+    assert L.zen_sort_pairs(_lib.ptr(dk), _lib.ptr(dv), cap, _lib.ptr(cnt), 20, _lib.ptr(ws), ws.numel(),
+                            _lib.stream_of(dk.device)) == 0
+    order = np.argsort(keys[:live], kind="stable")
+    assert np.array_equal(to_np(dk).view(np.uint32)[:live], keys[:live][order])
+    assert np.array_equal(to_np(dv).view(np.uint32)[:live], vals[:live][order])
+    assert np.array_equal(to_np(dk).view(np.uint32)[live:], keys[live:])  # tail untouched
+
+
+# ------------------------------------------------------------------ hash
+
+
+@pytest.mark.parametrize("n,P", [(1 << 20, 4), (1003, 4), (38597376 // 16, 16), (999983, 7), (64, 64)])
+def test_hash_index(zen, oracle, n, P):
+    idx = torch.full((n,), -7, dtype=torch.int32, device="cuda")
+    zen.hash_index(idx, P)
+    assert np.array_equal(to_np(idx), oracle.hash_index(n, P))
+
+
+def test_hash_index_rejects(zen):
+    with pytest.raises(ValueError):
+        zen.hash_index(torch.zeros(3, dtype=torch.int32, device="cuda"), 4)
+    with pytest.raises(AssertionError):
+        zen.hash_index(torch.zeros(8, dtype=torch.int64, device="cuda"), 4)
+
+
+@pytest.mark.parametrize("n,P", [(1 << 16, 8), (1003, 4), (300000, 16)])
+def test_calculate_mapping(zen, oracle, n, P):
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P), None, None)
+    got = lba.calculate_mapping(n)
+    want = oracle.mapping(n, P)
+    assert len(got) == P
+    for g, w in zip(got, want):
+        assert g.dtype == torch.int64 and np.array_equal(to_np(g), w)
+
+
+# ---------------------------------------------------------------- insert
+
+INSERT_CASES = [
+    (4096, 4, 0.01, 1), (4096, 4, 0.3, 1), (1 << 16, 16, 0.05, 1), (1 << 16, 8, 0.5, 1),
+    (100000, 5, 0.2, 1), (1 << 18, 32, 0.01, 1), (60000, 6, 0.35, 2), (50000, 4, 0.25, 1.5),
+    (1000000, 4, 0.4, 1),  # rehash 1: > 8192 serial entries per partition (sorted in global memory)
+]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("rehash", [1, 2, 3])
+@pytest.mark.parametrize("n,P,density,scale", INSERT_CASES)
+def test_sparse_balance_tables_byte_identical(zen, oracle, n, P, density, scale, rehash, dtype):
+    g = make_grad(oracle, n, density, dtype, seed=n + P)
+    g[0] = g[g != 0][0] if (g != 0).any() else 1  # index 0 nonzero: must never be stored
+    m, sn = oracle.table_sizes(n, P, scale)
+    mem_o, ser_o, off_o, st_o = oracle.sparse_balance(g, m, sn, P, rehash)
+    d = to_dev(g)
+    mem = torch.zeros(m, dtype=torch.int32, device="cuda")
+    ser = torch.zeros(sn, dtype=torch.int32, device="cuda")
+    pending = zen.sparse_balance(d, mem, ser, P, rehash)
+    assert np.array_equal(to_np(pending.offsets), off_o)
+    assert int(pending.status.item()) == st_o
+    assert np.array_equal(to_np(mem), mem_o)
+    if st_o == 0:
+        assert np.array_equal(to_np(ser), ser_o)
+
+
+def test_sparse_balance_overflow_is_flagged_not_oob(zen, oracle):
+    n, P = 40000, 4
+    g = np.ones(n, np.float32)
+    m, sn = oracle.table_sizes(n, P)
+    mem_o, _, off_o, st_o = oracle.sparse_balance(g, m, sn, P, 1)
+    assert st_o == oracle.SERIAL_OVERFLOW
+    mem = torch.zeros(m, dtype=torch.int32, device="cuda")
+    ser = torch.zeros(sn + 64, dtype=torch.int32, device="cuda")  # guard zone behind the table
+    pending = zen.sparse_balance(to_dev(g), mem, ser[:sn], P, 1)
+    assert int(pending.status.item()) & 1
+    with pytest.raises(RuntimeError):
+        pending.check()
+    assert np.array_equal(to_np(mem), mem_o)
+    assert np.array_equal(to_np(pending.offsets), off_o)
+    assert not to_np(ser)[sn:].any()
+
+
+def test_sparse_balance_argument_errors(zen):
+    g = torch.zeros(64, dtype=torch.bfloat16, device="cuda")
+    mem = torch.zeros(64, dtype=torch.int32, device="cuda")
+    ser = torch.zeros(4, dtype=torch.int32, device="cuda")
+    with pytest.raises(AssertionError):
+        zen.sparse_balance(g.cpu(), mem, ser, 4, 3)
+    with pytest.raises(AssertionError):
+        zen.sparse_balance(g.half(), mem, ser, 4, 3)
+    with pytest.raises(AssertionError):
+        zen.sparse_balance(g, mem.long(), ser, 4, 3)
+    with pytest.raises(RuntimeError):
+        zen.sparse_balance(g[::2], mem, ser, 4, 3)
+    with pytest.raises(ValueError):
+        zen.sparse_balance(g, mem[:62], ser, 4, 3)  # table not a multiple of P
+
+
+def test_reference_style_compaction_over_tables(zen, oracle):
+    # balance_sparse_tensor + get_sub_sparse_tensors, the reference's two-step route
+    n, P = 100000, 5
+    g = make_grad(oracle, n, 0.2, "bf16", seed=77)
+    tp = zen.TensorPartition(P, 1, 3)
+    d = to_dev(g)
+    mem, ser = tp.balance_sparse_tensor(d)
+    i1, v1, s1 = tp.get_sub_sparse_tensors(d, mem)
+    i2, v2, s2 = tp.get_sub_sparse_tensors(d, ser)
+    idx_o, val_o, splits_o, st = oracle.load_balance(g, P, 1, 3)
+    assert st == 0 and s2.sum().item() > 0  # the serial region is in use at this density
+    got_i = np.concatenate([np.concatenate([to_np(a), to_np(b)]) for a, b in zip(i1, i2)])
+    got_v = np.concatenate([np.concatenate([to_np(a), to_np(b)]) for a, b in zip(v1, v2)])
+    assert np.array_equal(got_i, idx_o) and np.array_equal(got_v, val_o)
+    assert np.array_equal(to_np(s1 + s2), splits_o)
+
+
+# ---------------------------------------------------------------- select
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("n", [5000, 1 << 16, 1 << 20, 3 * (1 << 20) + 17])
+def test_topk_threshold(zen, oracle, n, dtype):
+    g = make_grad(oracle, n, 1.0, dtype, seed=n)
+    d = to_dev(g)
+    for k in (1, 2, n // 200, n // 100, n // 3, n):
+        thr = zen.topk_threshold(d, k)
+        key, count = (int(x) & 0xFFFFFFFF for x in to_np(thr))
+        assert key == oracle.kth_key(g, k), (n, dtype, k)
+        keys = (g & 0x7FFF) if dtype == "bf16" else (g.view(np.uint32) & 0x7FFFFFFF)
+        assert count == int((keys >= key).sum())
+
+
+def test_topk_threshold_heavy_ties_and_zeros(zen, oracle):
+    n = 1 << 18
+    g = np.zeros(n, np.float32)
+    g[::7] = 0.5
+    g[::11] = -0.5
+    g[5::13] = 2.0
+    d = to_dev(g)
+    for k in (1, 1000, int((g != 0).sum()), n):
+        thr = zen.topk_threshold(d, k)
+        assert int(to_np(thr)[0]) == oracle.kth_key(g, k)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_compress_masked_copy(zen, oracle, dtype):
+    import importlib
+
+    C = importlib.import_module("zen_repro_amd.compress")
+
+    n = (1 << 18) + 5
+    g = make_grad(oracle, n, 1.0, dtype, seed=5)
+    d = to_dev(g)
+    k = n // 100
+    thr = C.topk_threshold(d, k)
+    want, kept = oracle.mask_dense(g, oracle.kth_key(g, k))
+    assert np.array_equal(to_np(C.mask_below(d, thr)), want)
+    # unaligned views take the scalar path
+    got = C.mask_below(d[1:], C.topk_threshold(d[1:], k))
+    want1, _ = oracle.mask_dense(g[1:], oracle.kth_key(g[1:], k))
+    assert np.array_equal(to_np(got), want1)
+    # the reference-shaped entry: caller-supplied sample positions
+    rng = np.random.default_rng(1)
+    sample = rng.integers(0, n, -(-n // 100))
+    out = zen.compress(5, d, torch.from_numpy(sample).cuda())
+    ks = len(sample) * 5 // 100
+    want2, _ = oracle.mask_dense(g, oracle.kth_key(g[sample], ks))
+    assert np.array_equal(to_np(out), want2)
+    small = d[:4096]
+    assert zen.compress(1, small) is small  # train.py:77-78
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("n,density", [(1, 1.0), (100, 0.5), (8192, 0.0), (8193, 1.0), (1 << 20, 0.01),
+                                       (5 * (1 << 20) + 3, 0.3)])
+def test_encode_sparse_tensor(zen, oracle, n, density, dtype):
+    g = make_grad(oracle, n, density, dtype, seed=n * 3 + 1)
+    if n > 4:
+        g[3] = 0x8000 if dtype == "bf16" else -0.0  # negative zero is a zero
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(4), None, None)
+    idx, val = lba.encode_sparse_tensor(to_dev(g))
+    idx_o, val_o = oracle.encode(g)
+    assert idx.dtype == torch.int64
+    assert np.array_equal(to_np(idx), idx_o) and np.array_equal(to_np(val), val_o)
+    if n > 64:
+        off = to_dev(g)[3:]
+        i2, v2 = lba.encode_sparse_tensor(off)
+        io, vo = oracle.encode(g[3:])
+        assert np.array_equal(to_np(i2), io) and np.array_equal(to_np(v2), vo)
+
+
+def test_select_capacity_flag(zen, oracle):
+    from zen_repro_amd import _lib
+
+    n = 100000
+    g = make_grad(oracle, n, 0.5, "f32", seed=2)
+    d = to_dev(g)
+    L = _lib.lib()
+    cap = 1000
+    oi = torch.full((cap + 16,), -1, dtype=torch.int32, device="cuda")
+    ov = torch.zeros(cap + 16, dtype=torch.float32, device="cuda")
+    cnt = torch.zeros(1, dtype=torch.int64, device="cuda")
+    st = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ws = torch.empty(L.zen_select_workspace(n, 0), dtype=torch.uint8, device="cuda")
+    assert L.zen_select(_lib.ptr(d), 0, n, None, _lib.ptr(oi), 0, _lib.ptr(ov), cap, _lib.ptr(cnt),
+                        _lib.ptr(ws), ws.numel(), _lib.ptr(st), _lib.stream_of(d.device)) == 0
+    io, _ = oracle.encode(g)
+    assert cnt.item() == len(io) and st.item() == _lib.STAT_CAPACITY
+    assert np.array_equal(to_np(oi)[:cap], io[:cap].astype(np.int32))
+    assert (to_np(oi)[cap:] == -1).all()
+
+
+# ---------------------------------------------------------- load balance
+
+LB_CASES = [
+    (8192, 4, 0.01, 1, 3), (1 << 16, 16, 0.005, 1, 3), (1 << 16, 8, 0.3, 1, 3), (1 << 18, 32, 0.05, 1, 2),
+    (100000, 5, 0.4, 1, 1), (1 << 20, 16, 0.01, 1, 3), (60000, 6, 0.2, 2, 3), (50000, 4, 0.25, 1.5, 3),
+    (1 << 20, 64, 0.001, 1, 3),
+]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("n,P,density,scale,rehash", LB_CASES)
+def test_load_balance_bit_exact(zen, oracle, n, P, density, scale, rehash, dtype):
+    g = make_grad(oracle, n, density, dtype, seed=n ^ P)
+    g[0] = 0x3F80 if dtype == "bf16" else 1.0
+    idx_o, val_o, splits_o, st_o = oracle.load_balance(g, P, scale, rehash)
+    tp = zen.TensorPartition(P, scale, rehash)
+    d = to_dev(g)
+    for rep in range(2):  # the second call reuses the (re-zeroed) owner table
+        if st_o:
+            with pytest.raises(RuntimeError):
+                tp.load_balance(d)
+            continue
+        indices, values, splits = tp.load_balance(d)
+        assert np.array_equal(to_np(splits), splits_o)
+        assert np.array_equal(np.concatenate([to_np(i) for i in indices]), idx_o)
+        assert np.array_equal(np.concatenate([to_np(v) for v in values]), val_o)
+        assert indices[0].dtype == torch.int32 and values[0].dtype == d.dtype
+    m, _ = oracle.table_sizes(n, P, scale)
+    assert not tp._table(d.device, m).any()  # left empty for the next call
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_topk_then_load_balance(zen, oracle, dtype):
+    n, P = 1 << 20, 16
+    g = make_grad(oracle, n, 1.0, dtype, seed=123)
+    k = n // 200
+    key = oracle.kth_key(g, k)
+    masked, kept = oracle.mask_dense(g, key)
+    idx_o, val_o, splits_o, st_o = oracle.load_balance(masked, P, 1, 3)
+    d = to_dev(g)
+    thr = zen.topk_threshold(d, k)
+    tp = zen.TensorPartition(P, 1, 3)
+    indices, values, splits = tp.load_balance(d, thr=thr, capacity=2 * k + 1024)
+    assert st_o == 0
+    assert np.array_equal(to_np(splits), splits_o)
+    assert np.array_equal(np.concatenate([to_np(i) for i in indices]), idx_o)
+    assert np.array_equal(np.concatenate([to_np(v) for v in values]), val_o)
+    part = oracle.hash_index(n, P)
+    for p, i in enumerate(indices):
+        assert (part[to_np(i)] == p).all()
+
+
+def test_load_balance_capacity_flag(zen, oracle):
+    n, P = 1 << 16, 4
+    g = make_grad(oracle, n, 0.5, "f32", seed=4)
+    tp = zen.TensorPartition(P, 1, 3)
+    with pytest.raises(RuntimeError, match="capacity"):
+        tp.load_balance(to_dev(g), capacity=100)
+
+
+# ----------------------------------------------------------------- merge
+
+
+def make_payloads(oracle, rng, n, peers, per_peer, overlap, dtype):
+    pool = rng.choice(n, max(1, int(per_peer * overlap)), replace=False)
+    idx, val = [], []
+    for _ in range(peers):
+        shared = rng.choice(pool, int(per_peer * overlap), replace=False) if overlap > 0 else np.empty(0, np.int64)
+        own = rng.integers(0, n, per_peer - len(shared))
+        i = np.concatenate([shared, own]).astype(np.int32)
+        rng.shuffle(i)
+        v = (rng.standard_normal(len(i)) * 1e-3).astype(np.float32)
+        idx.append(i)
+        val.append(oracle.f32_to_bf16_bits(v) if dtype == "bf16" else v)
+    return idx, val
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("n,peers,per_peer,overlap", [(1000, 4, 50, 0.2), (1 << 20, 16, 5000, 0.3),
+                                                      (1 << 22, 64, 3000, 0.4), (4096, 8, 4096, 0.9),
+                                                      (1 << 16, 1, 1, 0.0)])
+def test_merge_sparse(zen, oracle, n, peers, per_peer, overlap, dtype):
+    rng = np.random.default_rng(n + peers)
+    idx, val = make_payloads(oracle, rng, n, peers, per_peer, overlap, dtype)
+    ci, cv = np.concatenate(idx), np.concatenate(val)
+    want_i, want_v = oracle.merge_sparse(ci, cv, n)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(peers), None, None)
+    gi, gv = lba.merge_sparse([to_dev(i) for i in idx], [to_dev(v) for v in val], n)
+    assert gi.dtype == torch.int64 and gv.dtype == torch.float32
+    assert np.array_equal(to_np(gi), want_i)
+    # same adds in the same order: bit-exact against the sequential fp32 oracle
+    assert np.array_equal(to_np(gv).view(np.uint32), want_v.view(np.uint32))
+    # and within 1e-6 (relative to the summed magnitudes) of the fp64 truth
+    truth = oracle.decode(ci, cv, n, "f64")[want_i]
+    vf = oracle.bf16_bits_to_f32(cv) if dtype == "bf16" else cv
+    scale = np.zeros(n)
+    np.add.at(scale, ci, np.abs(vf.astype(np.float64)))
+    assert (np.abs(to_np(gv) - truth) <= 1e-6 * scale[want_i] + 1e-30).all()
+
+
+def test_merge_cancellation_nan_and_bad_index(zen, oracle):
+    from zen_repro_amd import _lib
+
+    n = 64
+    idx = np.array([5, 9, 5, 63, 9, 0, 0, 17], np.int32)
+    val = np.array([1.0, 2.0, -1.0, 4.0, np.nan, 3.0, -3.0, -0.0], np.float32)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(2), None, None)
+    gi, gv = lba.merge_sparse(to_dev(idx), to_dev(val), n)
+    wi, wv = oracle.merge_sparse(idx, val, n)
+    assert to_np(gi).tolist() == wi.tolist() == [9, 63]
+    assert np.array_equal(to_np(gv).view(np.uint32) & 0x7FC00000, wv.view(np.uint32) & 0x7FC00000)
+    bad = np.array([5, 64, -1, 7], np.int64)
+    i2, v2, cnt, st = lba.merge_sparse_flat(to_dev(bad), to_dev(np.ones(4, np.float32)), n, idx64=True)
+    assert cnt.item() == 2 and st.item() == _lib.STAT_BAD_INDEX
+    assert to_np(i2)[:2].tolist() == [5, 7]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_decode_sparse_tensors_dense(zen, oracle, dtype):
+    rng = np.random.default_rng(8)
+    n, peers = 1 << 18, 8
+    idx, val = make_payloads(oracle, rng, n, peers, 4000, 0.3, dtype)
+    ci, cv = np.concatenate(idx), np.concatenate(val)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(peers), None, None)
+    dense = lba.decode_sparse_tensors([to_dev(i) for i in idx], [to_dev(v) for v in val], n)
+    f32 = oracle.decode(ci, cv, n, "f32acc")
+    want = oracle.f32_to_bf16_bits(f32) if dtype == "bf16" else f32
+    got = to_np(dense)
+    assert dense.dtype == (torch.bfloat16 if dtype == "bf16" else torch.float32)
+    assert np.array_equal(got, want)
+    # single-tensor form with int64 indices (comm.py:40-44)
+    d2 = lba.decode_sparse_tensors(to_dev(ci.astype(np.int64)), to_dev(cv), n)
+    assert np.array_equal(to_np(d2), want)
+    if dtype == "bf16":
+        # against the reference's own accumulation dtype: 1e-3 relative
+        native = oracle.bf16_bits_to_f32(oracle.decode(ci, cv, n, "native"))
+        scale = np.zeros(n)
+        np.add.at(scale, ci, np.abs(oracle.bf16_bits_to_f32(cv).astype(np.float64)))
+        assert (np.abs(oracle.bf16_bits_to_f32(got) - native) <= 2e-2 * scale + 1e-30).all()
+
+
+def test_stack_tensors_views_are_not_copied(zen):
+    buf = torch.arange(100, device="cuda", dtype=torch.int32)
+    parts = [buf[0:10], buf[10:45], buf[45:100]]
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(3), None, None)
+    assert lba.stack_tensors(parts).data_ptr() == buf.data_ptr()
+    other = [buf[0:10], buf[20:30]]
+    assert lba.stack_tensors(other).tolist() == list(range(10)) + list(range(20, 30))

@@ -1,0 +1,159 @@
+"""Loader of libzen_hip.so (the C-ABI of include/zen_hip.h) and the small
+amount of torch plumbing every wrapper shares: dtype codes, stream handles,
+cached workspaces and status words.  There is no fallback: if the library is
+missing or a call fails, an exception is raised."""
+import ctypes
+import os
+
+import torch  # first: makes the process use torch's HIP runtime for libzen_hip too
+
+F32, BF16 = 0, 1
+OK, EINVAL, EHIP, EWORKSPACE = 0, -1, -2, -3
+STAT_SERIAL_OVERFLOW, STAT_CAPACITY, STAT_INTERNAL, STAT_BAD_INDEX = 1, 2, 4, 8
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libzen_hip.so")
+
+_lib = None
+
+
+def build():
+    """Compile libzen_hip.so for gfx950 with hipcc (cross-compiles without a GPU)."""
+    import subprocess
+
+    subprocess.check_call(["make", "-C", os.path.join(_HERE, "csrc"), "-B", "-j8", "all"],
+                          stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    return LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `make -C zen_repro_amd/csrc` "
+            "(or __graft_entry__.build()); there is no fallback path")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, i32, i64, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
+    sig = {
+        "zen_abi_version": (i32, []),
+        "zen_last_error": (ctypes.c_char_p, []),
+        "zen_hash_index": (i32, [vp, i64, i32, vp]),
+        "zen_mapping_workspace": (sz, [i64, i32]),
+        "zen_mapping": (i32, [i64, i32, vp, vp, vp, sz, vp]),
+        "zen_sparse_balance": (i32, [vp, i32, i64, vp, i64, vp, i64, vp, i32, i32, vp, vp]),
+        "zen_topk_threshold_workspace": (sz, []),
+        "zen_topk_threshold": (i32, [vp, i32, i64, i64, vp, vp, sz, vp]),
+        "zen_compress": (i32, [vp, i32, i64, vp, vp, vp]),
+        "zen_select_workspace": (sz, [i64, i32]),
+        "zen_select": (i32, [vp, i32, i64, vp, vp, i32, vp, i64, vp, vp, sz, vp, vp]),
+        "zen_load_balance_workspace": (sz, [i64, i32, i64, i32]),
+        "zen_load_balance": (i32, [vp, i32, i64, i64, i32, i32, vp, vp, vp, i64, vp, vp, vp, sz, vp, vp]),
+        "zen_merge_workspace": (sz, [i64]),
+        "zen_merge": (i32, [vp, i32, vp, i32, i64, i64, vp, i32, vp, i64, vp, vp, sz, vp, vp]),
+        "zen_decode_dense_workspace": (sz, [i64]),
+        "zen_decode_dense": (i32, [vp, i32, vp, i32, i64, vp, i64, vp, sz, vp, vp]),
+        "zen_sort_pairs_workspace": (sz, [i64]),
+        "zen_sort_pairs": (i32, [vp, vp, i64, vp, i32, vp, sz, vp]),
+        "zen_profile_enable": (i32, [i32]),
+        "zen_profile_tags": (i32, []),
+        "zen_profile_name": (ctypes.c_char_p, [i32]),
+        "zen_profile_read": (i32, [i32, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype, fn.argtypes = res, args
+    if L.zen_abi_version() != 1:
+        raise RuntimeError("libzen_hip.so: unexpected ABI version")
+    _lib = L
+    return L
+
+
+def check(code, what):
+    if code == OK:
+        return
+    msg = lib().zen_last_error().decode(errors="replace")
+    if code == EINVAL:
+        raise ValueError(f"{what}: {msg}")
+    raise RuntimeError(f"{what} failed ({code}): {msg}")
+
+
+def dtype_code(t):
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise AssertionError(f"gradient dtype must be bfloat16 or float32, got {t.dtype}")
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def stream_of(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def require_gpu(t, name):
+    # extensions/cuda/functions.py:5-7 asserts; functions_cuda.cpp:11-13 raises RuntimeError
+    assert t.is_cuda, f"{name} must be a GPU tensor"
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+class Scratch:
+    """Per-device cache of raw byte buffers, grown on demand and reused.  A
+    buffer is tied to the stream order of its users, like any torch tensor."""
+
+    def __init__(self):
+        self._bufs = {}
+
+    def get(self, device, name, nbytes, zero=False):
+        key = (torch.device(device).index if torch.device(device).index is not None
+               else torch.cuda.current_device(), name)
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < nbytes:
+            alloc = torch.zeros if zero else torch.empty
+            buf = alloc(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+            self._bufs[key] = buf
+        return buf
+
+    def drop(self):
+        self._bufs.clear()
+
+
+scratch = Scratch()
+
+
+def status_word(device):
+    return torch.zeros(1, dtype=torch.int32, device=device)
+
+
+def describe_status(bits):
+    names = []
+    if bits & STAT_SERIAL_OVERFLOW:
+        names.append("serial region overflow")
+    if bits & STAT_CAPACITY:
+        names.append("output capacity exceeded")
+    if bits & STAT_INTERNAL:
+        names.append("internal wait expired")
+    if bits & STAT_BAD_INDEX:
+        names.append("index out of range")
+    return ", ".join(names) or "ok"
+
+
+def profile_enable(on=True):
+    check(lib().zen_profile_enable(1 if on else 0), "profile_enable")
+
+
+def profile_read():
+    """{kernel name: (total ms, launches)} for every tag that recorded a launch."""
+    L = lib()
+    out = {}
+    for tag in range(L.zen_profile_tags()):
+        ms, cnt = ctypes.c_double(0), ctypes.c_int64(0)
+        check(L.zen_profile_read(tag, ctypes.byref(ms), ctypes.byref(cnt)), "profile_read")
+        if cnt.value:
+            out[L.zen_profile_name(tag).decode()] = (ms.value, cnt.value)
+    return out

@@ -1,0 +1,175 @@
+"""Drop-in for the encode / decode / mapping half of the reference's comm.py
+(LoadBalanceAllreduce).  The collectives around it are not part of this
+package: one GPU computes its own share, the full P-way partition of its
+gradient and the merge of P incoming payloads."""
+import torch
+
+from . import _lib
+from .functions import hash_index
+from .tensor_load_balance import TensorPartition
+
+
+class LocalGroup:
+    """Stands in for a torch.distributed process group when there is none: it
+    only answers size() and rank(), which is all this path asks of a group."""
+
+    def __init__(self, size, rank=0):
+        self._size, self._rank = size, rank
+
+    def size(self):
+        return self._size
+
+    def rank(self):
+        return self._rank
+
+
+def _select(tensor, thr, idx64, capacity=None):
+    """Ascending (indices, values, count) of the selected elements of a flat
+    tensor; count is a device int64[1] and may exceed capacity."""
+    flat = tensor.reshape(-1)
+    n = flat.numel()
+    dev = flat.device
+    if capacity is None:
+        capacity = n
+    L = _lib.lib()
+    code = _lib.dtype_code(flat)
+    out_idx = torch.empty(capacity, dtype=torch.int64 if idx64 else torch.int32, device=dev)
+    out_val = torch.empty(capacity, dtype=flat.dtype, device=dev)
+    count = torch.zeros(1, dtype=torch.int64, device=dev)
+    status = _lib.status_word(dev)
+    ws = _lib.scratch.get(dev, "select", L.zen_select_workspace(n, code))
+    rc = L.zen_select(_lib.ptr(flat), code, n, _lib.ptr(thr), _lib.ptr(out_idx), 1 if idx64 else 0,
+                      _lib.ptr(out_val), capacity, _lib.ptr(count), _lib.ptr(ws), ws.numel(),
+                      _lib.ptr(status), _lib.stream_of(dev))
+    _lib.check(rc, "select")
+    host = torch.cat([count, status.to(torch.int64)]).tolist()
+    if host[1]:
+        raise RuntimeError("select: " + _lib.describe_status(host[1]))
+    return out_idx[:host[0]], out_val[:host[0]], host[0]
+
+
+class LoadBalanceAllreduce:
+    """Constructor and method names of the reference class (comm.py:8-56)."""
+
+    def __init__(self, process_group, global_ranks, logger, memory_scale=1, rehash=3):
+        self.name = "LoadBalanceAllreduce"
+        self.device = torch.cuda.current_device()
+        self.process_group = process_group
+        self.global_ranks = global_ranks
+        self.partitions = process_group.size()
+        self.local_rank = process_group.rank() if hasattr(process_group, "rank") else 0
+        self.tensor_partition = self.get_tensor_partition_obj(memory_scale, rehash)
+        self.logger = logger
+        self.mapping = {}
+
+    def get_tensor_partition_obj(self, memory_scale, rehash):
+        return TensorPartition(partitions=self.partitions, memory_scale=memory_scale, rehash=rehash)
+
+    def stack_tensors(self, tensors, shape=-1):
+        # comm.py:25-29; payloads that already sit back to back in one buffer
+        # (what an all-to-all into a single flat buffer leaves) are not copied
+        if isinstance(tensors, (list, tuple)):
+            flat = _as_one_buffer(tensors)
+            return (flat if flat is not None else torch.cat(list(tensors))).reshape(shape)
+        return tensors.reshape(shape)
+
+    # ------------------------------------------------------------ merge
+    def decode_sparse_tensors(self, indices_tensors, values_tensors, alltoall_dense_size):
+        """Dense tensor of `alltoall_dense_size` elements in the value dtype with
+        every payload scatter-added into it (comm.py:32-44).  Sums are taken in
+        fp32 in payload order and rounded once."""
+        indices = self.stack_tensors(indices_tensors)
+        values = self.stack_tensors(values_tensors)
+        assert indices.dtype in (torch.int32, torch.int64)
+        _lib.require_gpu(indices, "indices")
+        _lib.require_gpu(values, "values")
+        dev = values.device
+        L = _lib.lib()
+        r = indices.numel()
+        dense = torch.empty(alltoall_dense_size, dtype=values.dtype, device=dev)
+        status = _lib.status_word(dev)
+        ws = _lib.scratch.get(dev, "decode", L.zen_decode_dense_workspace(r))
+        rc = L.zen_decode_dense(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(values),
+                                _lib.dtype_code(values), r, _lib.ptr(dense), alltoall_dense_size,
+                                _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
+        _lib.check(rc, "decode_sparse_tensors")
+        self._last_status = status
+        return dense
+
+    def encode_sparse_tensor(self, tensor):
+        """(ascending int64 indices of the nonzeros, their values), comm.py:47-50."""
+        _lib.require_gpu(tensor, "input")
+        idx, val, _ = _select(tensor, None, idx64=True)
+        return idx, val
+
+    def merge_sparse_flat(self, indices_tensors, values_tensors, dense_size, capacity=None, idx64=False):
+        """decode_sparse_tensors followed by encode_sparse_tensor (comm.py:125-127)
+        without the dense intermediate and without host synchronisation.
+        Returns (indices, fp32 sums, count int64[1], status int32[1]); the first
+        `count` entries are valid and ascending."""
+        indices = self.stack_tensors(indices_tensors)
+        values = self.stack_tensors(values_tensors)
+        _lib.require_gpu(indices, "indices")
+        _lib.require_gpu(values, "values")
+        dev = values.device
+        L = _lib.lib()
+        r = indices.numel()
+        if capacity is None:
+            capacity = r
+        out_idx = torch.empty(capacity, dtype=torch.int64 if idx64 else torch.int32, device=dev)
+        out_val = torch.empty(capacity, dtype=torch.float32, device=dev)
+        count = torch.zeros(1, dtype=torch.int64, device=dev)
+        status = _lib.status_word(dev)
+        ws = _lib.scratch.get(dev, "merge", L.zen_merge_workspace(r))
+        rc = L.zen_merge(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(values),
+                         _lib.dtype_code(values), r, dense_size, _lib.ptr(out_idx), 1 if idx64 else 0,
+                         _lib.ptr(out_val), capacity, _lib.ptr(count), _lib.ptr(ws), ws.numel(),
+                         _lib.ptr(status), _lib.stream_of(dev))
+        _lib.check(rc, "merge_sparse")
+        return out_idx, out_val, count, status
+
+    def merge_sparse(self, indices_tensors, values_tensors, dense_size):
+        """Synchronising form of merge_sparse_flat: (int64 indices, fp32 sums)."""
+        idx, val, count, status = self.merge_sparse_flat(indices_tensors, values_tensors, dense_size, idx64=True)
+        host = torch.cat([count, status.to(torch.int64)]).tolist()
+        if host[1]:
+            raise RuntimeError("merge_sparse: " + _lib.describe_status(host[1]))
+        return idx[:host[0]], val[:host[0]]
+
+    # ---------------------------------------------------------- mapping
+    def calculate_mapping(self, numel):
+        """List of P ascending int64 tensors: the indices of each partition
+        (comm.py:52-56)."""
+        L = _lib.lib()
+        dev = torch.device("cuda", self.device)
+        out = torch.empty(numel, dtype=torch.int64, device=dev)
+        counts = torch.zeros(self.partitions, dtype=torch.int64, device=dev)
+        ws = _lib.scratch.get(dev, "mapping", L.zen_mapping_workspace(numel, self.partitions))
+        rc = L.zen_mapping(numel, self.partitions, _lib.ptr(out), _lib.ptr(counts), _lib.ptr(ws), ws.numel(),
+                           _lib.stream_of(dev))
+        _lib.check(rc, "calculate_mapping")
+        sizes = counts.tolist()
+        mapping, at = [], 0
+        for c in sizes:
+            mapping.append(out[at:at + c])
+            at += c
+        return mapping
+
+
+def _as_one_buffer(tensors):
+    """If the 1-D tensors are consecutive views of one storage, the covering
+    view; else None."""
+    if not tensors:
+        return None
+    first = tensors[0]
+    if first.dim() != 1 or not first.is_contiguous():
+        return None
+    total = 0
+    base = first.data_ptr()
+    for t in tensors:
+        if (t.dim() != 1 or t.dtype != first.dtype or not t.is_contiguous()
+                or t.untyped_storage().data_ptr() != first.untyped_storage().data_ptr()
+                or t.data_ptr() != base + total * first.element_size()):
+            return None
+        total += t.numel()
+    return torch.as_strided(first, (total,), (1,))

@@ -1,0 +1,64 @@
+"""Magnitude selection: the reference's `compress` (train.py:75-84) and the
+exact top-k threshold BASELINE's configurations ask for."""
+import math
+
+import torch
+
+from . import _lib
+
+
+def topk_threshold(tensor, k):
+    """Device tensor uint32[2]: [magnitude key of the k-th largest |x|, number
+    of elements with key >= it].  The key is the bit pattern of |x| (bf16: 15
+    bits, fp32: 31 bits); for non-NaN values key order is magnitude order, so
+    this equals topk(|x|, k)[0].min() (train.py:81-82).  No host sync."""
+    _lib.require_gpu(tensor, "input")
+    flat = tensor.reshape(-1)
+    L = _lib.lib()
+    thr = torch.empty(2, dtype=torch.int32, device=flat.device)
+    nbytes = L.zen_topk_threshold_workspace()
+    ws = _lib.scratch.get(flat.device, "topk", nbytes)
+    rc = L.zen_topk_threshold(_lib.ptr(flat), _lib.dtype_code(flat), flat.numel(), int(k),
+                              _lib.ptr(thr), _lib.ptr(ws), ws.numel(), _lib.stream_of(flat.device))
+    _lib.check(rc, "topk_threshold")
+    return thr
+
+
+def threshold_value(tensor, thr):
+    """The threshold as a 0-dim tensor of tensor.dtype (synchronises)."""
+    key = int(thr[0].item()) & 0xFFFFFFFF
+    if tensor.dtype == torch.bfloat16:
+        return torch.tensor([key], dtype=torch.int16).view(torch.bfloat16)[0]
+    return torch.tensor([key], dtype=torch.int32).view(torch.float32)[0]
+
+
+def mask_below(tensor, thr):
+    """where(|x| >= threshold, x, 0) as a new dense tensor (train.py:83)."""
+    _lib.require_gpu(tensor, "input")
+    out = torch.empty_like(tensor)
+    rc = _lib.lib().zen_compress(_lib.ptr(tensor), _lib.dtype_code(tensor), tensor.numel(),
+                                 _lib.ptr(thr), _lib.ptr(out), _lib.stream_of(tensor.device))
+    _lib.check(rc, "compress")
+    return out
+
+
+def compress(top_k, tensor, sample_index=None):
+    """Same contract as the reference's compress (train.py:75-84): tensors of
+    at most 4096 elements pass through; otherwise the threshold is the
+    (n_s*top_k//100)-th largest magnitude of a 1 % sample drawn with
+    replacement, and everything below it is zeroed.  `sample_index` (int64
+    positions) replaces the reference's device RNG draw so that results can be
+    reproduced; None draws it with torch.randint like the reference."""
+    numel = tensor.numel()
+    if numel <= 4096:
+        return tensor
+    flat = tensor.reshape(-1)
+    if sample_index is None:
+        sample_index = torch.randint(0, numel, (math.ceil(0.01 * numel),), device=tensor.device)
+    sample = flat[sample_index]
+    k = sample.numel() * top_k // 100
+    if k < 1:
+        # torch.min of the empty topk result raises in the reference
+        raise RuntimeError("compress: top-k of the sample is empty")
+    thr = topk_threshold(sample, k)
+    return mask_below(flat, thr).view_as(tensor)

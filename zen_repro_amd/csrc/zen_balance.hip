@@ -1,0 +1,395 @@
+// Hash partitioning: hash_index, the in-place table insert (sparse_balance) and
+// the fused select + insert + slot-order compaction (load_balance).
+//
+// The reference insert (functions_cuda_kernel.cu:97-167) is a race: plain load,
+// plain store.  Run with its threads in ascending order it has one well-defined
+// result: a slot belongs to the smallest index that ever probes it, and an
+// index probes level l+1 only if a smaller index owns its level-l slot.  That
+// fixed point is computed here with atomicMax on the encoding 0 - index (so the
+// empty marker 0 stays the smallest value): a thread that takes a slot from a
+// larger index carries on with that index's probe sequence, so every lost
+// probe is continued exactly once and no rounds or flags are needed.
+#include "zen_select.h"
+
+namespace zen {
+namespace {
+
+__device__ inline void insert_chain(uint32_t *table, const Probe &g, uint32_t t) {
+  uint32_t cur = t;
+  int lv = 0;
+  for (;;) {
+    uint32_t part;
+    const uint32_t slot = probe_slot(g, cur, lv, &part);
+    const uint32_t mine = 0u - cur;
+    const uint32_t old = atomicMax(&table[slot], mine);
+    if (old > mine) {  // a smaller index owns the slot: cur moves on
+      if (++lv >= g.levels) return;  // out of levels: found later by its absence
+      continue;
+    }
+    if (old == 0u || old == mine) return;  // took an empty slot
+    // took the slot from a larger index w: w held it at its first level that
+    // maps here, and now continues from the next one
+    const uint32_t w = 0u - old;
+    int lw = 0;
+    while (lw < g.levels && probe_slot(g, w, lw, &part) != slot) ++lw;
+    cur = w;
+    lv = lw + 1;
+    if (lv >= g.levels) return;
+  }
+}
+
+// level at which t holds a slot, or -1; *slot_out / *part_out as found
+__device__ inline int find_level(const uint32_t *table, const Probe &g, uint32_t t, uint32_t *slot_out,
+                                 uint32_t *part_out) {
+  const uint32_t mine = 0u - t;
+  for (int lv = 0; lv < g.levels; ++lv) {
+    const uint32_t slot = probe_slot(g, t, lv, part_out);
+    if (table[slot] == mine) {
+      *slot_out = slot;
+      return lv;
+    }
+  }
+  return -1;
+}
+
+// ------------------------------------------------------------- hash_index
+
+__global__ __launch_bounds__(256) void k_hash_index(int32_t *__restrict__ out, uint32_t n, uint32_t per_part) {
+  for (uint32_t t = blockIdx.x * 256u + threadIdx.x; t < n; t += gridDim.x * 256u)
+    out[t] = (int32_t)(((poly(t) + kSeed1) % n) / per_part);
+}
+
+// ------------------------------------------------ in-place insert (dense)
+
+template <typename S, bool ALIGNED>
+__global__ __launch_bounds__(256) void k_insert_dense(const S *__restrict__ in, int64_t n, uint32_t *table,
+                                                      Probe g) {
+  constexpr int V = VecOf<S>::kN;
+  const int64_t nvec = (n + V - 1) / V;
+  for (int64_t v = blockIdx.x * (int64_t)256 + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * 256) {
+    S e[V];
+    const int live = load_vec<S, ALIGNED>(in, v * V, n, e);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const uint32_t t = (uint32_t)(v * V + i);
+      if (i < live && (e[i] & KeyOf<S>::kMask) != 0 && t != 0) insert_chain(table, g, t);
+    }
+  }
+}
+
+template <typename S, bool ALIGNED>
+__global__ __launch_bounds__(256) void k_finalize_dense(const S *__restrict__ in, int64_t n, uint32_t *table,
+                                                        Probe g, int32_t *serial, int64_t spp,
+                                                        int32_t *offset, int32_t *status) {
+  constexpr int V = VecOf<S>::kN;
+  const int64_t nvec = (n + V - 1) / V;
+  for (int64_t v = blockIdx.x * (int64_t)256 + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * 256) {
+    S e[V];
+    const int live = load_vec<S, ALIGNED>(in, v * V, n, e);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const uint32_t t = (uint32_t)(v * V + i);
+      if (!(i < live && (e[i] & KeyOf<S>::kMask) != 0 && t != 0)) continue;
+      uint32_t slot, part;
+      if (find_level(table, g, t, &slot, &part) >= 0) {
+        table[slot] = t;  // owner only: nobody else compares equal to this slot
+      } else {
+        const int64_t ticket = atomicAdd(&offset[part], 1);
+        if (ticket >= 0 && ticket < (int64_t)(part + 1) * spp)
+          serial[ticket] = (int32_t)t;
+        else
+          atomicOr(status, ZEN_STAT_SERIAL_OVERFLOW);
+      }
+    }
+  }
+}
+
+// Ascending compare-exchange network (bitonic with mirrored first step), valid
+// for any n: positions >= n act as +infinity and never move.
+__device__ inline void sort_network(uint32_t *a, uint32_t n) {
+  uint32_t n2 = 1;
+  while (n2 < n) n2 <<= 1;
+  const uint32_t half = n2 >> 1;
+  for (uint32_t k = 2; k <= n2; k <<= 1) {
+    const uint32_t hk = k >> 1;
+    for (uint32_t q = threadIdx.x; q < half; q += blockDim.x) {
+      const uint32_t blk = q / hk, r = q % hk;
+      const uint32_t i = blk * k + r, l = blk * k + (k - 1 - r);
+      if (l < n) {
+        const uint32_t x = a[i], y = a[l];
+        if (x > y) { a[i] = y; a[l] = x; }
+      }
+    }
+    __syncthreads();
+    for (uint32_t j = hk >> 1; j > 0; j >>= 1) {
+      for (uint32_t q = threadIdx.x; q < half; q += blockDim.x) {
+        const uint32_t i = (q / j) * 2 * j + (q % j), l = i + j;
+        if (l < n) {
+          const uint32_t x = a[i], y = a[l];
+          if (x > y) { a[i] = y; a[l] = x; }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+constexpr uint32_t kSerialLds = 8192;
+
+// Tickets are handed out in arrival order; the canonical order is ascending
+// index inside each partition's region, so each region is sorted in place.
+__global__ __launch_bounds__(256) void k_serial_sort(int32_t *serial, int64_t spp, const int32_t *offset) {
+  __shared__ uint32_t buf[kSerialLds];
+  const int p = blockIdx.x;
+  const int64_t begin = (int64_t)p * spp;
+  int64_t end = offset[p];
+  if (end > begin + spp) end = begin + spp;
+  if (end - begin < 2) return;
+  const uint32_t cnt = (uint32_t)(end - begin);
+  uint32_t *region = reinterpret_cast<uint32_t *>(serial + begin);
+  if (cnt <= kSerialLds) {
+    for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) buf[i] = region[i];
+    __syncthreads();
+    sort_network(buf, cnt);
+    for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) region[i] = buf[i];
+  } else {
+    sort_network(region, cnt);
+  }
+}
+
+// ------------------------------------------------- fused path (list based)
+
+__global__ __launch_bounds__(256) void k_insert_list(const int32_t *__restrict__ cand, const uint32_t *count,
+                                                     uint32_t *table, Probe g) {
+  const uint32_t j = blockIdx.x * 256u + threadIdx.x;
+  if (j >= *count) return;
+  const uint32_t t = (uint32_t)cand[j];
+  if (t != 0) insert_chain(table, g, t);
+}
+
+// Sort key = position in the output: partition-major, table slots before the
+// partition's serial entries (all serial entries of a partition share one key;
+// the stable sort keeps them in ascending index order).
+__global__ __launch_bounds__(256) void k_final_key(const int32_t *__restrict__ cand, const uint32_t *count,
+                                                   const uint32_t *__restrict__ table, Probe g,
+                                                   uint32_t drop_key, uint32_t *__restrict__ keys,
+                                                   uint32_t *__restrict__ perm) {
+  const uint32_t j = blockIdx.x * 256u + threadIdx.x;
+  if (j >= *count) return;
+  const uint32_t t = (uint32_t)cand[j];
+  uint32_t key = drop_key;  // index 0 is never transmitted
+  if (t != 0) {
+    uint32_t slot = 0, part = 0;
+    const int lv = find_level(table, g, t, &slot, &part);
+    key = part * (g.npp + 1u) + (lv >= 0 ? slot - part * g.npp : g.npp);
+  }
+  keys[j] = key;
+  perm[j] = j;
+}
+
+template <typename S>
+__global__ __launch_bounds__(256) void k_gather(const uint32_t *__restrict__ keys, const uint32_t *__restrict__ perm,
+                                                const uint32_t *count, const int32_t *__restrict__ cand_idx,
+                                                const S *__restrict__ cand_val, uint32_t drop_key, Probe g,
+                                                int32_t *__restrict__ out_idx, S *__restrict__ out_val,
+                                                uint32_t *table) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= *count) return;
+  const uint32_t key = keys[i];
+  if (key >= drop_key) return;
+  const uint32_t j = perm[i];
+  out_idx[i] = cand_idx[j];
+  out_val[i] = cand_val[j];
+  const uint32_t part = key / (g.npp + 1u), local = key % (g.npp + 1u);
+  if (local < g.npp) table[part * g.npp + local] = 0u;  // leave the table empty again
+}
+
+__device__ inline uint32_t lower_bound_u32(const uint32_t *a, uint32_t n, uint32_t x) {
+  uint32_t lo = 0, hi = n;
+  while (lo < hi) {
+    const uint32_t mid = lo + ((hi - lo) >> 1);
+    if (a[mid] < x) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+__global__ void k_splits(const uint32_t *__restrict__ keys, const uint32_t *count, int partitions, uint32_t npp,
+                         int64_t spp, int64_t *__restrict__ splits, int32_t *status) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= partitions) return;
+  const uint32_t n = *count;
+  const uint32_t first = (uint32_t)p * (npp + 1u);
+  const uint32_t lo = lower_bound_u32(keys, n, first);
+  const uint32_t ser = lower_bound_u32(keys, n, first + npp);
+  const uint32_t hi = lower_bound_u32(keys, n, first + npp + 1u);
+  splits[p] = (int64_t)(hi - lo);
+  if ((int64_t)(hi - ser) > spp) atomicOr(status, ZEN_STAT_SERIAL_OVERFLOW);
+}
+
+template <typename S>
+int sparse_balance_launch(const S *in, int64_t n, uint32_t *table, Probe g, int32_t *serial, int64_t spp,
+                          int32_t *offset, int partitions, int32_t *status, hipStream_t s) {
+  constexpr int V = VecOf<S>::kN;
+  const int64_t nvec = ceil_div(n, V);
+  int64_t blocks = ceil_div(nvec, 256);
+  if (blocks > 16384) blocks = 16384;
+  const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+  ProfScope prof(kProfInsertDense, s);
+  if (aligned) {
+    k_insert_dense<S, true><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(in, n, table, g);
+    ZEN_LAUNCH_CHECK("k_insert_dense");
+    k_finalize_dense<S, true><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(in, n, table, g, serial, spp, offset, status);
+  } else {
+    k_insert_dense<S, false><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(in, n, table, g);
+    ZEN_LAUNCH_CHECK("k_insert_dense");
+    k_finalize_dense<S, false><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(in, n, table, g, serial, spp, offset, status);
+  }
+  ZEN_LAUNCH_CHECK("k_finalize_dense");
+  if (spp > 0) {
+    k_serial_sort<<<dim3((unsigned)partitions), dim3(256), 0, s>>>(serial, spp, offset);
+    ZEN_LAUNCH_CHECK("k_serial_sort");
+  }
+  return ZEN_OK;
+}
+
+struct BalancePlan {
+  int32_t *cand_idx;
+  uint32_t *cand_val;  // 4 bytes per entry reserved; bf16 uses half
+  uint32_t *keys_a, *perm_a, *keys_b, *perm_b;
+  uint32_t *count;
+  void *select_scratch;
+  void *sort_scratch;
+  size_t bytes;
+};
+
+BalancePlan plan_balance(void *workspace, int64_t n, int dtype, int64_t capacity) {
+  Carver cv(workspace);
+  BalancePlan p;
+  const size_t cap = (size_t)(capacity > 0 ? capacity : 1);
+  p.cand_idx = cv.take<int32_t>(cap);
+  p.cand_val = cv.take<uint32_t>(cap);
+  p.keys_a = cv.take<uint32_t>(cap);
+  p.perm_a = cv.take<uint32_t>(cap);
+  p.keys_b = cv.take<uint32_t>(cap);
+  p.perm_b = cv.take<uint32_t>(cap);
+  p.count = cv.take<uint32_t>(1);
+  p.select_scratch = cv.take<char>(select_scratch_bytes(n, dtype));
+  p.sort_scratch = cv.take<char>(sort_scratch_bytes((int64_t)cap));
+  p.bytes = cv.used;
+  return p;
+}
+
+}  // namespace
+}  // namespace zen
+
+extern "C" {
+
+int zen_hash_index(int32_t *out, int64_t n, int partitions, void *stream) {
+  using namespace zen;
+  if (!out) return fail(ZEN_EINVAL, "zen_hash_index: null pointer");
+  if (n <= 0 || n > 0x7fffffffll || partitions <= 0 || n / partitions == 0)
+    return fail(ZEN_EINVAL, "zen_hash_index: need 0 < partitions <= n < 2^31");
+  int64_t blocks = ceil_div(n, 256 * 4);
+  if (blocks > 65536) blocks = 65536;
+  k_hash_index<<<dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      out, (uint32_t)n, (uint32_t)(n / partitions));
+  ZEN_LAUNCH_CHECK("k_hash_index");
+  return ZEN_OK;
+}
+
+int zen_sparse_balance(const void *input, int dtype, int64_t n, int32_t *memory, int64_t m, int32_t *serial,
+                       int64_t serial_n, int32_t *offset, int partitions, int rehash, int32_t *status,
+                       void *stream) {
+  using namespace zen;
+  if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_sparse_balance: bad dtype");
+  if (n < 0 || n > 0x7fffffffll || m <= 0 || m > 0x7fffffffll || partitions <= 0 || m % partitions != 0 ||
+      serial_n < 0 || serial_n > 0x7fffffffll)
+    return fail(ZEN_EINVAL, "zen_sparse_balance: need n, m < 2^31 and m a positive multiple of partitions");
+  if (n == 0) return ZEN_OK;
+  if (!input || !memory || !offset || !status || (serial_n > 0 && !serial))
+    return fail(ZEN_EINVAL, "zen_sparse_balance: null pointer");
+  Probe g;
+  g.m = (uint32_t)m;
+  g.npp = (uint32_t)(m / partitions);
+  g.levels = (rehash == 2 || rehash == 3) ? rehash : 1;  // functions_cuda_kernel.cu:192-198
+  const int64_t spp = serial_n / partitions;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint32_t *table = reinterpret_cast<uint32_t *>(memory);
+  if (dtype == ZEN_BF16)
+    return sparse_balance_launch(static_cast<const uint16_t *>(input), n, table, g, serial, spp, offset,
+                                 partitions, status, s);
+  return sparse_balance_launch(static_cast<const uint32_t *>(input), n, table, g, serial, spp, offset,
+                               partitions, status, s);
+}
+
+size_t zen_load_balance_workspace(int64_t n, int dtype, int64_t capacity, int partitions) {
+  (void)partitions;
+  if (n <= 0 || capacity < 0) return 0;
+  return zen::plan_balance(nullptr, n, dtype, capacity).bytes;
+}
+
+int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
+                     const uint32_t *thr, int32_t *out_idx, void *out_val, int64_t capacity, int64_t *splits,
+                     int32_t *table, void *workspace, size_t workspace_bytes, int32_t *status, void *stream) {
+  using namespace zen;
+  if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_load_balance: bad dtype");
+  if (n <= 0 || n > 0x7fffffffll || m <= 0 || m > 0x7fffffffll || partitions <= 0 || partitions > 65535 ||
+      m % partitions != 0 || capacity <= 0 || capacity > 0x7fffffffll)
+    return fail(ZEN_EINVAL, "zen_load_balance: need 0 < n, m < 2^31, m a multiple of partitions, capacity > 0");
+  if (!input || !out_idx || !out_val || !splits || !table || !workspace || !status)
+    return fail(ZEN_EINVAL, "zen_load_balance: null pointer");
+  if (workspace_bytes < zen_load_balance_workspace(n, dtype, capacity, partitions))
+    return fail(ZEN_EWORKSPACE, "zen_load_balance: workspace too small");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  Probe g;
+  g.m = (uint32_t)m;
+  g.npp = (uint32_t)(m / partitions);
+  g.levels = (rehash == 2 || rehash == 3) ? rehash : 1;
+  const int64_t spp = n / partitions / 10;  // tensor_load_balance.py:18
+  const uint32_t drop_key = (uint32_t)partitions * (g.npp + 1u);
+  const int bits = ceil_log2_u64(drop_key);
+  BalancePlan p = plan_balance(workspace, n, dtype, capacity);
+
+  int rc = select_compact(input, dtype, n, thr, p.cand_idx, 0, p.cand_val, capacity, nullptr, p.count,
+                          p.select_scratch, status, s);
+  if (rc != ZEN_OK) return rc;
+  const unsigned blocks = (unsigned)ceil_div(capacity, 256);
+  {
+    ProfScope prof(kProfInsertList, s);
+    k_insert_list<<<dim3(blocks), dim3(256), 0, s>>>(p.cand_idx, p.count, reinterpret_cast<uint32_t *>(table), g);
+    ZEN_LAUNCH_CHECK("k_insert_list");
+  }
+  {
+    ProfScope prof(kProfFinalKey, s);
+    k_final_key<<<dim3(blocks), dim3(256), 0, s>>>(p.cand_idx, p.count, reinterpret_cast<uint32_t *>(table), g,
+                                                   drop_key, p.keys_a, p.perm_a);
+    ZEN_LAUNCH_CHECK("k_final_key");
+  }
+  int where;
+  {
+    ProfScope prof(kProfSort, s);
+    where = sort_pairs(p.keys_a, p.perm_a, p.keys_b, p.perm_b, capacity, p.count, bits, p.sort_scratch, s);
+  }
+  if (where < 0) return where;
+  const uint32_t *sk = where ? p.keys_b : p.keys_a;
+  const uint32_t *sp = where ? p.perm_b : p.perm_a;
+  {
+  ProfScope prof(kProfGather, s);
+  if (dtype == ZEN_BF16)
+    k_gather<uint16_t><<<dim3(blocks), dim3(256), 0, s>>>(sk, sp, p.count, p.cand_idx,
+                                                          reinterpret_cast<const uint16_t *>(p.cand_val), drop_key, g,
+                                                          out_idx, static_cast<uint16_t *>(out_val),
+                                                          reinterpret_cast<uint32_t *>(table));
+  else
+    k_gather<uint32_t><<<dim3(blocks), dim3(256), 0, s>>>(sk, sp, p.count, p.cand_idx, p.cand_val, drop_key, g,
+                                                          out_idx, static_cast<uint32_t *>(out_val),
+                                                          reinterpret_cast<uint32_t *>(table));
+  ZEN_LAUNCH_CHECK("k_gather");
+  }
+  k_splits<<<dim3((unsigned)ceil_div(partitions, 64)), dim3(64), 0, s>>>(sk, p.count, partitions, g.npp, spp, splits,
+                                                                        status);
+  ZEN_LAUNCH_CHECK("k_splits");
+  return ZEN_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,89 @@
+// Optional per-kernel timing with HIP events recorded on the launch stream.
+// Off by default; when on, every tagged launch site records an event before
+// and after its kernel(s).  Reading a tag synchronises on its events.
+#include <mutex>
+#include <vector>
+
+#include "zen_common.h"
+
+namespace zen {
+namespace {
+
+struct Span {
+  int tag;
+  hipEvent_t start, stop;
+};
+
+std::mutex g_mu;
+bool g_on = false;
+std::vector<Span> g_spans;
+
+const char *const kNames[kProfCount] = {
+    "k_topk_hist", "k_select_compact", "k_insert_list", "k_final_key", "sort_pairs",
+    "k_gather",    "k_merge_prep",     "k_merge_reduce", "k_compress", "k_insert_dense",
+};
+
+void drop_spans() {
+  for (Span &s : g_spans) {
+    (void)hipEventDestroy(s.start);
+    (void)hipEventDestroy(s.stop);
+  }
+  g_spans.clear();
+}
+
+}  // namespace
+
+ProfScope::ProfScope(int tag, hipStream_t stream) : tag_(tag), stream_(stream), start_(nullptr), stop_(nullptr) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (!g_on) return;
+  if (hipEventCreate(&start_) != hipSuccess || hipEventCreate(&stop_) != hipSuccess) {
+    start_ = stop_ = nullptr;
+    return;
+  }
+  (void)hipEventRecord(start_, stream_);
+}
+
+ProfScope::~ProfScope() {
+  if (!start_) return;
+  (void)hipEventRecord(stop_, stream_);
+  std::lock_guard<std::mutex> lock(g_mu);
+  g_spans.push_back(Span{tag_, start_, stop_});
+}
+
+}  // namespace zen
+
+extern "C" {
+
+int zen_profile_enable(int on) {
+  std::lock_guard<std::mutex> lock(zen::g_mu);
+  zen::drop_spans();
+  zen::g_on = on != 0;
+  return ZEN_OK;
+}
+
+int zen_profile_tags(void) { return zen::kProfCount; }
+
+const char *zen_profile_name(int tag) {
+  return tag >= 0 && tag < zen::kProfCount ? zen::kNames[tag] : "";
+}
+
+int zen_profile_read(int tag, double *total_ms, int64_t *launches) {
+  using namespace zen;
+  if (!total_ms || !launches || tag < 0 || tag >= kProfCount) return fail(ZEN_EINVAL, "zen_profile_read: bad argument");
+  std::lock_guard<std::mutex> lock(g_mu);
+  double sum = 0;
+  int64_t count = 0;
+  for (const Span &s : g_spans) {
+    if (s.tag != tag) continue;
+    ZEN_HIP_CHECK(hipEventSynchronize(s.stop));
+    float ms = 0;
+    ZEN_HIP_CHECK(hipEventElapsedTime(&ms, s.start, s.stop));
+    sum += ms;
+    ++count;
+  }
+  *total_ms = sum;
+  *launches = count;
+  return ZEN_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,119 @@
+"""Drop-in for the reference's tensor_load_balance.py.  `load_balance` runs as
+one fused device pipeline (select, insert, slot-order compaction) instead of
+2P boolean-mask compactions with a host sync each."""
+import torch
+
+from . import _lib
+from .functions import sparse_balance
+
+
+class TensorPartition:
+    """Same constructor and methods as the reference class
+    (tensor_load_balance.py:5-51)."""
+
+    def __init__(self, partitions, memory_scale, rehash):
+        self.partitions = partitions
+        self.memory_scale = memory_scale
+        self.rehash = rehash
+        self.device = torch.cuda.current_device()
+        self._tables = {}
+
+    # ------------------------------------------------------------ sizes
+    def table_sizes(self, numel):
+        """(hash table size, serial table size), tensor_load_balance.py:14-18."""
+        memory_size = numel * self.memory_scale
+        memory_size = int(memory_size // self.partitions * self.partitions)
+        serial_memory_size = int(numel // self.partitions // 10 * self.partitions)
+        return memory_size, serial_memory_size
+
+    # ------------------------------------------- reference-shaped pieces
+    def balance_sparse_tensor(self, tensor):
+        """Allocates and fills the two tables (tensor_load_balance.py:13-21)."""
+        memory_size, serial_memory_size = self.table_sizes(tensor.numel())
+        memory = torch.zeros(memory_size, dtype=torch.int32, device=tensor.device)
+        serial_memory = torch.zeros(serial_memory_size, dtype=torch.int32, device=tensor.device)
+        sparse_balance(tensor, memory, serial_memory, self.partitions, rehash=self.rehash).check()
+        return memory, serial_memory
+
+    def get_sub_sparse_tensors(self, tensor, memory):
+        """Per-partition nonzero entries of a table and the values they point
+        at (tensor_load_balance.py:24-40), as one compaction over the table."""
+        flat = tensor.reshape(-1)
+        found = self._nonzero_int32(memory)
+        per_part = memory.numel() // self.partitions if self.partitions else 0
+        if per_part == 0:
+            bounds = torch.zeros(self.partitions + 1, dtype=torch.int64, device=memory.device)
+        else:
+            edges = torch.arange(self.partitions + 1, device=memory.device, dtype=torch.int64) * per_part
+            bounds = torch.searchsorted(found[0], edges)
+        splits = bounds[1:] - bounds[:-1]
+        cuts = bounds.tolist()
+        idx = found[1]
+        indices = [idx[cuts[p]:cuts[p + 1]] for p in range(self.partitions)]
+        values = [flat[i.long()] for i in indices]
+        return indices, values, splits
+
+    @staticmethod
+    def _nonzero_int32(table):
+        """(positions, entries) of the nonzero entries of an int32 table.  An
+        int32 is nonzero iff its bit pattern read as float32 has a nonzero
+        magnitude key, so the float compaction kernel serves."""
+        from .comm import _select
+
+        pos, val, _ = _select(table.view(torch.float32), None, idx64=True, capacity=table.numel())
+        return pos, val.view(torch.int32)
+
+    # ------------------------------------------------------- fused path
+    def _table(self, device, m):
+        key = (torch.device(device), m)
+        t = self._tables.get(key)
+        if t is None:
+            self._tables.clear()  # one table per partitioner: sizes rarely change
+            t = torch.zeros(m, dtype=torch.int32, device=device)
+            self._tables[key] = t
+        return t
+
+    def load_balance_flat(self, tensor, thr=None, capacity=None):
+        """Fused path without host synchronisation.  Returns (indices int32
+        [capacity], values [capacity], splits int64[P] on device, status int32[1]
+        on device); the first splits.sum() entries are valid, partition-major.
+        `thr` is the device tensor written by topk_threshold (None: nonzeros)."""
+        _lib.require_gpu(tensor, "input")
+        flat = tensor.reshape(-1)
+        n = flat.numel()
+        code = _lib.dtype_code(flat)
+        m, _ = self.table_sizes(n)
+        if capacity is None:
+            capacity = n
+        dev = flat.device
+        L = _lib.lib()
+        out_idx = torch.empty(capacity, dtype=torch.int32, device=dev)
+        out_val = torch.empty(capacity, dtype=flat.dtype, device=dev)
+        splits = torch.zeros(self.partitions, dtype=torch.int64, device=dev)
+        status = _lib.status_word(dev)
+        nbytes = L.zen_load_balance_workspace(n, code, capacity, self.partitions)
+        ws = _lib.scratch.get(dev, "load_balance", nbytes)
+        table = self._table(dev, m)
+        rc = L.zen_load_balance(
+            _lib.ptr(flat), code, n, m, self.partitions, self.rehash, _lib.ptr(thr),
+            _lib.ptr(out_idx), _lib.ptr(out_val), capacity, _lib.ptr(splits), _lib.ptr(table),
+            _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
+        _lib.check(rc, "load_balance")
+        return out_idx, out_val, splits, status
+
+    def load_balance(self, tensor, thr=None, capacity=None):
+        """Returns (indices[P], values[P], splits) like the reference
+        (tensor_load_balance.py:43-51).  The per-partition tensors are views of
+        two contiguous buffers; slicing them needs the split sizes on the
+        host, which is this call's only synchronisation."""
+        out_idx, out_val, splits, status = self.load_balance_flat(tensor, thr, capacity)
+        host = torch.cat([splits, status.to(torch.int64)]).tolist()
+        bits = host[-1]
+        if bits:
+            raise RuntimeError("load_balance: " + _lib.describe_status(bits))
+        indices, values, at = [], [], 0
+        for p in range(self.partitions):
+            indices.append(out_idx[at:at + host[p]])
+            values.append(out_val[at:at + host[p]])
+            at += host[p]
+        return indices, values, splits
