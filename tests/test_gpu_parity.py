@@ -233,7 +233,8 @@ def test_compress_masked_copy(zen, oracle, dtype):
 
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
 @pytest.mark.parametrize("n,density", [(1, 1.0), (100, 0.5), (8192, 0.0), (8193, 1.0), (1 << 20, 0.01),
-                                       (5 * (1 << 20) + 3, 0.3)])
+                                       (5 * (1 << 20) + 3, 0.3), (40 * 1000 * 1000 + 3, 0.5),
+                                       (70 * 1000 * 1000, 0.004)])
 def test_encode_sparse_tensor(zen, oracle, n, density, dtype):
     g = make_grad(oracle, n, density, dtype, seed=n * 3 + 1)
     if n > 4:

@@ -126,74 +126,129 @@ __global__ __launch_bounds__(256) void k_compress(const S *__restrict__ in, int6
 }  // namespace
 
 // ------------------------------------------------------ ordered compaction
+//
+// A tile is `subs` consecutive sub-tiles of kSelBlock * kSelVecs 16-byte
+// vectors.  A block walks its tile once, staging the selected (index, value)
+// pairs in LDS in ascending order; only then does it need the number of
+// selected elements in all earlier tiles, which it gets by look-back over one
+// descriptor per tile.  Large tiles keep the descriptor chain short (the
+// look-back frontier advances 64 tiles per memory round trip), the LDS stage
+// makes the write-out coalesced.  A tile with more selected elements than the
+// stage holds is walked a second time and written directly.
+
+constexpr int kSelStage = 4096;  // staged pairs per tile
+
+template <typename S, typename I, bool ALIGNED, bool STAGED>
+__device__ inline uint32_t select_walk_tile(const S *__restrict__ in, int64_t n, uint32_t floor_key,
+                                            int64_t tile_base, int subs, uint64_t *s_scan, int32_t *st_idx,
+                                            S *st_val, I *__restrict__ out_idx, S *__restrict__ out_val,
+                                            uint64_t out_base, int64_t capacity) {
+  constexpr int V = VecOf<S>::kN;
+  constexpr int kSub = kSelBlock * kSelVecs * V;
+  uint32_t running = 0;
+  for (int sub = 0; sub < subs; ++sub) {
+    const int64_t sub_base = tile_base + (int64_t)sub * kSub;
+    if (sub_base >= n) break;
+    S e[kSelVecs][V];
+    uint32_t bits[kSelVecs];
+    uint64_t packed = 0;  // four 16-bit counters, one per vector of this thread
+#pragma unroll
+    for (int j = 0; j < kSelVecs; ++j) {
+      const int64_t first = sub_base + ((int64_t)j * kSelBlock + threadIdx.x) * V;
+      const int live = first < n ? load_vec<S, ALIGNED>(in, first, n, e[j]) : 0;
+      uint32_t b = 0;
+#pragma unroll
+      for (int i = 0; i < V; ++i)
+        if (i < live && (e[j][i] & KeyOf<S>::kMask) >= floor_key) b |= 1u << i;
+      bits[j] = b;
+      packed |= (uint64_t)__popc(b) << (16 * j);
+    }
+    uint64_t totals;
+    const uint64_t before = block_exclusive_scan<uint64_t, kSelBlock>(packed, s_scan, &totals);
+    uint32_t vec_start = running;
+#pragma unroll
+    for (int j = 0; j < kSelVecs; ++j) {
+      uint32_t pos = vec_start + (uint32_t)((before >> (16 * j)) & 0xffffu);
+      const int64_t first = sub_base + ((int64_t)j * kSelBlock + threadIdx.x) * V;
+      const uint32_t b = bits[j];
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        if (b & (1u << i)) {
+          if (STAGED) {
+            if (pos < (uint32_t)kSelStage) {
+              st_idx[pos] = (int32_t)(first + i);
+              st_val[pos] = e[j][i];
+            }
+          } else if (out_base + pos < (uint64_t)capacity) {
+            out_idx[out_base + pos] = (I)(first + i);
+            out_val[out_base + pos] = e[j][i];
+          }
+          ++pos;
+        }
+      }
+      vec_start += (uint32_t)((totals >> (16 * j)) & 0xffffu);
+    }
+    running = vec_start;
+  }
+  return running;
+}
 
 template <typename S, typename I, bool ALIGNED>
 __global__ __launch_bounds__(kSelBlock) void k_select_compact(
     const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, I *__restrict__ out_idx,
-    S *__restrict__ out_val, int64_t capacity, unsigned long long *desc, uint32_t *ticket, int ntiles,
+    S *__restrict__ out_val, int64_t capacity, unsigned long long *desc, uint32_t *ticket, int ntiles, int subs,
     int64_t *out_count, uint32_t *out_count32, int32_t *status) {
   constexpr int V = VecOf<S>::kN;
-  constexpr int kTile = kSelBlock * kSelVecs * V;
+  constexpr int kSub = kSelBlock * kSelVecs * V;
   __shared__ uint64_t s_scan[kSelBlock / 64 + 1];
   __shared__ uint64_t s_bcast;
   __shared__ int s_tile;
+  __shared__ int32_t st_idx[kSelStage];
+  __shared__ S st_val[kSelStage];
   if (threadIdx.x == 0) s_tile = (int)atomicAdd(ticket, 1u);
   __syncthreads();
   const int tile = s_tile;
   if (tile >= ntiles) return;
   uint32_t floor_key = thr ? thr[0] : 1u;
-  if (floor_key == 0) floor_key = 1u;  // a zero is never selected (Q: index/value 0 = empty)
-  const int64_t tile_base = (int64_t)tile * kTile;
+  if (floor_key == 0) floor_key = 1u;  // zeros are never selected
+  const int64_t tile_base = (int64_t)tile * subs * kSub;
 
-  S e[kSelVecs][V];
-  uint32_t bits[kSelVecs];
-  uint64_t packed = 0;  // four 16-bit counters, one per vector of this thread
-#pragma unroll
-  for (int j = 0; j < kSelVecs; ++j) {
-    const int64_t first = tile_base + ((int64_t)j * kSelBlock + threadIdx.x) * V;
-    const int live = first < n ? load_vec<S, ALIGNED>(in, first, n, e[j]) : 0;
-    uint32_t b = 0;
-#pragma unroll
-    for (int i = 0; i < V; ++i)
-      if (i < live && (e[j][i] & KeyOf<S>::kMask) >= floor_key) b |= 1u << i;
-    bits[j] = b;
-    packed |= (uint64_t)__popc(b) << (16 * j);
-  }
-  uint64_t totals;
-  const uint64_t before = block_exclusive_scan<uint64_t, kSelBlock>(packed, s_scan, &totals);
-  uint64_t aggregate = 0;
-#pragma unroll
-  for (int j = 0; j < kSelVecs; ++j) aggregate += (totals >> (16 * j)) & 0xffffu;
-  const uint64_t tile_start = lookback_exclusive(desc, tile, aggregate, status, &s_bcast);
+  const uint32_t found = select_walk_tile<S, I, ALIGNED, true>(in, n, floor_key, tile_base, subs, s_scan, st_idx,
+                                                               st_val, out_idx, out_val, 0, capacity);
+  const uint64_t tile_start = lookback_exclusive(desc, tile, found, status, &s_bcast);
   if (tile == ntiles - 1 && threadIdx.x == 0) {
-    const uint64_t all = tile_start + aggregate;
+    const uint64_t all = tile_start + found;
     if (out_count) *out_count = (int64_t)all;
     if (out_count32) *out_count32 = (uint32_t)(all < (uint64_t)capacity ? all : (uint64_t)capacity);
     if (all > (uint64_t)capacity) atomicOr(status, ZEN_STAT_CAPACITY);
   }
-  uint64_t vec_start = tile_start;
-#pragma unroll
-  for (int j = 0; j < kSelVecs; ++j) {
-    uint64_t pos = vec_start + ((before >> (16 * j)) & 0xffffu);
-    const int64_t first = tile_base + ((int64_t)j * kSelBlock + threadIdx.x) * V;
-    uint32_t b = bits[j];
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-      if (b & (1u << i)) {
-        if (pos < (uint64_t)capacity) {
-          out_idx[pos] = (I)(first + i);
-          out_val[pos] = e[j][i];
-        }
-        ++pos;
+  if (found <= (uint32_t)kSelStage) {
+    for (uint32_t i = threadIdx.x; i < found; i += kSelBlock) {
+      const uint64_t pos = tile_start + i;
+      if (pos < (uint64_t)capacity) {
+        out_idx[pos] = (I)st_idx[i];
+        out_val[pos] = st_val[i];
       }
     }
-    vec_start += (totals >> (16 * j)) & 0xffffu;
+  } else {
+    select_walk_tile<S, I, ALIGNED, false>(in, n, floor_key, tile_base, subs, s_scan, st_idx, st_val, out_idx,
+                                           out_val, tile_start, capacity);
   }
+}
+
+// Sub-tiles per tile: large tiles for large inputs, but never so large that
+// the grid falls below a few workgroups per compute unit.
+static int select_subs(int64_t n, int dtype) {
+  const int v = dtype == ZEN_BF16 ? 8 : 4;
+  const int64_t sub = (int64_t)kSelBlock * kSelVecs * v;
+  int subs = 16;
+  while (subs > 1 && ceil_div(n, sub * subs) < 2048) subs >>= 1;
+  return subs;
 }
 
 size_t select_scratch_bytes(int64_t n, int dtype) {
   const int v = dtype == ZEN_BF16 ? 8 : 4;
-  const int64_t tile = (int64_t)kSelBlock * kSelVecs * v;
+  const int64_t tile = (int64_t)kSelBlock * kSelVecs * v * select_subs(n > 0 ? n : 1, dtype);
   const int64_t ntiles = ceil_div(n > 0 ? n : 1, tile);
   return align_up((size_t)(ntiles + 2) * sizeof(unsigned long long), 256);
 }
@@ -203,7 +258,8 @@ static int select_launch(const S *in, int64_t n, const uint32_t *thr, I *out_idx
                          int64_t capacity, int64_t *out_count, uint32_t *out_count32, void *scratch,
                          int32_t *status, hipStream_t stream) {
   constexpr int V = VecOf<S>::kN;
-  const int64_t tile = (int64_t)kSelBlock * kSelVecs * V;
+  const int subs = select_subs(n, sizeof(S) == 2 ? ZEN_BF16 : ZEN_F32);
+  const int64_t tile = (int64_t)kSelBlock * kSelVecs * V * subs;
   const int64_t ntiles = ceil_div(n, tile);
   if (ntiles > 0x7fffffff) return fail(ZEN_EINVAL, "select: too many tiles");
   // descriptors followed by the ticket counter, cleared together
@@ -215,10 +271,10 @@ static int select_launch(const S *in, int64_t n, const uint32_t *thr, I *out_idx
   ProfScope prof(kProfSelectCompact, stream);
   if (aligned)
     k_select_compact<S, I, true><<<dim3((unsigned)ntiles), dim3(kSelBlock), 0, stream>>>(
-        in, n, thr, out_idx, out_val, capacity, desc, ticket, (int)ntiles, out_count, out_count32, status);
+        in, n, thr, out_idx, out_val, capacity, desc, ticket, (int)ntiles, subs, out_count, out_count32, status);
   else
     k_select_compact<S, I, false><<<dim3((unsigned)ntiles), dim3(kSelBlock), 0, stream>>>(
-        in, n, thr, out_idx, out_val, capacity, desc, ticket, (int)ntiles, out_count, out_count32, status);
+        in, n, thr, out_idx, out_val, capacity, desc, ticket, (int)ntiles, subs, out_count, out_count32, status);
   ZEN_LAUNCH_CHECK("k_select_compact");
   return ZEN_OK;
 }
