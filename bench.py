@@ -1,9 +1,9 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-gradient encode + decode path on one MI355X.
 
-One step = exact top-k threshold + fused select/hash-partition/compaction of
-the rank's own gradient + merge of the P peer payloads addressed to rank 0,
-all inputs resident in HBM.  Prints one JSON line (see README / DESIGN).
+One step = exact top-k selection fused with the hash partition and slot-order
+compaction of the rank's own gradient + merge of the P peer payloads addressed
+to rank 0, all inputs resident in HBM.  Prints one JSON line (see README / DESIGN).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--shrink S]
 """
@@ -94,10 +94,9 @@ def main():
     received = flat_idx.numel()
 
     def step():
-        thr = topk_threshold(grad, cfg.k) if cfg.k else None
-        enc = tp.load_balance_flat(grad, thr, capacity)
+        enc = tp.load_balance_flat(grad, None, capacity, k=cfg.k)
         mrg = lba.merge_sparse_flat(flat_idx, flat_val, n, capacity=received)
-        return thr, enc, mrg
+        return enc, mrg
 
     for _ in range(args.warmup):
         out = step()
@@ -112,7 +111,7 @@ def main():
     kernels = {} if args.no_kernel_timing else _lib.profile_read()
     _lib.profile_enable(False)
 
-    thr, (o_idx, o_val, splits, st_enc), (m_idx, m_val, m_count, st_mrg) = out
+    (o_idx, o_val, splits, st_enc), (m_idx, m_val, m_count, st_mrg) = out
     nnz = int(splits.sum())
     merged = int(m_count)
     flags = int(st_enc) | int(st_mrg)

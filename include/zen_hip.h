@@ -44,6 +44,12 @@ extern "C" {
 #define ZEN_STAT_CAPACITY 2        /* more output entries than `capacity`; the excess was dropped */
 #define ZEN_STAT_INTERNAL 4        /* a bounded in-kernel wait expired; outputs are invalid */
 #define ZEN_STAT_BAD_INDEX 8       /* merge/decode saw an index outside [0, dense_n); it was skipped */
+#define ZEN_STAT_RETRY 16          /* the fast path met keys piled on a few values and produced nothing:
+                                      call again with ZEN_MODE_GENERAL */
+
+/* `mode` argument of the sort-based entry points */
+#define ZEN_MODE_FAST 0    /* two-level bin sort; flags ZEN_STAT_RETRY on pathological key distributions */
+#define ZEN_MODE_GENERAL 1 /* one radix pass per 8 key bits; any input */
 
 int zen_abi_version(void);
 
@@ -69,7 +75,7 @@ int zen_hash_index(int32_t *out, int64_t n, int partitions, void *stream);
  */
 size_t zen_mapping_workspace(int64_t n, int partitions);
 int zen_mapping(int64_t n, int partitions, int64_t *out, int64_t *counts,
-                void *workspace, size_t workspace_bytes, void *stream);
+                void *workspace, size_t workspace_bytes, int32_t *status, void *stream);
 
 /* ---------------------------------------------------------------- insert */
 
@@ -130,7 +136,13 @@ int zen_select(const void *input, int dtype, int64_t n, const uint32_t *thr,
 /*
  * Fused select + insert + slot-order compaction.  Replaces
  * TensorPartition.load_balance (tensor_load_balance.py:13-51) and, with
- * thr != NULL, the masked copy of compress (train.py:83) in front of it.
+ * thr != NULL or k > 0, compress (train.py:75-84) in front of it.
+ * Selection: thr == NULL and k == 0: the nonzero elements; thr != NULL: key >=
+ * max(thr[0], 1); k > 0: the k largest magnitudes, ties at the k-th kept (thr
+ * must be NULL; thr_out, if not NULL, receives that key and the number
+ * selected).  In ZEN_MODE_FAST the k-th largest is found with one pass over
+ * the tensor (sampled floor, exact refinement among the candidates); if the
+ * sample misleads, ZEN_STAT_RETRY is raised and nothing valid is produced.
  * Output: out_idx / out_val hold partition 0's entries, then partition 1's,
  * ...; inside a partition, table entries in ascending slot order followed by
  * that partition's serial entries in ascending index order; splits[p] (int64)
@@ -142,9 +154,9 @@ int zen_select(const void *input, int dtype, int64_t n, const uint32_t *thr,
  */
 size_t zen_load_balance_workspace(int64_t n, int dtype, int64_t capacity, int partitions);
 int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m,
-                     int partitions, int rehash, const uint32_t *thr,
-                     int32_t *out_idx, void *out_val, int64_t capacity,
-                     int64_t *splits, int32_t *table,
+                     int partitions, int rehash, const uint32_t *thr, int64_t k,
+                     uint32_t *thr_out, int32_t *out_idx, void *out_val,
+                     int64_t capacity, int64_t *splits, int32_t *table, int mode,
                      void *workspace, size_t workspace_bytes,
                      int32_t *status, void *stream);
 
@@ -157,12 +169,13 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m,
  * encode_sparse_tensor of the first exchange (comm.py:32-50, 125-127) without
  * the dense intermediate.  idx is int32 (idx64_in == 0) or int64.  out_idx is
  * int64 when idx64_out != 0.  out_val is fp32.  *out_count is int64.
+ * `mode` is ZEN_MODE_FAST or ZEN_MODE_GENERAL; both give identical results.
  */
-size_t zen_merge_workspace(int64_t r);
+size_t zen_merge_workspace(int64_t r, int64_t dense_n);
 int zen_merge(const void *idx, int idx64_in, const void *val, int dtype,
               int64_t r, int64_t dense_n,
               void *out_idx, int idx64_out, float *out_val, int64_t capacity,
-              int64_t *out_count, void *workspace, size_t workspace_bytes,
+              int64_t *out_count, int mode, void *workspace, size_t workspace_bytes,
               int32_t *status, void *stream);
 
 /*
@@ -170,9 +183,9 @@ int zen_merge(const void *idx, int idx64_in, const void *val, int dtype,
  * in entry order, rounded once to `dtype`.  Replaces decode_sparse_tensors
  * (comm.py:32-44), whose result is a dense tensor in the value dtype.
  */
-size_t zen_decode_dense_workspace(int64_t r);
+size_t zen_decode_dense_workspace(int64_t r, int64_t dense_n);
 int zen_decode_dense(const void *idx, int idx64_in, const void *val, int dtype,
-                     int64_t r, void *dense, int64_t dense_n,
+                     int64_t r, void *dense, int64_t dense_n, int mode,
                      void *workspace, size_t workspace_bytes,
                      int32_t *status, void *stream);
 
@@ -188,7 +201,7 @@ int zen_decode_dense(const void *idx, int idx64_in, const void *val, int dtype,
 size_t zen_sort_pairs_workspace(int64_t max_count);
 int zen_sort_pairs(uint32_t *keys, uint32_t *vals, int64_t max_count,
                    const uint32_t *count_dev, int bits,
-                   void *workspace, size_t workspace_bytes, void *stream);
+                   void *workspace, size_t workspace_bytes, int32_t *status, void *stream);
 
 /*
  * Per-kernel timing with HIP events recorded on the launch stream, for

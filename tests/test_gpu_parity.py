@@ -43,9 +43,10 @@ def test_sort_pairs_is_stable_sort(zen, count, bits):
     dv = to_dev(vals.view(np.int32))
     L = _lib.lib()
     ws = torch.empty(L.zen_sort_pairs_workspace(count), dtype=torch.uint8, device="cuda")
+    st = torch.zeros(1, dtype=torch.int32, device="cuda")
     rc = L.zen_sort_pairs(_lib.ptr(dk), _lib.ptr(dv), count, None, bits, _lib.ptr(ws), ws.numel(),
-                          _lib.stream_of(dk.device))
-    assert rc == 0
+                          _lib.ptr(st), _lib.stream_of(dk.device))
+    assert rc == 0 and st.item() == 0
     order = np.argsort(keys, kind="stable")
     assert np.array_equal(to_np(dk).view(np.uint32), keys[order])
     assert np.array_equal(to_np(dv).view(np.uint32), vals[order])
@@ -62,8 +63,9 @@ def test_sort_pairs_device_count(zen):
     cnt = torch.tensor([live], dtype=torch.int32, device="cuda")
     L = _lib.lib()
     ws = torch.empty(L.zen_sort_pairs_workspace(cap), dtype=torch.uint8, device="cuda")
+    st = torch.zeros(1, dtype=torch.int32, device="cuda")
     assert L.zen_sort_pairs(_lib.ptr(dk), _lib.ptr(dv), cap, _lib.ptr(cnt), 20, _lib.ptr(ws), ws.numel(),
-                            _lib.stream_of(dk.device)) == 0
+                            _lib.ptr(st), _lib.stream_of(dk.device)) == 0
     order = np.argsort(keys[:live], kind="stable")
     assert np.array_equal(to_np(dk).view(np.uint32)[:live], keys[:live][order])
     assert np.array_equal(to_np(dv).view(np.uint32)[:live], vals[:live][order])
@@ -324,6 +326,62 @@ def test_topk_then_load_balance(zen, oracle, dtype):
         assert (part[to_np(i)] == p).all()
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("dtype,shape", [("bf16", "flat"), ("f32", "flat"), ("bf16", "columns")])
+def test_load_balance_fused_topk(zen, oracle, dtype, shape, mode):
+    """k-largest selection inside the call: the one-pass sampled route (mode 0,
+    tensors of 2^24 elements and more) and the exact full-histogram route must
+    both equal oracle top-k followed by oracle load balance."""
+    from zen_repro_amd import _lib
+
+    n, P = (1 << 25) + 4096, 16
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    if shape == "columns":  # a few hot columns of a 4096-wide matrix: a stride-aligned sample would be fooled
+        x.reshape(-1, 4096)[:, ::509] *= 50.0
+    g = oracle.f32_to_bf16_bits(x) if dtype == "bf16" else x
+    k = n // 200
+    key = oracle.kth_key(g, k)
+    masked, kept = oracle.mask_dense(g, key)
+    idx_o, val_o, splits_o, st_o = oracle.load_balance(masked, P, 1, 3)
+    assert st_o == 0
+    tp = zen.TensorPartition(P, 1, 3)
+    d = to_dev(g)
+    thr_out = torch.zeros(2, dtype=torch.int32, device="cuda")
+    oi, ov, splits, status = tp.load_balance_flat(d, capacity=int(1.3 * k) + 4096, k=k, mode=mode, thr_out=thr_out)
+    assert status.item() == 0
+    assert to_np(thr_out).tolist() == [key, kept]
+    assert np.array_equal(to_np(splits), splits_o)
+    total = int(splits_o.sum())
+    assert np.array_equal(to_np(oi)[:total], idx_o)
+    assert np.array_equal(to_np(ov)[:total], val_o)
+    if mode == 0:  # the reference-shaped call picks the mode by itself
+        indices, values, _ = tp.load_balance(d, capacity=int(1.3 * k) + 4096, k=k)
+        assert np.array_equal(np.concatenate([to_np(i) for i in indices]), idx_o)
+
+
+def test_load_balance_sampled_floor_too_high_asks_for_retry(zen, oracle):
+    """k larger than the number of nonzeros the floor lets through cannot
+    happen with a fair sample; force it with a tensor whose large values all
+    hide from the 1-in-256 sample's expectation: nearly all zeros."""
+    from zen_repro_amd import _lib
+
+    n, P = 1 << 25, 8
+    g = np.zeros(n, np.float32)
+    rng = np.random.default_rng(5)
+    hot = rng.choice(n, 3000, replace=False)
+    g[hot] = rng.standard_normal(3000).astype(np.float32)
+    k = 2000
+    tp = zen.TensorPartition(P, 1, 3)
+    d = to_dev(g)
+    indices, values, splits = tp.load_balance(d, capacity=8192, k=k)  # retries in general mode if it must
+    key = oracle.kth_key(g, k)
+    masked, _ = oracle.mask_dense(g, key)
+    idx_o, val_o, splits_o, _ = oracle.load_balance(masked, P, 1, 3)
+    assert np.array_equal(to_np(splits), splits_o)
+    assert np.array_equal(np.concatenate([to_np(i) for i in indices]), idx_o)
+
+
 def test_load_balance_capacity_flag(zen, oracle):
     n, P = 1 << 16, 4
     g = make_grad(oracle, n, 0.5, "f32", seed=4)
@@ -372,6 +430,37 @@ def test_merge_sparse(zen, oracle, n, peers, per_peer, overlap, dtype):
     assert (np.abs(to_np(gv) - truth) <= 1e-6 * scale[want_i] + 1e-30).all()
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+def test_merge_modes_agree_with_oracle(zen, oracle, mode):
+    rng = np.random.default_rng(77 + mode)
+    n = 3000017
+    idx, val = make_payloads(oracle, rng, n, 16, 20000, 0.3, "bf16")
+    ci, cv = np.concatenate(idx), np.concatenate(val)
+    want_i, want_v = oracle.merge_sparse(ci, cv, n)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(16), None, None)
+    gi, gv, cnt, st = lba.merge_sparse_flat(to_dev(ci), to_dev(cv), n, mode=mode)
+    assert st.item() == 0 and cnt.item() == len(want_i)
+    assert np.array_equal(to_np(gi)[:len(want_i)], want_i.astype(np.int32))
+    assert np.array_equal(to_np(gv)[:len(want_i)].view(np.uint32), want_v.view(np.uint32))
+
+
+def test_merge_piled_up_keys_fall_back_to_general_mode(zen, oracle):
+    from zen_repro_amd import _lib
+
+    n = 1 << 20
+    rng = np.random.default_rng(3)
+    idx = np.concatenate([np.full(20000, 12345), rng.integers(0, n, 5000)]).astype(np.int32)
+    val = (rng.standard_normal(len(idx)) * 1e-3).astype(np.float32)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(4), None, None)
+    _, _, cnt, st = lba.merge_sparse_flat(to_dev(idx), to_dev(val), n, mode=_lib.MODE_FAST)
+    assert st.item() == _lib.STAT_RETRY and cnt.item() == 0
+    gi, gv = lba.merge_sparse(to_dev(idx), to_dev(val), n)  # retries by itself
+    wi, wv = oracle.merge_sparse(idx, val, n)
+    assert np.array_equal(to_np(gi), wi) and np.array_equal(to_np(gv).view(np.uint32), wv.view(np.uint32))
+    dense = lba.decode_sparse_tensors(to_dev(idx), to_dev(val), n)
+    assert np.array_equal(to_np(dense), oracle.decode(idx, val, n, "f32acc"))
+
+
 def test_merge_cancellation_nan_and_bad_index(zen, oracle):
     from zen_repro_amd import _lib
 
@@ -384,9 +473,10 @@ def test_merge_cancellation_nan_and_bad_index(zen, oracle):
     assert to_np(gi).tolist() == wi.tolist() == [9, 63]
     assert np.array_equal(to_np(gv).view(np.uint32) & 0x7FC00000, wv.view(np.uint32) & 0x7FC00000)
     bad = np.array([5, 64, -1, 7], np.int64)
-    i2, v2, cnt, st = lba.merge_sparse_flat(to_dev(bad), to_dev(np.ones(4, np.float32)), n, idx64=True)
-    assert cnt.item() == 2 and st.item() == _lib.STAT_BAD_INDEX
-    assert to_np(i2)[:2].tolist() == [5, 7]
+    for mode in (0, 1):
+        i2, v2, cnt, st = lba.merge_sparse_flat(to_dev(bad), to_dev(np.ones(4, np.float32)), n, idx64=True, mode=mode)
+        assert cnt.item() == 2 and st.item() == _lib.STAT_BAD_INDEX
+        assert to_np(i2)[:2].tolist() == [5, 7]
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])

@@ -37,11 +37,11 @@ def test_workspace_queries_are_host_only(L):
     assert L.zen_topk_threshold_workspace() >= 2048 * 4
     a, b = L.zen_sort_pairs_workspace(1000), L.zen_sort_pairs_workspace(1 << 20)
     assert 0 < a < b
-    assert L.zen_merge_workspace(1 << 20) >= 4 * 4 * (1 << 20)
+    assert L.zen_merge_workspace(1 << 20, 1 << 30) >= 5 * 4 * (1 << 20)
     assert L.zen_load_balance_workspace(1 << 24, 1, 1 << 18, 16) >= 6 * 4 * (1 << 18)
     assert L.zen_select_workspace(1 << 24, 1) >= (1 << 24) // 8192 * 8
     assert L.zen_mapping_workspace(1 << 20, 8) >= 16 * (1 << 20)
-    assert L.zen_decode_dense_workspace(1000) > L.zen_merge_workspace(1000)
+    assert L.zen_decode_dense_workspace(1000, 5000) > L.zen_merge_workspace(1000, 5000)
 
 
 def test_bad_arguments_are_rejected_on_the_host(L):
@@ -60,11 +60,13 @@ def test_bad_arguments_are_rejected_on_the_host(L):
     assert L.zen_topk_threshold(one, 0, 100, 0, one, one, 1 << 20, None) == _lib.EINVAL    # k < 1
     assert L.zen_topk_threshold(one, 0, 100, 101, one, one, 1 << 20, None) == _lib.EINVAL  # k > n
     assert L.zen_topk_threshold(one, 0, 100, 5, one, one, 16, None) == _lib.EWORKSPACE
-    assert L.zen_load_balance(one, 1, 1024, 1022, 4, 3, None, one, one, 64, one, one, one, 1 << 30, one, None) == _lib.EINVAL
-    assert L.zen_load_balance(one, 1, 1024, 1024, 4, 3, None, one, one, 64, one, one, one, 16, one, None) == _lib.EWORKSPACE
-    assert L.zen_merge(one, 0, one, 0, 10, 0, one, 0, one, 10, one, one, 1 << 20, one, None) == _lib.EINVAL  # dense_n
-    assert L.zen_merge(one, 0, one, 0, 10, 100, one, 0, one, 10, one, one, 16, one, None) == _lib.EWORKSPACE
-    assert L.zen_sort_pairs(one, one, 100, None, 33, one, 1 << 20, None) == _lib.EINVAL
+    assert L.zen_load_balance(one, 1, 1024, 1022, 4, 3, None, 0, None, one, one, 64, one, one, 0, one, 1 << 30, one, None) == _lib.EINVAL
+    assert L.zen_load_balance(one, 1, 1024, 1024, 4, 3, one, 5, None, one, one, 64, one, one, 0, one, 1 << 30, one, None) == _lib.EINVAL  # thr and k
+    assert L.zen_load_balance(one, 1, 1024, 1024, 4, 3, None, 0, None, one, one, 64, one, one, 0, one, 16, one, None) == _lib.EWORKSPACE
+    assert L.zen_merge(one, 0, one, 0, 10, 0, one, 0, one, 10, one, 0, one, 1 << 20, one, None) == _lib.EINVAL  # dense_n
+    assert L.zen_merge(one, 0, one, 0, 10, 100, one, 0, one, 10, one, 7, one, 1 << 20, one, None) == _lib.EINVAL  # mode
+    assert L.zen_merge(one, 0, one, 0, 10, 100, one, 0, one, 10, one, 0, one, 16, one, None) == _lib.EWORKSPACE
+    assert L.zen_sort_pairs(one, one, 100, None, 33, one, 1 << 20, one, None) == _lib.EINVAL
     with pytest.raises(ValueError):
         _lib.check(_lib.EINVAL, "x")
     with pytest.raises(RuntimeError):

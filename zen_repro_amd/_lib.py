@@ -9,7 +9,8 @@ import torch  # first: makes the process use torch's HIP runtime for libzen_hip 
 
 F32, BF16 = 0, 1
 OK, EINVAL, EHIP, EWORKSPACE = 0, -1, -2, -3
-STAT_SERIAL_OVERFLOW, STAT_CAPACITY, STAT_INTERNAL, STAT_BAD_INDEX = 1, 2, 4, 8
+STAT_SERIAL_OVERFLOW, STAT_CAPACITY, STAT_INTERNAL, STAT_BAD_INDEX, STAT_RETRY = 1, 2, 4, 8, 16
+MODE_FAST, MODE_GENERAL = 0, 1
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libzen_hip.so")
@@ -41,7 +42,7 @@ def lib():
         "zen_last_error": (ctypes.c_char_p, []),
         "zen_hash_index": (i32, [vp, i64, i32, vp]),
         "zen_mapping_workspace": (sz, [i64, i32]),
-        "zen_mapping": (i32, [i64, i32, vp, vp, vp, sz, vp]),
+        "zen_mapping": (i32, [i64, i32, vp, vp, vp, sz, vp, vp]),
         "zen_sparse_balance": (i32, [vp, i32, i64, vp, i64, vp, i64, vp, i32, i32, vp, vp]),
         "zen_topk_threshold_workspace": (sz, []),
         "zen_topk_threshold": (i32, [vp, i32, i64, i64, vp, vp, sz, vp]),
@@ -49,13 +50,13 @@ def lib():
         "zen_select_workspace": (sz, [i64, i32]),
         "zen_select": (i32, [vp, i32, i64, vp, vp, i32, vp, i64, vp, vp, sz, vp, vp]),
         "zen_load_balance_workspace": (sz, [i64, i32, i64, i32]),
-        "zen_load_balance": (i32, [vp, i32, i64, i64, i32, i32, vp, vp, vp, i64, vp, vp, vp, sz, vp, vp]),
-        "zen_merge_workspace": (sz, [i64]),
-        "zen_merge": (i32, [vp, i32, vp, i32, i64, i64, vp, i32, vp, i64, vp, vp, sz, vp, vp]),
-        "zen_decode_dense_workspace": (sz, [i64]),
-        "zen_decode_dense": (i32, [vp, i32, vp, i32, i64, vp, i64, vp, sz, vp, vp]),
+        "zen_load_balance": (i32, [vp, i32, i64, i64, i32, i32, vp, i64, vp, vp, vp, i64, vp, vp, i32, vp, sz, vp, vp]),
+        "zen_merge_workspace": (sz, [i64, i64]),
+        "zen_merge": (i32, [vp, i32, vp, i32, i64, i64, vp, i32, vp, i64, vp, i32, vp, sz, vp, vp]),
+        "zen_decode_dense_workspace": (sz, [i64, i64]),
+        "zen_decode_dense": (i32, [vp, i32, vp, i32, i64, vp, i64, i32, vp, sz, vp, vp]),
         "zen_sort_pairs_workspace": (sz, [i64]),
-        "zen_sort_pairs": (i32, [vp, vp, i64, vp, i32, vp, sz, vp]),
+        "zen_sort_pairs": (i32, [vp, vp, i64, vp, i32, vp, sz, vp, vp]),
         "zen_profile_enable": (i32, [i32]),
         "zen_profile_tags": (i32, []),
         "zen_profile_name": (ctypes.c_char_p, [i32]),
@@ -140,6 +141,8 @@ def describe_status(bits):
         names.append("internal wait expired")
     if bits & STAT_BAD_INDEX:
         names.append("index out of range")
+    if bits & STAT_RETRY:
+        names.append("fast path declined the input (retry in general mode)")
     return ", ".join(names) or "ok"
 
 

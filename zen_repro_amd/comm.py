@@ -87,13 +87,18 @@ class LoadBalanceAllreduce:
         L = _lib.lib()
         r = indices.numel()
         dense = torch.empty(alltoall_dense_size, dtype=values.dtype, device=dev)
-        status = _lib.status_word(dev)
-        ws = _lib.scratch.get(dev, "decode", L.zen_decode_dense_workspace(r))
-        rc = L.zen_decode_dense(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(values),
-                                _lib.dtype_code(values), r, _lib.ptr(dense), alltoall_dense_size,
-                                _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
-        _lib.check(rc, "decode_sparse_tensors")
-        self._last_status = status
+        ws = _lib.scratch.get(dev, "decode", L.zen_decode_dense_workspace(r, alltoall_dense_size))
+        for mode in (_lib.MODE_FAST, _lib.MODE_GENERAL):
+            status = _lib.status_word(dev)
+            rc = L.zen_decode_dense(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(values),
+                                    _lib.dtype_code(values), r, _lib.ptr(dense), alltoall_dense_size, mode,
+                                    _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
+            _lib.check(rc, "decode_sparse_tensors")
+            bits = int(status.item())  # the reference's scatter_add_ raises on a bad index, also a sync
+            if not bits & _lib.STAT_RETRY:
+                break
+        if bits:
+            raise RuntimeError("decode_sparse_tensors: " + _lib.describe_status(bits))
         return dense
 
     def encode_sparse_tensor(self, tensor):
@@ -102,11 +107,14 @@ class LoadBalanceAllreduce:
         idx, val, _ = _select(tensor, None, idx64=True)
         return idx, val
 
-    def merge_sparse_flat(self, indices_tensors, values_tensors, dense_size, capacity=None, idx64=False):
+    def merge_sparse_flat(self, indices_tensors, values_tensors, dense_size, capacity=None, idx64=False,
+                          mode=_lib.MODE_GENERAL):
         """decode_sparse_tensors followed by encode_sparse_tensor (comm.py:125-127)
         without the dense intermediate and without host synchronisation.
         Returns (indices, fp32 sums, count int64[1], status int32[1]); the first
-        `count` entries are valid and ascending."""
+        `count` entries are valid and ascending.  In fast mode a status with
+        STAT_RETRY means nothing was produced and the call must be repeated
+        with mode=MODE_GENERAL (merge_sparse does that by itself)."""
         indices = self.stack_tensors(indices_tensors)
         values = self.stack_tensors(values_tensors)
         _lib.require_gpu(indices, "indices")
@@ -120,18 +128,22 @@ class LoadBalanceAllreduce:
         out_val = torch.empty(capacity, dtype=torch.float32, device=dev)
         count = torch.zeros(1, dtype=torch.int64, device=dev)
         status = _lib.status_word(dev)
-        ws = _lib.scratch.get(dev, "merge", L.zen_merge_workspace(r))
+        ws = _lib.scratch.get(dev, "merge", L.zen_merge_workspace(r, dense_size))
         rc = L.zen_merge(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(values),
                          _lib.dtype_code(values), r, dense_size, _lib.ptr(out_idx), 1 if idx64 else 0,
-                         _lib.ptr(out_val), capacity, _lib.ptr(count), _lib.ptr(ws), ws.numel(),
+                         _lib.ptr(out_val), capacity, _lib.ptr(count), mode, _lib.ptr(ws), ws.numel(),
                          _lib.ptr(status), _lib.stream_of(dev))
         _lib.check(rc, "merge_sparse")
         return out_idx, out_val, count, status
 
     def merge_sparse(self, indices_tensors, values_tensors, dense_size):
         """Synchronising form of merge_sparse_flat: (int64 indices, fp32 sums)."""
-        idx, val, count, status = self.merge_sparse_flat(indices_tensors, values_tensors, dense_size, idx64=True)
-        host = torch.cat([count, status.to(torch.int64)]).tolist()
+        for mode in (_lib.MODE_FAST, _lib.MODE_GENERAL):
+            idx, val, count, status = self.merge_sparse_flat(indices_tensors, values_tensors, dense_size,
+                                                             idx64=True, mode=mode)
+            host = torch.cat([count, status.to(torch.int64)]).tolist()
+            if not host[1] & _lib.STAT_RETRY:
+                break
         if host[1]:
             raise RuntimeError("merge_sparse: " + _lib.describe_status(host[1]))
         return idx[:host[0]], val[:host[0]]
@@ -145,10 +157,13 @@ class LoadBalanceAllreduce:
         out = torch.empty(numel, dtype=torch.int64, device=dev)
         counts = torch.zeros(self.partitions, dtype=torch.int64, device=dev)
         ws = _lib.scratch.get(dev, "mapping", L.zen_mapping_workspace(numel, self.partitions))
+        status = _lib.status_word(dev)
         rc = L.zen_mapping(numel, self.partitions, _lib.ptr(out), _lib.ptr(counts), _lib.ptr(ws), ws.numel(),
-                           _lib.stream_of(dev))
+                           _lib.ptr(status), _lib.stream_of(dev))
         _lib.check(rc, "calculate_mapping")
-        sizes = counts.tolist()
+        sizes = torch.cat([counts, status.to(torch.int64)]).tolist()
+        if sizes.pop():
+            raise RuntimeError("calculate_mapping: " + _lib.describe_status(int(status.item())))
         mapping, at = [], 0
         for c in sizes:
             mapping.append(out[at:at + c])

@@ -213,17 +213,44 @@ __device__ inline uint32_t lower_bound_u32(const uint32_t *a, uint32_t n, uint32
   return lo;
 }
 
-__global__ void k_splits(const uint32_t *__restrict__ keys, const uint32_t *count, int partitions, uint32_t npp,
-                         int64_t spp, int64_t *__restrict__ splits, int32_t *status) {
-  const int p = blockIdx.x * blockDim.x + threadIdx.x;
-  if (p >= partitions) return;
-  const uint32_t n = *count;
-  const uint32_t first = (uint32_t)p * (npp + 1u);
-  const uint32_t lo = lower_bound_u32(keys, n, first);
-  const uint32_t ser = lower_bound_u32(keys, n, first + npp);
-  const uint32_t hi = lower_bound_u32(keys, n, first + npp + 1u);
-  splits[p] = (int64_t)(hi - lo);
-  if ((int64_t)(hi - ser) > spp) atomicOr(status, ZEN_STAT_SERIAL_OVERFLOW);
+// One block per partition: its length from the sorted keys, and the canonical
+// order of its serial tail.  The selected list arrives tile by tile in no
+// particular order and all serial entries of a partition share one sort key, so
+// the stable sort leaves them in arrival order; the reference order (tickets
+// handed out to ascending indices) is restored by sorting the tail by index and
+// fetching the values again.
+template <typename S>
+__global__ __launch_bounds__(256) void k_splits_serial(const uint32_t *__restrict__ keys, const uint32_t *count,
+                                                       uint32_t npp, int64_t spp, const S *__restrict__ dense,
+                                                       int32_t *__restrict__ out_idx, S *__restrict__ out_val,
+                                                       int64_t *__restrict__ splits, int32_t *status) {
+  __shared__ uint32_t s_bound[3];
+  __shared__ uint32_t buf[kSerialLds];
+  const uint32_t p = blockIdx.x;
+  if (threadIdx.x < 3) {
+    const uint32_t first = p * (npp + 1u);
+    const uint32_t probe = threadIdx.x == 0 ? first : (threadIdx.x == 1 ? first + npp : first + npp + 1u);
+    s_bound[threadIdx.x] = lower_bound_u32(keys, *count, probe);
+  }
+  __syncthreads();
+  const uint32_t lo = s_bound[0], ser = s_bound[1], hi = s_bound[2];
+  if (threadIdx.x == 0) {
+    splits[p] = (int64_t)(hi - lo);
+    if ((int64_t)(hi - ser) > spp) atomicOr(status, ZEN_STAT_SERIAL_OVERFLOW);
+  }
+  const uint32_t cnt = hi - ser;
+  if (cnt < 2) return;
+  uint32_t *region = reinterpret_cast<uint32_t *>(out_idx + ser);
+  if (cnt <= kSerialLds) {
+    for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) buf[i] = region[i];
+    __syncthreads();
+    sort_network(buf, cnt);
+    for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) region[i] = buf[i];
+  } else {
+    sort_network(region, cnt);
+  }
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) out_val[ser + i] = dense[region[i]];
 }
 
 template <typename S>
@@ -252,12 +279,19 @@ int sparse_balance_launch(const S *in, int64_t n, uint32_t *table, Probe g, int3
   return ZEN_OK;
 }
 
+constexpr int64_t kSampleMinElems = 1ll << 24;  // below this the exact full-tensor histogram is cheap anyway
+
 struct BalancePlan {
-  int32_t *cand_idx;
-  uint32_t *cand_val;  // 4 bytes per entry reserved; bf16 uses half
+  int32_t *cand_idx;   // first-stage candidates of the sampled top-k (2 * capacity)
+  uint32_t *cand_val;
+  int32_t *sel_idx;    // the selected entries (capacity); 4 bytes per value reserved, bf16 uses half
+  uint32_t *sel_val;
   uint32_t *keys_a, *perm_a, *keys_b, *perm_b;
-  uint32_t *count;
+  uint32_t *count;     // [0] selected, [1] candidates
+  uint32_t *thr;       // [0..1] exact threshold + count, [2..3] sampled floor
+  void *topk_scratch;
   void *select_scratch;
+  void *list_scratch;
   void *sort_scratch;
   size_t bytes;
 };
@@ -266,17 +300,69 @@ BalancePlan plan_balance(void *workspace, int64_t n, int dtype, int64_t capacity
   Carver cv(workspace);
   BalancePlan p;
   const size_t cap = (size_t)(capacity > 0 ? capacity : 1);
-  p.cand_idx = cv.take<int32_t>(cap);
-  p.cand_val = cv.take<uint32_t>(cap);
+  p.cand_idx = cv.take<int32_t>(2 * cap);
+  p.cand_val = cv.take<uint32_t>(2 * cap);
+  p.sel_idx = cv.take<int32_t>(cap);
+  p.sel_val = cv.take<uint32_t>(cap);
   p.keys_a = cv.take<uint32_t>(cap);
   p.perm_a = cv.take<uint32_t>(cap);
   p.keys_b = cv.take<uint32_t>(cap);
   p.perm_b = cv.take<uint32_t>(cap);
-  p.count = cv.take<uint32_t>(1);
+  p.count = cv.take<uint32_t>(2);
+  p.thr = cv.take<uint32_t>(4);
+  p.topk_scratch = cv.take<char>(topk_scratch_bytes());
   p.select_scratch = cv.take<char>(select_scratch_bytes(n, dtype));
+  p.list_scratch = cv.take<char>(select_scratch_bytes((int64_t)(2 * cap), dtype));
   p.sort_scratch = cv.take<char>(sort_scratch_bytes((int64_t)cap));
   p.bytes = cv.used;
   return p;
+}
+
+// Stage 1 of load balance: the selected (index, value) list in p.sel_*, its
+// length in p.count[0].  k > 0 asks for the k largest magnitudes (ties at the
+// threshold kept); then the threshold goes to p.thr[0..1].
+int select_stage(const BalancePlan &p, const void *input, int dtype, int64_t n, const uint32_t *thr, int64_t k,
+                 int64_t capacity, int mode, int32_t *status, hipStream_t s) {
+  SelectArgs sel;
+  sel.in = input;
+  sel.dtype = dtype;
+  sel.n = n;
+  sel.thr = thr;
+  sel.out_idx = p.sel_idx;
+  sel.out_val = p.sel_val;
+  sel.capacity = capacity;
+  sel.out_count32 = &p.count[0];
+  sel.ordered = false;  // the sort below fixes the order
+  sel.scratch = p.select_scratch;
+  sel.status = status;
+  if (k <= 0) return select_compact(sel, s);
+  int rc;
+  if (mode == ZEN_MODE_GENERAL || n < kSampleMinElems) {
+    // exact radix select over the whole tensor, then one compaction pass
+    if ((rc = topk_exact(input, dtype, n, nullptr, k, p.thr, p.topk_scratch, status, 0, s)) != ZEN_OK) return rc;
+    sel.thr = p.thr;
+    return select_compact(sel, s);
+  }
+  // one pass: compact everything at or above a floor estimated from a sample,
+  // find the exact threshold among those candidates, filter them
+  if ((rc = topk_sampled_floor(input, dtype, n, k, p.thr + 2, p.topk_scratch, status, s)) != ZEN_OK) return rc;
+  SelectArgs cand = sel;
+  cand.thr = p.thr + 2;
+  cand.out_idx = p.cand_idx;
+  cand.out_val = p.cand_val;
+  cand.capacity = 2 * capacity;
+  cand.out_count32 = &p.count[1];
+  if ((rc = select_compact(cand, s)) != ZEN_OK) return rc;
+  if ((rc = topk_exact(p.cand_val, dtype, 2 * capacity, &p.count[1], k, p.thr, p.topk_scratch, status,
+                       ZEN_STAT_RETRY, s)) != ZEN_OK)
+    return rc;
+  sel.in = p.cand_val;
+  sel.n = 2 * capacity;
+  sel.n_dev = &p.count[1];
+  sel.src_idx = p.cand_idx;
+  sel.thr = p.thr;
+  sel.scratch = p.list_scratch;
+  return select_compact(sel, s);
 }
 
 }  // namespace
@@ -329,13 +415,16 @@ size_t zen_load_balance_workspace(int64_t n, int dtype, int64_t capacity, int pa
 }
 
 int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
-                     const uint32_t *thr, int32_t *out_idx, void *out_val, int64_t capacity, int64_t *splits,
-                     int32_t *table, void *workspace, size_t workspace_bytes, int32_t *status, void *stream) {
+                     const uint32_t *thr, int64_t k, uint32_t *thr_out, int32_t *out_idx, void *out_val,
+                     int64_t capacity, int64_t *splits, int32_t *table, int mode, void *workspace,
+                     size_t workspace_bytes, int32_t *status, void *stream) {
   using namespace zen;
   if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_load_balance: bad dtype");
+  if (mode != ZEN_MODE_FAST && mode != ZEN_MODE_GENERAL) return fail(ZEN_EINVAL, "zen_load_balance: bad mode");
   if (n <= 0 || n > 0x7fffffffll || m <= 0 || m > 0x7fffffffll || partitions <= 0 || partitions > 65535 ||
-      m % partitions != 0 || capacity <= 0 || capacity > 0x7fffffffll)
-    return fail(ZEN_EINVAL, "zen_load_balance: need 0 < n, m < 2^31, m a multiple of partitions, capacity > 0");
+      m % partitions != 0 || capacity <= 0 || capacity > 0x3fffffffll)
+    return fail(ZEN_EINVAL, "zen_load_balance: need 0 < n, m < 2^31, m a multiple of partitions, 0 < capacity < 2^30");
+  if (k < 0 || k > n || (k > 0 && thr)) return fail(ZEN_EINVAL, "zen_load_balance: need 0 <= k <= n and no thr with k");
   if (!input || !out_idx || !out_val || !splits || !table || !workspace || !status)
     return fail(ZEN_EINVAL, "zen_load_balance: null pointer");
   if (workspace_bytes < zen_load_balance_workspace(n, dtype, capacity, partitions))
@@ -350,45 +439,51 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
   const int bits = ceil_log2_u64(drop_key);
   BalancePlan p = plan_balance(workspace, n, dtype, capacity);
 
-  int rc = select_compact(input, dtype, n, thr, p.cand_idx, 0, p.cand_val, capacity, nullptr, p.count,
-                          p.select_scratch, status, s);
+  int rc = select_stage(p, input, dtype, n, thr, k, capacity, mode, status, s);
   if (rc != ZEN_OK) return rc;
+  if (k > 0 && thr_out) ZEN_HIP_CHECK(hipMemcpyAsync(thr_out, p.thr, 2 * sizeof(uint32_t), hipMemcpyDeviceToDevice, s));
   const unsigned blocks = (unsigned)ceil_div(capacity, 256);
   {
     ProfScope prof(kProfInsertList, s);
-    k_insert_list<<<dim3(blocks), dim3(256), 0, s>>>(p.cand_idx, p.count, reinterpret_cast<uint32_t *>(table), g);
+    k_insert_list<<<dim3(blocks), dim3(256), 0, s>>>(p.sel_idx, p.count, reinterpret_cast<uint32_t *>(table), g);
     ZEN_LAUNCH_CHECK("k_insert_list");
   }
   {
     ProfScope prof(kProfFinalKey, s);
-    k_final_key<<<dim3(blocks), dim3(256), 0, s>>>(p.cand_idx, p.count, reinterpret_cast<uint32_t *>(table), g,
+    k_final_key<<<dim3(blocks), dim3(256), 0, s>>>(p.sel_idx, p.count, reinterpret_cast<uint32_t *>(table), g,
                                                    drop_key, p.keys_a, p.perm_a);
     ZEN_LAUNCH_CHECK("k_final_key");
   }
   int where;
   {
     ProfScope prof(kProfSort, s);
-    where = sort_pairs(p.keys_a, p.perm_a, p.keys_b, p.perm_b, capacity, p.count, bits, p.sort_scratch, s);
+    where = sort_pairs(p.keys_a, p.perm_a, p.keys_b, p.perm_b, capacity, p.count, bits, p.sort_scratch, status, s);
   }
   if (where < 0) return where;
   const uint32_t *sk = where ? p.keys_b : p.keys_a;
   const uint32_t *sp = where ? p.perm_b : p.perm_a;
   {
-  ProfScope prof(kProfGather, s);
-  if (dtype == ZEN_BF16)
-    k_gather<uint16_t><<<dim3(blocks), dim3(256), 0, s>>>(sk, sp, p.count, p.cand_idx,
-                                                          reinterpret_cast<const uint16_t *>(p.cand_val), drop_key, g,
-                                                          out_idx, static_cast<uint16_t *>(out_val),
-                                                          reinterpret_cast<uint32_t *>(table));
-  else
-    k_gather<uint32_t><<<dim3(blocks), dim3(256), 0, s>>>(sk, sp, p.count, p.cand_idx, p.cand_val, drop_key, g,
-                                                          out_idx, static_cast<uint32_t *>(out_val),
-                                                          reinterpret_cast<uint32_t *>(table));
-  ZEN_LAUNCH_CHECK("k_gather");
+    ProfScope prof(kProfGather, s);
+    if (dtype == ZEN_BF16)
+      k_gather<uint16_t><<<dim3(blocks), dim3(256), 0, s>>>(sk, sp, p.count, p.sel_idx,
+                                                            reinterpret_cast<const uint16_t *>(p.sel_val), drop_key, g,
+                                                            out_idx, static_cast<uint16_t *>(out_val),
+                                                            reinterpret_cast<uint32_t *>(table));
+    else
+      k_gather<uint32_t><<<dim3(blocks), dim3(256), 0, s>>>(sk, sp, p.count, p.sel_idx, p.sel_val, drop_key, g,
+                                                            out_idx, static_cast<uint32_t *>(out_val),
+                                                            reinterpret_cast<uint32_t *>(table));
+    ZEN_LAUNCH_CHECK("k_gather");
   }
-  k_splits<<<dim3((unsigned)ceil_div(partitions, 64)), dim3(64), 0, s>>>(sk, p.count, partitions, g.npp, spp, splits,
-                                                                        status);
-  ZEN_LAUNCH_CHECK("k_splits");
+  if (dtype == ZEN_BF16)
+    k_splits_serial<uint16_t><<<dim3((unsigned)partitions), dim3(256), 0, s>>>(
+        sk, p.count, g.npp, spp, static_cast<const uint16_t *>(input), out_idx, static_cast<uint16_t *>(out_val), splits,
+        status);
+  else
+    k_splits_serial<uint32_t><<<dim3((unsigned)partitions), dim3(256), 0, s>>>(
+        sk, p.count, g.npp, spp, static_cast<const uint32_t *>(input), out_idx, static_cast<uint32_t *>(out_val), splits,
+        status);
+  ZEN_LAUNCH_CHECK("k_splits_serial");
   return ZEN_OK;
 }
 

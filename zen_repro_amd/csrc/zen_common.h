@@ -187,15 +187,37 @@ __device__ inline T block_exclusive_scan(T v, T *smem, T *total) {
   return wave_base + incl - v;
 }
 
-// ----------------------------------------------- single-pass prefix (look-back)
-// One 64-bit descriptor per tile: 2 flag bits + 62 value bits, so flag and
-// value are published by one atomic store.  Tiles take their id from a ticket
-// counter, which guarantees that every lower-numbered tile already runs.
+// ------------------------------------------------ single-pass prefix over tiles
+// Decoupled look-back.  One 64-bit descriptor per tile holds 2 flag bits and a
+// 62-bit value, so flag and value are published by one atomic store: first the
+// tile's own count (aggregate), later its inclusive prefix.  A tile sums the
+// aggregates of its predecessors, 64 at a time, back to the nearest one that
+// already shows a prefix.  Tiles take their id from a ticket counter, so every
+// lower-numbered tile already runs and the wait cannot deadlock; it is also
+// bounded.  The prefix frontier advances 64 tiles per memory round trip, so
+// kernels keep their tile count in the low thousands.
+//
+// Scratch layout (all zero before the launch): ntiles descriptors and one
+// ticket word = scan_words(ntiles) uint64.
 
 constexpr uint64_t kDescAggregate = 1ull << 62;
 constexpr uint64_t kDescPrefix = 2ull << 62;
 constexpr uint64_t kDescValue = (1ull << 62) - 1;
 constexpr uint32_t kSpinLimit = 1u << 22;  // bounded wait: flag ZEN_STAT_INTERNAL instead of hanging
+
+inline size_t scan_words(int64_t ntiles) { return (size_t)ntiles + 2; }
+
+struct ScanState {
+  unsigned long long *desc;
+  uint32_t *ticket;
+};
+
+inline ScanState scan_state(void *scratch, int64_t ntiles) {
+  ScanState st;
+  st.desc = static_cast<unsigned long long *>(scratch);
+  st.ticket = reinterpret_cast<uint32_t *>(st.desc + ntiles);
+  return st;
+}
 
 __device__ inline uint64_t desc_load(const unsigned long long *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -206,8 +228,9 @@ __device__ inline void desc_store(unsigned long long *p, uint64_t v) {
 
 // Called by every thread of the block.  Returns the sum of the aggregates of
 // all tiles before `tile`.  smem: one uint64.
-__device__ inline uint64_t lookback_exclusive(unsigned long long *desc, int tile, uint64_t aggregate,
+__device__ inline uint64_t lookback_exclusive(const ScanState &st, int tile, uint64_t aggregate,
                                               int32_t *status, uint64_t *smem) {
+  unsigned long long *desc = st.desc;
   if (threadIdx.x < 64) {
     const int lane = lane_id();
     if (lane == 0) desc_store(&desc[tile], (tile == 0 ? kDescPrefix : kDescAggregate) | aggregate);
@@ -271,6 +294,6 @@ inline void launch_fill(T *p, T v, size_t count, hipStream_t s) {
 size_t sort_scratch_bytes(int64_t max_count);
 int sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *vals_b,
                int64_t max_count, const uint32_t *count_dev, int bits, void *scratch,
-               hipStream_t stream);
+               int32_t *status, hipStream_t stream);
 
 }  // namespace zen

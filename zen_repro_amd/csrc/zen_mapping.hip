@@ -49,9 +49,9 @@ size_t zen_mapping_workspace(int64_t n, int partitions) {
 }
 
 int zen_mapping(int64_t n, int partitions, int64_t *out, int64_t *counts, void *workspace, size_t workspace_bytes,
-                void *stream) {
+                int32_t *status, void *stream) {
   using namespace zen;
-  if (!out || !counts || !workspace) return fail(ZEN_EINVAL, "zen_mapping: null pointer");
+  if (!out || !counts || !workspace || !status) return fail(ZEN_EINVAL, "zen_mapping: null pointer");
   if (n <= 0 || n > 0x7fffffffll || partitions <= 0 || n / partitions == 0)
     return fail(ZEN_EINVAL, "zen_mapping: need 0 < partitions <= n < 2^31");
   if (workspace_bytes < zen_mapping_workspace(n, partitions)) return fail(ZEN_EWORKSPACE, "zen_mapping: workspace too small");
@@ -64,7 +64,7 @@ int zen_mapping(int64_t n, int partitions, int64_t *out, int64_t *counts, void *
   if (blocks > 65536) blocks = 65536;
   k_map_prep<<<dim3((unsigned)blocks), dim3(256), 0, s>>>((uint32_t)n, (uint32_t)(n / partitions), ka, va);
   ZEN_LAUNCH_CHECK("k_map_prep");
-  const int where = sort_pairs(ka, va, kb, vb, n, nullptr, ceil_log2_u64((uint64_t)partitions), scratch, s);
+  const int where = sort_pairs(ka, va, kb, vb, n, nullptr, ceil_log2_u64((uint64_t)partitions), scratch, status, s);
   if (where < 0) return where;
   const uint32_t *sk = where ? kb : ka, *sv = where ? vb : va;
   k_map_out<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(sk, sv, (uint32_t)n, (uint32_t)partitions, out);

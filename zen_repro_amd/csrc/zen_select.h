@@ -34,12 +34,43 @@ __device__ inline int load_vec(const S *__restrict__ in, int64_t first, int64_t 
 constexpr int kSelBlock = 256;
 constexpr int kSelVecs = 4;  // 16-byte vectors per thread and tile
 
-// Ascending (index, value) list of the elements with key >= max(thr[0], 1);
-// thr == nullptr means "nonzero".  out_count (int64) and out_count32 (clamped
-// to capacity) are optional.  scratch: select_scratch_bytes(n, dtype).
+// Compaction of the elements with key >= max(thr[0], 1) (thr == nullptr: the
+// nonzero ones) into (index, value) lists.
+struct SelectArgs {
+  const void *in = nullptr;           // dense tensor, or the values of a list
+  int dtype = ZEN_F32;
+  int64_t n = 0;                      // elements (capacity of the list when n_dev is set)
+  const uint32_t *n_dev = nullptr;    // optional device-side element count (<= n)
+  const uint32_t *thr = nullptr;      // optional device threshold key
+  const int32_t *src_idx = nullptr;   // list input: the index each element carries
+  void *out_idx = nullptr;
+  int idx64 = 0;                      // out_idx is int64 instead of int32
+  void *out_val = nullptr;
+  int64_t capacity = 0;
+  int64_t *out_count = nullptr;       // optional: number found (may exceed capacity)
+  uint32_t *out_count32 = nullptr;    // optional: the same clamped to capacity
+  bool ordered = true;                // ascending output (false: tiles in arrival order)
+  void *scratch = nullptr;            // select_scratch_bytes(n, dtype)
+  int32_t *status = nullptr;
+};
+
 size_t select_scratch_bytes(int64_t n, int dtype);
-int select_compact(const void *in, int dtype, int64_t n, const uint32_t *thr, void *out_idx, int idx64,
-                   void *out_val, int64_t capacity, int64_t *out_count, uint32_t *out_count32,
-                   void *scratch, int32_t *status, hipStream_t stream);
+int select_compact(const SelectArgs &args, hipStream_t stream);
+
+// Exact k-th largest magnitude key by radix select: thr[0] = key, thr[1] = number
+// of elements with key >= it.  `in` is a dense tensor or any array of values;
+// n_dev optionally holds the live element count.  Fewer than k elements:
+// thr = (0, count) and `short_bit` (if nonzero) is OR-ed into *status.
+size_t topk_scratch_bytes();
+int topk_exact(const void *in, int dtype, int64_t n, const uint32_t *n_dev, int64_t k, uint32_t *thr,
+               void *scratch, int32_t *status, int short_bit, hipStream_t stream);
+
+// Lower bound for that key from a 1/256 sample: thr_lo[0] is the lowest key of
+// the 11-bit magnitude bin in which the sample reaches the (padded) expected
+// rank.  Almost surely at least k elements of the tensor lie at or above it;
+// selecting them and running topk_exact on the selection gives the exact
+// threshold with one pass over the tensor (the caller checks the count).
+int topk_sampled_floor(const void *in, int dtype, int64_t n, int64_t k, uint32_t *thr_lo, void *scratch,
+                       int32_t *status, hipStream_t stream);
 
 }  // namespace zen

@@ -2,6 +2,8 @@
 // magnitude bit pattern (train.py:81-82), the masked dense copy
 // (train.py:83), and the ordered single-pass compaction that turns a dense
 // tensor into ascending (index, value) lists (comm.py:47-50).
+#include <math.h>
+
 #include "zen_select.h"
 
 namespace zen {
@@ -11,6 +13,7 @@ namespace {
 
 constexpr int kHistBins = 2048;
 constexpr int kHistBlock = 256;
+constexpr int kSampleLog2 = 8;  // the sample is one 16-byte vector in 256
 
 struct TopkState {
   uint32_t prefix;    // key bits fixed so far (right aligned)
@@ -32,12 +35,15 @@ __global__ void k_topk_init(TopkState *st, uint32_t *hist, uint32_t k) {
 // Histogram of the digit (key >> shift) & (2^width - 1) over elements whose
 // higher bits equal the prefix found so far.
 template <typename S, bool ALIGNED>
-__global__ __launch_bounds__(kHistBlock) void k_topk_hist(const S *__restrict__ in, int64_t n,
+__global__ __launch_bounds__(kHistBlock) void k_topk_hist(const S *__restrict__ in, int64_t n_max,
+                                                          const uint32_t *__restrict__ n_dev,
                                                           const TopkState *__restrict__ st, int shift,
                                                           int width, int pass,
                                                           uint32_t *__restrict__ hist) {
   constexpr int V = VecOf<S>::kN;
   __shared__ uint32_t bins[kHistBins];
+  int64_t n = n_max;
+  if (n_dev && (int64_t)*n_dev < n) n = (int64_t)*n_dev;
   for (int i = threadIdx.x; i < kHistBins; i += kHistBlock) bins[i] = 0;
   __syncthreads();
   const uint32_t prefix = st->prefix;
@@ -63,9 +69,12 @@ __global__ __launch_bounds__(kHistBlock) void k_topk_hist(const S *__restrict__ 
 }
 
 // One block: find the digit that holds the k_rem-th largest match, extend the
-// prefix, clear the histogram for the next pass.
-__global__ __launch_bounds__(kHistBlock) void k_topk_pick(TopkState *st, uint32_t *hist, int width,
-                                                          int last, uint32_t *thr_out) {
+// prefix, clear the histogram for the next pass.  On the last pass the result
+// goes to thr_out as (prefix << final_shift, number of elements >= it).  Fewer
+// than k_rem matches: thr_out = (0, matches) and `short_bit` is raised.
+__global__ __launch_bounds__(kHistBlock) void k_topk_pick(TopkState *st, uint32_t *hist, int width, int last,
+                                                          int final_shift, uint32_t *thr_out, int32_t *status,
+                                                          int short_bit) {
   constexpr int kPer = kHistBins / kHistBlock;
   __shared__ uint32_t smem[kHistBlock / 64 + 1];
   const uint32_t prefix = st->prefix, k_rem = st->k_rem, count_gt = st->count_gt;
@@ -80,23 +89,64 @@ __global__ __launch_bounds__(kHistBlock) void k_topk_pick(TopkState *st, uint32_
   uint32_t total;
   uint32_t above = block_exclusive_scan<uint32_t, kHistBlock>(mine, smem, &total);
   __syncthreads();
-#pragma unroll
-  for (int j = 0; j < kPer; ++j) {
-    if (above < k_rem && k_rem <= above + c[j]) {
-      const uint32_t bin = kHistBins - 1 - (threadIdx.x * kPer + j);
-      const uint32_t np = (prefix << width) | bin;
-      st->prefix = np;
-      st->k_rem = k_rem - above;
-      st->count_gt = count_gt + above;
+  if (total < k_rem) {
+    if (threadIdx.x == 0) {
+      st->prefix = 0;
       if (last) {
-        thr_out[0] = np;
-        thr_out[1] = count_gt + above + c[j];
+        thr_out[0] = 0;
+        thr_out[1] = count_gt + total;
       }
+      if (short_bit) atomicOr(status, short_bit);
     }
-    above += c[j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      if (above < k_rem && k_rem <= above + c[j]) {
+        const uint32_t bin = kHistBins - 1 - (threadIdx.x * kPer + j);
+        const uint32_t np = (prefix << width) | bin;
+        st->prefix = np;
+        st->k_rem = k_rem - above;
+        st->count_gt = count_gt + above;
+        if (last) {
+          thr_out[0] = np << final_shift;
+          thr_out[1] = count_gt + above + c[j];
+        }
+      }
+      above += c[j];
+    }
   }
 #pragma unroll
   for (int j = 0; j < kPer; ++j) hist[kHistBins - 1 - (threadIdx.x * kPer + j)] = 0;
+}
+
+// Histogram of the top 11 key bits over a sample: one 16-byte vector out of
+// every 2^block_log2 consecutive vectors, at a pseudo-random place inside its
+// block so that regular layouts (rows, columns) are not sampled in lockstep.
+template <typename S, bool ALIGNED>
+__global__ __launch_bounds__(kHistBlock) void k_sample_hist(const S *__restrict__ in, int64_t n, int block_log2,
+                                                            uint32_t *__restrict__ hist) {
+  constexpr int V = VecOf<S>::kN;
+  constexpr int kShift = KeyOf<S>::kBits - 11;
+  __shared__ uint32_t bins[kHistBins];
+  for (int i = threadIdx.x; i < kHistBins; i += kHistBlock) bins[i] = 0;
+  __syncthreads();
+  const int64_t nvec = (n + V - 1) / V;
+  const int64_t nblocks = (nvec + (1ll << block_log2) - 1) >> block_log2;
+  for (int64_t b = blockIdx.x * (int64_t)kHistBlock + threadIdx.x; b < nblocks;
+       b += (int64_t)gridDim.x * kHistBlock) {
+    const int64_t v = (b << block_log2) + (poly((uint32_t)b) >> 7 & ((1u << block_log2) - 1u));
+    if (v >= nvec) continue;
+    S e[V];
+    const int live = load_vec<S, ALIGNED>(in, v * V, n, e);
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+      if (i < live) atomicAdd(&bins[(e[i] & KeyOf<S>::kMask) >> kShift], 1u);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < kHistBins; i += kHistBlock) {
+    const uint32_t c = bins[i];
+    if (c) atomicAdd(&hist[i], c);
+  }
 }
 
 // ------------------------------------------------------------- masked copy
@@ -125,99 +175,206 @@ __global__ __launch_bounds__(256) void k_compress(const S *__restrict__ in, int6
 
 }  // namespace
 
-// ------------------------------------------------------ ordered compaction
+// ------------------------------------------------------ stream compaction
 //
-// A tile is `subs` consecutive sub-tiles of kSelBlock * kSelVecs 16-byte
-// vectors.  A block walks its tile once, staging the selected (index, value)
-// pairs in LDS in ascending order; only then does it need the number of
-// selected elements in all earlier tiles, which it gets by look-back over one
-// descriptor per tile.  Large tiles keep the descriptor chain short (the
-// look-back frontier advances 64 tiles per memory round trip), the LDS stage
-// makes the write-out coalesced.  A tile with more selected elements than the
-// stage holds is walked a second time and written directly.
+// A tile is `subs` consecutive sub-tiles; in a sub-tile every thread owns
+// kSelVecs consecutive 16-byte vectors (64 contiguous bytes), so element order
+// is thread order and one block scan of per-thread counts places everything.
+// A block walks its tile once, staging the selected (index, value) pairs in
+// LDS in ascending order; only then does it need its place in the output.
+// Ordered mode gets it from the tile-prefix protocol (the output is ascending
+// in the index); unordered mode reserves a range with one atomic add (tiles
+// land in arrival order, each tile's entries stay ascending), which callers
+// that sort afterwards prefer because no tile ever waits.  The LDS stage makes
+// the write-out coalesced.  A tile with more selected elements than the stage
+// holds is walked a second time and written directly.
+//
+// A CDNA compute unit retires 64 lane-operations per clock while HBM delivers
+// about 8 bytes per clock and unit, so a bf16 stream has ~16 operations per
+// element before the vector ALU, not memory, sets the pace.  The predicate is
+// therefore evaluated two bf16 at a time on packed words (3 operations per
+// pair), the flags of a thread's 32 elements end in one register, and only the
+// few selected elements take the longer extraction path.
+// The input is a dense tensor (an element's index is its position) or a list
+// (src_idx gives the index carried by each element).
 
-constexpr int kSelStage = 4096;  // staged pairs per tile
+constexpr int kSelStage = 4096;    // staged pairs per tile
+constexpr int kReserveShift = 40;  // unordered mode: tiles done above, entries reserved below
+
+// Inclusive prefix sum across the 64 lanes with DPP row shifts and broadcasts.
+__device__ inline uint32_t wave_inclusive_scan_dpp(uint32_t x) {
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x111, 0xf, 0xf, false);  // row_shr:1
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x112, 0xf, 0xf, false);  // row_shr:2
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x114, 0xf, 0xf, false);  // row_shr:4
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x118, 0xf, 0xf, false);  // row_shr:8
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1,3
+  x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2,3
+  return x;
+}
+
+// Flags of the elements a thread owns in one sub-tile, one bit per element,
+// plus the translation between bit positions and element offsets.
+template <typename S>
+struct Flags;
+
+// bf16: element (vector j, word w, half h) sits at bit 4j + w + 16h, i.e. the
+// even elements fill the low half-word and the odd ones the high half-word.
+template <>
+struct Flags<uint16_t> {
+  static constexpr int kElems = kSelVecs * 8;
+  static __device__ inline uint32_t build(const uint4 (&q)[kSelVecs], uint32_t floor_key) {
+    // per 16-bit lane: key + (0x8000 - floor) carries into bit 15 iff key >= floor
+    const uint32_t c = (0x8000u - floor_key) * 0x00010001u;
+    uint32_t x = 0;
+#pragma unroll
+    for (int j = 0; j < kSelVecs; ++j) {
+      const uint32_t m0 = ((q[j].x & 0x7fff7fffu) + c) & 0x80008000u;
+      const uint32_t m1 = ((q[j].y & 0x7fff7fffu) + c) & 0x80008000u;
+      const uint32_t m2 = ((q[j].z & 0x7fff7fffu) + c) & 0x80008000u;
+      const uint32_t m3 = ((q[j].w & 0x7fff7fffu) + c) & 0x80008000u;
+      const uint32_t v = (m0 >> 15) | (m1 >> 14) | (m2 >> 13) | (m3 >> 12);  // bits 0-3 and 16-19
+      x |= v << (4 * j);
+    }
+    return x;
+  }
+  // flags of the elements whose offset is below `count`
+  static __device__ inline uint32_t below(int count) {
+    const int a = (count >> 3) * 4 + ((count & 7) >> 1), h = count & 1;
+    return (uint32_t)((1ull << (a + h)) - 1ull) | ((uint32_t)((1ull << a) - 1ull) << 16);
+  }
+  static __device__ inline int offset_of(int bit) {  // element offset of a flag bit
+    const int a = bit & 15;
+    return ((a >> 2) << 3) + ((a & 3) << 1) + (bit >> 4);
+  }
+};
+
+// fp32: element e sits at bit e.
+template <>
+struct Flags<uint32_t> {
+  static constexpr int kElems = kSelVecs * 4;
+  static __device__ inline uint32_t build(const uint4 (&q)[kSelVecs], uint32_t floor_key) {
+    uint32_t x = 0;
+#pragma unroll
+    for (int j = 0; j < kSelVecs; ++j) {
+      x |= (uint32_t)((q[j].x & 0x7fffffffu) >= floor_key) << (4 * j);
+      x |= (uint32_t)((q[j].y & 0x7fffffffu) >= floor_key) << (4 * j + 1);
+      x |= (uint32_t)((q[j].z & 0x7fffffffu) >= floor_key) << (4 * j + 2);
+      x |= (uint32_t)((q[j].w & 0x7fffffffu) >= floor_key) << (4 * j + 3);
+    }
+    return x;
+  }
+  static __device__ inline uint32_t below(int count) { return (uint32_t)((1ull << count) - 1ull); }
+  static __device__ inline int offset_of(int bit) { return bit; }
+};
 
 template <typename S, typename I, bool ALIGNED, bool STAGED>
 __device__ inline uint32_t select_walk_tile(const S *__restrict__ in, int64_t n, uint32_t floor_key,
-                                            int64_t tile_base, int subs, uint64_t *s_scan, int32_t *st_idx,
-                                            S *st_val, I *__restrict__ out_idx, S *__restrict__ out_val,
-                                            uint64_t out_base, int64_t capacity) {
+                                            int64_t tile_base, int subs, const int32_t *__restrict__ src_idx,
+                                            uint32_t *s_wave, int32_t *st_idx, S *st_val, I *__restrict__ out_idx,
+                                            S *__restrict__ out_val, uint64_t out_base, int64_t capacity) {
   constexpr int V = VecOf<S>::kN;
-  constexpr int kSub = kSelBlock * kSelVecs * V;
+  constexpr int kChunk = Flags<S>::kElems;  // elements per thread and sub-tile
+  constexpr int kSub = kSelBlock * kChunk;
+  const int wave = threadIdx.x >> 6;
   uint32_t running = 0;
   for (int sub = 0; sub < subs; ++sub) {
     const int64_t sub_base = tile_base + (int64_t)sub * kSub;
     if (sub_base >= n) break;
-    S e[kSelVecs][V];
-    uint32_t bits[kSelVecs];
-    uint64_t packed = 0;  // four 16-bit counters, one per vector of this thread
+    const int64_t first = sub_base + (int64_t)threadIdx.x * kChunk;
+    uint4 q[kSelVecs];
+    if (ALIGNED && first + kChunk <= n) {
+      const uint4 *src = reinterpret_cast<const uint4 *>(in + first);
 #pragma unroll
-    for (int j = 0; j < kSelVecs; ++j) {
-      const int64_t first = sub_base + ((int64_t)j * kSelBlock + threadIdx.x) * V;
-      const int live = first < n ? load_vec<S, ALIGNED>(in, first, n, e[j]) : 0;
-      uint32_t b = 0;
+      for (int j = 0; j < kSelVecs; ++j) q[j] = src[j];
+    } else {
 #pragma unroll
-      for (int i = 0; i < V; ++i)
-        if (i < live && (e[j][i] & KeyOf<S>::kMask) >= floor_key) b |= 1u << i;
-      bits[j] = b;
-      packed |= (uint64_t)__popc(b) << (16 * j);
-    }
-    uint64_t totals;
-    const uint64_t before = block_exclusive_scan<uint64_t, kSelBlock>(packed, s_scan, &totals);
-    uint32_t vec_start = running;
-#pragma unroll
-    for (int j = 0; j < kSelVecs; ++j) {
-      uint32_t pos = vec_start + (uint32_t)((before >> (16 * j)) & 0xffffu);
-      const int64_t first = sub_base + ((int64_t)j * kSelBlock + threadIdx.x) * V;
-      const uint32_t b = bits[j];
-#pragma unroll
-      for (int i = 0; i < V; ++i) {
-        if (b & (1u << i)) {
-          if (STAGED) {
-            if (pos < (uint32_t)kSelStage) {
-              st_idx[pos] = (int32_t)(first + i);
-              st_val[pos] = e[j][i];
-            }
-          } else if (out_base + pos < (uint64_t)capacity) {
-            out_idx[out_base + pos] = (I)(first + i);
-            out_val[out_base + pos] = e[j][i];
-          }
-          ++pos;
-        }
+      for (int j = 0; j < kSelVecs; ++j) {
+        S e[V];
+        load_vec<S, false>(in, first + j * V, n, e);
+        __builtin_memcpy(&q[j], e, 16);
       }
-      vec_start += (uint32_t)((totals >> (16 * j)) & 0xffffu);
     }
-    running = vec_start;
+    uint32_t x = Flags<S>::build(q, floor_key);
+    if (first + kChunk > n) x &= first < n ? Flags<S>::below((int)(n - first)) : 0u;
+    const uint32_t cnt = (uint32_t)__popc(x);
+    // block-wide exclusive prefix of cnt
+    const uint32_t incl = wave_inclusive_scan_dpp(cnt);
+    if ((threadIdx.x & 63) == 63) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t before = running + incl - cnt, total = 0;
+#pragma unroll
+    for (int w = 0; w < kSelBlock / 64; ++w) {
+      const uint32_t t = s_wave[w];
+      if (w < wave) before += t;
+      total += t;
+    }
+    __syncthreads();
+    const uint32_t all = x;
+    while (x) {
+      const int bit = __ffs((int)x) - 1;
+      x &= x - 1;
+      const int off = Flags<S>::offset_of(bit);
+      const uint32_t pos = before + (uint32_t)__popc(all & Flags<S>::below(off));
+      const S v = in[first + off];  // just streamed through the cache; selected elements are few
+      if (STAGED) {
+        if (pos < (uint32_t)kSelStage) {
+          st_idx[pos] = (int32_t)(first + off);
+          st_val[pos] = v;
+        }
+      } else if (out_base + pos < (uint64_t)capacity) {
+        out_idx[out_base + pos] = (I)(src_idx ? src_idx[first + off] : first + off);
+        out_val[out_base + pos] = v;
+      }
+    }
+    running += total;
   }
   return running;
 }
 
-template <typename S, typename I, bool ALIGNED>
+template <typename S, typename I, bool ALIGNED, bool ORDERED>
 __global__ __launch_bounds__(kSelBlock) void k_select_compact(
-    const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, I *__restrict__ out_idx,
-    S *__restrict__ out_val, int64_t capacity, unsigned long long *desc, uint32_t *ticket, int ntiles, int subs,
-    int64_t *out_count, uint32_t *out_count32, int32_t *status) {
-  constexpr int V = VecOf<S>::kN;
-  constexpr int kSub = kSelBlock * kSelVecs * V;
-  __shared__ uint64_t s_scan[kSelBlock / 64 + 1];
+    const S *__restrict__ in, int64_t n_max, const uint32_t *__restrict__ n_dev, const uint32_t *__restrict__ thr,
+    const int32_t *__restrict__ src_idx, I *__restrict__ out_idx, S *__restrict__ out_val, int64_t capacity,
+    ScanState st, int ntiles, int subs, int64_t *out_count, uint32_t *out_count32, int32_t *status) {
+  constexpr int kSub = kSelBlock * Flags<S>::kElems;
+  __shared__ uint32_t s_wave[kSelBlock / 64];
   __shared__ uint64_t s_bcast;
   __shared__ int s_tile;
   __shared__ int32_t st_idx[kSelStage];
   __shared__ S st_val[kSelStage];
-  if (threadIdx.x == 0) s_tile = (int)atomicAdd(ticket, 1u);
-  __syncthreads();
-  const int tile = s_tile;
-  if (tile >= ntiles) return;
+  int tile = (int)blockIdx.x;
+  if (ORDERED) {
+    if (threadIdx.x == 0) s_tile = (int)atomicAdd(st.ticket, 1u);
+    __syncthreads();
+    tile = s_tile;
+    if (tile >= ntiles) return;
+  }
+  int64_t n = n_max;
+  if (n_dev && (int64_t)*n_dev < n) n = (int64_t)*n_dev;
   uint32_t floor_key = thr ? thr[0] : 1u;
   if (floor_key == 0) floor_key = 1u;  // zeros are never selected
+  if (floor_key > KeyOf<S>::kMask) floor_key = KeyOf<S>::kMask + 1u;  // nothing qualifies
   const int64_t tile_base = (int64_t)tile * subs * kSub;
 
-  const uint32_t found = select_walk_tile<S, I, ALIGNED, true>(in, n, floor_key, tile_base, subs, s_scan, st_idx,
-                                                               st_val, out_idx, out_val, 0, capacity);
-  const uint64_t tile_start = lookback_exclusive(desc, tile, found, status, &s_bcast);
-  if (tile == ntiles - 1 && threadIdx.x == 0) {
-    const uint64_t all = tile_start + found;
+  const uint32_t found = select_walk_tile<S, I, ALIGNED, true>(in, n, floor_key, tile_base, subs, src_idx, s_wave,
+                                                               st_idx, st_val, out_idx, out_val, 0, capacity);
+  uint64_t tile_start, all = 0;
+  bool last;
+  if (ORDERED) {
+    tile_start = lookback_exclusive(st, tile, found, status, &s_bcast);
+    last = tile == ntiles - 1;
+    all = tile_start + found;
+  } else {
+    if (threadIdx.x == 0)
+      s_bcast = __hip_atomic_fetch_add(st.desc, (1ull << kReserveShift) | found, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const uint64_t old = s_bcast;
+    tile_start = old & ((1ull << kReserveShift) - 1);
+    last = (int)(old >> kReserveShift) == ntiles - 1;  // every other tile has reserved already
+    all = tile_start + found;
+  }
+  if (last && threadIdx.x == 0) {
     if (out_count) *out_count = (int64_t)all;
     if (out_count32) *out_count32 = (uint32_t)(all < (uint64_t)capacity ? all : (uint64_t)capacity);
     if (all > (uint64_t)capacity) atomicOr(status, ZEN_STAT_CAPACITY);
@@ -226,18 +383,20 @@ __global__ __launch_bounds__(kSelBlock) void k_select_compact(
     for (uint32_t i = threadIdx.x; i < found; i += kSelBlock) {
       const uint64_t pos = tile_start + i;
       if (pos < (uint64_t)capacity) {
-        out_idx[pos] = (I)st_idx[i];
+        const int32_t at = st_idx[i];
+        out_idx[pos] = (I)(src_idx ? src_idx[at] : at);
         out_val[pos] = st_val[i];
       }
     }
   } else {
-    select_walk_tile<S, I, ALIGNED, false>(in, n, floor_key, tile_base, subs, s_scan, st_idx, st_val, out_idx,
-                                           out_val, tile_start, capacity);
+    select_walk_tile<S, I, ALIGNED, false>(in, n, floor_key, tile_base, subs, src_idx, s_wave, st_idx, st_val,
+                                           out_idx, out_val, tile_start, capacity);
   }
 }
 
-// Sub-tiles per tile: large tiles for large inputs, but never so large that
-// the grid falls below a few workgroups per compute unit.
+// Sub-tiles per tile: large tiles for large inputs (few descriptors, few
+// atomics), but never so large that the grid falls below a few workgroups per
+// compute unit.
 static int select_subs(int64_t n, int dtype) {
   const int v = dtype == ZEN_BF16 ? 8 : 4;
   const int64_t sub = (int64_t)kSelBlock * kSelVecs * v;
@@ -250,58 +409,49 @@ size_t select_scratch_bytes(int64_t n, int dtype) {
   const int v = dtype == ZEN_BF16 ? 8 : 4;
   const int64_t tile = (int64_t)kSelBlock * kSelVecs * v * select_subs(n > 0 ? n : 1, dtype);
   const int64_t ntiles = ceil_div(n > 0 ? n : 1, tile);
-  return align_up((size_t)(ntiles + 2) * sizeof(unsigned long long), 256);
+  return align_up(scan_words(ntiles) * sizeof(unsigned long long), 256);
 }
 
 template <typename S, typename I>
-static int select_launch(const S *in, int64_t n, const uint32_t *thr, I *out_idx, S *out_val,
-                         int64_t capacity, int64_t *out_count, uint32_t *out_count32, void *scratch,
-                         int32_t *status, hipStream_t stream) {
+static int select_launch(const SelectArgs &a, hipStream_t stream) {
   constexpr int V = VecOf<S>::kN;
-  const int subs = select_subs(n, sizeof(S) == 2 ? ZEN_BF16 : ZEN_F32);
+  const int subs = select_subs(a.n, a.dtype);
   const int64_t tile = (int64_t)kSelBlock * kSelVecs * V * subs;
-  const int64_t ntiles = ceil_div(n, tile);
-  if (ntiles > 0x7fffffff) return fail(ZEN_EINVAL, "select: too many tiles");
-  // descriptors followed by the ticket counter, cleared together
-  unsigned long long *desc = static_cast<unsigned long long *>(scratch);
-  uint32_t *ticket = reinterpret_cast<uint32_t *>(desc + ntiles);
-  launch_fill<unsigned long long>(desc, 0ull, (size_t)ntiles + 1, stream);
-  ZEN_LAUNCH_CHECK("select: clear descriptors");
+  const int64_t ntiles = ceil_div(a.n, tile);
+  if (ntiles > 0xffffff) return fail(ZEN_EINVAL, "select: too many tiles");
+  const ScanState st = scan_state(a.scratch, ntiles);
+  launch_fill<unsigned long long>(st.desc, 0ull, a.ordered ? scan_words(ntiles) : 1, stream);
+  ZEN_LAUNCH_CHECK("select: clear scan state");
+  const S *in = static_cast<const S *>(a.in);
+  I *out_idx = static_cast<I *>(a.out_idx);
+  S *out_val = static_cast<S *>(a.out_val);
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+  const dim3 grid((unsigned)ntiles), block(kSelBlock);
   ProfScope prof(kProfSelectCompact, stream);
-  if (aligned)
-    k_select_compact<S, I, true><<<dim3((unsigned)ntiles), dim3(kSelBlock), 0, stream>>>(
-        in, n, thr, out_idx, out_val, capacity, desc, ticket, (int)ntiles, subs, out_count, out_count32, status);
-  else
-    k_select_compact<S, I, false><<<dim3((unsigned)ntiles), dim3(kSelBlock), 0, stream>>>(
-        in, n, thr, out_idx, out_val, capacity, desc, ticket, (int)ntiles, subs, out_count, out_count32, status);
+#define ZEN_SELECT_GO(AL, ORD)                                                                                 \
+  k_select_compact<S, I, AL, ORD><<<grid, block, 0, stream>>>(in, a.n, a.n_dev, a.thr, a.src_idx, out_idx,   \
+                                                              out_val, a.capacity, st, (int)ntiles, subs,    \
+                                                              a.out_count, a.out_count32, a.status)
+  if (aligned && a.ordered) ZEN_SELECT_GO(true, true);
+  else if (aligned) ZEN_SELECT_GO(true, false);
+  else if (a.ordered) ZEN_SELECT_GO(false, true);
+  else ZEN_SELECT_GO(false, false);
+#undef ZEN_SELECT_GO
   ZEN_LAUNCH_CHECK("k_select_compact");
   return ZEN_OK;
 }
 
-int select_compact(const void *in, int dtype, int64_t n, const uint32_t *thr, void *out_idx, int idx64,
-                   void *out_val, int64_t capacity, int64_t *out_count, uint32_t *out_count32,
-                   void *scratch, int32_t *status, hipStream_t stream) {
-  if (dtype == ZEN_BF16) {
-    auto *p = static_cast<const uint16_t *>(in);
-    auto *v = static_cast<uint16_t *>(out_val);
-    return idx64 ? select_launch<uint16_t, int64_t>(p, n, thr, static_cast<int64_t *>(out_idx), v, capacity,
-                                                    out_count, out_count32, scratch, status, stream)
-                 : select_launch<uint16_t, int32_t>(p, n, thr, static_cast<int32_t *>(out_idx), v, capacity,
-                                                    out_count, out_count32, scratch, status, stream);
-  }
-  auto *p = static_cast<const uint32_t *>(in);
-  auto *v = static_cast<uint32_t *>(out_val);
-  return idx64 ? select_launch<uint32_t, int64_t>(p, n, thr, static_cast<int64_t *>(out_idx), v, capacity,
-                                                  out_count, out_count32, scratch, status, stream)
-               : select_launch<uint32_t, int32_t>(p, n, thr, static_cast<int32_t *>(out_idx), v, capacity,
-                                                  out_count, out_count32, scratch, status, stream);
+int select_compact(const SelectArgs &a, hipStream_t stream) {
+  if (a.dtype == ZEN_BF16)
+    return a.idx64 ? select_launch<uint16_t, int64_t>(a, stream) : select_launch<uint16_t, int32_t>(a, stream);
+  return a.idx64 ? select_launch<uint32_t, int64_t>(a, stream) : select_launch<uint32_t, int32_t>(a, stream);
 }
 
 namespace {
 
 template <typename S>
-int topk_launch(const S *in, int64_t n, int64_t k, uint32_t *thr, void *workspace, hipStream_t stream) {
+int topk_launch(const S *in, int64_t n, const uint32_t *n_dev, int64_t k, uint32_t *thr, void *workspace,
+                int32_t *status, int short_bit, hipStream_t stream) {
   Carver cv(workspace);
   TopkState *st = cv.take<TopkState>(1);
   uint32_t *hist = cv.take<uint32_t>(kHistBins);
@@ -323,16 +473,47 @@ int topk_launch(const S *in, int64_t n, int64_t k, uint32_t *thr, void *workspac
     {
       ProfScope prof(kProfTopkHist, stream);
       if (aligned)
-        k_topk_hist<S, true><<<dim3((unsigned)blocks), dim3(kHistBlock), 0, stream>>>(in, n, st, shift,
+        k_topk_hist<S, true><<<dim3((unsigned)blocks), dim3(kHistBlock), 0, stream>>>(in, n, n_dev, st, shift,
                                                                                       widths[p], p, hist);
       else
-        k_topk_hist<S, false><<<dim3((unsigned)blocks), dim3(kHistBlock), 0, stream>>>(in, n, st, shift,
+        k_topk_hist<S, false><<<dim3((unsigned)blocks), dim3(kHistBlock), 0, stream>>>(in, n, n_dev, st, shift,
                                                                                        widths[p], p, hist);
       ZEN_LAUNCH_CHECK("k_topk_hist");
     }
-    k_topk_pick<<<dim3(1), dim3(kHistBlock), 0, stream>>>(st, hist, widths[p], p == npass - 1, thr);
+    k_topk_pick<<<dim3(1), dim3(kHistBlock), 0, stream>>>(st, hist, widths[p], p == npass - 1, 0, thr, status,
+                                                          short_bit);
     ZEN_LAUNCH_CHECK("k_topk_pick");
   }
+  return ZEN_OK;
+}
+
+template <typename S>
+int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *workspace, int32_t *status,
+                  hipStream_t stream) {
+  constexpr int V = VecOf<S>::kN;
+  Carver cv(workspace);
+  TopkState *st = cv.take<TopkState>(1);
+  uint32_t *hist = cv.take<uint32_t>(kHistBins);
+  const int64_t nvec = ceil_div(n, V);
+  const int64_t nblocks = ceil_div(nvec, 1ll << kSampleLog2);
+  // rank to look for in the sample: the expected one plus six standard
+  // deviations of a binomial count, so that the full tensor almost surely holds
+  // at least k elements at or above the bin found (callers verify and retry)
+  const double expect = (double)k * ((double)nblocks * V) / (double)n;
+  const double want = expect + 6.0 * sqrt(expect) + 16.0;
+  const uint32_t rank = want > 4.0e9 ? 0xffffffffu : (uint32_t)want;
+  k_topk_init<<<dim3(1), dim3(256), 0, stream>>>(st, hist, rank);
+  ZEN_LAUNCH_CHECK("k_topk_init");
+  int64_t blocks = ceil_div(nblocks, kHistBlock);
+  if (blocks > 512) blocks = 512;
+  const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+  if (aligned)
+    k_sample_hist<S, true><<<dim3((unsigned)blocks), dim3(kHistBlock), 0, stream>>>(in, n, kSampleLog2, hist);
+  else
+    k_sample_hist<S, false><<<dim3((unsigned)blocks), dim3(kHistBlock), 0, stream>>>(in, n, kSampleLog2, hist);
+  ZEN_LAUNCH_CHECK("k_sample_hist");
+  k_topk_pick<<<dim3(1), dim3(kHistBlock), 0, stream>>>(st, hist, 11, 1, KeyOf<S>::kBits - 11, thr_lo, status, 0);
+  ZEN_LAUNCH_CHECK("k_topk_pick");
   return ZEN_OK;
 }
 
@@ -354,13 +535,28 @@ int compress_launch(const S *in, int64_t n, const uint32_t *thr, S *out, hipStre
 }
 
 }  // namespace
+
+size_t topk_scratch_bytes() { return align_up(sizeof(TopkState), 256) + align_up(kHistBins * sizeof(uint32_t), 256); }
+
+int topk_exact(const void *in, int dtype, int64_t n, const uint32_t *n_dev, int64_t k, uint32_t *thr,
+               void *scratch, int32_t *status, int short_bit, hipStream_t stream) {
+  if (dtype == ZEN_BF16)
+    return topk_launch(static_cast<const uint16_t *>(in), n, n_dev, k, thr, scratch, status, short_bit, stream);
+  return topk_launch(static_cast<const uint32_t *>(in), n, n_dev, k, thr, scratch, status, short_bit, stream);
+}
+
+int topk_sampled_floor(const void *in, int dtype, int64_t n, int64_t k, uint32_t *thr_lo, void *scratch,
+                       int32_t *status, hipStream_t stream) {
+  if (dtype == ZEN_BF16)
+    return sample_launch(static_cast<const uint16_t *>(in), n, k, thr_lo, scratch, status, stream);
+  return sample_launch(static_cast<const uint32_t *>(in), n, k, thr_lo, scratch, status, stream);
+}
+
 }  // namespace zen
 
 extern "C" {
 
-size_t zen_topk_threshold_workspace(void) {
-  return zen::align_up(sizeof(zen::TopkState), 256) + zen::align_up(zen::kHistBins * sizeof(uint32_t), 256);
-}
+size_t zen_topk_threshold_workspace(void) { return zen::topk_scratch_bytes(); }
 
 int zen_topk_threshold(const void *input, int dtype, int64_t n, int64_t k, uint32_t *thr, void *workspace,
                        size_t workspace_bytes, void *stream) {
@@ -370,8 +566,7 @@ int zen_topk_threshold(const void *input, int dtype, int64_t n, int64_t k, uint3
   if (n <= 0 || n > 0x7fffffffll || k < 1 || k > n) return fail(ZEN_EINVAL, "zen_topk_threshold: need 1 <= k <= n < 2^31");
   if (workspace_bytes < zen_topk_threshold_workspace()) return fail(ZEN_EWORKSPACE, "zen_topk_threshold: workspace too small");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == ZEN_BF16) return topk_launch(static_cast<const uint16_t *>(input), n, k, thr, workspace, s);
-  return topk_launch(static_cast<const uint32_t *>(input), n, k, thr, workspace, s);
+  return topk_exact(input, dtype, n, nullptr, k, thr, workspace, nullptr, 0, s);
 }
 
 int zen_compress(const void *input, int dtype, int64_t n, const uint32_t *thr, void *out, void *stream) {
@@ -404,8 +599,20 @@ int zen_select(const void *input, int dtype, int64_t n, const uint32_t *thr, voi
   if (!input || !workspace || (capacity > 0 && (!out_idx || !out_val)))
     return fail(ZEN_EINVAL, "zen_select: null pointer");
   if (workspace_bytes < zen_select_workspace(n, dtype)) return fail(ZEN_EWORKSPACE, "zen_select: workspace too small");
-  return select_compact(input, dtype, n, thr, out_idx, idx64, out_val, capacity, out_count, nullptr,
-                        workspace, status, s);
+  SelectArgs a;
+  a.in = input;
+  a.dtype = dtype;
+  a.n = n;
+  a.thr = thr;
+  a.out_idx = out_idx;
+  a.idx64 = idx64;
+  a.out_val = out_val;
+  a.capacity = capacity;
+  a.out_count = out_count;
+  a.ordered = true;
+  a.scratch = workspace;
+  a.status = status;
+  return select_compact(a, s);
 }
 
 }  // extern "C"

@@ -73,11 +73,15 @@ class TensorPartition:
             self._tables[key] = t
         return t
 
-    def load_balance_flat(self, tensor, thr=None, capacity=None):
+    def load_balance_flat(self, tensor, thr=None, capacity=None, k=0, mode=_lib.MODE_FAST, thr_out=None):
         """Fused path without host synchronisation.  Returns (indices int32
         [capacity], values [capacity], splits int64[P] on device, status int32[1]
         on device); the first splits.sum() entries are valid, partition-major.
-        `thr` is the device tensor written by topk_threshold (None: nonzeros)."""
+        Selection: `k` > 0 keeps the k largest magnitudes (ties kept; `thr_out`,
+        an int32[2] device tensor, receives the threshold key and the count);
+        else `thr` is the device tensor written by topk_threshold; else the
+        nonzeros.  A status with STAT_RETRY (fast mode only) means the call
+        must be repeated with mode=MODE_GENERAL; load_balance does that."""
         _lib.require_gpu(tensor, "input")
         flat = tensor.reshape(-1)
         n = flat.numel()
@@ -95,20 +99,23 @@ class TensorPartition:
         ws = _lib.scratch.get(dev, "load_balance", nbytes)
         table = self._table(dev, m)
         rc = L.zen_load_balance(
-            _lib.ptr(flat), code, n, m, self.partitions, self.rehash, _lib.ptr(thr),
-            _lib.ptr(out_idx), _lib.ptr(out_val), capacity, _lib.ptr(splits), _lib.ptr(table),
+            _lib.ptr(flat), code, n, m, self.partitions, self.rehash, _lib.ptr(thr), int(k), _lib.ptr(thr_out),
+            _lib.ptr(out_idx), _lib.ptr(out_val), capacity, _lib.ptr(splits), _lib.ptr(table), mode,
             _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
         _lib.check(rc, "load_balance")
         return out_idx, out_val, splits, status
 
-    def load_balance(self, tensor, thr=None, capacity=None):
+    def load_balance(self, tensor, thr=None, capacity=None, k=0):
         """Returns (indices[P], values[P], splits) like the reference
         (tensor_load_balance.py:43-51).  The per-partition tensors are views of
         two contiguous buffers; slicing them needs the split sizes on the
         host, which is this call's only synchronisation."""
-        out_idx, out_val, splits, status = self.load_balance_flat(tensor, thr, capacity)
-        host = torch.cat([splits, status.to(torch.int64)]).tolist()
-        bits = host[-1]
+        for mode in (_lib.MODE_FAST, _lib.MODE_GENERAL):
+            out_idx, out_val, splits, status = self.load_balance_flat(tensor, thr, capacity, k, mode)
+            host = torch.cat([splits, status.to(torch.int64)]).tolist()
+            bits = host[-1]
+            if not bits & _lib.STAT_RETRY:
+                break
         if bits:
             raise RuntimeError("load_balance: " + _lib.describe_status(bits))
         indices, values, at = [], [], 0
