@@ -159,26 +159,39 @@ __global__ __launch_bounds__(256) void k_serial_sort(int32_t *serial, int64_t sp
 
 // ------------------------------------------------- fused path (list based)
 
-__global__ __launch_bounds__(256) void k_insert_list(const int32_t *__restrict__ cand, const uint32_t *count,
+// The list may hold candidates of a sampled top-k: entries whose magnitude key
+// is below the exact threshold (thr, optional) are not selected after all.
+template <typename S>
+__device__ inline bool list_selected(const int32_t *cand, const S *vals, const uint32_t *thr, uint32_t j,
+                                     uint32_t *t_out) {
+  const uint32_t t = (uint32_t)cand[j];
+  *t_out = t;
+  if (t == 0) return false;  // index 0 is never transmitted
+  return !thr || (vals[j] & KeyOf<S>::kMask) >= thr[0];
+}
+
+template <typename S>
+__global__ __launch_bounds__(256) void k_insert_list(const int32_t *__restrict__ cand, const S *__restrict__ vals,
+                                                     const uint32_t *count, const uint32_t *__restrict__ thr,
                                                      uint32_t *table, Probe g) {
   const uint32_t j = blockIdx.x * 256u + threadIdx.x;
   if (j >= *count) return;
-  const uint32_t t = (uint32_t)cand[j];
-  if (t != 0) insert_chain(table, g, t);
+  uint32_t t;
+  if (list_selected<S>(cand, vals, thr, j, &t)) insert_chain(table, g, t);
 }
 
 // Sort key = position in the output: partition-major, table slots before the
-// partition's serial entries (all serial entries of a partition share one key;
-// the stable sort keeps them in ascending index order).
-__global__ __launch_bounds__(256) void k_final_key(const int32_t *__restrict__ cand, const uint32_t *count,
-                                                   const uint32_t *__restrict__ table, Probe g,
-                                                   uint32_t drop_key, uint32_t *__restrict__ keys,
-                                                   uint32_t *__restrict__ perm) {
+// partition's serial entries (all serial entries of a partition share one key).
+template <typename S>
+__global__ __launch_bounds__(256) void k_final_key(const int32_t *__restrict__ cand, const S *__restrict__ vals,
+                                                   const uint32_t *count, const uint32_t *__restrict__ thr,
+                                                   const uint32_t *__restrict__ table, Probe g, uint32_t drop_key,
+                                                   uint32_t *__restrict__ keys, uint32_t *__restrict__ perm) {
   const uint32_t j = blockIdx.x * 256u + threadIdx.x;
   if (j >= *count) return;
-  const uint32_t t = (uint32_t)cand[j];
-  uint32_t key = drop_key;  // index 0 is never transmitted
-  if (t != 0) {
+  uint32_t t;
+  uint32_t key = drop_key;
+  if (list_selected<S>(cand, vals, thr, j, &t)) {
     uint32_t slot = 0, part = 0;
     const int lv = find_level(table, g, t, &slot, &part);
     key = part * (g.npp + 1u) + (lv >= 0 ? slot - part * g.npp : g.npp);
@@ -192,14 +205,16 @@ __global__ __launch_bounds__(256) void k_gather(const uint32_t *__restrict__ key
                                                 const uint32_t *count, const int32_t *__restrict__ cand_idx,
                                                 const S *__restrict__ cand_val, uint32_t drop_key, Probe g,
                                                 int32_t *__restrict__ out_idx, S *__restrict__ out_val,
-                                                uint32_t *table) {
+                                                uint32_t capacity, uint32_t *table) {
   const uint32_t i = blockIdx.x * 256u + threadIdx.x;
   if (i >= *count) return;
   const uint32_t key = keys[i];
   if (key >= drop_key) return;
   const uint32_t j = perm[i];
-  out_idx[i] = cand_idx[j];
-  out_val[i] = cand_val[j];
+  if (i < capacity) {
+    out_idx[i] = cand_idx[j];
+    out_val[i] = cand_val[j];
+  }
   const uint32_t part = key / (g.npp + 1u), local = key % (g.npp + 1u);
   if (local < g.npp) table[part * g.npp + local] = 0u;  // leave the table empty again
 }
@@ -221,9 +236,10 @@ __device__ inline uint32_t lower_bound_u32(const uint32_t *a, uint32_t n, uint32
 // fetching the values again.
 template <typename S>
 __global__ __launch_bounds__(256) void k_splits_serial(const uint32_t *__restrict__ keys, const uint32_t *count,
-                                                       uint32_t npp, int64_t spp, const S *__restrict__ dense,
-                                                       int32_t *__restrict__ out_idx, S *__restrict__ out_val,
-                                                       int64_t *__restrict__ splits, int32_t *status) {
+                                                       uint32_t npp, int64_t spp, uint32_t capacity,
+                                                       const S *__restrict__ dense, int32_t *__restrict__ out_idx,
+                                                       S *__restrict__ out_val, int64_t *__restrict__ splits,
+                                                       int32_t *status) {
   __shared__ uint32_t s_bound[3];
   __shared__ uint32_t buf[kSerialLds];
   const uint32_t p = blockIdx.x;
@@ -237,9 +253,10 @@ __global__ __launch_bounds__(256) void k_splits_serial(const uint32_t *__restric
   if (threadIdx.x == 0) {
     splits[p] = (int64_t)(hi - lo);
     if ((int64_t)(hi - ser) > spp) atomicOr(status, ZEN_STAT_SERIAL_OVERFLOW);
+    if (hi > capacity) atomicOr(status, ZEN_STAT_CAPACITY);
   }
   const uint32_t cnt = hi - ser;
-  if (cnt < 2) return;
+  if (cnt < 2 || hi > capacity) return;
   uint32_t *region = reinterpret_cast<uint32_t *>(out_idx + ser);
   if (cnt <= kSerialLds) {
     for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) buf[i] = region[i];
@@ -281,17 +298,19 @@ int sparse_balance_launch(const S *in, int64_t n, uint32_t *table, Probe g, int3
 
 constexpr int64_t kSampleMinElems = 1ll << 24;  // below this the exact full-tensor histogram is cheap anyway
 
+// Room for the candidates of a sampled top-k (the selected plus those between
+// the sampled floor and the exact threshold).
+inline int64_t list_capacity(int64_t capacity) { return capacity + capacity / 2 + 4096; }
+
 struct BalancePlan {
-  int32_t *cand_idx;   // first-stage candidates of the sampled top-k (2 * capacity)
-  uint32_t *cand_val;
-  int32_t *sel_idx;    // the selected entries (capacity); 4 bytes per value reserved, bf16 uses half
-  uint32_t *sel_val;
+  int32_t *sel_idx;    // the selected entries or candidates (list_capacity)
+  uint32_t *sel_val;   // 4 bytes per value reserved, bf16 uses half
   uint32_t *keys_a, *perm_a, *keys_b, *perm_b;
-  uint32_t *count;     // [0] selected, [1] candidates
+  uint32_t *count;     // entries in sel_*
   uint32_t *thr;       // [0..1] exact threshold + count, [2..3] sampled floor
+  uint32_t *cand_hist;
   void *topk_scratch;
   void *select_scratch;
-  void *list_scratch;
   void *sort_scratch;
   size_t bytes;
 };
@@ -299,9 +318,7 @@ struct BalancePlan {
 BalancePlan plan_balance(void *workspace, int64_t n, int dtype, int64_t capacity) {
   Carver cv(workspace);
   BalancePlan p;
-  const size_t cap = (size_t)(capacity > 0 ? capacity : 1);
-  p.cand_idx = cv.take<int32_t>(2 * cap);
-  p.cand_val = cv.take<uint32_t>(2 * cap);
+  const size_t cap = (size_t)list_capacity(capacity > 0 ? capacity : 1);
   p.sel_idx = cv.take<int32_t>(cap);
   p.sel_val = cv.take<uint32_t>(cap);
   p.keys_a = cv.take<uint32_t>(cap);
@@ -310,19 +327,20 @@ BalancePlan plan_balance(void *workspace, int64_t n, int dtype, int64_t capacity
   p.perm_b = cv.take<uint32_t>(cap);
   p.count = cv.take<uint32_t>(2);
   p.thr = cv.take<uint32_t>(4);
+  p.cand_hist = cv.take<uint32_t>((size_t)kCandRows * kCandBins);
   p.topk_scratch = cv.take<char>(topk_scratch_bytes());
   p.select_scratch = cv.take<char>(select_scratch_bytes(n, dtype));
-  p.list_scratch = cv.take<char>(select_scratch_bytes((int64_t)(2 * cap), dtype));
   p.sort_scratch = cv.take<char>(sort_scratch_bytes((int64_t)cap));
   p.bytes = cv.used;
   return p;
 }
 
-// Stage 1 of load balance: the selected (index, value) list in p.sel_*, its
-// length in p.count[0].  k > 0 asks for the k largest magnitudes (ties at the
-// threshold kept); then the threshold goes to p.thr[0..1].
+// Stage 1 of load balance: an (index, value) list in p.sel_* with its length in
+// p.count[0], and in *filter the threshold the later stages must still apply to
+// it (nullptr: every entry is selected).  k > 0 asks for the k largest
+// magnitudes (ties at the threshold kept); the threshold goes to p.thr[0..1].
 int select_stage(const BalancePlan &p, const void *input, int dtype, int64_t n, const uint32_t *thr, int64_t k,
-                 int64_t capacity, int mode, int32_t *status, hipStream_t s) {
+                 int64_t capacity, int mode, const uint32_t **filter, int32_t *status, hipStream_t s) {
   SelectArgs sel;
   sel.in = input;
   sel.dtype = dtype;
@@ -330,11 +348,12 @@ int select_stage(const BalancePlan &p, const void *input, int dtype, int64_t n, 
   sel.thr = thr;
   sel.out_idx = p.sel_idx;
   sel.out_val = p.sel_val;
-  sel.capacity = capacity;
+  sel.capacity = list_capacity(capacity);
   sel.out_count32 = &p.count[0];
   sel.ordered = false;  // the sort below fixes the order
   sel.scratch = p.select_scratch;
   sel.status = status;
+  *filter = nullptr;
   if (k <= 0) return select_compact(sel, s);
   int rc;
   if (mode == ZEN_MODE_GENERAL || n < kSampleMinElems) {
@@ -344,25 +363,24 @@ int select_stage(const BalancePlan &p, const void *input, int dtype, int64_t n, 
     return select_compact(sel, s);
   }
   // one pass: compact everything at or above a floor estimated from a sample,
-  // find the exact threshold among those candidates, filter them
-  if ((rc = topk_sampled_floor(input, dtype, n, k, p.thr + 2, p.topk_scratch, status, s)) != ZEN_OK) return rc;
-  SelectArgs cand = sel;
-  cand.thr = p.thr + 2;
-  cand.out_idx = p.cand_idx;
-  cand.out_val = p.cand_val;
-  cand.capacity = 2 * capacity;
-  cand.out_count32 = &p.count[1];
-  if ((rc = select_compact(cand, s)) != ZEN_OK) return rc;
-  if ((rc = topk_exact(p.cand_val, dtype, 2 * capacity, &p.count[1], k, p.thr, p.topk_scratch, status,
-                       ZEN_STAT_RETRY, s)) != ZEN_OK)
-    return rc;
-  sel.in = p.cand_val;
-  sel.n = 2 * capacity;
-  sel.n_dev = &p.count[1];
-  sel.src_idx = p.cand_idx;
-  sel.thr = p.thr;
-  sel.scratch = p.list_scratch;
-  return select_compact(sel, s);
+  // histogram those candidates on the way, read the exact threshold off the
+  // histogram; entries between floor and threshold stay in the list and are
+  // filtered by the later stages
+  if ((rc = topk_sampled_floor(input, dtype, n, k, p.thr + 2, p.topk_scratch, s)) != ZEN_OK) return rc;
+  launch_fill<uint32_t>(p.cand_hist, 0u, (size_t)kCandRows * kCandBins, s);
+  ZEN_LAUNCH_CHECK("clear candidate histogram");
+  sel.thr = p.thr + 2;
+  sel.cand_hist = p.cand_hist;
+  if ((rc = select_compact(sel, s)) != ZEN_OK) return rc;
+  if ((rc = cand_pick(p.cand_hist, p.thr + 2, k, dtype, p.thr, status, s)) != ZEN_OK) return rc;
+  if (dtype == ZEN_F32) {
+    // the histogram resolved 15 key bits; the remaining 16 need the radix select, over the candidates only
+    if ((rc = topk_exact(p.sel_val, dtype, sel.capacity, &p.count[0], k, p.thr, p.topk_scratch, status,
+                         ZEN_STAT_RETRY, s)) != ZEN_OK)
+      return rc;
+  }
+  *filter = p.thr;
+  return ZEN_OK;
 }
 
 }  // namespace
@@ -439,25 +457,36 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
   const int bits = ceil_log2_u64(drop_key);
   BalancePlan p = plan_balance(workspace, n, dtype, capacity);
 
-  int rc = select_stage(p, input, dtype, n, thr, k, capacity, mode, status, s);
+  const uint32_t *filter = nullptr;
+  int rc = select_stage(p, input, dtype, n, thr, k, capacity, mode, &filter, status, s);
   if (rc != ZEN_OK) return rc;
   if (k > 0 && thr_out) ZEN_HIP_CHECK(hipMemcpyAsync(thr_out, p.thr, 2 * sizeof(uint32_t), hipMemcpyDeviceToDevice, s));
-  const unsigned blocks = (unsigned)ceil_div(capacity, 256);
+  const int64_t lcap = list_capacity(capacity);
+  const unsigned blocks = (unsigned)ceil_div(lcap, 256);
+  uint32_t *tab = reinterpret_cast<uint32_t *>(table);
+  const uint16_t *val16 = reinterpret_cast<const uint16_t *>(p.sel_val);
   {
     ProfScope prof(kProfInsertList, s);
-    k_insert_list<<<dim3(blocks), dim3(256), 0, s>>>(p.sel_idx, p.count, reinterpret_cast<uint32_t *>(table), g);
+    if (dtype == ZEN_BF16)
+      k_insert_list<uint16_t><<<dim3(blocks), dim3(256), 0, s>>>(p.sel_idx, val16, p.count, filter, tab, g);
+    else
+      k_insert_list<uint32_t><<<dim3(blocks), dim3(256), 0, s>>>(p.sel_idx, p.sel_val, p.count, filter, tab, g);
     ZEN_LAUNCH_CHECK("k_insert_list");
   }
   {
     ProfScope prof(kProfFinalKey, s);
-    k_final_key<<<dim3(blocks), dim3(256), 0, s>>>(p.sel_idx, p.count, reinterpret_cast<uint32_t *>(table), g,
-                                                   drop_key, p.keys_a, p.perm_a);
+    if (dtype == ZEN_BF16)
+      k_final_key<uint16_t><<<dim3(blocks), dim3(256), 0, s>>>(p.sel_idx, val16, p.count, filter, tab, g, drop_key,
+                                                               p.keys_a, p.perm_a);
+    else
+      k_final_key<uint32_t><<<dim3(blocks), dim3(256), 0, s>>>(p.sel_idx, p.sel_val, p.count, filter, tab, g, drop_key,
+                                                               p.keys_a, p.perm_a);
     ZEN_LAUNCH_CHECK("k_final_key");
   }
   int where;
   {
     ProfScope prof(kProfSort, s);
-    where = sort_pairs(p.keys_a, p.perm_a, p.keys_b, p.perm_b, capacity, p.count, bits, p.sort_scratch, status, s);
+    where = sort_pairs(p.keys_a, p.perm_a, p.keys_b, p.perm_b, lcap, p.count, bits, p.sort_scratch, status, s);
   }
   if (where < 0) return where;
   const uint32_t *sk = where ? p.keys_b : p.keys_a;
@@ -465,24 +494,21 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
   {
     ProfScope prof(kProfGather, s);
     if (dtype == ZEN_BF16)
-      k_gather<uint16_t><<<dim3(blocks), dim3(256), 0, s>>>(sk, sp, p.count, p.sel_idx,
-                                                            reinterpret_cast<const uint16_t *>(p.sel_val), drop_key, g,
-                                                            out_idx, static_cast<uint16_t *>(out_val),
-                                                            reinterpret_cast<uint32_t *>(table));
+      k_gather<uint16_t><<<dim3(blocks), dim3(256), 0, s>>>(sk, sp, p.count, p.sel_idx, val16, drop_key, g, out_idx,
+                                                            static_cast<uint16_t *>(out_val), (uint32_t)capacity, tab);
     else
-      k_gather<uint32_t><<<dim3(blocks), dim3(256), 0, s>>>(sk, sp, p.count, p.sel_idx, p.sel_val, drop_key, g,
-                                                            out_idx, static_cast<uint32_t *>(out_val),
-                                                            reinterpret_cast<uint32_t *>(table));
+      k_gather<uint32_t><<<dim3(blocks), dim3(256), 0, s>>>(sk, sp, p.count, p.sel_idx, p.sel_val, drop_key, g, out_idx,
+                                                            static_cast<uint32_t *>(out_val), (uint32_t)capacity, tab);
     ZEN_LAUNCH_CHECK("k_gather");
   }
   if (dtype == ZEN_BF16)
     k_splits_serial<uint16_t><<<dim3((unsigned)partitions), dim3(256), 0, s>>>(
-        sk, p.count, g.npp, spp, static_cast<const uint16_t *>(input), out_idx, static_cast<uint16_t *>(out_val), splits,
-        status);
+        sk, p.count, g.npp, spp, (uint32_t)capacity, static_cast<const uint16_t *>(input), out_idx,
+        static_cast<uint16_t *>(out_val), splits, status);
   else
     k_splits_serial<uint32_t><<<dim3((unsigned)partitions), dim3(256), 0, s>>>(
-        sk, p.count, g.npp, spp, static_cast<const uint32_t *>(input), out_idx, static_cast<uint32_t *>(out_val), splits,
-        status);
+        sk, p.count, g.npp, spp, (uint32_t)capacity, static_cast<const uint32_t *>(input), out_idx,
+        static_cast<uint32_t *>(out_val), splits, status);
   ZEN_LAUNCH_CHECK("k_splits_serial");
   return ZEN_OK;
 }

@@ -119,33 +119,118 @@ __global__ __launch_bounds__(kHistBlock) void k_topk_pick(TopkState *st, uint32_
   for (int j = 0; j < kPer; ++j) hist[kHistBins - 1 - (threadIdx.x * kPer + j)] = 0;
 }
 
-// Histogram of the top 11 key bits over a sample: one 16-byte vector out of
-// every 2^block_log2 consecutive vectors, at a pseudo-random place inside its
-// block so that regular layouts (rows, columns) are not sampled in lockstep.
+// Histogram of the top 15 key bits (for bf16: the whole key) over a sample: one
+// 16-byte vector out of every 2^block_log2 consecutive vectors, at a
+// pseudo-random place inside its block so that regular layouts (rows, columns)
+// are not sampled in lockstep.  The block's histogram lives in LDS as 32768
+// 16-bit counters packed two per word; a block never sees more than 65535
+// sample elements, so they cannot overflow into each other.
+constexpr int kFineBins = 32768;
+constexpr int kSampleBlock = 1024;
+
 template <typename S, bool ALIGNED>
-__global__ __launch_bounds__(kHistBlock) void k_sample_hist(const S *__restrict__ in, int64_t n, int block_log2,
-                                                            uint32_t *__restrict__ hist) {
+__global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restrict__ in, int64_t n, int block_log2,
+                                                              uint32_t *__restrict__ hist) {
   constexpr int V = VecOf<S>::kN;
-  constexpr int kShift = KeyOf<S>::kBits - 11;
-  __shared__ uint32_t bins[kHistBins];
-  for (int i = threadIdx.x; i < kHistBins; i += kHistBlock) bins[i] = 0;
+  constexpr int kShift = KeyOf<S>::kBits - 15;
+  __shared__ uint32_t bins[kFineBins / 2];
+  for (int i = threadIdx.x; i < kFineBins / 2; i += kSampleBlock) bins[i] = 0;
   __syncthreads();
   const int64_t nvec = (n + V - 1) / V;
   const int64_t nblocks = (nvec + (1ll << block_log2) - 1) >> block_log2;
-  for (int64_t b = blockIdx.x * (int64_t)kHistBlock + threadIdx.x; b < nblocks;
-       b += (int64_t)gridDim.x * kHistBlock) {
+  for (int64_t b = blockIdx.x * (int64_t)kSampleBlock + threadIdx.x; b < nblocks;
+       b += (int64_t)gridDim.x * kSampleBlock) {
     const int64_t v = (b << block_log2) + (poly((uint32_t)b) >> 7 & ((1u << block_log2) - 1u));
     if (v >= nvec) continue;
     S e[V];
     const int live = load_vec<S, ALIGNED>(in, v * V, n, e);
 #pragma unroll
-    for (int i = 0; i < V; ++i)
-      if (i < live) atomicAdd(&bins[(e[i] & KeyOf<S>::kMask) >> kShift], 1u);
+    for (int i = 0; i < V; ++i) {
+      if (i < live) {
+        const uint32_t bin = (e[i] & KeyOf<S>::kMask) >> kShift;
+        atomicAdd(&bins[bin >> 1], 1u << (16 * (bin & 1u)));
+      }
+    }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < kHistBins; i += kHistBlock) {
+  for (int i = threadIdx.x; i < kFineBins / 2; i += kSampleBlock) {
     const uint32_t c = bins[i];
-    if (c) atomicAdd(&hist[i], c);
+    if (c & 0xffffu) atomicAdd(&hist[2 * i], c & 0xffffu);
+    if (c >> 16) atomicAdd(&hist[2 * i + 1], c >> 16);
+  }
+}
+
+// One block: the lowest fine bin b such that `rank` sample elements lie in bins
+// >= b; floor_out[0] = lowest key of that bin (0 if the sample is too small).
+__global__ __launch_bounds__(kSampleBlock) void k_sample_pick(uint32_t *hist, uint32_t rank, int key_shift,
+                                                              uint32_t *floor_out) {
+  constexpr int kPer = kFineBins / kSampleBlock;
+  __shared__ uint32_t smem[kSampleBlock / 64 + 1];
+  uint32_t c[kPer];
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    c[j] = hist[kFineBins - 1 - (threadIdx.x * kPer + j)];
+    mine += c[j];
+  }
+  uint32_t total;
+  uint32_t above = block_exclusive_scan<uint32_t, kSampleBlock>(mine, smem, &total);
+  if (total < rank) {
+    if (threadIdx.x == 0) floor_out[0] = 0;
+  } else {
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      if (above < rank && rank <= above + c[j]) floor_out[0] = (uint32_t)(kFineBins - 1 - (threadIdx.x * kPer + j)) << key_shift;
+      above += c[j];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) hist[kFineBins - 1 - (threadIdx.x * kPer + j)] = 0;
+}
+
+// One block over the candidate histogram the compaction kernel filled (bin =
+// min((key - floor) >> shift, kHistBins-1)): the exact k-th largest key when the
+// bins are single keys (shift 0), else the lowest key of its bin.
+// thr_out = (key, number of candidates >= key).  Too few candidates, or the
+// k-th lies in the clipped last bin: ZEN_STAT_RETRY.
+__global__ __launch_bounds__(kHistBlock) void k_cand_pick(uint32_t *hist, const uint32_t *floor_key, uint32_t k,
+                                                          int shift, uint32_t *thr_out, int32_t *status) {
+  constexpr int kPer = kHistBins / kHistBlock;
+  __shared__ uint32_t smem[kHistBlock / 64 + 1];
+  uint32_t c[kPer];
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int bin = kHistBins - 1 - (threadIdx.x * kPer + j);
+    uint32_t sum = 0;
+    for (int row = 0; row < kCandRows; ++row) {
+      sum += hist[row * kHistBins + bin];
+      hist[row * kHistBins + bin] = 0;
+    }
+    c[j] = sum;
+    mine += sum;
+  }
+  uint32_t total;
+  uint32_t above = block_exclusive_scan<uint32_t, kHistBlock>(mine, smem, &total);
+  uint32_t base = floor_key[0];
+  if (base == 0) base = 1;  // the compaction treats a zero floor as "nonzero"
+  if (total < k) {
+    if (threadIdx.x == 0) {
+      thr_out[0] = 0;
+      thr_out[1] = total;
+      atomicOr(status, ZEN_STAT_RETRY);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      if (above < k && k <= above + c[j]) {
+        const uint32_t bin = kHistBins - 1 - (threadIdx.x * kPer + j);
+        thr_out[0] = base + (bin << shift);
+        thr_out[1] = above + c[j];
+        if (bin == kHistBins - 1) atomicOr(status, ZEN_STAT_RETRY);
+      }
+      above += c[j];
+    }
   }
 }
 
@@ -198,7 +283,7 @@ __global__ __launch_bounds__(256) void k_compress(const S *__restrict__ in, int6
 // The input is a dense tensor (an element's index is its position) or a list
 // (src_idx gives the index carried by each element).
 
-constexpr int kSelStage = 4096;    // staged pairs per tile
+constexpr int kSelStage = 3072;    // staged pairs per tile
 constexpr int kReserveShift = 40;  // unordered mode: tiles done above, entries reserved below
 
 // Inclusive prefix sum across the 64 lanes with DPP row shifts and broadcasts.
@@ -270,8 +355,9 @@ struct Flags<uint32_t> {
 template <typename S, typename I, bool ALIGNED, bool STAGED>
 __device__ inline uint32_t select_walk_tile(const S *__restrict__ in, int64_t n, uint32_t floor_key,
                                             int64_t tile_base, int subs, const int32_t *__restrict__ src_idx,
-                                            uint32_t *s_wave, int32_t *st_idx, S *st_val, I *__restrict__ out_idx,
-                                            S *__restrict__ out_val, uint64_t out_base, int64_t capacity) {
+                                            uint32_t *s_wave, int32_t *st_idx, S *st_val, uint32_t *s_hist,
+                                            I *__restrict__ out_idx, S *__restrict__ out_val, uint64_t out_base,
+                                            int64_t capacity) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kChunk = Flags<S>::kElems;  // elements per thread and sub-tile
   constexpr int kSub = kSelBlock * kChunk;
@@ -317,6 +403,10 @@ __device__ inline uint32_t select_walk_tile(const S *__restrict__ in, int64_t n,
       const uint32_t pos = before + (uint32_t)__popc(all & Flags<S>::below(off));
       const S v = in[first + off];  // just streamed through the cache; selected elements are few
       if (STAGED) {
+        if (s_hist) {
+          const uint32_t bin = ((v & KeyOf<S>::kMask) - floor_key) >> (sizeof(S) == 2 ? 0 : 16);
+          atomicAdd(&s_hist[bin < (uint32_t)kCandBins - 1u ? bin : (uint32_t)kCandBins - 1u], 1u);
+        }
         if (pos < (uint32_t)kSelStage) {
           st_idx[pos] = (int32_t)(first + off);
           st_val[pos] = v;
@@ -335,62 +425,81 @@ template <typename S, typename I, bool ALIGNED, bool ORDERED>
 __global__ __launch_bounds__(kSelBlock) void k_select_compact(
     const S *__restrict__ in, int64_t n_max, const uint32_t *__restrict__ n_dev, const uint32_t *__restrict__ thr,
     const int32_t *__restrict__ src_idx, I *__restrict__ out_idx, S *__restrict__ out_val, int64_t capacity,
-    ScanState st, int ntiles, int subs, int64_t *out_count, uint32_t *out_count32, int32_t *status) {
+    ScanState st, int ntiles, int subs, uint32_t *cand_hist, int64_t *out_count, uint32_t *out_count32,
+    int32_t *status) {
   constexpr int kSub = kSelBlock * Flags<S>::kElems;
   __shared__ uint32_t s_wave[kSelBlock / 64];
   __shared__ uint64_t s_bcast;
   __shared__ int s_tile;
   __shared__ int32_t st_idx[kSelStage];
   __shared__ S st_val[kSelStage];
-  int tile = (int)blockIdx.x;
-  if (ORDERED) {
-    if (threadIdx.x == 0) s_tile = (int)atomicAdd(st.ticket, 1u);
+  __shared__ uint32_t s_hist[ORDERED ? 1 : kCandBins];
+  uint32_t *hist = (!ORDERED && cand_hist) ? s_hist : nullptr;
+  if (hist) {
+    for (int i = threadIdx.x; i < kCandBins; i += kSelBlock) s_hist[i] = 0;
     __syncthreads();
-    tile = s_tile;
-    if (tile >= ntiles) return;
   }
   int64_t n = n_max;
   if (n_dev && (int64_t)*n_dev < n) n = (int64_t)*n_dev;
   uint32_t floor_key = thr ? thr[0] : 1u;
   if (floor_key == 0) floor_key = 1u;  // zeros are never selected
   if (floor_key > KeyOf<S>::kMask) floor_key = KeyOf<S>::kMask + 1u;  // nothing qualifies
-  const int64_t tile_base = (int64_t)tile * subs * kSub;
 
-  const uint32_t found = select_walk_tile<S, I, ALIGNED, true>(in, n, floor_key, tile_base, subs, src_idx, s_wave,
-                                                               st_idx, st_val, out_idx, out_val, 0, capacity);
-  uint64_t tile_start, all = 0;
-  bool last;
-  if (ORDERED) {
-    tile_start = lookback_exclusive(st, tile, found, status, &s_bcast);
-    last = tile == ntiles - 1;
-    all = tile_start + found;
-  } else {
-    if (threadIdx.x == 0)
-      s_bcast = __hip_atomic_fetch_add(st.desc, (1ull << kReserveShift) | found, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    const uint64_t old = s_bcast;
-    tile_start = old & ((1ull << kReserveShift) - 1);
-    last = (int)(old >> kReserveShift) == ntiles - 1;  // every other tile has reserved already
-    all = tile_start + found;
-  }
-  if (last && threadIdx.x == 0) {
-    if (out_count) *out_count = (int64_t)all;
-    if (out_count32) *out_count32 = (uint32_t)(all < (uint64_t)capacity ? all : (uint64_t)capacity);
-    if (all > (uint64_t)capacity) atomicOr(status, ZEN_STAT_CAPACITY);
-  }
-  if (found <= (uint32_t)kSelStage) {
-    for (uint32_t i = threadIdx.x; i < found; i += kSelBlock) {
-      const uint64_t pos = tile_start + i;
-      if (pos < (uint64_t)capacity) {
-        const int32_t at = st_idx[i];
-        out_idx[pos] = (I)(src_idx ? src_idx[at] : at);
-        out_val[pos] = st_val[i];
-      }
+  // ordered: tiles are taken by ticket, so that every earlier tile already runs
+  {
+    int tile = (int)blockIdx.x;
+    if (ORDERED) {
+      if (threadIdx.x == 0) s_tile = (int)atomicAdd(st.ticket, 1u);
+      __syncthreads();
+      tile = s_tile;
     }
-  } else {
-    select_walk_tile<S, I, ALIGNED, false>(in, n, floor_key, tile_base, subs, src_idx, s_wave, st_idx, st_val,
-                                           out_idx, out_val, tile_start, capacity);
+    if (tile >= ntiles) return;
+    const int64_t tile_base = (int64_t)tile * subs * kSub;
+    const uint32_t found = select_walk_tile<S, I, ALIGNED, true>(in, n, floor_key, tile_base, subs, src_idx, s_wave,
+                                                                 st_idx, st_val, hist, out_idx, out_val, 0, capacity);
+    uint64_t tile_start, all = 0;
+    bool last;
+    if (ORDERED) {
+      tile_start = lookback_exclusive(st, tile, found, status, &s_bcast);
+      last = tile == ntiles - 1;
+      all = tile_start + found;
+    } else {
+      if (threadIdx.x == 0)
+        s_bcast = __hip_atomic_fetch_add(st.desc, (1ull << kReserveShift) | found, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      const uint64_t old = s_bcast;
+      tile_start = old & ((1ull << kReserveShift) - 1);
+      last = (int)(old >> kReserveShift) == ntiles - 1;  // every other tile has reserved already
+      all = tile_start + found;
+    }
+    if (last && threadIdx.x == 0) {
+      if (out_count) *out_count = (int64_t)all;
+      if (out_count32) *out_count32 = (uint32_t)(all < (uint64_t)capacity ? all : (uint64_t)capacity);
+      if (all > (uint64_t)capacity) atomicOr(status, ZEN_STAT_CAPACITY);
+    }
+    if (found <= (uint32_t)kSelStage) {
+      for (uint32_t i = threadIdx.x; i < found; i += kSelBlock) {
+        const uint64_t pos = tile_start + i;
+        if (pos < (uint64_t)capacity) {
+          const int32_t at = st_idx[i];
+          out_idx[pos] = (I)(src_idx ? src_idx[at] : at);
+          out_val[pos] = st_val[i];
+        }
+      }
+    } else {
+      select_walk_tile<S, I, ALIGNED, false>(in, n, floor_key, tile_base, subs, src_idx, s_wave, st_idx, st_val,
+                                             nullptr, out_idx, out_val, tile_start, capacity);
+    }
+  }
+  if (hist) {
+    // spread over kCandRows partial histograms: fewer blocks meet on one counter
+    __syncthreads();
+    uint32_t *row = cand_hist + (size_t)(blockIdx.x % kCandRows) * kCandBins;
+    for (int i = threadIdx.x; i < kCandBins; i += kSelBlock) {
+      const uint32_t c = s_hist[i];
+      if (c) atomicAdd(&row[i], c);
+    }
   }
 }
 
@@ -431,7 +540,7 @@ static int select_launch(const SelectArgs &a, hipStream_t stream) {
 #define ZEN_SELECT_GO(AL, ORD)                                                                                 \
   k_select_compact<S, I, AL, ORD><<<grid, block, 0, stream>>>(in, a.n, a.n_dev, a.thr, a.src_idx, out_idx,   \
                                                               out_val, a.capacity, st, (int)ntiles, subs,    \
-                                                              a.out_count, a.out_count32, a.status)
+                                                              a.cand_hist, a.out_count, a.out_count32, a.status)
   if (aligned && a.ordered) ZEN_SELECT_GO(true, true);
   else if (aligned) ZEN_SELECT_GO(true, false);
   else if (a.ordered) ZEN_SELECT_GO(false, true);
@@ -488,12 +597,9 @@ int topk_launch(const S *in, int64_t n, const uint32_t *n_dev, int64_t k, uint32
 }
 
 template <typename S>
-int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *workspace, int32_t *status,
-                  hipStream_t stream) {
+int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *workspace, hipStream_t stream) {
   constexpr int V = VecOf<S>::kN;
-  Carver cv(workspace);
-  TopkState *st = cv.take<TopkState>(1);
-  uint32_t *hist = cv.take<uint32_t>(kHistBins);
+  uint32_t *hist = static_cast<uint32_t *>(workspace);
   const int64_t nvec = ceil_div(n, V);
   const int64_t nblocks = ceil_div(nvec, 1ll << kSampleLog2);
   // rank to look for in the sample: the expected one plus six standard
@@ -502,18 +608,22 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
   const double expect = (double)k * ((double)nblocks * V) / (double)n;
   const double want = expect + 6.0 * sqrt(expect) + 16.0;
   const uint32_t rank = want > 4.0e9 ? 0xffffffffu : (uint32_t)want;
-  k_topk_init<<<dim3(1), dim3(256), 0, stream>>>(st, hist, rank);
-  ZEN_LAUNCH_CHECK("k_topk_init");
-  int64_t blocks = ceil_div(nblocks, kHistBlock);
-  if (blocks > 512) blocks = 512;
+  launch_fill<uint32_t>(hist, 0u, kFineBins, stream);
+  ZEN_LAUNCH_CHECK("sample: clear histogram");
+  // every block must see fewer than 65536 sample elements (16-bit LDS counters)
+  int64_t blocks = ceil_div(nblocks * V, 32768);
+  if (blocks < 128) blocks = 128;
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
-  if (aligned)
-    k_sample_hist<S, true><<<dim3((unsigned)blocks), dim3(kHistBlock), 0, stream>>>(in, n, kSampleLog2, hist);
-  else
-    k_sample_hist<S, false><<<dim3((unsigned)blocks), dim3(kHistBlock), 0, stream>>>(in, n, kSampleLog2, hist);
-  ZEN_LAUNCH_CHECK("k_sample_hist");
-  k_topk_pick<<<dim3(1), dim3(kHistBlock), 0, stream>>>(st, hist, 11, 1, KeyOf<S>::kBits - 11, thr_lo, status, 0);
-  ZEN_LAUNCH_CHECK("k_topk_pick");
+  {
+    ProfScope prof(kProfTopkHist, stream);
+    if (aligned)
+      k_sample_hist<S, true><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist);
+    else
+      k_sample_hist<S, false><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist);
+    ZEN_LAUNCH_CHECK("k_sample_hist");
+  }
+  k_sample_pick<<<dim3(1), dim3(kSampleBlock), 0, stream>>>(hist, rank, KeyOf<S>::kBits - 15, thr_lo);
+  ZEN_LAUNCH_CHECK("k_sample_pick");
   return ZEN_OK;
 }
 
@@ -536,7 +646,19 @@ int compress_launch(const S *in, int64_t n, const uint32_t *thr, S *out, hipStre
 
 }  // namespace
 
-size_t topk_scratch_bytes() { return align_up(sizeof(TopkState), 256) + align_up(kHistBins * sizeof(uint32_t), 256); }
+size_t topk_scratch_bytes() {
+  const size_t exact = align_up(sizeof(TopkState), 256) + align_up(kHistBins * sizeof(uint32_t), 256);
+  const size_t sampled = align_up(kFineBins * sizeof(uint32_t), 256);
+  return exact > sampled ? exact : sampled;
+}
+
+int cand_pick(uint32_t *cand_hist, const uint32_t *floor_key, int64_t k, int dtype, uint32_t *thr, int32_t *status,
+              hipStream_t stream) {
+  k_cand_pick<<<dim3(1), dim3(kHistBlock), 0, stream>>>(cand_hist, floor_key, (uint32_t)k, dtype == ZEN_BF16 ? 0 : 16,
+                                                        thr, status);
+  ZEN_LAUNCH_CHECK("k_cand_pick");
+  return ZEN_OK;
+}
 
 int topk_exact(const void *in, int dtype, int64_t n, const uint32_t *n_dev, int64_t k, uint32_t *thr,
                void *scratch, int32_t *status, int short_bit, hipStream_t stream) {
@@ -546,10 +668,9 @@ int topk_exact(const void *in, int dtype, int64_t n, const uint32_t *n_dev, int6
 }
 
 int topk_sampled_floor(const void *in, int dtype, int64_t n, int64_t k, uint32_t *thr_lo, void *scratch,
-                       int32_t *status, hipStream_t stream) {
-  if (dtype == ZEN_BF16)
-    return sample_launch(static_cast<const uint16_t *>(in), n, k, thr_lo, scratch, status, stream);
-  return sample_launch(static_cast<const uint32_t *>(in), n, k, thr_lo, scratch, status, stream);
+                       hipStream_t stream) {
+  if (dtype == ZEN_BF16) return sample_launch(static_cast<const uint16_t *>(in), n, k, thr_lo, scratch, stream);
+  return sample_launch(static_cast<const uint32_t *>(in), n, k, thr_lo, scratch, stream);
 }
 
 }  // namespace zen
