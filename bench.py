@@ -15,6 +15,12 @@ import time
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch of the dominant kernel on the full c3 workload, from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by what the same counters read
+# for a plain 1 GiB copy (profiles/c3_select_compact_hbm_traffic.txt).  Other
+# workloads report null.
+MEASURED_TRAFFIC = {("c3", 1, "k_select_compact"): 1.519e9}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -164,7 +170,8 @@ def main():
         avg_ms = total_ms / launches
         achieved = per_launch[dom] / (avg_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                    "traffic": MEASURED_TRAFFIC.get((cfg.name, args.shrink, dom)),
                     "avg_launch_ms": round(avg_ms, 4), "launches_per_step": launches // args.steps,
                     "algorithmic_bytes_per_launch": per_launch[dom]}
 

@@ -78,7 +78,7 @@ int topk_exact(const void *in, int dtype, int64_t n, const uint32_t *n_dev, int6
 int topk_sampled_floor(const void *in, int dtype, int64_t n, int64_t k, uint32_t *thr_lo, void *scratch,
                        hipStream_t stream);
 constexpr int kCandBins = 2048;
-constexpr int kCandRows = 64;  // partial candidate histograms (blocks spread over them), summed by cand_pick
+constexpr int kCandRows = 8;   // partial candidate histograms (blocks spread over them), summed by cand_pick
 int cand_pick(uint32_t *cand_hist, const uint32_t *floor_key, int64_t k, int dtype, uint32_t *thr, int32_t *status,
               hipStream_t stream);
 

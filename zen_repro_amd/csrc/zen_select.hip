@@ -203,10 +203,10 @@ __global__ __launch_bounds__(kHistBlock) void k_cand_pick(uint32_t *hist, const 
   for (int j = 0; j < kPer; ++j) {
     const int bin = kHistBins - 1 - (threadIdx.x * kPer + j);
     uint32_t sum = 0;
-    for (int row = 0; row < kCandRows; ++row) {
-      sum += hist[row * kHistBins + bin];
-      hist[row * kHistBins + bin] = 0;
-    }
+#pragma unroll
+    for (int row = 0; row < kCandRows; ++row) sum += hist[row * kHistBins + bin];
+#pragma unroll
+    for (int row = 0; row < kCandRows; ++row) hist[row * kHistBins + bin] = 0;
     c[j] = sum;
     mine += sum;
   }

@@ -116,6 +116,8 @@ class TensorPartition:
             bits = host[-1]
             if not bits & _lib.STAT_RETRY:
                 break
+            m, _ = self.table_sizes(tensor.numel())
+            self._table(tensor.device, m).zero_()  # a declined call may leave entries behind
         if bits:
             raise RuntimeError("load_balance: " + _lib.describe_status(bits))
         indices, values, at = [], [], 0
