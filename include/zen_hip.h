@@ -150,9 +150,14 @@ int zen_select(const void *input, int dtype, int64_t n, const uint32_t *thr,
  * tensor_load_balance.py:15-16; the serial capacity is n / partitions / 10
  * per partition (tensor_load_balance.py:18).
  * `table` is int32[m] scratch that must be all zero on entry and is all zero
- * again on return (so one allocation serves every call).
+ * again on return (so one allocation serves every call); after a call that
+ * raised ZEN_STAT_RETRY or ZEN_STAT_INTERNAL its contents are undefined and the
+ * caller clears it.  ZEN_MODE_GENERAL keeps the owner of every probed slot in
+ * it, like the reference; ZEN_MODE_FAST sorts the selected entries by their
+ * level-1 slot instead and only borrows a corner of the table as a hash map
+ * for the few entries that collide (ZEN_STAT_RETRY if there are too many).
  */
-size_t zen_load_balance_workspace(int64_t n, int dtype, int64_t capacity, int partitions);
+size_t zen_load_balance_workspace(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions);
 int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m,
                      int partitions, int rehash, const uint32_t *thr, int64_t k,
                      uint32_t *thr_out, int32_t *out_idx, void *out_val,

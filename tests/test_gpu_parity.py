@@ -283,9 +283,11 @@ LB_CASES = [
 ]
 
 
+@pytest.mark.parametrize("mode", [0, 1])
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
 @pytest.mark.parametrize("n,P,density,scale,rehash", LB_CASES)
-def test_load_balance_bit_exact(zen, oracle, n, P, density, scale, rehash, dtype):
+def test_load_balance_bit_exact(zen, oracle, n, P, density, scale, rehash, dtype, mode):
+    """mode 0: sort-based owner resolution; mode 1: owner table like the reference."""
     g = make_grad(oracle, n, density, dtype, seed=n ^ P)
     g[0] = 0x3F80 if dtype == "bf16" else 1.0
     idx_o, val_o, splits_o, st_o = oracle.load_balance(g, P, scale, rehash)
@@ -294,9 +296,9 @@ def test_load_balance_bit_exact(zen, oracle, n, P, density, scale, rehash, dtype
     for rep in range(2):  # the second call reuses the (re-zeroed) owner table
         if st_o:
             with pytest.raises(RuntimeError):
-                tp.load_balance(d)
+                tp.load_balance(d, mode=mode)
             continue
-        indices, values, splits = tp.load_balance(d)
+        indices, values, splits = tp.load_balance(d, mode=mode)
         assert np.array_equal(to_np(splits), splits_o)
         assert np.array_equal(np.concatenate([to_np(i) for i in indices]), idx_o)
         assert np.array_equal(np.concatenate([to_np(v) for v in values]), val_o)

@@ -1,0 +1,116 @@
+// Helpers shared by the two load-balance back ends (owner table in
+// zen_balance.hip, sort-based resolution in zen_resolve.hip).
+#pragma once
+
+#include "zen_select.h"
+
+namespace zen {
+
+constexpr uint32_t kSerialLds = 8192;  // serial tails up to this size are sorted in LDS
+
+// Ascending compare-exchange network (bitonic with mirrored first step), valid
+// for any n: positions >= n act as +infinity and never move.
+__device__ inline void sort_network(uint32_t *a, uint32_t n) {
+  uint32_t n2 = 1;
+  while (n2 < n) n2 <<= 1;
+  const uint32_t half = n2 >> 1;
+  for (uint32_t k = 2; k <= n2; k <<= 1) {
+    const uint32_t hk = k >> 1;
+    for (uint32_t q = threadIdx.x; q < half; q += blockDim.x) {
+      const uint32_t blk = q / hk, r = q % hk;
+      const uint32_t i = blk * k + r, l = blk * k + (k - 1 - r);
+      if (l < n) {
+        const uint32_t x = a[i], y = a[l];
+        if (x > y) { a[i] = y; a[l] = x; }
+      }
+    }
+    __syncthreads();
+    for (uint32_t j = hk >> 1; j > 0; j >>= 1) {
+      for (uint32_t q = threadIdx.x; q < half; q += blockDim.x) {
+        const uint32_t i = (q / j) * 2 * j + (q % j), l = i + j;
+        if (l < n) {
+          const uint32_t x = a[i], y = a[l];
+          if (x > y) { a[i] = y; a[l] = x; }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+
+
+__device__ inline uint32_t lower_bound_u32(const uint32_t *a, uint32_t n, uint32_t x) {
+  uint32_t lo = 0, hi = n;
+  while (lo < hi) {
+    const uint32_t mid = lo + ((hi - lo) >> 1);
+    if (a[mid] < x) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+
+// Room for the candidates of a sampled top-k (the selected plus those between
+// the sampled floor and the exact threshold).
+inline int64_t list_capacity(int64_t capacity) { return capacity + capacity / 2 + 4096; }
+
+// A list entry (candidate index, value) is selected if its index is not 0
+// (index 0 is never transmitted) and, when the list still holds candidates of a
+// sampled top-k, its magnitude key reaches the exact threshold.
+template <typename S>
+__device__ inline bool list_selected(const int32_t *cand, const S *vals, const uint32_t *thr, uint32_t j,
+                                     uint32_t *t_out) {
+  const uint32_t t = (uint32_t)cand[j];
+  *t_out = t;
+  if (t == 0) return false;
+  return !thr || (vals[j] & KeyOf<S>::kMask) >= thr[0];
+}
+
+// Canonical order of a partition's serial tail out_idx[ser .. ser+cnt): ascending
+// index (the reference hands tickets to ascending indices), values fetched
+// again from the dense gradient.  Called by every thread of one block.
+template <typename S>
+__device__ inline void fix_serial_tail(int32_t *out_idx, S *out_val, const S *dense, uint32_t ser, uint32_t cnt,
+                                       uint32_t *lds_buf) {
+  if (cnt < 2) return;
+  uint32_t *region = reinterpret_cast<uint32_t *>(out_idx + ser);
+  if (cnt <= kSerialLds) {
+    for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) lds_buf[i] = region[i];
+    __syncthreads();
+    sort_network(lds_buf, cnt);
+    for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) region[i] = lds_buf[i];
+  } else {
+    sort_network(region, cnt);
+  }
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) out_val[ser + i] = dense[region[i]];
+}
+
+// Sort-based owner resolution (zen_resolve.hip): everything after the selected
+// list exists, without touching a table of the reference's size.
+struct ResolveArgs {
+  const void *dense;          // the gradient (serial tails re-fetch their values)
+  int dtype;
+  Probe g;
+  int partitions;
+  int64_t spp;                // serial slots per partition
+  const int32_t *list_idx;    // selected / candidate list
+  const void *list_val;
+  const uint32_t *count;      // its length (device)
+  const uint32_t *filter;     // optional exact threshold still to apply
+  int64_t list_cap;
+  uint32_t *keys_a, *perm_a, *more_a, *keys_b, *perm_b, *more_b;  // list_cap each
+  void *sort_scratch;
+  unsigned long long *hash;   // zeroed cells for slot -> smallest index, zero again on return
+  uint32_t hash_log2;
+  void *scratch;              // resolve_scratch_bytes(list_cap)
+  int32_t *out_idx;
+  void *out_val;
+  int64_t capacity;
+  int64_t *splits;
+  int32_t *status;
+};
+size_t resolve_scratch_bytes(int64_t list_cap, uint64_t key_limit);  // key_limit = P * (m / P + 1) + 1
+int resolve_and_place(const ResolveArgs &a, hipStream_t stream);
+
+}  // namespace zen

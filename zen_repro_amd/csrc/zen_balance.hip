@@ -9,7 +9,7 @@
 // empty marker 0 stays the smallest value): a thread that takes a slot from a
 // larger index carries on with that index's probe sequence, so every lost
 // probe is continued exactly once and no rounds or flags are needed.
-#include "zen_select.h"
+#include "zen_balance.h"
 
 namespace zen {
 namespace {
@@ -104,38 +104,6 @@ __global__ __launch_bounds__(256) void k_finalize_dense(const S *__restrict__ in
   }
 }
 
-// Ascending compare-exchange network (bitonic with mirrored first step), valid
-// for any n: positions >= n act as +infinity and never move.
-__device__ inline void sort_network(uint32_t *a, uint32_t n) {
-  uint32_t n2 = 1;
-  while (n2 < n) n2 <<= 1;
-  const uint32_t half = n2 >> 1;
-  for (uint32_t k = 2; k <= n2; k <<= 1) {
-    const uint32_t hk = k >> 1;
-    for (uint32_t q = threadIdx.x; q < half; q += blockDim.x) {
-      const uint32_t blk = q / hk, r = q % hk;
-      const uint32_t i = blk * k + r, l = blk * k + (k - 1 - r);
-      if (l < n) {
-        const uint32_t x = a[i], y = a[l];
-        if (x > y) { a[i] = y; a[l] = x; }
-      }
-    }
-    __syncthreads();
-    for (uint32_t j = hk >> 1; j > 0; j >>= 1) {
-      for (uint32_t q = threadIdx.x; q < half; q += blockDim.x) {
-        const uint32_t i = (q / j) * 2 * j + (q % j), l = i + j;
-        if (l < n) {
-          const uint32_t x = a[i], y = a[l];
-          if (x > y) { a[i] = y; a[l] = x; }
-        }
-      }
-      __syncthreads();
-    }
-  }
-}
-
-constexpr uint32_t kSerialLds = 8192;
-
 // Tickets are handed out in arrival order; the canonical order is ascending
 // index inside each partition's region, so each region is sorted in place.
 __global__ __launch_bounds__(256) void k_serial_sort(int32_t *serial, int64_t spp, const int32_t *offset) {
@@ -158,17 +126,6 @@ __global__ __launch_bounds__(256) void k_serial_sort(int32_t *serial, int64_t sp
 }
 
 // ------------------------------------------------- fused path (list based)
-
-// The list may hold candidates of a sampled top-k: entries whose magnitude key
-// is below the exact threshold (thr, optional) are not selected after all.
-template <typename S>
-__device__ inline bool list_selected(const int32_t *cand, const S *vals, const uint32_t *thr, uint32_t j,
-                                     uint32_t *t_out) {
-  const uint32_t t = (uint32_t)cand[j];
-  *t_out = t;
-  if (t == 0) return false;  // index 0 is never transmitted
-  return !thr || (vals[j] & KeyOf<S>::kMask) >= thr[0];
-}
 
 template <typename S>
 __global__ __launch_bounds__(256) void k_insert_list(const int32_t *__restrict__ cand, const S *__restrict__ vals,
@@ -219,15 +176,6 @@ __global__ __launch_bounds__(256) void k_gather(const uint32_t *__restrict__ key
   if (local < g.npp) table[part * g.npp + local] = 0u;  // leave the table empty again
 }
 
-__device__ inline uint32_t lower_bound_u32(const uint32_t *a, uint32_t n, uint32_t x) {
-  uint32_t lo = 0, hi = n;
-  while (lo < hi) {
-    const uint32_t mid = lo + ((hi - lo) >> 1);
-    if (a[mid] < x) lo = mid + 1; else hi = mid;
-  }
-  return lo;
-}
-
 // One block per partition: its length from the sorted keys, and the canonical
 // order of its serial tail.  The selected list arrives tile by tile in no
 // particular order and all serial entries of a partition share one sort key, so
@@ -255,19 +203,8 @@ __global__ __launch_bounds__(256) void k_splits_serial(const uint32_t *__restric
     if ((int64_t)(hi - ser) > spp) atomicOr(status, ZEN_STAT_SERIAL_OVERFLOW);
     if (hi > capacity) atomicOr(status, ZEN_STAT_CAPACITY);
   }
-  const uint32_t cnt = hi - ser;
-  if (cnt < 2 || hi > capacity) return;
-  uint32_t *region = reinterpret_cast<uint32_t *>(out_idx + ser);
-  if (cnt <= kSerialLds) {
-    for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) buf[i] = region[i];
-    __syncthreads();
-    sort_network(buf, cnt);
-    for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) region[i] = buf[i];
-  } else {
-    sort_network(region, cnt);
-  }
-  __syncthreads();
-  for (uint32_t i = threadIdx.x; i < cnt; i += blockDim.x) out_val[ser + i] = dense[region[i]];
+  if (hi > capacity) return;
+  fix_serial_tail<S>(out_idx, out_val, dense, ser, hi - ser, buf);
 }
 
 template <typename S>
@@ -298,24 +235,21 @@ int sparse_balance_launch(const S *in, int64_t n, uint32_t *table, Probe g, int3
 
 constexpr int64_t kSampleMinElems = 1ll << 24;  // below this the exact full-tensor histogram is cheap anyway
 
-// Room for the candidates of a sampled top-k (the selected plus those between
-// the sampled floor and the exact threshold).
-inline int64_t list_capacity(int64_t capacity) { return capacity + capacity / 2 + 4096; }
-
 struct BalancePlan {
   int32_t *sel_idx;    // the selected entries or candidates (list_capacity)
   uint32_t *sel_val;   // 4 bytes per value reserved, bf16 uses half
-  uint32_t *keys_a, *perm_a, *keys_b, *perm_b;
+  uint32_t *keys_a, *perm_a, *more_a, *keys_b, *perm_b, *more_b;
   uint32_t *count;     // entries in sel_*
   uint32_t *thr;       // [0..1] exact threshold + count, [2..3] sampled floor
   uint32_t *cand_hist;
   void *topk_scratch;
   void *select_scratch;
   void *sort_scratch;
+  void *resolve_scratch;
   size_t bytes;
 };
 
-BalancePlan plan_balance(void *workspace, int64_t n, int dtype, int64_t capacity) {
+BalancePlan plan_balance(void *workspace, int64_t n, int64_t m, int dtype, int64_t capacity) {
   Carver cv(workspace);
   BalancePlan p;
   const size_t cap = (size_t)list_capacity(capacity > 0 ? capacity : 1);
@@ -325,12 +259,16 @@ BalancePlan plan_balance(void *workspace, int64_t n, int dtype, int64_t capacity
   p.perm_a = cv.take<uint32_t>(cap);
   p.keys_b = cv.take<uint32_t>(cap);
   p.perm_b = cv.take<uint32_t>(cap);
+  p.more_a = cv.take<uint32_t>(cap);
+  p.more_b = cv.take<uint32_t>(cap);
   p.count = cv.take<uint32_t>(2);
   p.thr = cv.take<uint32_t>(4);
   p.cand_hist = cv.take<uint32_t>((size_t)kCandRows * kCandBins);
   p.topk_scratch = cv.take<char>(topk_scratch_bytes());
   p.select_scratch = cv.take<char>(select_scratch_bytes(n, dtype));
   p.sort_scratch = cv.take<char>(sort_scratch_bytes((int64_t)cap));
+  // m + P + 1 <= 2 m + 1 bounds the final-position keys whatever the partition count
+  p.resolve_scratch = cv.take<char>(resolve_scratch_bytes((int64_t)cap, 2ull * (uint64_t)m + 1));
   p.bytes = cv.used;
   return p;
 }
@@ -426,10 +364,10 @@ int zen_sparse_balance(const void *input, int dtype, int64_t n, int32_t *memory,
                                partitions, status, s);
 }
 
-size_t zen_load_balance_workspace(int64_t n, int dtype, int64_t capacity, int partitions) {
+size_t zen_load_balance_workspace(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions) {
   (void)partitions;
-  if (n <= 0 || capacity < 0) return 0;
-  return zen::plan_balance(nullptr, n, dtype, capacity).bytes;
+  if (n <= 0 || m <= 0 || capacity < 0) return 0;
+  return zen::plan_balance(nullptr, n, m, dtype, capacity).bytes;
 }
 
 int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
@@ -440,12 +378,12 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
   if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_load_balance: bad dtype");
   if (mode != ZEN_MODE_FAST && mode != ZEN_MODE_GENERAL) return fail(ZEN_EINVAL, "zen_load_balance: bad mode");
   if (n <= 0 || n > 0x7fffffffll || m <= 0 || m > 0x7fffffffll || partitions <= 0 || partitions > 65535 ||
-      m % partitions != 0 || capacity <= 0 || capacity > 0x3fffffffll)
-    return fail(ZEN_EINVAL, "zen_load_balance: need 0 < n, m < 2^31, m a multiple of partitions, 0 < capacity < 2^30");
+      m % partitions != 0 || capacity <= 0 || capacity > 0x1fffffffll)
+    return fail(ZEN_EINVAL, "zen_load_balance: need 0 < n, m < 2^31, m a multiple of partitions, 0 < capacity < 2^29");
   if (k < 0 || k > n || (k > 0 && thr)) return fail(ZEN_EINVAL, "zen_load_balance: need 0 <= k <= n and no thr with k");
   if (!input || !out_idx || !out_val || !splits || !table || !workspace || !status)
     return fail(ZEN_EINVAL, "zen_load_balance: null pointer");
-  if (workspace_bytes < zen_load_balance_workspace(n, dtype, capacity, partitions))
+  if (workspace_bytes < zen_load_balance_workspace(n, m, dtype, capacity, partitions))
     return fail(ZEN_EWORKSPACE, "zen_load_balance: workspace too small");
   hipStream_t s = static_cast<hipStream_t>(stream);
   Probe g;
@@ -455,13 +393,45 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
   const int64_t spp = n / partitions / 10;  // tensor_load_balance.py:18
   const uint32_t drop_key = (uint32_t)partitions * (g.npp + 1u);
   const int bits = ceil_log2_u64(drop_key);
-  BalancePlan p = plan_balance(workspace, n, dtype, capacity);
+  BalancePlan p = plan_balance(workspace, n, m, dtype, capacity);
 
   const uint32_t *filter = nullptr;
   int rc = select_stage(p, input, dtype, n, thr, k, capacity, mode, &filter, status, s);
   if (rc != ZEN_OK) return rc;
   if (k > 0 && thr_out) ZEN_HIP_CHECK(hipMemcpyAsync(thr_out, p.thr, 2 * sizeof(uint32_t), hipMemcpyDeviceToDevice, s));
   const int64_t lcap = list_capacity(capacity);
+  if (mode == ZEN_MODE_FAST && m >= 4096 && (reinterpret_cast<uintptr_t>(table) & 7u) == 0) {
+    // sort-based resolution: the table only lends its (zero) memory to a small hash map
+    ResolveArgs ra;
+    ra.dense = input;
+    ra.dtype = dtype;
+    ra.g = g;
+    ra.partitions = partitions;
+    ra.spp = spp;
+    ra.list_idx = p.sel_idx;
+    ra.list_val = p.sel_val;
+    ra.count = p.count;
+    ra.filter = filter;
+    ra.list_cap = lcap;
+    ra.keys_a = p.keys_a;
+    ra.perm_a = p.perm_a;
+    ra.keys_b = p.keys_b;
+    ra.perm_b = p.perm_b;
+    ra.more_a = p.more_a;
+    ra.more_b = p.more_b;
+    ra.sort_scratch = p.sort_scratch;
+    ra.hash = reinterpret_cast<unsigned long long *>(table);
+    uint32_t log2 = 0;
+    while (log2 < 24 && (2ull << log2) <= (uint64_t)m / 2) ++log2;
+    ra.hash_log2 = log2;
+    ra.scratch = p.resolve_scratch;
+    ra.out_idx = out_idx;
+    ra.out_val = out_val;
+    ra.capacity = capacity;
+    ra.splits = splits;
+    ra.status = status;
+    return resolve_and_place(ra, s);
+  }
   const unsigned blocks = (unsigned)ceil_div(lcap, 256);
   uint32_t *tab = reinterpret_cast<uint32_t *>(table);
   const uint16_t *val16 = reinterpret_cast<const uint16_t *>(p.sel_val);

@@ -4,7 +4,9 @@ namespace zen {
 namespace {
 
 __device__ inline uint32_t live_count(const uint32_t *count_dev, uint32_t count_imm) {
-  return count_dev ? *count_dev : count_imm;
+  if (!count_dev) return count_imm;
+  const uint32_t c = *count_dev;
+  return c < count_imm ? c : count_imm;
 }
 
 // Exclusive prefix of the bin histogram in one pass (look-back over tiles).

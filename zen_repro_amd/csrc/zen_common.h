@@ -291,9 +291,10 @@ inline void launch_fill(T *p, T v, size_t count, hipStream_t s) {
 // Stable LSD radix sort of (key, val) pairs on the low `bits` bits.  The result
 // ends in (keys_a, vals_a) when the returned value is 0 and in (keys_b,
 // vals_b) when it is 1; negative = error.  `scratch` from sort_scratch_bytes.
+// more_a / more_b: an optional second payload moved along with the first.
 size_t sort_scratch_bytes(int64_t max_count);
 int sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *vals_b,
                int64_t max_count, const uint32_t *count_dev, int bits, void *scratch,
-               int32_t *status, hipStream_t stream);
+               int32_t *status, hipStream_t stream, uint32_t *more_a = nullptr, uint32_t *more_b = nullptr);
 
 }  // namespace zen

@@ -9,15 +9,20 @@
 namespace zen {
 namespace {
 
-constexpr int kMrgBlock = 256;
+constexpr int kMrgBlock = 512;
 constexpr int kMrgItems = 16;  // consecutive sorted entries per thread (few, large tiles: short prefix chain)
 constexpr int kMrgTile = kMrgBlock * kMrgItems;
 
 // Validated sort keys; in fast mode also the coarse-bin histogram.
-template <typename I>
-__global__ __launch_bounds__(256) void k_merge_prep(const I *__restrict__ idx, uint32_t r, uint32_t dense_n,
-                                                    uint32_t *__restrict__ keys, uint32_t *__restrict__ perm,
-                                                    uint32_t *hist, int bshift, int32_t *status) {
+// In general mode the payload that travels with a key is the value itself (as
+// fp32 bits): the stable sort keeps arrival order, and the reduce kernel needs
+// no gather.  The bin sort needs distinct (key, payload) pairs, so in fast mode
+// the payload is the entry's position.
+template <typename I, typename S>
+__global__ __launch_bounds__(256) void k_merge_prep(const I *__restrict__ idx, const S *__restrict__ val, uint32_t r,
+                                                    uint32_t dense_n, uint32_t *__restrict__ keys,
+                                                    uint32_t *__restrict__ perm, uint32_t *hist, int bshift,
+                                                    int32_t *status) {
   const uint32_t j = blockIdx.x * 256u + threadIdx.x;
   if (j >= r) return;
   const I k = idx[j];
@@ -25,8 +30,10 @@ __global__ __launch_bounds__(256) void k_merge_prep(const I *__restrict__ idx, u
   if (!ok) atomicOr(status, ZEN_STAT_BAD_INDEX);
   const uint32_t key = ok ? (uint32_t)k : dense_n;  // bad indices sort behind every good one
   keys[j] = key;
-  if (perm) perm[j] = j;
-  if (hist) atomicAdd(&hist[key >> bshift], 1u);
+  if (hist)
+    atomicAdd(&hist[key >> bshift], 1u);
+  else
+    perm[j] = __float_as_uint(KeyOf<S>::to_f32(val[j]));
 }
 
 // One tile = kMrgTile consecutive sorted entries.  The tile's keys and values
@@ -41,7 +48,7 @@ template <typename S, typename I>
 __global__ __launch_bounds__(kMrgBlock) void k_merge_reduce(
     const uint32_t *__restrict__ keys, const uint32_t *__restrict__ perm, const S *__restrict__ val, uint32_t r,
     uint32_t dense_n, I *__restrict__ out_idx, float *__restrict__ out_val, int64_t capacity,
-    ScanState st, int ntiles, int64_t *out_count, const uint32_t *retry,
+    ScanState st, int ntiles, int64_t *out_count, const uint32_t *retry, bool payload_is_value,
     int32_t *status) {
   __shared__ uint32_t s_scan[kMrgBlock / 64 + 1];
   __shared__ uint64_t s_bcast;
@@ -68,7 +75,7 @@ __global__ __launch_bounds__(kMrgBlock) void k_merge_reduce(
     float v = 0.0f;
     if (i < r) {
       k = keys[i];
-      v = KeyOf<S>::to_f32(val[perm[i]]);
+      v = payload_is_value ? __uint_as_float(perm[i]) : KeyOf<S>::to_f32(val[perm[i]]);
     }
     s_key[mrg_slot(local)] = k;
     s_val[mrg_slot(local)] = v;
@@ -91,7 +98,8 @@ __global__ __launch_bounds__(kMrgBlock) void k_merge_reduce(
       int u = local;
       while (u < kMrgTile && s_key[mrg_slot(u)] == k[q]) acc += s_val[mrg_slot(u++)];
       if (u == kMrgTile)
-        for (uint32_t g = tile_base + kMrgTile; g < r && keys[g] == k[q]; ++g) acc += KeyOf<S>::to_f32(val[perm[g]]);
+        for (uint32_t g = tile_base + kMrgTile; g < r && keys[g] == k[q]; ++g)
+          acc += payload_is_value ? __uint_as_float(perm[g]) : KeyOf<S>::to_f32(val[perm[g]]);
       sum[q] = acc;
       if (acc != 0.0f) keep |= 1u << q;  // torch.nonzero keeps NaN, drops +-0
     }
@@ -104,15 +112,23 @@ __global__ __launch_bounds__(kMrgBlock) void k_merge_reduce(
     *out_count = (int64_t)all;
     if (all > (uint64_t)capacity) atomicOr(status, ZEN_STAT_CAPACITY);
   }
-  uint64_t pos = tile_start + before;
+  // compact the kept entries in LDS (everybody is past reading the staged tile:
+  // the scan above synchronised), then write them out with consecutive lanes
+  uint32_t li = before;
 #pragma unroll
   for (int q = 0; q < kMrgItems; ++q) {
     if (keep & (1u << q)) {
-      if (pos < (uint64_t)capacity) {
-        out_idx[pos] = (I)k[q];
-        out_val[pos] = sum[q];
-      }
-      ++pos;
+      s_key[li] = k[q];
+      s_val[li] = sum[q];
+      ++li;
+    }
+  }
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < total; i += kMrgBlock) {
+    const uint64_t pos = tile_start + i;
+    if (pos < (uint64_t)capacity) {
+      out_idx[pos] = (I)s_key[i];
+      out_val[pos] = s_val[i];
     }
   }
 }
@@ -177,11 +193,13 @@ int merge_launch(const void *idx, int idx64_in, const S *val, int64_t r, int64_t
   {
     ProfScope prof(kProfMergePrep, s);
     if (idx64_in)
-      k_merge_prep<int64_t><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const int64_t *>(idx), (uint32_t)r,
-                                                               (uint32_t)dense_n, p.keys, perm, hist, p.bs.bshift, status);
+      k_merge_prep<int64_t, S><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const int64_t *>(idx), val, (uint32_t)r,
+                                                                  (uint32_t)dense_n, p.keys, perm, hist, p.bs.bshift,
+                                                                  status);
     else
-      k_merge_prep<int32_t><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const int32_t *>(idx), (uint32_t)r,
-                                                               (uint32_t)dense_n, p.keys, perm, hist, p.bs.bshift, status);
+      k_merge_prep<int32_t, S><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const int32_t *>(idx), val, (uint32_t)r,
+                                                                  (uint32_t)dense_n, p.keys, perm, hist, p.bs.bshift,
+                                                                  status);
     ZEN_LAUNCH_CHECK("k_merge_prep");
   }
   const uint32_t *sk, *sp;
@@ -207,11 +225,11 @@ int merge_launch(const void *idx, int idx64_in, const S *val, int64_t r, int64_t
   if (idx64_out)
     k_merge_reduce<S, int64_t><<<dim3((unsigned)p.ntiles), dim3(kMrgBlock), 0, s>>>(
         sk, sp, val, (uint32_t)r, (uint32_t)dense_n, static_cast<int64_t *>(out_idx), out_val, capacity, st,
-        p.ntiles, out_count, retry, status);
+        p.ntiles, out_count, retry, !fast, status);
   else
     k_merge_reduce<S, int32_t><<<dim3((unsigned)p.ntiles), dim3(kMrgBlock), 0, s>>>(
         sk, sp, val, (uint32_t)r, (uint32_t)dense_n, static_cast<int32_t *>(out_idx), out_val, capacity, st,
-        p.ntiles, out_count, retry, status);
+        p.ntiles, out_count, retry, !fast, status);
   ZEN_LAUNCH_CHECK("k_merge_reduce");
   return ZEN_OK;
 }

@@ -79,7 +79,8 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_scan(uint32_t *__restrict__
 
 __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
     const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
-    uint32_t *__restrict__ keys_out, uint32_t *__restrict__ vals_out, const uint32_t *count_dev,
+    const uint32_t *__restrict__ more_in, uint32_t *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
+    uint32_t *__restrict__ more_out, const uint32_t *count_dev,
     uint32_t count_imm, int shift, uint32_t mask, int nblk, const uint32_t *__restrict__ offsets) {
   __shared__ uint32_t wcnt[kSortBlock / 64][kRadix];  // per wave: count, then start inside the tile
   __shared__ uint32_t gshift[kRadix];                 // global position = gshift[digit] + position in the tile
@@ -163,6 +164,17 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
     keys_out[g] = k;
     vals_out[g] = sval[j];
   }
+  if (!more_in) return;
+  // a second payload travels through the same LDS buffer in a second round
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kSortItems; ++i) {
+    const uint32_t at = wave_base + i * 64;
+    if (at < count) sval[wcnt[wave][(key[i] >> shift) & mask] + rank[i]] = more_in[at];
+  }
+  __syncthreads();
+  for (uint32_t j = threadIdx.x; j < tile_count; j += kSortBlock)
+    more_out[gshift[(skey[j] >> shift) & mask] + j] = sval[j];
 }
 
 __global__ void k_copy_pairs(const uint32_t *__restrict__ ka, const uint32_t *__restrict__ va,
@@ -190,7 +202,7 @@ size_t sort_scratch_bytes(int64_t max_count) {
 
 int sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *vals_b,
                int64_t max_count, const uint32_t *count_dev, int bits, void *scratch, int32_t *status,
-               hipStream_t stream) {
+               hipStream_t stream, uint32_t *more_a, uint32_t *more_b) {
   if (max_count < 0 || max_count > 0x7fffffffll || bits < 0 || bits > 32)
     return fail(ZEN_EINVAL, "sort_pairs: bad count or bits");
   if (max_count == 0 || bits == 0) return 0;
@@ -201,7 +213,7 @@ int sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *v
   launch_fill<unsigned long long>(scan, 0ull, kMaxPasses * scan_words(kRadix), stream);
   ZEN_LAUNCH_CHECK("sort: clear scan state");
   const int passes = (bits + 7) / 8;
-  uint32_t *ks = keys_a, *vs = vals_a, *kd = keys_b, *vd = vals_b;
+  uint32_t *ks = keys_a, *vs = vals_a, *kd = keys_b, *vd = vals_b, *ms = more_a, *md = more_b;
   for (int p = 0; p < passes; ++p) {
     const int shift = p * 8;
     const int width = bits - shift < 8 ? bits - shift : 8;
@@ -212,11 +224,12 @@ int sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *v
     k_sort_scan<<<dim3(kRadix), dim3(kSortBlock), 0, stream>>>(
         hist, nblk, scan_state(scan + (size_t)p * scan_words(kRadix), kRadix), status);
     ZEN_LAUNCH_CHECK("k_sort_scan");
-    k_sort_scatter<<<dim3(nblk), dim3(kSortBlock), 0, stream>>>(ks, vs, kd, vd, count_dev,
+    k_sort_scatter<<<dim3(nblk), dim3(kSortBlock), 0, stream>>>(ks, vs, ms, kd, vd, md, count_dev,
                                                                 (uint32_t)max_count, shift, mask, nblk, hist);
     ZEN_LAUNCH_CHECK("k_sort_scatter");
     uint32_t *t = ks; ks = kd; kd = t;
     t = vs; vs = vd; vd = t;
+    t = ms; ms = md; md = t;
   }
   return passes & 1;
 }

@@ -95,7 +95,7 @@ class TensorPartition:
         out_val = torch.empty(capacity, dtype=flat.dtype, device=dev)
         splits = torch.zeros(self.partitions, dtype=torch.int64, device=dev)
         status = _lib.status_word(dev)
-        nbytes = L.zen_load_balance_workspace(n, code, capacity, self.partitions)
+        nbytes = L.zen_load_balance_workspace(n, m, code, capacity, self.partitions)
         ws = _lib.scratch.get(dev, "load_balance", nbytes)
         table = self._table(dev, m)
         rc = L.zen_load_balance(
@@ -105,12 +105,12 @@ class TensorPartition:
         _lib.check(rc, "load_balance")
         return out_idx, out_val, splits, status
 
-    def load_balance(self, tensor, thr=None, capacity=None, k=0):
+    def load_balance(self, tensor, thr=None, capacity=None, k=0, mode=None):
         """Returns (indices[P], values[P], splits) like the reference
         (tensor_load_balance.py:43-51).  The per-partition tensors are views of
         two contiguous buffers; slicing them needs the split sizes on the
         host, which is this call's only synchronisation."""
-        for mode in (_lib.MODE_FAST, _lib.MODE_GENERAL):
+        for mode in ((_lib.MODE_FAST, _lib.MODE_GENERAL) if mode is None else (mode,)):
             out_idx, out_val, splits, status = self.load_balance_flat(tensor, thr, capacity, k, mode)
             host = torch.cat([splits, status.to(torch.int64)]).tolist()
             bits = host[-1]
