@@ -1,10 +1,10 @@
-// Stable LSD radix sort of (uint32 key, uint32 value) pairs, 8-bit digits.
-// Three kernels per digit: per-tile histogram, scan, stable scatter.  The
-// scatter ranks its tile in LDS (wave ballots + per-wave digit counters),
-// reorders the tile in LDS and writes every digit's run with consecutive lanes,
-// so global stores are contiguous runs instead of 4-byte scatters.  The element
-// count may live on the device, so grids are sized by the capacity and surplus
-// tiles retire immediately.
+// Stable LSD radix sort of (uint32 key, uint32 value[, uint32 value]) records.
+// Four kernels per digit: per-tile histogram, digit totals, offsets, stable
+// scatter.  The scatter ranks its tile in LDS (wave ballots + per-wave digit
+// counters), reorders the tile in LDS and writes every digit's run with
+// consecutive lanes, so global stores are contiguous runs instead of 4-byte
+// scatters.  The element count may live on the device, so grids are sized by
+// the capacity and surplus tiles retire immediately.
 #include "zen_common.h"
 
 namespace zen {
@@ -17,22 +17,25 @@ constexpr int kSortBlock = 256;
 constexpr int kSortItems = 16;                       // keys per thread
 constexpr int kSortTile = kSortBlock * kSortItems;   // 4096 keys per tile
 constexpr int kWaveSpan = 64 * kSortItems;           // contiguous keys owned by one wave
-constexpr int kRadix = 256;
-constexpr int kMaxPasses = 4;
+constexpr int kMaxRadix = 1024;
 
 __device__ inline uint32_t live_count(const uint32_t *count_dev, uint32_t count_imm) {
-  return count_dev ? *count_dev : count_imm;
+  if (!count_dev) return count_imm;
+  const uint32_t c = *count_dev;
+  return c < count_imm ? c : count_imm;
 }
 
 // hist[d * nblk + tile] = number of keys of this tile whose digit is d
+template <int RB>
 __global__ __launch_bounds__(kSortBlock) void k_sort_hist(const uint32_t *__restrict__ keys,
                                                           const uint32_t *count_dev, uint32_t count_imm,
                                                           int shift, uint32_t mask, int nblk,
                                                           uint32_t *__restrict__ hist) {
-  __shared__ uint32_t bins[kRadix];
+  constexpr int R = 1 << RB;
+  __shared__ uint32_t bins[R];
   const uint32_t count = live_count(count_dev, count_imm);
   const uint32_t base = blockIdx.x * (uint32_t)kSortTile;
-  bins[threadIdx.x] = 0;
+  for (int d = threadIdx.x; d < R; d += kSortBlock) bins[d] = 0;
   __syncthreads();
   if (base < count) {
     const uint32_t wave_base = base + (threadIdx.x >> 6) * kWaveSpan + (threadIdx.x & 63);
@@ -47,26 +50,32 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_hist(const uint32_t *__rest
       if (wave_base + i * 64 < count) atomicAdd(&bins[(k[i] >> shift) & mask], 1u);
   }
   __syncthreads();
-  hist[(size_t)threadIdx.x * nblk + blockIdx.x] = bins[threadIdx.x];
+  for (int d = threadIdx.x; d < R; d += kSortBlock) hist[(size_t)d * nblk + blockIdx.x] = bins[d];
 }
 
-// One block per digit (taken in ticket order): the digit's total goes through
-// the tile-prefix protocol to give the sum of all lower digits, then the row of
-// per-tile counts becomes per-tile global start offsets.
-__global__ __launch_bounds__(kSortBlock) void k_sort_scan(uint32_t *__restrict__ hist, int nblk, ScanState st,
-                                                          int32_t *status) {
+// Block d: totals[d] = sum of row d.
+__global__ __launch_bounds__(kSortBlock) void k_sort_totals(const uint32_t *__restrict__ hist, int nblk,
+                                                            uint32_t *__restrict__ totals) {
   __shared__ uint32_t smem[kSortBlock / 64 + 1];
-  __shared__ uint64_t s_bcast;
-  __shared__ int s_digit;
-  if (threadIdx.x == 0) s_digit = (int)atomicAdd(st.ticket, 1u);
-  __syncthreads();
-  const int d = s_digit;
-  uint32_t *row = hist + (size_t)d * nblk;
+  const uint32_t *row = hist + (size_t)blockIdx.x * nblk;
   uint32_t mine = 0;
   for (int b = threadIdx.x; b < nblk; b += kSortBlock) mine += row[b];
-  uint32_t row_total;
-  block_exclusive_scan<uint32_t, kSortBlock>(mine, smem, &row_total);
-  uint32_t running = (uint32_t)lookback_exclusive(st, d, row_total, status, &s_bcast);
+  uint32_t total;
+  block_exclusive_scan<uint32_t, kSortBlock>(mine, smem, &total);
+  if (threadIdx.x == 0) totals[blockIdx.x] = total;
+}
+
+// Block d: the row of per-tile counts becomes per-tile global start offsets
+// (keys of all lower digits first, then this digit's keys of earlier tiles).
+__global__ __launch_bounds__(kSortBlock) void k_sort_offsets(uint32_t *__restrict__ hist, int nblk,
+                                                             const uint32_t *__restrict__ totals) {
+  __shared__ uint32_t smem[kSortBlock / 64 + 1];
+  const int d = blockIdx.x;
+  uint32_t below = 0;
+  for (int e = threadIdx.x; e < d; e += kSortBlock) below += totals[e];
+  uint32_t running;
+  block_exclusive_scan<uint32_t, kSortBlock>(below, smem, &running);
+  uint32_t *row = hist + (size_t)d * nblk;
   for (int b0 = 0; b0 < nblk; b0 += kSortBlock) {
     const int b = b0 + threadIdx.x;
     const uint32_t v = b < nblk ? row[b] : 0u;
@@ -77,13 +86,16 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_scan(uint32_t *__restrict__
   }
 }
 
+template <int RB>
 __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
     const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
     const uint32_t *__restrict__ more_in, uint32_t *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
     uint32_t *__restrict__ more_out, const uint32_t *count_dev,
     uint32_t count_imm, int shift, uint32_t mask, int nblk, const uint32_t *__restrict__ offsets) {
-  __shared__ uint32_t wcnt[kSortBlock / 64][kRadix];  // per wave: count, then start inside the tile
-  __shared__ uint32_t gshift[kRadix];                 // global position = gshift[digit] + position in the tile
+  constexpr int R = 1 << RB;
+  constexpr int kPer = R / kSortBlock;  // digits per thread in the prefix step
+  __shared__ uint32_t wcnt[kSortBlock / 64][R];  // per wave: count, then start inside the tile
+  __shared__ uint32_t gshift[R];                 // global position = gshift[digit] + position in the tile
   __shared__ uint32_t smem[kSortBlock / 64 + 1];
   __shared__ uint32_t skey[kSortTile];
   __shared__ uint32_t sval[kSortTile];
@@ -93,8 +105,8 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
   const uint32_t tile_count = count - base < (uint32_t)kSortTile ? count - base : (uint32_t)kSortTile;
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
-#pragma unroll
-  for (int w = 0; w < kSortBlock / 64; ++w) wcnt[w][threadIdx.x] = 0;
+  for (int w = 0; w < kSortBlock / 64; ++w)
+    for (int d = threadIdx.x; d < R; d += kSortBlock) wcnt[w][d] = 0;
   __syncthreads();
 
   const uint32_t wave_base = base + wave * kWaveSpan + lane;
@@ -113,7 +125,7 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
     // lanes of this wave holding the same digit
     uint64_t peers = __ballot(valid);
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
+    for (int b = 0; b < RB; ++b) {
       const bool bit = (d >> b) & 1u;
       const uint64_t vote = __ballot(valid && bit);
       peers &= bit ? vote : ~vote;
@@ -130,21 +142,27 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
   }
   __syncthreads();
   {
-    // thread = digit: start of the digit inside the tile, then one start per wave
-    uint32_t c[kSortBlock / 64];
-    uint32_t total = 0;
+    // thread owns kPer consecutive digits: start of each digit inside the tile, then one start per wave
+    uint32_t c[kPer][kSortBlock / 64];
+    uint32_t mine = 0;
 #pragma unroll
-    for (int w = 0; w < kSortBlock / 64; ++w) {
-      c[w] = wcnt[w][threadIdx.x];
-      total += c[w];
-    }
+    for (int e = 0; e < kPer; ++e)
+#pragma unroll
+      for (int w = 0; w < kSortBlock / 64; ++w) {
+        c[e][w] = wcnt[w][threadIdx.x * kPer + e];
+        mine += c[e][w];
+      }
     uint32_t unused;
-    uint32_t running = block_exclusive_scan<uint32_t, kSortBlock>(total, smem, &unused);
-    gshift[threadIdx.x] = offsets[(size_t)threadIdx.x * nblk + blockIdx.x] - running;
+    uint32_t running = block_exclusive_scan<uint32_t, kSortBlock>(mine, smem, &unused);
 #pragma unroll
-    for (int w = 0; w < kSortBlock / 64; ++w) {
-      wcnt[w][threadIdx.x] = running;
-      running += c[w];
+    for (int e = 0; e < kPer; ++e) {
+      const int d = threadIdx.x * kPer + e;
+      gshift[d] = offsets[(size_t)d * nblk + blockIdx.x] - running;
+#pragma unroll
+      for (int w = 0; w < kSortBlock / 64; ++w) {
+        wcnt[w][d] = running;
+        running += c[e][w];
+      }
     }
   }
   __syncthreads();
@@ -196,37 +214,52 @@ inline int num_tiles(int64_t max_count) {
 
 size_t sort_scratch_bytes(int64_t max_count) {
   const size_t nblk = (size_t)num_tiles(max_count);
-  return align_up(nblk * kRadix * sizeof(uint32_t), 256) +
-         align_up(kMaxPasses * scan_words(kRadix) * sizeof(unsigned long long), 256);
+  return align_up(nblk * kMaxRadix * sizeof(uint32_t), 256) + align_up(kMaxRadix * sizeof(uint32_t), 256);
+}
+
+template <int RB>
+static int sort_pass(uint32_t *ks, uint32_t *vs, uint32_t *ms, uint32_t *kd, uint32_t *vd, uint32_t *md,
+                     int64_t max_count, const uint32_t *count_dev, int shift, uint32_t mask, int nblk,
+                     uint32_t *hist, uint32_t *totals, hipStream_t stream) {
+  constexpr int R = 1 << RB;
+  k_sort_hist<RB><<<dim3(nblk), dim3(kSortBlock), 0, stream>>>(ks, count_dev, (uint32_t)max_count, shift, mask, nblk,
+                                                               hist);
+  ZEN_LAUNCH_CHECK("k_sort_hist");
+  k_sort_totals<<<dim3(R), dim3(kSortBlock), 0, stream>>>(hist, nblk, totals);
+  ZEN_LAUNCH_CHECK("k_sort_totals");
+  k_sort_offsets<<<dim3(R), dim3(kSortBlock), 0, stream>>>(hist, nblk, totals);
+  ZEN_LAUNCH_CHECK("k_sort_offsets");
+  k_sort_scatter<RB><<<dim3(nblk), dim3(kSortBlock), 0, stream>>>(ks, vs, ms, kd, vd, md, count_dev,
+                                                                  (uint32_t)max_count, shift, mask, nblk, hist);
+  ZEN_LAUNCH_CHECK("k_sort_scatter");
+  return ZEN_OK;
 }
 
 int sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *vals_b,
                int64_t max_count, const uint32_t *count_dev, int bits, void *scratch, int32_t *status,
                hipStream_t stream, uint32_t *more_a, uint32_t *more_b) {
+  (void)status;
   if (max_count < 0 || max_count > 0x7fffffffll || bits < 0 || bits > 32)
     return fail(ZEN_EINVAL, "sort_pairs: bad count or bits");
   if (max_count == 0 || bits == 0) return 0;
   const int nblk = num_tiles(max_count);
   Carver cv(scratch);
-  uint32_t *hist = cv.take<uint32_t>((size_t)nblk * kRadix);
-  unsigned long long *scan = cv.take<unsigned long long>(kMaxPasses * scan_words(kRadix));
-  launch_fill<unsigned long long>(scan, 0ull, kMaxPasses * scan_words(kRadix), stream);
-  ZEN_LAUNCH_CHECK("sort: clear scan state");
-  const int passes = (bits + 7) / 8;
+  uint32_t *hist = cv.take<uint32_t>((size_t)nblk * kMaxRadix);
+  uint32_t *totals = cv.take<uint32_t>(kMaxRadix);
+  // 8-bit digits: 10-bit ones would save a pass on 25..30-bit keys, but with 4096-key tiles a digit's run
+  // shrinks to 4 keys and the scatter loses more than the pass gains (measured on MI355X)
+  const int rb = 8;
+  const int passes = (bits + rb - 1) / rb;
   uint32_t *ks = keys_a, *vs = vals_a, *kd = keys_b, *vd = vals_b, *ms = more_a, *md = more_b;
   for (int p = 0; p < passes; ++p) {
-    const int shift = p * 8;
-    const int width = bits - shift < 8 ? bits - shift : 8;
+    const int shift = p * rb;
+    const int width = bits - shift < rb ? bits - shift : rb;
     const uint32_t mask = (1u << width) - 1u;
-    k_sort_hist<<<dim3(nblk), dim3(kSortBlock), 0, stream>>>(ks, count_dev, (uint32_t)max_count, shift, mask, nblk,
-                                                             hist);
-    ZEN_LAUNCH_CHECK("k_sort_hist");
-    k_sort_scan<<<dim3(kRadix), dim3(kSortBlock), 0, stream>>>(
-        hist, nblk, scan_state(scan + (size_t)p * scan_words(kRadix), kRadix), status);
-    ZEN_LAUNCH_CHECK("k_sort_scan");
-    k_sort_scatter<<<dim3(nblk), dim3(kSortBlock), 0, stream>>>(ks, vs, ms, kd, vd, md, count_dev,
-                                                                (uint32_t)max_count, shift, mask, nblk, hist);
-    ZEN_LAUNCH_CHECK("k_sort_scatter");
+    const int rc = rb == 10 ? sort_pass<10>(ks, vs, ms, kd, vd, md, max_count, count_dev, shift, mask, nblk, hist,
+                                            totals, stream)
+                            : sort_pass<8>(ks, vs, ms, kd, vd, md, max_count, count_dev, shift, mask, nblk, hist,
+                                           totals, stream);
+    if (rc != ZEN_OK) return rc;
     uint32_t *t = ks; ks = kd; kd = t;
     t = vs; vs = vd; vd = t;
     t = ms; ms = md; md = t;
