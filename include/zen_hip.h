@@ -44,11 +44,11 @@ extern "C" {
 #define ZEN_STAT_CAPACITY 2        /* more output entries than `capacity`; the excess was dropped */
 #define ZEN_STAT_INTERNAL 4        /* a bounded in-kernel wait expired; outputs are invalid */
 #define ZEN_STAT_BAD_INDEX 8       /* merge/decode saw an index outside [0, dense_n); it was skipped */
-#define ZEN_STAT_RETRY 16          /* the fast path met keys piled on a few values and produced nothing:
+#define ZEN_STAT_RETRY 16          /* the fast path met keys piled on a few values; outputs unspecified:
                                       call again with ZEN_MODE_GENERAL */
 
 /* `mode` argument of the sort-based entry points */
-#define ZEN_MODE_FAST 0    /* two-level bin sort; flags ZEN_STAT_RETRY on pathological key distributions */
+#define ZEN_MODE_FAST 0    /* bucket sort in LDS; flags ZEN_STAT_RETRY on pathological key distributions */
 #define ZEN_MODE_GENERAL 1 /* one radix pass per 8 key bits; any input */
 
 int zen_abi_version(void);
@@ -207,6 +207,20 @@ size_t zen_sort_pairs_workspace(int64_t max_count);
 int zen_sort_pairs(uint32_t *keys, uint32_t *vals, int64_t max_count,
                    const uint32_t *count_dev, int bits,
                    void *workspace, size_t workspace_bytes, int32_t *status, void *stream);
+
+/*
+ * The same for keys that spread evenly over [0, sentinel), as hash slots and
+ * hashed indices do: one scatter pass into 511 key ranges, then every range
+ * sorted inside LDS.  Pairs with key >= sentinel come last in no particular
+ * order.  A key range too full for LDS sets ZEN_STAT_RETRY in *status (order
+ * then unspecified; use zen_sort_pairs).  zen_bucket_sort_fits tells whether
+ * (max_count, sentinel) is in the supported range; workspace as zen_sort_pairs.
+ * No counterpart in the reference.
+ */
+int zen_bucket_sort_fits(int64_t max_count, uint32_t sentinel);
+int zen_bucket_sort_pairs(uint32_t *keys, uint32_t *vals, int64_t max_count,
+                          const uint32_t *count_dev, uint32_t sentinel,
+                          void *workspace, size_t workspace_bytes, int32_t *status, void *stream);
 
 /*
  * Per-kernel timing with HIP events recorded on the launch stream, for

@@ -72,6 +72,59 @@ def test_sort_pairs_device_count(zen):
     assert np.array_equal(to_np(dk).view(np.uint32)[live:], keys[live:])  # tail untouched
 
 
+@pytest.mark.parametrize("count,sentinel,live,distinct", [
+    (1 << 16, 1 << 20, None, None), (70001, 743440384, None, None), (1 << 20, (1 << 30) + 7, None, None),
+    (3800000, 743440384, None, None), (1 << 20, 5000011, 300000, None), (1 << 18, 1 << 24, None, 700),
+])
+def test_bucket_sort_pairs_is_stable_sort(zen, count, sentinel, live, distinct):
+    """Evenly spread keys below the sentinel, some at or above it; duplicates keep their arrival order."""
+    from zen_repro_amd import _lib
+
+    rng = np.random.default_rng(count + sentinel % 1000)
+    keys = rng.integers(0, sentinel, count, dtype=np.uint64).astype(np.uint32)
+    if distinct:  # many equal keys
+        keys = (keys // np.uint32(sentinel // distinct) * np.uint32(sentinel // distinct)).astype(np.uint32)
+    tail = rng.random(count) < 0.05
+    keys[tail] = sentinel + (rng.integers(0, 2, int(tail.sum())).astype(np.uint32))
+    vals = np.arange(count, dtype=np.uint32)
+    dk, dv = to_dev(keys.view(np.int32)), to_dev(vals.view(np.int32))
+    n = count if live is None else live
+    cnt = None if live is None else torch.tensor([live], dtype=torch.int32, device="cuda")
+    L = _lib.lib()
+    assert L.zen_bucket_sort_fits(count, sentinel)
+    ws = torch.empty(L.zen_sort_pairs_workspace(count), dtype=torch.uint8, device="cuda")
+    st = torch.zeros(1, dtype=torch.int32, device="cuda")
+    rc = L.zen_bucket_sort_pairs(_lib.ptr(dk), _lib.ptr(dv), count, _lib.ptr(cnt), sentinel, _lib.ptr(ws),
+                                 ws.numel(), _lib.ptr(st), _lib.stream_of(dk.device))
+    assert rc == 0 and st.item() == 0
+    below = np.flatnonzero(keys[:n] < sentinel)
+    order = below[np.argsort(keys[below], kind="stable")]
+    got_k, got_v = to_np(dk).view(np.uint32), to_np(dv).view(np.uint32)
+    assert np.array_equal(got_k[:len(order)], keys[order])
+    assert np.array_equal(got_v[:len(order)], vals[order])
+    rest = np.flatnonzero(keys[:n] >= sentinel)  # behind, as a set, each still with its own value
+    assert np.array_equal(np.sort(got_v[len(order):n]), rest)
+    assert np.array_equal(got_k[len(order):n], keys[got_v[len(order):n]])
+    assert np.array_equal(got_k[n:], keys[n:])
+
+
+def test_bucket_sort_pairs_crowded_range_asks_for_retry(zen):
+    from zen_repro_amd import _lib
+
+    count, sentinel = 1 << 17, 1 << 24
+    keys = np.random.default_rng(5).integers(0, 20000, count, dtype=np.uint64).astype(np.uint32)  # one key range
+    dk, dv = to_dev(keys.view(np.int32)), to_dev(np.arange(count, dtype=np.int32))
+    L = _lib.lib()
+    ws = torch.empty(L.zen_sort_pairs_workspace(count), dtype=torch.uint8, device="cuda")
+    st = torch.zeros(1, dtype=torch.int32, device="cuda")
+    assert L.zen_bucket_sort_pairs(_lib.ptr(dk), _lib.ptr(dv), count, None, sentinel, _lib.ptr(ws), ws.numel(),
+                                   _lib.ptr(st), _lib.stream_of(dk.device)) == 0
+    assert st.item() == _lib.STAT_RETRY
+    assert not L.zen_bucket_sort_fits(1000, sentinel) and not L.zen_bucket_sort_fits(count, 1000)
+    assert L.zen_bucket_sort_pairs(_lib.ptr(dk), _lib.ptr(dv), 1000, None, sentinel, _lib.ptr(ws), ws.numel(),
+                                   _lib.ptr(st), _lib.stream_of(dk.device)) == _lib.EINVAL
+
+
 # ------------------------------------------------------------------ hash
 
 
@@ -451,11 +504,11 @@ def test_merge_piled_up_keys_fall_back_to_general_mode(zen, oracle):
 
     n = 1 << 20
     rng = np.random.default_rng(3)
-    idx = np.concatenate([np.full(20000, 12345), rng.integers(0, n, 5000)]).astype(np.int32)
+    idx = np.concatenate([np.full(100000, 12345), rng.integers(0, n, 50000)]).astype(np.int32)
     val = (rng.standard_normal(len(idx)) * 1e-3).astype(np.float32)
     lba = zen.LoadBalanceAllreduce(zen.LocalGroup(4), None, None)
     _, _, cnt, st = lba.merge_sparse_flat(to_dev(idx), to_dev(val), n, mode=_lib.MODE_FAST)
-    assert st.item() == _lib.STAT_RETRY and cnt.item() == 0
+    assert st.item() == _lib.STAT_RETRY  # one key range holds more than a workgroup sorts in LDS
     gi, gv = lba.merge_sparse(to_dev(idx), to_dev(val), n)  # retries by itself
     wi, wv = oracle.merge_sparse(idx, val, n)
     assert np.array_equal(to_np(gi), wi) and np.array_equal(to_np(gv).view(np.uint32), wv.view(np.uint32))

@@ -37,7 +37,7 @@ def test_workspace_queries_are_host_only(L):
     assert L.zen_topk_threshold_workspace() >= 2048 * 4
     a, b = L.zen_sort_pairs_workspace(1000), L.zen_sort_pairs_workspace(1 << 20)
     assert 0 < a < b
-    assert L.zen_merge_workspace(1 << 20, 1 << 30) >= 5 * 4 * (1 << 20)
+    assert L.zen_merge_workspace(1 << 20, 1 << 30) >= 4 * 4 * (1 << 20)
     assert L.zen_load_balance_workspace(1 << 24, 1 << 24, 1, 1 << 18, 16) >= 6 * 4 * (1 << 18)
     assert L.zen_select_workspace(1 << 24, 1) >= (1 << 24) // 8192 * 8
     assert L.zen_mapping_workspace(1 << 20, 8) >= 16 * (1 << 20)

@@ -57,6 +57,8 @@ def lib():
         "zen_decode_dense": (i32, [vp, i32, vp, i32, i64, vp, i64, i32, vp, sz, vp, vp]),
         "zen_sort_pairs_workspace": (sz, [i64]),
         "zen_sort_pairs": (i32, [vp, vp, i64, vp, i32, vp, sz, vp, vp]),
+        "zen_bucket_sort_fits": (i32, [i64, ctypes.c_uint32]),
+        "zen_bucket_sort_pairs": (i32, [vp, vp, i64, vp, ctypes.c_uint32, vp, sz, vp, vp]),
         "zen_profile_enable": (i32, [i32]),
         "zen_profile_tags": (i32, []),
         "zen_profile_name": (ctypes.c_char_p, [i32]),

@@ -108,12 +108,12 @@ class LoadBalanceAllreduce:
         return idx, val
 
     def merge_sparse_flat(self, indices_tensors, values_tensors, dense_size, capacity=None, idx64=False,
-                          mode=_lib.MODE_GENERAL):
+                          mode=_lib.MODE_FAST):
         """decode_sparse_tensors followed by encode_sparse_tensor (comm.py:125-127)
         without the dense intermediate and without host synchronisation.
         Returns (indices, fp32 sums, count int64[1], status int32[1]); the first
         `count` entries are valid and ascending.  In fast mode a status with
-        STAT_RETRY means nothing was produced and the call must be repeated
+        STAT_RETRY means the outputs are unspecified and the call must be repeated
         with mode=MODE_GENERAL (merge_sparse does that by itself)."""
         indices = self.stack_tensors(indices_tensors)
         values = self.stack_tensors(values_tensors)

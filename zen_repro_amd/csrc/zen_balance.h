@@ -99,6 +99,7 @@ struct ResolveArgs {
   const uint32_t *count;      // its length (device)
   const uint32_t *filter;     // optional exact threshold still to apply
   int64_t list_cap;
+  int64_t expected;           // how many entries the caller expects the list to hold
   uint32_t *keys_a, *perm_a, *more_a, *keys_b, *perm_b, *more_b;  // list_cap each
   void *sort_scratch;
   unsigned long long *hash;   // zeroed cells for slot -> smallest index, zero again on return

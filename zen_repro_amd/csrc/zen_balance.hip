@@ -413,6 +413,7 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
     ra.count = p.count;
     ra.filter = filter;
     ra.list_cap = lcap;
+    ra.expected = k > 0 ? k + k / 16 + 1024 : capacity;
     ra.keys_a = p.keys_a;
     ra.perm_a = p.perm_a;
     ra.keys_b = p.keys_b;

@@ -297,4 +297,15 @@ int sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *v
                int64_t max_count, const uint32_t *count_dev, int bits, void *scratch,
                int32_t *status, hipStream_t stream, uint32_t *more_a = nullptr, uint32_t *more_b = nullptr);
 
+// Stable sort of records whose keys spread evenly over [0, sentinel) (hash slots, hashed indices): one
+// scatter pass into 511 key ranges, then each range sorted inside LDS by one workgroup.  Records with
+// key >= sentinel come last, in no particular order.  The result is in the b arrays (returns 1; negative =
+// error).  A key range holding more records than fit in LDS sets ZEN_STAT_RETRY in *status and the order
+// is then unspecified.  bucket_sort_fits: whether `expected` records (the live count may sit on the device)
+// leave the key ranges room to spare; same scratch as sort_pairs.
+bool bucket_sort_fits(int64_t expected, uint32_t sentinel);
+int bucket_sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *vals_b, int64_t max_count,
+                      const uint32_t *count_dev, uint32_t sentinel, void *scratch, int32_t *status,
+                      hipStream_t stream, uint32_t *more_a = nullptr, uint32_t *more_b = nullptr);
+
 }  // namespace zen

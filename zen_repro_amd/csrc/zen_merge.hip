@@ -4,7 +4,7 @@
 // are stably sorted by index, equal indices are summed in fp32 in arrival order
 // (the order a sequential scatter_add_ uses, so the result is reproducible),
 // zero sums are dropped and the survivors leave in ascending index order.
-#include "zen_binsort.h"
+#include "zen_common.h"
 
 namespace zen {
 namespace {
@@ -13,16 +13,13 @@ constexpr int kMrgBlock = 512;
 constexpr int kMrgItems = 16;  // consecutive sorted entries per thread (few, large tiles: short prefix chain)
 constexpr int kMrgTile = kMrgBlock * kMrgItems;
 
-// Validated sort keys; in fast mode also the coarse-bin histogram.
-// In general mode the payload that travels with a key is the value itself (as
-// fp32 bits): the stable sort keeps arrival order, and the reduce kernel needs
-// no gather.  The bin sort needs distinct (key, payload) pairs, so in fast mode
-// the payload is the entry's position.
+// Validated sort keys.  The payload that travels with a key is the value itself
+// (as fp32 bits): the stable sort keeps arrival order, and the reduce kernel
+// needs no gather.
 template <typename I, typename S>
 __global__ __launch_bounds__(256) void k_merge_prep(const I *__restrict__ idx, const S *__restrict__ val, uint32_t r,
                                                     uint32_t dense_n, uint32_t *__restrict__ keys,
-                                                    uint32_t *__restrict__ perm, uint32_t *hist, int bshift,
-                                                    int32_t *status) {
+                                                    uint32_t *__restrict__ perm, int32_t *status) {
   const uint32_t j = blockIdx.x * 256u + threadIdx.x;
   if (j >= r) return;
   const I k = idx[j];
@@ -30,38 +27,25 @@ __global__ __launch_bounds__(256) void k_merge_prep(const I *__restrict__ idx, c
   if (!ok) atomicOr(status, ZEN_STAT_BAD_INDEX);
   const uint32_t key = ok ? (uint32_t)k : dense_n;  // bad indices sort behind every good one
   keys[j] = key;
-  if (hist)
-    atomicAdd(&hist[key >> bshift], 1u);
-  else
-    perm[j] = __float_as_uint(KeyOf<S>::to_f32(val[j]));
+  perm[j] = __float_as_uint(KeyOf<S>::to_f32(val[j]));
 }
 
 // One tile = kMrgTile consecutive sorted entries.  The tile's keys and values
-// (gathered through the sort permutation) are first brought into LDS with
-// independent, coalesced loads, so the latency of the gather is paid once per
-// tile instead of once per entry; each thread then walks kMrgItems consecutive
-// entries in LDS.  A run that continues past the tile is finished from global
+// are first brought into LDS with coalesced loads; each thread then walks
+// kMrgItems consecutive entries in LDS.  A run that continues past the tile is finished from global
 // memory by the thread that owns its head.
 __device__ inline int mrg_slot(int i) { return i + (i >> 4); }  // one pad word per 16: conflict-free strides
 
-template <typename S, typename I>
+template <typename I>
 __global__ __launch_bounds__(kMrgBlock) void k_merge_reduce(
-    const uint32_t *__restrict__ keys, const uint32_t *__restrict__ perm, const S *__restrict__ val, uint32_t r,
+    const uint32_t *__restrict__ keys, const uint32_t *__restrict__ perm, uint32_t r,
     uint32_t dense_n, I *__restrict__ out_idx, float *__restrict__ out_val, int64_t capacity,
-    ScanState st, int ntiles, int64_t *out_count, const uint32_t *retry, bool payload_is_value,
-    int32_t *status) {
+    ScanState st, int ntiles, int64_t *out_count, int32_t *status) {
   __shared__ uint32_t s_scan[kMrgBlock / 64 + 1];
   __shared__ uint64_t s_bcast;
   __shared__ int s_tile;
   __shared__ uint32_t s_key[kMrgTile + kMrgTile / 16];
   __shared__ float s_val[kMrgTile + kMrgTile / 16];
-  if (retry && *retry) {  // the bin sort gave up: nothing was sorted
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
-      *out_count = 0;
-      atomicOr(status, ZEN_STAT_RETRY);
-    }
-    return;
-  }
   if (threadIdx.x == 0) s_tile = (int)atomicAdd(st.ticket, 1u);
   __syncthreads();
   const int tile = s_tile;
@@ -75,7 +59,7 @@ __global__ __launch_bounds__(kMrgBlock) void k_merge_reduce(
     float v = 0.0f;
     if (i < r) {
       k = keys[i];
-      v = payload_is_value ? __uint_as_float(perm[i]) : KeyOf<S>::to_f32(val[perm[i]]);
+      v = __uint_as_float(perm[i]);
     }
     s_key[mrg_slot(local)] = k;
     s_val[mrg_slot(local)] = v;
@@ -99,7 +83,7 @@ __global__ __launch_bounds__(kMrgBlock) void k_merge_reduce(
       while (u < kMrgTile && s_key[mrg_slot(u)] == k[q]) acc += s_val[mrg_slot(u++)];
       if (u == kMrgTile)
         for (uint32_t g = tile_base + kMrgTile; g < r && keys[g] == k[q]; ++g)
-          acc += payload_is_value ? __uint_as_float(perm[g]) : KeyOf<S>::to_f32(val[perm[g]]);
+          acc += __uint_as_float(perm[g]);
       sum[q] = acc;
       if (acc != 0.0f) keep |= 1u << q;  // torch.nonzero keeps NaN, drops +-0
     }
@@ -152,9 +136,8 @@ __global__ __launch_bounds__(256) void k_scatter_dense<uint16_t>(const int32_t *
 }
 
 struct MergePlan {
-  uint32_t *keys, *tmp_k, *tmp_v, *sort_k, *sort_v;
-  void *scan;  // prefix state of the reduce kernel (inside the bin sort's cleared area)
-  BinSort bs;
+  uint32_t *keys, *tmp_v, *sort_k, *sort_v;
+  void *scan;  // prefix state of the reduce kernel
   void *sort_scratch;
   size_t bytes;
   int ntiles;
@@ -164,16 +147,13 @@ MergePlan plan_merge(void *workspace, int64_t r, int64_t dense_n) {
   Carver cv(workspace);
   MergePlan p;
   const size_t cap = (size_t)(r > 0 ? r : 1);
+  (void)dense_n;
   p.keys = cv.take<uint32_t>(cap);
-  p.tmp_k = cv.take<uint32_t>(cap);
   p.tmp_v = cv.take<uint32_t>(cap);
   p.sort_k = cv.take<uint32_t>(cap);
   p.sort_v = cv.take<uint32_t>(cap);
   p.ntiles = (int)ceil_div((int64_t)cap, kMrgTile);
-  const size_t desc_bytes = scan_words(p.ntiles) * sizeof(unsigned long long);
-  char *bs_base = cv.take<char>(plan_binsort(nullptr, (uint64_t)dense_n + 1, (int64_t)cap, desc_bytes).bytes);
-  p.bs = plan_binsort(workspace ? bs_base : nullptr, (uint64_t)dense_n + 1, (int64_t)cap, desc_bytes);
-  p.scan = p.bs.extra;
+  p.scan = cv.take<unsigned long long>(scan_words(p.ntiles));
   p.sort_scratch = cv.take<char>(sort_scratch_bytes((int64_t)cap));
   p.bytes = cv.used;
   return p;
@@ -184,52 +164,44 @@ int merge_launch(const void *idx, int idx64_in, const S *val, int64_t r, int64_t
                  int idx64_out, float *out_val, int64_t capacity, int64_t *out_count, int mode, void *workspace,
                  int32_t *status, hipStream_t s) {
   MergePlan p = plan_merge(workspace, r, dense_n);
-  const bool fast = mode == ZEN_MODE_FAST;
   const unsigned blocks = (unsigned)ceil_div(r, 256);
-  int rc = binsort_clear(p.bs, s);  // also clears the reduce descriptors
-  if (rc != ZEN_OK) return rc;
-  uint32_t *perm = fast ? nullptr : p.tmp_v;
-  uint32_t *hist = fast ? p.bs.hist : nullptr;
+  launch_fill<unsigned long long>(static_cast<unsigned long long *>(p.scan), 0ull, scan_words(p.ntiles), s);
   {
     ProfScope prof(kProfMergePrep, s);
     if (idx64_in)
       k_merge_prep<int64_t, S><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const int64_t *>(idx), val, (uint32_t)r,
-                                                                  (uint32_t)dense_n, p.keys, perm, hist, p.bs.bshift,
-                                                                  status);
+                                                                  (uint32_t)dense_n, p.keys, p.tmp_v, status);
     else
       k_merge_prep<int32_t, S><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const int32_t *>(idx), val, (uint32_t)r,
-                                                                  (uint32_t)dense_n, p.keys, perm, hist, p.bs.bshift,
-                                                                  status);
+                                                                  (uint32_t)dense_n, p.keys, p.tmp_v, status);
     ZEN_LAUNCH_CHECK("k_merge_prep");
   }
   const uint32_t *sk, *sp;
   {
+    // fast mode: indices that a hash assigned to one destination spread evenly over the dense length, so
+    // the bucket sort applies; a crowded key range makes it raise ZEN_STAT_RETRY
     ProfScope prof(kProfSort, s);
-    if (fast) {
-      if ((rc = binsort_scan(p.bs, status, s)) != ZEN_OK) return rc;
-      if ((rc = binsort_scatter(p.bs, p.keys, nullptr, r, nullptr, p.tmp_k, p.tmp_v, s)) != ZEN_OK) return rc;
-      if ((rc = binsort_rank(p.bs, p.tmp_k, p.tmp_v, r, nullptr, p.sort_k, p.sort_v, s)) != ZEN_OK) return rc;
-      sk = p.sort_k;
-      sp = p.sort_v;
-    } else {
-      const int bits = ceil_log2_u64((uint64_t)dense_n);
-      const int where = sort_pairs(p.keys, p.tmp_v, p.sort_k, p.sort_v, r, nullptr, bits, p.sort_scratch, status, s);
-      if (where < 0) return where;
-      sk = where ? p.sort_k : p.keys;
-      sp = where ? p.sort_v : p.tmp_v;
-    }
+    int where;
+    if (mode == ZEN_MODE_FAST && bucket_sort_fits(r, (uint32_t)dense_n))
+      where = bucket_sort_pairs(p.keys, p.tmp_v, p.sort_k, p.sort_v, r, nullptr, (uint32_t)dense_n, p.sort_scratch,
+                                status, s);
+    else
+      where = sort_pairs(p.keys, p.tmp_v, p.sort_k, p.sort_v, r, nullptr, ceil_log2_u64((uint64_t)dense_n),
+                         p.sort_scratch, status, s);
+    if (where < 0) return where;
+    sk = where ? p.sort_k : p.keys;
+    sp = where ? p.sort_v : p.tmp_v;
   }
   const ScanState st = scan_state(p.scan, p.ntiles);
-  const uint32_t *retry = fast ? p.bs.retry : nullptr;
   ProfScope prof(kProfMergeReduce, s);
   if (idx64_out)
-    k_merge_reduce<S, int64_t><<<dim3((unsigned)p.ntiles), dim3(kMrgBlock), 0, s>>>(
-        sk, sp, val, (uint32_t)r, (uint32_t)dense_n, static_cast<int64_t *>(out_idx), out_val, capacity, st,
-        p.ntiles, out_count, retry, !fast, status);
+    k_merge_reduce<int64_t><<<dim3((unsigned)p.ntiles), dim3(kMrgBlock), 0, s>>>(
+        sk, sp, (uint32_t)r, (uint32_t)dense_n, static_cast<int64_t *>(out_idx), out_val, capacity, st, p.ntiles,
+        out_count, status);
   else
-    k_merge_reduce<S, int32_t><<<dim3((unsigned)p.ntiles), dim3(kMrgBlock), 0, s>>>(
-        sk, sp, val, (uint32_t)r, (uint32_t)dense_n, static_cast<int32_t *>(out_idx), out_val, capacity, st,
-        p.ntiles, out_count, retry, !fast, status);
+    k_merge_reduce<int32_t><<<dim3((unsigned)p.ntiles), dim3(kMrgBlock), 0, s>>>(
+        sk, sp, (uint32_t)r, (uint32_t)dense_n, static_cast<int32_t *>(out_idx), out_val, capacity, st, p.ntiles,
+        out_count, status);
   ZEN_LAUNCH_CHECK("k_merge_reduce");
   return ZEN_OK;
 }

@@ -448,8 +448,13 @@ int resolve_launch(const ResolveArgs &a, hipStream_t s) {
   int where;
   {
     ProfScope prof(kProfSort, s);
-    where = sort_pairs(a.keys_a, a.perm_a, a.keys_b, a.perm_b, a.list_cap, a.count, ceil_log2_u64(g.m),
-                       a.sort_scratch, a.status, s, a.more_a, a.more_b);
+    // level-1 slots are hash values: they spread evenly over [0, m), filtered entries carry the key m
+    if (bucket_sort_fits(a.expected, g.m))
+      where = bucket_sort_pairs(a.keys_a, a.perm_a, a.keys_b, a.perm_b, a.list_cap, a.count, g.m, a.sort_scratch,
+                                a.status, s, a.more_a, a.more_b);
+    else
+      where = sort_pairs(a.keys_a, a.perm_a, a.keys_b, a.perm_b, a.list_cap, a.count, ceil_log2_u64(g.m),
+                         a.sort_scratch, a.status, s, a.more_a, a.more_b);
   }
   if (where < 0) return where;
   uint32_t *sk = where ? a.keys_b : a.keys_a, *st = where ? a.perm_b : a.perm_a, *sv = where ? a.more_b : a.more_a;

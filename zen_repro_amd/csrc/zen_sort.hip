@@ -19,6 +19,25 @@ constexpr int kSortTile = kSortBlock * kSortItems;   // 4096 keys per tile
 constexpr int kWaveSpan = 64 * kSortItems;           // contiguous keys owned by one wave
 constexpr int kMaxRadix = 1024;
 
+// Digit of a key: a bit field (LSD passes), or a monotone map of [0, sentinel) onto `last` equal ranges
+// with every key >= sentinel in a range of its own (bucket pass).
+struct DigitField {
+  int shift;
+  uint32_t mask;
+  __device__ uint32_t operator()(uint32_t k) const { return (k >> shift) & mask; }
+};
+struct DigitRange {
+  uint32_t mult;      // floor(last * 2^32 / sentinel)
+  uint32_t sentinel;
+  uint32_t last;      // number of real ranges = index of the sentinel's own
+  __device__ uint32_t operator()(uint32_t k) const {
+    return k >= sentinel ? last : (uint32_t)(((uint64_t)k * mult) >> 32);
+  }
+  __device__ uint32_t first_key(uint32_t b) const {  // smallest key of range b
+    return (uint32_t)((((uint64_t)b << 32) + mult - 1) / mult);
+  }
+};
+
 __device__ inline uint32_t live_count(const uint32_t *count_dev, uint32_t count_imm) {
   if (!count_dev) return count_imm;
   const uint32_t c = *count_dev;
@@ -26,10 +45,10 @@ __device__ inline uint32_t live_count(const uint32_t *count_dev, uint32_t count_
 }
 
 // hist[d * nblk + tile] = number of keys of this tile whose digit is d
-template <int RB>
+template <int RB, typename Digit>
 __global__ __launch_bounds__(kSortBlock) void k_sort_hist(const uint32_t *__restrict__ keys,
                                                           const uint32_t *count_dev, uint32_t count_imm,
-                                                          int shift, uint32_t mask, int nblk,
+                                                          Digit digit, int nblk,
                                                           uint32_t *__restrict__ hist) {
   constexpr int R = 1 << RB;
   __shared__ uint32_t bins[R];
@@ -47,7 +66,7 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_hist(const uint32_t *__rest
     }
 #pragma unroll
     for (int i = 0; i < kSortItems; ++i)
-      if (wave_base + i * 64 < count) atomicAdd(&bins[(k[i] >> shift) & mask], 1u);
+      if (wave_base + i * 64 < count) atomicAdd(&bins[digit(k[i])], 1u);
   }
   __syncthreads();
   for (int d = threadIdx.x; d < R; d += kSortBlock) hist[(size_t)d * nblk + blockIdx.x] = bins[d];
@@ -86,12 +105,12 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_offsets(uint32_t *__restric
   }
 }
 
-template <int RB>
+template <int RB, typename Digit>
 __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
     const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
     const uint32_t *__restrict__ more_in, uint32_t *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
     uint32_t *__restrict__ more_out, const uint32_t *count_dev,
-    uint32_t count_imm, int shift, uint32_t mask, int nblk, const uint32_t *__restrict__ offsets) {
+    uint32_t count_imm, Digit digit, int nblk, const uint32_t *__restrict__ offsets) {
   constexpr int R = 1 << RB;
   constexpr int kPer = R / kSortBlock;  // digits per thread in the prefix step
   __shared__ uint32_t wcnt[kSortBlock / 64][R];  // per wave: count, then start inside the tile
@@ -121,7 +140,7 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
 #pragma unroll
   for (int i = 0; i < kSortItems; ++i) {
     const bool valid = wave_base + i * 64 < count;
-    const uint32_t d = (key[i] >> shift) & mask;
+    const uint32_t d = digit(key[i]);
     // lanes of this wave holding the same digit
     uint64_t peers = __ballot(valid);
 #pragma unroll
@@ -170,7 +189,7 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
   for (int i = 0; i < kSortItems; ++i) {
     const uint32_t at = wave_base + i * 64;
     if (at < count) {
-      const uint32_t pos = wcnt[wave][(key[i] >> shift) & mask] + rank[i];
+      const uint32_t pos = wcnt[wave][digit(key[i])] + rank[i];
       skey[pos] = key[i];
       sval[pos] = vals_in[at];
     }
@@ -178,7 +197,7 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
   __syncthreads();
   for (uint32_t j = threadIdx.x; j < tile_count; j += kSortBlock) {
     const uint32_t k = skey[j];
-    const uint32_t g = gshift[(k >> shift) & mask] + j;
+    const uint32_t g = gshift[digit(k)] + j;
     keys_out[g] = k;
     vals_out[g] = sval[j];
   }
@@ -188,11 +207,11 @@ __global__ __launch_bounds__(kSortBlock) void k_sort_scatter(
 #pragma unroll
   for (int i = 0; i < kSortItems; ++i) {
     const uint32_t at = wave_base + i * 64;
-    if (at < count) sval[wcnt[wave][(key[i] >> shift) & mask] + rank[i]] = more_in[at];
+    if (at < count) sval[wcnt[wave][digit(key[i])] + rank[i]] = more_in[at];
   }
   __syncthreads();
   for (uint32_t j = threadIdx.x; j < tile_count; j += kSortBlock)
-    more_out[gshift[(skey[j] >> shift) & mask] + j] = sval[j];
+    more_out[gshift[digit(skey[j])] + j] = sval[j];
 }
 
 __global__ void k_copy_pairs(const uint32_t *__restrict__ ka, const uint32_t *__restrict__ va,
@@ -217,20 +236,20 @@ size_t sort_scratch_bytes(int64_t max_count) {
   return align_up(nblk * kMaxRadix * sizeof(uint32_t), 256) + align_up(kMaxRadix * sizeof(uint32_t), 256);
 }
 
-template <int RB>
+template <int RB, typename Digit>
 static int sort_pass(uint32_t *ks, uint32_t *vs, uint32_t *ms, uint32_t *kd, uint32_t *vd, uint32_t *md,
-                     int64_t max_count, const uint32_t *count_dev, int shift, uint32_t mask, int nblk,
+                     int64_t max_count, const uint32_t *count_dev, Digit digit, int nblk,
                      uint32_t *hist, uint32_t *totals, hipStream_t stream) {
   constexpr int R = 1 << RB;
-  k_sort_hist<RB><<<dim3(nblk), dim3(kSortBlock), 0, stream>>>(ks, count_dev, (uint32_t)max_count, shift, mask, nblk,
-                                                               hist);
+  k_sort_hist<RB, Digit><<<dim3(nblk), dim3(kSortBlock), 0, stream>>>(ks, count_dev, (uint32_t)max_count, digit,
+                                                                      nblk, hist);
   ZEN_LAUNCH_CHECK("k_sort_hist");
   k_sort_totals<<<dim3(R), dim3(kSortBlock), 0, stream>>>(hist, nblk, totals);
   ZEN_LAUNCH_CHECK("k_sort_totals");
   k_sort_offsets<<<dim3(R), dim3(kSortBlock), 0, stream>>>(hist, nblk, totals);
   ZEN_LAUNCH_CHECK("k_sort_offsets");
-  k_sort_scatter<RB><<<dim3(nblk), dim3(kSortBlock), 0, stream>>>(ks, vs, ms, kd, vd, md, count_dev,
-                                                                  (uint32_t)max_count, shift, mask, nblk, hist);
+  k_sort_scatter<RB, Digit><<<dim3(nblk), dim3(kSortBlock), 0, stream>>>(ks, vs, ms, kd, vd, md, count_dev,
+                                                                         (uint32_t)max_count, digit, nblk, hist);
   ZEN_LAUNCH_CHECK("k_sort_scatter");
   return ZEN_OK;
 }
@@ -248,17 +267,15 @@ int sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *v
   uint32_t *totals = cv.take<uint32_t>(kMaxRadix);
   // 8-bit digits: 10-bit ones would save a pass on 25..30-bit keys, but with 4096-key tiles a digit's run
   // shrinks to 4 keys and the scatter loses more than the pass gains (measured on MI355X)
-  const int rb = 8;
+  constexpr int rb = 8;
   const int passes = (bits + rb - 1) / rb;
   uint32_t *ks = keys_a, *vs = vals_a, *kd = keys_b, *vd = vals_b, *ms = more_a, *md = more_b;
   for (int p = 0; p < passes; ++p) {
     const int shift = p * rb;
     const int width = bits - shift < rb ? bits - shift : rb;
     const uint32_t mask = (1u << width) - 1u;
-    const int rc = rb == 10 ? sort_pass<10>(ks, vs, ms, kd, vd, md, max_count, count_dev, shift, mask, nblk, hist,
-                                            totals, stream)
-                            : sort_pass<8>(ks, vs, ms, kd, vd, md, max_count, count_dev, shift, mask, nblk, hist,
-                                           totals, stream);
+    const int rc = sort_pass<8>(ks, vs, ms, kd, vd, md, max_count, count_dev, DigitField{shift, mask}, nblk, hist,
+                                totals, stream);
     if (rc != ZEN_OK) return rc;
     uint32_t *t = ks; ks = kd; kd = t;
     t = vs; vs = vd; vd = t;
@@ -266,6 +283,170 @@ int sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *v
   }
   return passes & 1;
 }
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// Bucket sort for keys that spread evenly over [0, sentinel): one scatter pass
+// by DigitRange puts every key range into a contiguous bucket, then one
+// workgroup per bucket sorts its records completely inside LDS (stable LSD
+// passes of 7 bits over key - first key of the bucket) and writes them back in
+// place.  Records with key >= sentinel end up behind all buckets, unsorted.
+// A bucket beyond kBktCap records raises ZEN_STAT_RETRY and stays unsorted.
+
+constexpr int kBktBlock = 1024;
+constexpr int kBktItems = 10;
+constexpr int kBktCap = kBktBlock * kBktItems;  // 10240 records: 120 KB of LDS
+constexpr int kBktWaves = kBktBlock / 64;
+constexpr int kBktSpan = 64 * kBktItems;        // records ranked by one wave
+constexpr int kBktRB = 7;
+constexpr int kBktR = 1 << kBktRB;
+constexpr int kBktDigitBits = 9;                // 511 buckets + the sentinel's
+
+template <bool MORE>
+__global__ __launch_bounds__(kBktBlock) void k_bucket_sort(uint32_t *__restrict__ keys, uint32_t *__restrict__ vals,
+                                                           uint32_t *__restrict__ more,
+                                                           const uint32_t *__restrict__ totals, DigitRange digit,
+                                                           int rel_bits, int32_t *status) {
+  __shared__ uint32_t skey[kBktCap];
+  __shared__ uint32_t sval[kBktCap];
+  __shared__ uint32_t smore[MORE ? kBktCap : 1];
+  __shared__ uint32_t wcnt[kBktWaves][kBktR];
+  __shared__ uint32_t smem[kBktWaves + 1];
+  const uint32_t b = blockIdx.x;
+  uint32_t before = 0;
+  for (uint32_t e = threadIdx.x; e < b; e += kBktBlock) before += totals[e];
+  uint32_t start;
+  block_exclusive_scan<uint32_t, kBktBlock>(before, smem, &start);
+  const uint32_t n = totals[b];
+  if (n > (uint32_t)kBktCap) {
+    if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
+    return;
+  }
+  if (n < 2) return;
+  const uint32_t lo = digit.first_key(b);
+  for (uint32_t j = threadIdx.x; j < n; j += kBktBlock) {
+    skey[j] = keys[start + j] - lo;
+    sval[j] = vals[start + j];
+    if (MORE) smore[j] = more[start + j];
+  }
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const uint32_t mine = wave * kBktSpan + lane;
+  const uint64_t below = lanes_below();
+  for (int shift = 0; shift < rel_bits; shift += kBktRB) {
+    const uint32_t mask = (1u << (rel_bits - shift < kBktRB ? rel_bits - shift : kBktRB)) - 1u;
+    for (int d = threadIdx.x; d < kBktWaves * kBktR; d += kBktBlock) (&wcnt[0][0])[d] = 0;
+    __syncthreads();
+    uint32_t k[kBktItems], v[kBktItems], m[kBktItems], rank[kBktItems];
+#pragma unroll
+    for (int i = 0; i < kBktItems; ++i) {
+      const uint32_t at = mine + i * 64;
+      const bool valid = at < n;
+      k[i] = valid ? skey[at] : 0u;
+      v[i] = valid ? sval[at] : 0u;
+      m[i] = (MORE && valid) ? smore[at] : 0u;
+    }
+    if ((uint32_t)(wave * kBktSpan) < n) {
+#pragma unroll
+      for (int i = 0; i < kBktItems; ++i) {
+        const bool valid = mine + i * 64 < n;
+        const uint32_t d = (k[i] >> shift) & mask;
+        uint64_t peers = __ballot(valid);
+#pragma unroll
+        for (int bit = 0; bit < kBktRB; ++bit) {
+          const bool set = (d >> bit) & 1u;
+          const uint64_t vote = __ballot(valid && set);
+          peers &= set ? vote : ~vote;
+        }
+        uint32_t old = 0;
+        const int leader = valid ? __ffsll((unsigned long long)peers) - 1 : lane;
+        if (valid && lane == leader) {
+          old = wcnt[wave][d];
+          wcnt[wave][d] = old + (uint32_t)__popcll(peers);
+        }
+        old = __shfl(old, leader, 64);
+        rank[i] = old + (uint32_t)__popcll(peers & below);
+        __builtin_amdgcn_wave_barrier();
+      }
+    }
+    __syncthreads();
+    {
+      // thread d < 128 owns digit d: its start inside the bucket, then one start per wave
+      uint32_t c[kBktWaves];
+      uint32_t sum = 0;
+      if (threadIdx.x < kBktR) {
+#pragma unroll
+        for (int w = 0; w < kBktWaves; ++w) {
+          c[w] = wcnt[w][threadIdx.x];
+          sum += c[w];
+        }
+      }
+      uint32_t unused;
+      uint32_t running = block_exclusive_scan<uint32_t, kBktBlock>(sum, smem, &unused);
+      if (threadIdx.x < kBktR) {
+#pragma unroll
+        for (int w = 0; w < kBktWaves; ++w) {
+          wcnt[w][threadIdx.x] = running;
+          running += c[w];
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kBktItems; ++i) {
+      if (mine + i * 64 < n) {
+        const uint32_t pos = wcnt[wave][(k[i] >> shift) & mask] + rank[i];
+        skey[pos] = k[i];
+        sval[pos] = v[i];
+        if (MORE) smore[pos] = m[i];
+      }
+    }
+    __syncthreads();
+  }
+  for (uint32_t j = threadIdx.x; j < n; j += kBktBlock) {
+    keys[start + j] = skey[j] + lo;
+    vals[start + j] = sval[j];
+    if (MORE) more[start + j] = smore[j];
+  }
+}
+
+}  // namespace
+
+bool bucket_sort_fits(int64_t expected, uint32_t sentinel) {
+  // an even spread must leave the buckets a fifth of their capacity to spare
+  return expected >= (1 << 16) && expected <= (int64_t)((1 << kBktDigitBits) - 1) * (kBktCap * 4 / 5) &&
+         sentinel >= (1u << 20);
+}
+
+int bucket_sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint32_t *vals_b, int64_t max_count,
+                      const uint32_t *count_dev, uint32_t sentinel, void *scratch, int32_t *status,
+                      hipStream_t stream, uint32_t *more_a, uint32_t *more_b) {
+  if (max_count < 1 || max_count > 0x7fffffffll || sentinel < (1u << 20))
+    return fail(ZEN_EINVAL, "bucket_sort_pairs: size out of range");
+  const int nblk = num_tiles(max_count);
+  Carver cv(scratch);
+  uint32_t *hist = cv.take<uint32_t>((size_t)nblk * kMaxRadix);
+  uint32_t *totals = cv.take<uint32_t>(kMaxRadix);
+  DigitRange digit;
+  digit.last = (1u << kBktDigitBits) - 1u;
+  digit.sentinel = sentinel;
+  digit.mult = (uint32_t)((((uint64_t)digit.last) << 32) / sentinel);
+  const uint64_t width = ((1ull << 32) + digit.mult - 1) / digit.mult + 1;  // keys per bucket, at most
+  const int rel_bits = ceil_log2_u64(width);
+  const int rc = sort_pass<kBktDigitBits>(keys_a, vals_a, more_a, keys_b, vals_b, more_b, max_count, count_dev, digit,
+                                          nblk, hist, totals, stream);
+  if (rc != ZEN_OK) return rc;
+  if (more_a)
+    k_bucket_sort<true><<<dim3(digit.last), dim3(kBktBlock), 0, stream>>>(keys_b, vals_b, more_b, totals, digit,
+                                                                          rel_bits, status);
+  else
+    k_bucket_sort<false><<<dim3(digit.last), dim3(kBktBlock), 0, stream>>>(keys_b, vals_b, nullptr, totals, digit,
+                                                                           rel_bits, status);
+  ZEN_LAUNCH_CHECK("k_bucket_sort");
+  return 1;
+}
+
 
 }  // namespace zen
 
@@ -300,6 +481,30 @@ int zen_sort_pairs(uint32_t *keys, uint32_t *vals, int64_t max_count, const uint
         kb, vb, keys, vals, count_dev, (uint32_t)max_count);
     ZEN_LAUNCH_CHECK("k_copy_pairs");
   }
+  return ZEN_OK;
+}
+
+int zen_bucket_sort_fits(int64_t max_count, uint32_t sentinel) { return zen::bucket_sort_fits(max_count, sentinel); }
+
+int zen_bucket_sort_pairs(uint32_t *keys, uint32_t *vals, int64_t max_count, const uint32_t *count_dev,
+                          uint32_t sentinel, void *workspace, size_t workspace_bytes, int32_t *status,
+                          void *stream) {
+  using namespace zen;
+  if (!keys || !vals || !workspace || !status) return fail(ZEN_EINVAL, "zen_bucket_sort_pairs: null pointer");
+  if (!bucket_sort_fits(max_count, sentinel)) return fail(ZEN_EINVAL, "zen_bucket_sort_pairs: size out of range");
+  if (workspace_bytes < zen_sort_pairs_workspace(max_count))
+    return fail(ZEN_EWORKSPACE, "zen_bucket_sort_pairs: workspace too small");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  Carver cv(workspace);
+  uint32_t *kb = cv.take<uint32_t>((size_t)max_count);
+  uint32_t *vb = cv.take<uint32_t>((size_t)max_count);
+  void *scratch = cv.take<char>(sort_scratch_bytes(max_count));
+  const int where = bucket_sort_pairs(keys, vals, kb, vb, max_count, count_dev, sentinel, scratch, status, s);
+  if (where < 0) return where;
+  const int64_t blocks = ceil_div(max_count, 1024);
+  k_copy_pairs<<<dim3((unsigned)(blocks < 2048 ? blocks : 2048)), dim3(256), 0, s>>>(kb, vb, keys, vals, count_dev,
+                                                                                     (uint32_t)max_count);
+  ZEN_LAUNCH_CHECK("k_copy_pairs");
   return ZEN_OK;
 }
 
