@@ -289,30 +289,37 @@ namespace {
 // ---------------------------------------------------------------------------
 // Bucket sort for keys that spread evenly over [0, sentinel): one scatter pass
 // by DigitRange puts every key range into a contiguous bucket, then one
-// workgroup per bucket sorts its records completely inside LDS (stable LSD
-// passes of 7 bits over key - first key of the bucket) and writes them back in
-// place.  Records with key >= sentinel end up behind all buckets, unsorted.
-// A bucket beyond kBktCap records raises ZEN_STAT_RETRY and stays unsorted.
+// workgroup per bucket sorts its records inside LDS and writes them back in
+// place.  Inside a bucket the keys spread evenly as well, so the workgroup
+// distributes them over up to kBktSubs narrow key ranges with one LDS atomic
+// each (about one record per range), and every record finds its place inside
+// its range by counting the range's records that precede it in (key, arrival)
+// order, which one packed word per record decides: equal keys keep their
+// arrival order.  Records with key >= sentinel end up behind all buckets,
+// unsorted.  A bucket beyond kBktCap records, or a narrow range beyond
+// kBktGroupLimit, raises ZEN_STAT_RETRY and the bucket stays unsorted.
 
 constexpr int kBktBlock = 1024;
 constexpr int kBktItems = 10;
-constexpr int kBktCap = kBktBlock * kBktItems;  // 10240 records: 120 KB of LDS
-constexpr int kBktWaves = kBktBlock / 64;
-constexpr int kBktSpan = 64 * kBktItems;        // records ranked by one wave
-constexpr int kBktRB = 7;
-constexpr int kBktR = 1 << kBktRB;
+constexpr int kBktCap = kBktBlock * kBktItems;  // 10240 records
+constexpr int kBktSubs = 8192;
+constexpr int kBktSubsPer = kBktSubs / kBktBlock;
+constexpr int kBktGroupLimit = 2048;            // bounds the counting loop on piled-up keys
 constexpr int kBktDigitBits = 9;                // 511 buckets + the sentinel's
 
 template <bool MORE>
 __global__ __launch_bounds__(kBktBlock) void k_bucket_sort(uint32_t *__restrict__ keys, uint32_t *__restrict__ vals,
                                                            uint32_t *__restrict__ more,
                                                            const uint32_t *__restrict__ totals, DigitRange digit,
-                                                           int rel_bits, int32_t *status) {
-  __shared__ uint32_t skey[kBktCap];
-  __shared__ uint32_t sval[kBktCap];
-  __shared__ uint32_t smore[MORE ? kBktCap : 1];
-  __shared__ uint32_t wcnt[kBktWaves][kBktR];
-  __shared__ uint32_t smem[kBktWaves + 1];
+                                                           int sub_shift, int32_t *status) {
+  // first the records grouped by narrow range, as (key bits below the range << 14 | arrival position); in
+  // the end the sorted keys
+  __shared__ uint32_t s_a[kBktCap];
+  __shared__ uint32_t s_b[kBktCap];
+  __shared__ uint32_t s_c[MORE ? kBktCap : 1];
+  __shared__ uint32_t s_cnt[kBktSubs + 1];
+  __shared__ uint32_t smem[kBktBlock / 64 + 1];
+  __shared__ uint32_t s_bad;
   const uint32_t b = blockIdx.x;
   uint32_t before = 0;
   for (uint32_t e = threadIdx.x; e < b; e += kBktBlock) before += totals[e];
@@ -325,89 +332,85 @@ __global__ __launch_bounds__(kBktBlock) void k_bucket_sort(uint32_t *__restrict_
   }
   if (n < 2) return;
   const uint32_t lo = digit.first_key(b);
-  for (uint32_t j = threadIdx.x; j < n; j += kBktBlock) {
-    skey[j] = keys[start + j] - lo;
-    sval[j] = vals[start + j];
-    if (MORE) smore[j] = more[start + j];
+  for (int d = threadIdx.x; d <= kBktSubs; d += kBktBlock) s_cnt[d] = 0;
+  if (threadIdx.x == 0) s_bad = 0;
+  __syncthreads();
+  uint32_t k[kBktItems], v[kBktItems], m[kBktItems], sub[kBktItems], at[kBktItems];
+#pragma unroll
+  for (int i = 0; i < kBktItems; ++i) {
+    const uint32_t j = threadIdx.x + i * kBktBlock;
+    k[i] = v[i] = m[i] = sub[i] = at[i] = 0;
+    if (j < n) {
+      k[i] = keys[start + j] - lo;
+      v[i] = vals[start + j];
+      if (MORE) m[i] = more[start + j];
+    }
   }
-  const int wave = threadIdx.x >> 6;
-  const int lane = threadIdx.x & 63;
-  const uint32_t mine = wave * kBktSpan + lane;
-  const uint64_t below = lanes_below();
-  for (int shift = 0; shift < rel_bits; shift += kBktRB) {
-    const uint32_t mask = (1u << (rel_bits - shift < kBktRB ? rel_bits - shift : kBktRB)) - 1u;
-    for (int d = threadIdx.x; d < kBktWaves * kBktR; d += kBktBlock) (&wcnt[0][0])[d] = 0;
-    __syncthreads();
-    uint32_t k[kBktItems], v[kBktItems], m[kBktItems], rank[kBktItems];
 #pragma unroll
-    for (int i = 0; i < kBktItems; ++i) {
-      const uint32_t at = mine + i * 64;
-      const bool valid = at < n;
-      k[i] = valid ? skey[at] : 0u;
-      v[i] = valid ? sval[at] : 0u;
-      m[i] = (MORE && valid) ? smore[at] : 0u;
+  for (int i = 0; i < kBktItems; ++i) {
+    if (threadIdx.x + i * kBktBlock < n) {
+      sub[i] = k[i] >> sub_shift;
+      at[i] = atomicAdd(&s_cnt[sub[i]], 1u);
     }
-    if ((uint32_t)(wave * kBktSpan) < n) {
-#pragma unroll
-      for (int i = 0; i < kBktItems; ++i) {
-        const bool valid = mine + i * 64 < n;
-        const uint32_t d = (k[i] >> shift) & mask;
-        uint64_t peers = __ballot(valid);
-#pragma unroll
-        for (int bit = 0; bit < kBktRB; ++bit) {
-          const bool set = (d >> bit) & 1u;
-          const uint64_t vote = __ballot(valid && set);
-          peers &= set ? vote : ~vote;
-        }
-        uint32_t old = 0;
-        const int leader = valid ? __ffsll((unsigned long long)peers) - 1 : lane;
-        if (valid && lane == leader) {
-          old = wcnt[wave][d];
-          wcnt[wave][d] = old + (uint32_t)__popcll(peers);
-        }
-        old = __shfl(old, leader, 64);
-        rank[i] = old + (uint32_t)__popcll(peers & below);
-        __builtin_amdgcn_wave_barrier();
-      }
-    }
-    __syncthreads();
-    {
-      // thread d < 128 owns digit d: its start inside the bucket, then one start per wave
-      uint32_t c[kBktWaves];
-      uint32_t sum = 0;
-      if (threadIdx.x < kBktR) {
-#pragma unroll
-        for (int w = 0; w < kBktWaves; ++w) {
-          c[w] = wcnt[w][threadIdx.x];
-          sum += c[w];
-        }
-      }
-      uint32_t unused;
-      uint32_t running = block_exclusive_scan<uint32_t, kBktBlock>(sum, smem, &unused);
-      if (threadIdx.x < kBktR) {
-#pragma unroll
-        for (int w = 0; w < kBktWaves; ++w) {
-          wcnt[w][threadIdx.x] = running;
-          running += c[w];
-        }
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < kBktItems; ++i) {
-      if (mine + i * 64 < n) {
-        const uint32_t pos = wcnt[wave][(k[i] >> shift) & mask] + rank[i];
-        skey[pos] = k[i];
-        sval[pos] = v[i];
-        if (MORE) smore[pos] = m[i];
-      }
-    }
-    __syncthreads();
   }
+  __syncthreads();
+  {
+    // counts become range starts; s_cnt[kBktSubs] = n
+    uint32_t c[kBktSubsPer];
+    uint32_t sum = 0, big = 0;
+#pragma unroll
+    for (int e = 0; e < kBktSubsPer; ++e) {
+      c[e] = s_cnt[threadIdx.x * kBktSubsPer + e];
+      sum += c[e];
+      big |= c[e] > (uint32_t)kBktGroupLimit;
+    }
+    if (big) s_bad = 1;
+    uint32_t unused;
+    uint32_t running = block_exclusive_scan<uint32_t, kBktBlock>(sum, smem, &unused);
+#pragma unroll
+    for (int e = 0; e < kBktSubsPer; ++e) {
+      s_cnt[threadIdx.x * kBktSubsPer + e] = running;
+      running += c[e];
+    }
+    if (threadIdx.x == kBktBlock - 1) s_cnt[kBktSubs] = running;
+  }
+  __syncthreads();
+  if (s_bad) {
+    if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
+    return;
+  }
+  const uint32_t low_mask = (1u << sub_shift) - 1u;
+#pragma unroll
+  for (int i = 0; i < kBktItems; ++i) {
+    const uint32_t j = threadIdx.x + i * kBktBlock;
+    if (j < n) s_a[s_cnt[sub[i]] + at[i]] = ((k[i] & low_mask) << 14) | j;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kBktItems; ++i) {
+    const uint32_t j = threadIdx.x + i * kBktBlock;
+    if (j < n) {
+      const uint32_t g0 = s_cnt[sub[i]], g1 = s_cnt[sub[i] + 1];
+      const uint32_t mine = ((k[i] & low_mask) << 14) | j;
+      uint32_t less = 0;
+      for (uint32_t u = g0; u < g1; ++u) less += s_a[u] < mine;
+      at[i] = g0 + less;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kBktItems; ++i) {
+    if (threadIdx.x + i * kBktBlock < n) {
+      s_a[at[i]] = k[i];
+      s_b[at[i]] = v[i];
+      if (MORE) s_c[at[i]] = m[i];
+    }
+  }
+  __syncthreads();
   for (uint32_t j = threadIdx.x; j < n; j += kBktBlock) {
-    keys[start + j] = skey[j] + lo;
-    vals[start + j] = sval[j];
-    if (MORE) more[start + j] = smore[j];
+    keys[start + j] = s_a[j] + lo;
+    vals[start + j] = s_b[j];
+    if (MORE) more[start + j] = s_c[j];
   }
 }
 
@@ -433,16 +436,18 @@ int bucket_sort_pairs(uint32_t *keys_a, uint32_t *vals_a, uint32_t *keys_b, uint
   digit.sentinel = sentinel;
   digit.mult = (uint32_t)((((uint64_t)digit.last) << 32) / sentinel);
   const uint64_t width = ((1ull << 32) + digit.mult - 1) / digit.mult + 1;  // keys per bucket, at most
-  const int rel_bits = ceil_log2_u64(width);
+  static_assert(kBktCap <= (1 << 14), "arrival positions are packed into 14 bits");
+  const int width_bits = ceil_log2_u64(width);  // at most 24 (mult >= 511), so sub_shift + 14 fits a word
+  const int sub_shift = width_bits > 13 ? width_bits - 13 : 0;
   const int rc = sort_pass<kBktDigitBits>(keys_a, vals_a, more_a, keys_b, vals_b, more_b, max_count, count_dev, digit,
                                           nblk, hist, totals, stream);
   if (rc != ZEN_OK) return rc;
   if (more_a)
     k_bucket_sort<true><<<dim3(digit.last), dim3(kBktBlock), 0, stream>>>(keys_b, vals_b, more_b, totals, digit,
-                                                                          rel_bits, status);
+                                                                          sub_shift, status);
   else
     k_bucket_sort<false><<<dim3(digit.last), dim3(kBktBlock), 0, stream>>>(keys_b, vals_b, nullptr, totals, digit,
-                                                                           rel_bits, status);
+                                                                           sub_shift, status);
   ZEN_LAUNCH_CHECK("k_bucket_sort");
   return 1;
 }
