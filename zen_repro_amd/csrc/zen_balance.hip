@@ -263,7 +263,7 @@ BalancePlan plan_balance(void *workspace, int64_t n, int64_t m, int dtype, int64
   p.more_b = cv.take<uint32_t>(cap);
   p.count = cv.take<uint32_t>(2);
   p.thr = cv.take<uint32_t>(4);
-  p.cand_hist = cv.take<uint32_t>((size_t)kCandRows * kCandBins);
+  p.cand_hist = cv.take<uint32_t>((size_t)kCandHistWords);
   p.topk_scratch = cv.take<char>(topk_scratch_bytes());
   p.select_scratch = cv.take<char>(select_scratch_bytes(n, dtype));
   p.sort_scratch = cv.take<char>(sort_scratch_bytes((int64_t)cap));
@@ -305,12 +305,13 @@ int select_stage(const BalancePlan &p, const void *input, int dtype, int64_t n, 
   // histogram; entries between floor and threshold stay in the list and are
   // filtered by the later stages
   if ((rc = topk_sampled_floor(input, dtype, n, k, p.thr + 2, p.topk_scratch, s)) != ZEN_OK) return rc;
-  launch_fill<uint32_t>(p.cand_hist, 0u, (size_t)kCandRows * kCandBins, s);
+  launch_fill<uint32_t>(p.cand_hist, 0u, (size_t)kCandHistWords, s);
   ZEN_LAUNCH_CHECK("clear candidate histogram");
   sel.thr = p.thr + 2;
   sel.cand_hist = p.cand_hist;
+  sel.pick_k = k;
+  sel.pick_thr = p.thr;
   if ((rc = select_compact(sel, s)) != ZEN_OK) return rc;
-  if ((rc = cand_pick(p.cand_hist, p.thr + 2, k, dtype, p.thr, status, s)) != ZEN_OK) return rc;
   if (dtype == ZEN_F32) {
     // the histogram resolved 15 key bits; the remaining 16 need the radix select, over the candidates only
     if ((rc = topk_exact(p.sel_val, dtype, sel.capacity, &p.count[0], k, p.thr, p.topk_scratch, status,

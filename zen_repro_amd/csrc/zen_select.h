@@ -50,8 +50,13 @@ struct SelectArgs {
   int64_t *out_count = nullptr;       // optional: number found (may exceed capacity)
   uint32_t *out_count32 = nullptr;    // optional: the same clamped to capacity
   bool ordered = true;                // ascending output (false: tiles in arrival order)
-  uint32_t *cand_hist = nullptr;      // optional (unordered mode): kCandRows x kCandBins counters, zero on entry, of
-                                      // min((key - floor) >> (bf16: 0, fp32: 16), kCandBins-1) over the selected
+  uint32_t *cand_hist = nullptr;      // optional (unordered mode): kCandHistWords counters, zero on entry: kCandRows
+                                      // partial histograms of min((key - floor) >> (bf16: 0, fp32: 16), kCandBins-1)
+                                      // over the selected, then a count of finished blocks
+  int64_t pick_k = 0;                 // with cand_hist and pick_thr: the block that finishes last writes
+  uint32_t *pick_thr = nullptr;       // pick_thr[0] = k-th largest key as far as the histogram resolves it (bf16:
+                                      // exactly; fp32: its top 15 bits), pick_thr[1] = candidates at or above it;
+                                      // ZEN_STAT_RETRY if the candidates are fewer than k
   void *scratch = nullptr;            // select_scratch_bytes(n, dtype)
   int32_t *status = nullptr;
 };
@@ -71,15 +76,14 @@ int topk_exact(const void *in, int dtype, int64_t n, const uint32_t *n_dev, int6
 // the 15-bit magnitude bin (for bf16: the key itself) in which the sample
 // reaches the expected rank plus a safety margin.  Almost surely at least k
 // elements of the tensor lie at or above it; compacting them with a candidate
-// histogram (SelectArgs::cand_hist) and cand_pick give the exact threshold with
-// one pass over the tensor.  cand_pick raises ZEN_STAT_RETRY if the candidates
-// are fewer than k after all.  For fp32 cand_pick resolves the top 15 key bits
-// only; topk_exact over the candidates finishes the job.
+// histogram (SelectArgs::cand_hist, pick_k, pick_thr) gives the exact
+// threshold with one pass over the tensor, or ZEN_STAT_RETRY if the
+// candidates are fewer than k after all.  For fp32 the histogram resolves the
+// top 15 key bits only; topk_exact over the candidates finishes the job.
 int topk_sampled_floor(const void *in, int dtype, int64_t n, int64_t k, uint32_t *thr_lo, void *scratch,
                        hipStream_t stream);
 constexpr int kCandBins = 2048;
-constexpr int kCandRows = 8;   // partial candidate histograms (blocks spread over them), summed by cand_pick
-int cand_pick(uint32_t *cand_hist, const uint32_t *floor_key, int64_t k, int dtype, uint32_t *thr, int32_t *status,
-              hipStream_t stream);
+constexpr int kCandRows = 8;   // partial candidate histograms (blocks spread over them)
+constexpr int kCandHistWords = kCandRows * kCandBins + 1;
 
 }  // namespace zen

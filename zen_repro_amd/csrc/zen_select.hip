@@ -128,12 +128,45 @@ __global__ __launch_bounds__(kHistBlock) void k_topk_pick(TopkState *st, uint32_
 constexpr int kFineBins = 32768;
 constexpr int kSampleBlock = 1024;
 
+// Run by one whole block once the histogram is complete: the lowest fine bin b
+// such that `rank` sample elements lie in bins >= b; floor_out[0] = lowest key
+// of that bin (0 if the sample is too small).
+__device__ inline uint32_t load_fresh(const uint32_t *p) {  // written by other blocks' atomics: read at L2
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ inline void sample_pick_block(const uint32_t *hist, uint32_t rank, int key_shift, uint32_t *floor_out,
+                                         uint32_t *smem) {
+  constexpr int kPer = kFineBins / kSampleBlock;
+  uint32_t c[kPer];
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    c[j] = load_fresh(&hist[kFineBins - 1 - (threadIdx.x * kPer + j)]);
+    mine += c[j];
+  }
+  uint32_t total;
+  uint32_t above = block_exclusive_scan<uint32_t, kSampleBlock>(mine, smem, &total);
+  if (total < rank) {
+    if (threadIdx.x == 0) floor_out[0] = 0;
+  } else {
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      if (above < rank && rank <= above + c[j]) floor_out[0] = (uint32_t)(kFineBins - 1 - (threadIdx.x * kPer + j)) << key_shift;
+      above += c[j];
+    }
+  }
+}
+
 template <typename S, bool ALIGNED>
 __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restrict__ in, int64_t n, int block_log2,
-                                                              uint32_t *__restrict__ hist) {
+                                                              uint32_t *__restrict__ hist, uint32_t rank,
+                                                              uint32_t *floor_out) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kShift = KeyOf<S>::kBits - 15;
   __shared__ uint32_t bins[kFineBins / 2];
+  __shared__ uint32_t smem[kSampleBlock / 64 + 1];
+  __shared__ bool s_last;
   for (int i = threadIdx.x; i < kFineBins / 2; i += kSampleBlock) bins[i] = 0;
   __syncthreads();
   const int64_t nvec = (n + V - 1) / V;
@@ -153,67 +186,46 @@ __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restric
     }
   }
   __syncthreads();
+  uint32_t landed = 0;
   for (int i = threadIdx.x; i < kFineBins / 2; i += kSampleBlock) {
     const uint32_t c = bins[i];
-    if (c & 0xffffu) atomicAdd(&hist[2 * i], c & 0xffffu);
-    if (c >> 16) atomicAdd(&hist[2 * i + 1], c >> 16);
+    if (c & 0xffffu) landed += atomicAdd(&hist[2 * i], c & 0xffffu);
+    if (c >> 16) landed += atomicAdd(&hist[2 * i + 1], c >> 16);
   }
+  // The block that finishes last reads the threshold off the complete histogram (hist[kFineBins] counts
+  // finished blocks).  No fence: every add above has returned its old value, so it has been carried out
+  // where atomics are carried out, before this block's count goes up; the reader loads from that place.
+  // (A device-wide fence in every block would write back and invalidate the caches each time.)
+  if (__syncthreads_or(landed == 0xffffffffu)) return;  // never true: keeps the returns alive
+  if (threadIdx.x == 0) s_last = atomicAdd(&hist[kFineBins], 1u) == gridDim.x - 1;
+  __syncthreads();
+  if (!s_last) return;
+  sample_pick_block(hist, rank, kShift, floor_out, smem);
 }
 
-// One block: the lowest fine bin b such that `rank` sample elements lie in bins
-// >= b; floor_out[0] = lowest key of that bin (0 if the sample is too small).
-__global__ __launch_bounds__(kSampleBlock) void k_sample_pick(uint32_t *hist, uint32_t rank, int key_shift,
-                                                              uint32_t *floor_out) {
-  constexpr int kPer = kFineBins / kSampleBlock;
-  __shared__ uint32_t smem[kSampleBlock / 64 + 1];
+// Run by one whole block (kSelBlock threads) over the complete candidate
+// histogram (bin = min((key - floor) >> shift, kCandBins-1), kCandRows partial
+// rows): the exact k-th largest key when the bins are single keys (shift 0),
+// else the lowest key of its bin.  thr_out = (key, number of candidates >=
+// key).  Too few candidates, or the k-th lies in the clipped last bin:
+// ZEN_STAT_RETRY.
+template <int BLOCK>
+__device__ inline void cand_pick_block(const uint32_t *hist, uint32_t base, uint32_t k, int shift,
+                                       uint32_t *thr_out, int32_t *status, uint32_t *smem) {
+  constexpr int kPer = kCandBins / BLOCK;
   uint32_t c[kPer];
   uint32_t mine = 0;
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
-    c[j] = hist[kFineBins - 1 - (threadIdx.x * kPer + j)];
-    mine += c[j];
-  }
-  uint32_t total;
-  uint32_t above = block_exclusive_scan<uint32_t, kSampleBlock>(mine, smem, &total);
-  if (total < rank) {
-    if (threadIdx.x == 0) floor_out[0] = 0;
-  } else {
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-      if (above < rank && rank <= above + c[j]) floor_out[0] = (uint32_t)(kFineBins - 1 - (threadIdx.x * kPer + j)) << key_shift;
-      above += c[j];
-    }
-  }
-#pragma unroll
-  for (int j = 0; j < kPer; ++j) hist[kFineBins - 1 - (threadIdx.x * kPer + j)] = 0;
-}
-
-// One block over the candidate histogram the compaction kernel filled (bin =
-// min((key - floor) >> shift, kHistBins-1)): the exact k-th largest key when the
-// bins are single keys (shift 0), else the lowest key of its bin.
-// thr_out = (key, number of candidates >= key).  Too few candidates, or the
-// k-th lies in the clipped last bin: ZEN_STAT_RETRY.
-__global__ __launch_bounds__(kHistBlock) void k_cand_pick(uint32_t *hist, const uint32_t *floor_key, uint32_t k,
-                                                          int shift, uint32_t *thr_out, int32_t *status) {
-  constexpr int kPer = kHistBins / kHistBlock;
-  __shared__ uint32_t smem[kHistBlock / 64 + 1];
-  uint32_t c[kPer];
-  uint32_t mine = 0;
-#pragma unroll
-  for (int j = 0; j < kPer; ++j) {
-    const int bin = kHistBins - 1 - (threadIdx.x * kPer + j);
+    const int bin = kCandBins - 1 - (threadIdx.x * kPer + j);
     uint32_t sum = 0;
 #pragma unroll
-    for (int row = 0; row < kCandRows; ++row) sum += hist[row * kHistBins + bin];
-#pragma unroll
-    for (int row = 0; row < kCandRows; ++row) hist[row * kHistBins + bin] = 0;
+    for (int row = 0; row < kCandRows; ++row) sum += load_fresh(&hist[row * kCandBins + bin]);
     c[j] = sum;
     mine += sum;
   }
   uint32_t total;
-  uint32_t above = block_exclusive_scan<uint32_t, kHistBlock>(mine, smem, &total);
-  uint32_t base = floor_key[0];
-  if (base == 0) base = 1;  // the compaction treats a zero floor as "nonzero"
+  uint32_t above = block_exclusive_scan<uint32_t, BLOCK>(mine, smem, &total);
   if (total < k) {
     if (threadIdx.x == 0) {
       thr_out[0] = 0;
@@ -224,10 +236,10 @@ __global__ __launch_bounds__(kHistBlock) void k_cand_pick(uint32_t *hist, const 
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       if (above < k && k <= above + c[j]) {
-        const uint32_t bin = kHistBins - 1 - (threadIdx.x * kPer + j);
+        const uint32_t bin = kCandBins - 1 - (threadIdx.x * kPer + j);
         thr_out[0] = base + (bin << shift);
         thr_out[1] = above + c[j];
-        if (bin == kHistBins - 1) atomicOr(status, ZEN_STAT_RETRY);
+        if (bin == kCandBins - 1) atomicOr(status, ZEN_STAT_RETRY);
       }
       above += c[j];
     }
@@ -425,8 +437,8 @@ template <typename S, typename I, bool ALIGNED, bool ORDERED>
 __global__ __launch_bounds__(kSelBlock) void k_select_compact(
     const S *__restrict__ in, int64_t n_max, const uint32_t *__restrict__ n_dev, const uint32_t *__restrict__ thr,
     const int32_t *__restrict__ src_idx, I *__restrict__ out_idx, S *__restrict__ out_val, int64_t capacity,
-    ScanState st, int ntiles, int subs, uint32_t *cand_hist, int64_t *out_count, uint32_t *out_count32,
-    int32_t *status) {
+    ScanState st, int ntiles, int subs, uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr,
+    int64_t *out_count, uint32_t *out_count32, int32_t *status) {
   constexpr int kSub = kSelBlock * Flags<S>::kElems;
   __shared__ uint32_t s_wave[kSelBlock / 64];
   __shared__ uint64_t s_bcast;
@@ -496,9 +508,24 @@ __global__ __launch_bounds__(kSelBlock) void k_select_compact(
     // spread over kCandRows partial histograms: fewer blocks meet on one counter
     __syncthreads();
     uint32_t *row = cand_hist + (size_t)(blockIdx.x % kCandRows) * kCandBins;
+    uint32_t landed = 0;
     for (int i = threadIdx.x; i < kCandBins; i += kSelBlock) {
       const uint32_t c = s_hist[i];
-      if (c) atomicAdd(&row[i], c);
+      if (c) landed += atomicAdd(&row[i], c);
+    }
+    if (pick_thr) {
+      // The block that finishes last reads the exact threshold off the complete histogram
+      // (cand_hist[kCandRows * kCandBins] counts finished blocks).  No fence: the adds above have returned,
+      // so they have been carried out before this block's count goes up, and the reader loads from the
+      // place where atomics are carried out.
+      __shared__ bool s_last;
+      if (__syncthreads_or(landed == 0xffffffffu)) return;  // never true: keeps the returns alive
+      if (threadIdx.x == 0) s_last = atomicAdd(&cand_hist[kCandRows * kCandBins], 1u) == (uint32_t)ntiles - 1u;
+      __syncthreads();
+      if (s_last) {
+        cand_pick_block<kSelBlock>(cand_hist, floor_key, pick_k, KeyOf<S>::kBits == 15 ? 0 : 16, pick_thr, status,
+                                   reinterpret_cast<uint32_t *>(st_idx));
+      }
     }
   }
 }
@@ -540,7 +567,8 @@ static int select_launch(const SelectArgs &a, hipStream_t stream) {
 #define ZEN_SELECT_GO(AL, ORD)                                                                                 \
   k_select_compact<S, I, AL, ORD><<<grid, block, 0, stream>>>(in, a.n, a.n_dev, a.thr, a.src_idx, out_idx,   \
                                                               out_val, a.capacity, st, (int)ntiles, subs,    \
-                                                              a.cand_hist, a.out_count, a.out_count32, a.status)
+                                                              a.cand_hist, (uint32_t)a.pick_k, a.pick_thr,   \
+                                                              a.out_count, a.out_count32, a.status)
   if (aligned && a.ordered) ZEN_SELECT_GO(true, true);
   else if (aligned) ZEN_SELECT_GO(true, false);
   else if (a.ordered) ZEN_SELECT_GO(false, true);
@@ -608,7 +636,7 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
   const double expect = (double)k * ((double)nblocks * V) / (double)n;
   const double want = expect + 6.0 * sqrt(expect) + 16.0;
   const uint32_t rank = want > 4.0e9 ? 0xffffffffu : (uint32_t)want;
-  launch_fill<uint32_t>(hist, 0u, kFineBins, stream);
+  launch_fill<uint32_t>(hist, 0u, kFineBins + 1, stream);
   ZEN_LAUNCH_CHECK("sample: clear histogram");
   // every block must see fewer than 65536 sample elements (16-bit LDS counters)
   int64_t blocks = ceil_div(nblocks * V, 32768);
@@ -617,13 +645,13 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
   {
     ProfScope prof(kProfTopkHist, stream);
     if (aligned)
-      k_sample_hist<S, true><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist);
+      k_sample_hist<S, true><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist, rank,
+                                                                                        thr_lo);
     else
-      k_sample_hist<S, false><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist);
+      k_sample_hist<S, false><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist,
+                                                                                         rank, thr_lo);
     ZEN_LAUNCH_CHECK("k_sample_hist");
   }
-  k_sample_pick<<<dim3(1), dim3(kSampleBlock), 0, stream>>>(hist, rank, KeyOf<S>::kBits - 15, thr_lo);
-  ZEN_LAUNCH_CHECK("k_sample_pick");
   return ZEN_OK;
 }
 
@@ -648,16 +676,8 @@ int compress_launch(const S *in, int64_t n, const uint32_t *thr, S *out, hipStre
 
 size_t topk_scratch_bytes() {
   const size_t exact = align_up(sizeof(TopkState), 256) + align_up(kHistBins * sizeof(uint32_t), 256);
-  const size_t sampled = align_up(kFineBins * sizeof(uint32_t), 256);
+  const size_t sampled = align_up((kFineBins + 1) * sizeof(uint32_t), 256);
   return exact > sampled ? exact : sampled;
-}
-
-int cand_pick(uint32_t *cand_hist, const uint32_t *floor_key, int64_t k, int dtype, uint32_t *thr, int32_t *status,
-              hipStream_t stream) {
-  k_cand_pick<<<dim3(1), dim3(kHistBlock), 0, stream>>>(cand_hist, floor_key, (uint32_t)k, dtype == ZEN_BF16 ? 0 : 16,
-                                                        thr, status);
-  ZEN_LAUNCH_CHECK("k_cand_pick");
-  return ZEN_OK;
 }
 
 int topk_exact(const void *in, int dtype, int64_t n, const uint32_t *n_dev, int64_t k, uint32_t *thr,
