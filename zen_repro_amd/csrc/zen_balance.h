@@ -111,6 +111,31 @@ struct ResolveArgs {
   int64_t *splits;
   int32_t *status;
 };
+// Load balance on bucket slabs (zen_slab_encode.hip): select, sort and place in six launches, for sizes
+// slab_balance_fits accepts.
+struct SlabBalanceArgs {
+  const void *input;          // the dense gradient
+  int dtype;
+  int64_t n;
+  Probe g;
+  int partitions;
+  int64_t spp;                // serial slots per partition
+  const uint32_t *thr;        // optional threshold key (device); with k == 0 and no thr: the nonzeros
+  int64_t k;                  // > 0: the k largest magnitudes, ties kept (bf16 only)
+  uint32_t *thr_out;          // optional, k > 0: receives (threshold key, number selected)
+  int32_t *out_idx;
+  void *out_val;
+  int64_t capacity;
+  int64_t *splits;
+  unsigned long long *hash;   // zeroed cells for slot -> smallest index, zero again on return
+  uint32_t hash_log2;
+  void *workspace;            // slab_balance_bytes(...)
+  int32_t *status;
+};
+bool slab_balance_fits(int64_t n, int64_t m, int partitions, int dtype, int64_t capacity, int64_t k, SlabGeom *geo);
+size_t slab_balance_bytes(int64_t m, int partitions, int dtype, int64_t capacity);
+int slab_load_balance(const SlabBalanceArgs &a, hipStream_t stream);
+
 size_t resolve_scratch_bytes(int64_t list_cap, uint64_t key_limit);  // key_limit = P * (m / P + 1) + 1
 int resolve_and_place(const ResolveArgs &a, hipStream_t stream);
 

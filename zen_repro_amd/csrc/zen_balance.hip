@@ -366,9 +366,10 @@ int zen_sparse_balance(const void *input, int dtype, int64_t n, int32_t *memory,
 }
 
 size_t zen_load_balance_workspace(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions) {
-  (void)partitions;
   if (n <= 0 || m <= 0 || capacity < 0) return 0;
-  return zen::plan_balance(nullptr, n, m, dtype, capacity).bytes;
+  const size_t general = zen::plan_balance(nullptr, n, m, dtype, capacity).bytes;
+  const size_t slabs = partitions > 0 && m % partitions == 0 ? zen::slab_balance_bytes(m, partitions, dtype, capacity) : 0;
+  return general > slabs ? general : slabs;
 }
 
 int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
@@ -394,6 +395,30 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
   const int64_t spp = n / partitions / 10;  // tensor_load_balance.py:18
   const uint32_t drop_key = (uint32_t)partitions * (g.npp + 1u);
   const int bits = ceil_log2_u64(drop_key);
+  if (mode == ZEN_MODE_FAST && (reinterpret_cast<uintptr_t>(table) & 7u) == 0 &&
+      slab_balance_fits(n, m, partitions, dtype, capacity, k, nullptr)) {
+    SlabBalanceArgs sa;
+    sa.input = input;
+    sa.dtype = dtype;
+    sa.n = n;
+    sa.g = g;
+    sa.partitions = partitions;
+    sa.spp = spp;
+    sa.thr = thr;
+    sa.k = k;
+    sa.thr_out = thr_out;
+    sa.out_idx = out_idx;
+    sa.out_val = out_val;
+    sa.capacity = capacity;
+    sa.splits = splits;
+    sa.hash = reinterpret_cast<unsigned long long *>(table);
+    uint32_t log2 = 0;
+    while (log2 < 24 && (2ull << log2) <= (uint64_t)m / 2) ++log2;
+    sa.hash_log2 = log2;
+    sa.workspace = workspace;
+    sa.status = status;
+    return slab_load_balance(sa, s);
+  }
   BalancePlan p = plan_balance(workspace, n, m, dtype, capacity);
 
   const uint32_t *filter = nullptr;

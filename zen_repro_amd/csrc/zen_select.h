@@ -3,6 +3,7 @@
 #pragma once
 
 #include "zen_common.h"
+#include "zen_slab.h"
 
 namespace zen {
 
@@ -81,9 +82,33 @@ int topk_exact(const void *in, int dtype, int64_t n, const uint32_t *n_dev, int6
 // candidates are fewer than k after all.  For fp32 the histogram resolves the
 // top 15 key bits only; topk_exact over the candidates finishes the job.
 int topk_sampled_floor(const void *in, int dtype, int64_t n, int64_t k, uint32_t *thr_lo, void *scratch,
-                       hipStream_t stream);
+                       hipStream_t stream, bool scratch_is_zero = false);
+size_t sampled_floor_zero_bytes();  // leading part of the scratch that must be zero (scratch_is_zero: the caller did it)
 constexpr int kCandBins = 2048;
 constexpr int kCandRows = 8;   // partial candidate histograms (blocks spread over them)
 constexpr int kCandHistWords = kCandRows * kCandBins + 1;
+
+// One pass over a dense tensor that appends every element with key >= max(thr[0], 1) (thr == nullptr: the
+// nonzero ones), as (index, value), to the bucket slab of its level-1 hash slot.  cursor[nbuckets], *ticket and
+// cand_hist must be zero on entry.  A slab that fills up raises ZEN_STAT_RETRY.  With cand_hist / pick_k /
+// pick_thr the exact k-th largest key is read off the candidates' histogram as in SelectArgs (and copied to
+// thr_copy if that is not null).
+struct ScatterArgs {
+  const void *in = nullptr;
+  int dtype = ZEN_F32;
+  int64_t n = 0;
+  const uint32_t *thr = nullptr;
+  SlabGeom geo;
+  uint32_t *cursor = nullptr;      // [nbuckets] records appended per bucket (may exceed kSlabCap: then RETRY)
+  int32_t *slab_idx = nullptr;     // [nbuckets * kSlabCap]
+  void *slab_val = nullptr;        // [nbuckets * kSlabCap] elements of the tensor's type
+  uint32_t *ticket = nullptr;
+  uint32_t *cand_hist = nullptr;
+  int64_t pick_k = 0;
+  uint32_t *pick_thr = nullptr;
+  uint32_t *thr_copy = nullptr;
+  int32_t *status = nullptr;
+};
+int select_scatter(const ScatterArgs &a, hipStream_t stream);
 
 }  // namespace zen

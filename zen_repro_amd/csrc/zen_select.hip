@@ -584,6 +584,276 @@ int select_compact(const SelectArgs &a, hipStream_t stream) {
   return a.idx64 ? select_launch<uint32_t, int64_t>(a, stream) : select_launch<uint32_t, int32_t>(a, stream);
 }
 
+// ------------------------------------------- compaction into bucket slabs
+//
+// The fused encode does not need its candidates in any order: they are sorted
+// by hash slot afterwards.  So this kernel runs as a few persistent workgroups
+// per compute unit, reads the tensor with fully coalesced non-temporal loads
+// (the next sub-tile is already in flight while the current one is examined),
+// needs one barrier per sub-tile (the wave totals are double buffered), and
+// stages candidates in LDS until kScatStage of them are there.  A full stage
+// is flushed: every entry's bucket (range of its level-1 hash slot) is counted
+// in LDS, a range in each bucket's slab is reserved with one atomic per bucket
+// and flush, and the entries are written there.  The candidate histogram is
+// taken at flush time.
+
+constexpr int kScatStage = 4096;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename S, bool ALIGNED>
+__device__ inline void scatter_load(const S *__restrict__ in, int64_t n, int64_t sub_base, uint4 (&q)[kSelVecs]) {
+  constexpr int V = VecOf<S>::kN;
+#pragma unroll
+  for (int j = 0; j < kSelVecs; ++j) {
+    const int64_t first = sub_base + ((int64_t)j * kSelBlock + threadIdx.x) * V;
+    if (ALIGNED && first + V <= n) {
+      const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(in + first));
+      q[j] = make_uint4(v.x, v.y, v.z, v.w);
+    } else if (first < n) {
+      S e[V];
+      load_vec<S, false>(in, first, n, e);  // elements past the end read as zero: never selected
+      __builtin_memcpy(&q[j], e, 16);
+    } else {
+      q[j] = make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+}
+
+// Word w (0..15) of the 64 bytes a thread holds, without indexing registers dynamically.
+__device__ inline uint32_t pick_word(const uint4 (&q)[kSelVecs], int w) {
+  uint32_t r = 0;
+#pragma unroll
+  for (int j = 0; j < kSelVecs; ++j) {
+    r = w == 4 * j ? q[j].x : r;
+    r = w == 4 * j + 1 ? q[j].y : r;
+    r = w == 4 * j + 2 ? q[j].z : r;
+    r = w == 4 * j + 3 ? q[j].w : r;
+  }
+  return r;
+}
+template <typename S>
+__device__ inline S pick_elem(const uint4 (&q)[kSelVecs], int off);
+template <>
+__device__ inline uint16_t pick_elem<uint16_t>(const uint4 (&q)[kSelVecs], int off) {
+  const uint32_t w = pick_word(q, off >> 1);
+  return (uint16_t)((off & 1) ? (w >> 16) : (w & 0xffffu));
+}
+template <>
+__device__ inline uint32_t pick_elem<uint32_t>(const uint4 (&q)[kSelVecs], int off) {
+  return pick_word(q, off);
+}
+
+// Called by the whole block after a barrier made the staged entries visible.
+// Nothing is kept in registers between the counting pass and the writing pass
+// (an entry's bucket is computed again): this runs rarely, and the streaming
+// loop around it should not pay for its registers.
+template <typename S>
+__device__ __noinline__ void scatter_flush(uint32_t count, const int32_t *st_idx, const S *st_val, uint32_t *s_bcnt,
+                                           uint32_t *s_hist, uint32_t floor_key, const SlabGeom &geo,
+                                           uint32_t *cursor, int32_t *__restrict__ slab_idx,
+                                           S *__restrict__ slab_val, int32_t *status) {
+  for (uint32_t b = threadIdx.x; b < geo.nbuckets; b += kSelBlock) s_bcnt[b] = 0;
+  __syncthreads();
+  for (uint32_t e = threadIdx.x; e < count; e += kSelBlock) {
+    const uint32_t t = (uint32_t)st_idx[e];
+    atomicAdd(&s_bcnt[geo.bucket_of((poly(t) + kSeed1) % geo.m)], 1u);
+    if (s_hist) {
+      const uint32_t bin = ((st_val[e] & KeyOf<S>::kMask) - floor_key) >> (sizeof(S) == 2 ? 0 : 16);
+      atomicAdd(&s_hist[bin < (uint32_t)kCandBins - 1u ? bin : (uint32_t)kCandBins - 1u], 1u);
+    }
+  }
+  __syncthreads();
+  for (uint32_t b = threadIdx.x; b < geo.nbuckets; b += kSelBlock) {
+    const uint32_t c = s_bcnt[b];
+    if (c) {
+      const uint32_t base = atomicAdd(&cursor[b], c);
+      if (base + c > (uint32_t)kSlabCap) atomicOr(status, ZEN_STAT_RETRY);
+      s_bcnt[b] = base;  // from here on: the next free place in the bucket's slab
+    }
+  }
+  __syncthreads();
+  for (uint32_t e = threadIdx.x; e < count; e += kSelBlock) {
+    const uint32_t t = (uint32_t)st_idx[e];
+    const uint32_t b = geo.bucket_of((poly(t) + kSeed1) % geo.m);
+    const uint32_t pos = atomicAdd(&s_bcnt[b], 1u);
+    if (pos < (uint32_t)kSlabCap) {
+      const size_t dst = (size_t)b * kSlabCap + pos;
+      slab_idx[dst] = (int32_t)t;
+      slab_val[dst] = st_val[e];
+    }
+  }
+  __syncthreads();
+}
+
+template <typename S, bool ALIGNED>
+__global__ __launch_bounds__(kSelBlock, 3) void k_select_scatter(
+    const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, SlabGeom geo, uint32_t *cursor,
+    int32_t *__restrict__ slab_idx, S *__restrict__ slab_val, uint32_t *ticket, int ntiles, int subs,
+    uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *thr_copy, int32_t *status) {
+  constexpr int V = VecOf<S>::kN;
+  constexpr int kSub = kSelBlock * kSelVecs * V;
+  constexpr int kWaves = kSelBlock / 64;
+  __shared__ uint32_t s_wave[2][kWaves];
+  __shared__ int s_next[2];
+  __shared__ int32_t st_idx[kScatStage];
+  __shared__ S st_val[kScatStage];
+  __shared__ uint32_t s_bcnt[kSlabMaxBuckets];
+  __shared__ uint32_t s_hist[kCandBins];
+  uint32_t *hist = cand_hist ? s_hist : nullptr;
+  if (hist)
+    for (int i = threadIdx.x; i < kCandBins; i += kSelBlock) s_hist[i] = 0;
+  uint32_t floor_key = thr ? thr[0] : 1u;
+  if (floor_key == 0) floor_key = 1u;  // zeros are never selected
+  if (floor_key > KeyOf<S>::kMask) floor_key = KeyOf<S>::kMask + 1u;  // nothing qualifies
+  const int wave = threadIdx.x >> 6;
+
+  // The first tile is the block's own number, later ones come from the ticket counter; the ticket for the
+  // tile after the current one is drawn while the current one is processed.  Two register sets take turns:
+  // while one sub-tile is examined the loads of the next one are in flight.
+  int tile = (int)blockIdx.x;
+  int turn = 0;        // tiles this block has started
+  uint32_t par = 0;    // sub-tiles this block has processed
+  uint32_t count = 0;  // staged entries
+  int next_tile = ntiles;
+  int64_t sub_base = 0;
+  int sub = 0;
+  uint4 qa[kSelVecs], qb[kSelVecs];
+
+  // one sub-tile: cur holds its data, nxt receives the following sub-tile's
+  auto body = [&](uint4 (&cur)[kSelVecs], uint4 (&nxt)[kSelVecs]) {
+    uint32_t x = Flags<S>::build(cur, floor_key);
+    const uint32_t cnt = (uint32_t)__popc(x);
+    const uint32_t incl = wave_inclusive_scan_dpp(cnt);
+    if ((threadIdx.x & 63) == 63) s_wave[par & 1][wave] = incl;
+    __syncthreads();
+    // what comes next: the following sub-tile of this tile, or the first one of the next tile
+    if (sub + 1 < subs) {
+      scatter_load<S, ALIGNED>(in, n, sub_base + kSub, nxt);
+    } else {
+      next_tile = s_next[turn & 1];
+      if (next_tile < ntiles) scatter_load<S, ALIGNED>(in, n, (int64_t)next_tile * subs * kSub, nxt);
+    }
+    uint32_t before = incl - cnt, total = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const uint32_t t = s_wave[par & 1][w];
+      if (w < wave) before += t;
+      total += t;
+    }
+    const uint32_t all = x;
+    uint32_t done = 0;
+    for (;;) {
+      const uint32_t room = (uint32_t)kScatStage - count;
+      const uint32_t hi = done + room;
+      uint32_t y = x;
+      while (y) {
+        const int bit = __ffs((int)y) - 1;
+        y &= y - 1;
+        const int off = Flags<S>::offset_of(bit);
+        const uint32_t pos = before + (uint32_t)__popc(all & Flags<S>::below(off));
+        if (pos < hi) {
+          x &= ~(1u << bit);
+          const uint32_t at = count + pos - done;
+          st_idx[at] = (int32_t)(sub_base + ((int64_t)(off / V) * kSelBlock + threadIdx.x) * V + (off % V));
+          st_val[at] = pick_elem<S>(cur, off);
+        }
+      }
+      const uint32_t take = total - done < room ? total - done : room;
+      count += take;
+      done += take;
+      if (count < (uint32_t)kScatStage) break;
+      __syncthreads();
+      scatter_flush<S>(count, st_idx, st_val, s_bcnt, hist, floor_key, geo, cursor, slab_idx, slab_val, status);
+      count = 0;
+      if (done == total) break;
+    }
+  };
+
+  if (tile < ntiles) scatter_load<S, ALIGNED>(in, n, (int64_t)tile * subs * kSub, qa);
+  while (tile < ntiles) {
+    if (threadIdx.x == 0) s_next[turn & 1] = (int)gridDim.x + (int)atomicAdd(ticket, 1u);
+    const int64_t tile_base = (int64_t)tile * subs * kSub;
+    for (sub = 0; sub < subs; ++sub, ++par) {
+      sub_base = tile_base + (int64_t)sub * kSub;
+      if (par & 1)
+        body(qb, qa);
+      else
+        body(qa, qb);
+    }
+    tile = next_tile;
+    ++turn;
+  }
+  __syncthreads();
+  if (count) scatter_flush<S>(count, st_idx, st_val, s_bcnt, hist, floor_key, geo, cursor, slab_idx, slab_val, status);
+  if (hist) {
+    __syncthreads();
+    uint32_t *row = cand_hist + (size_t)(blockIdx.x % kCandRows) * kCandBins;
+    uint32_t landed = 0;
+    for (int i = threadIdx.x; i < kCandBins; i += kSelBlock) {
+      const uint32_t c = s_hist[i];
+      if (c) landed += atomicAdd(&row[i], c);
+    }
+    if (pick_thr) {
+      // the block that finishes last reads the exact threshold off the complete histogram (the adds above
+      // have returned, so they are carried out before this block's count goes up)
+      __shared__ bool s_last;
+      if (__syncthreads_or(landed == 0xffffffffu)) return;  // never true: keeps the returns alive
+      if (threadIdx.x == 0) s_last = atomicAdd(&cand_hist[kCandRows * kCandBins], 1u) == gridDim.x - 1u;
+      __syncthreads();
+      if (s_last) {
+        cand_pick_block<kSelBlock>(cand_hist, floor_key, pick_k, KeyOf<S>::kBits == 15 ? 0 : 16, pick_thr, status,
+                                   s_bcnt);
+        __syncthreads();
+        if (thr_copy && threadIdx.x < 2)
+          thr_copy[threadIdx.x] = __hip_atomic_load(&pick_thr[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+}
+
+static int device_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      cus = v;
+    else
+      cus = 256;
+  }
+  return cus;
+}
+
+template <typename S>
+static int scatter_launch(const ScatterArgs &a, hipStream_t stream) {
+  constexpr int V = VecOf<S>::kN;
+  const int subs = select_subs(a.n, a.dtype);
+  const int64_t tile = (int64_t)kSelBlock * kSelVecs * V * subs;
+  const int64_t ntiles = ceil_div(a.n, tile);
+  if (ntiles > 0x3fffffff) return fail(ZEN_EINVAL, "select_scatter: too many tiles");
+  int64_t blocks = (int64_t)device_cus() * 3;
+  if (blocks > ntiles) blocks = ntiles;
+  const S *in = static_cast<const S *>(a.in);
+  const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+  ProfScope prof(kProfSelectCompact, stream);
+  if (aligned)
+    k_select_scatter<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
+        in, a.n, a.thr, a.geo, a.cursor, a.slab_idx, static_cast<S *>(a.slab_val), a.ticket, (int)ntiles, subs,
+        a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
+  else
+    k_select_scatter<S, false><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
+        in, a.n, a.thr, a.geo, a.cursor, a.slab_idx, static_cast<S *>(a.slab_val), a.ticket, (int)ntiles, subs,
+        a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
+  ZEN_LAUNCH_CHECK("k_select_scatter");
+  return ZEN_OK;
+}
+
+int select_scatter(const ScatterArgs &a, hipStream_t stream) {
+  if (a.dtype == ZEN_BF16) return scatter_launch<uint16_t>(a, stream);
+  return scatter_launch<uint32_t>(a, stream);
+}
+
 namespace {
 
 template <typename S>
@@ -625,7 +895,8 @@ int topk_launch(const S *in, int64_t n, const uint32_t *n_dev, int64_t k, uint32
 }
 
 template <typename S>
-int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *workspace, hipStream_t stream) {
+int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *workspace, hipStream_t stream,
+                  bool is_zero) {
   constexpr int V = VecOf<S>::kN;
   uint32_t *hist = static_cast<uint32_t *>(workspace);
   const int64_t nvec = ceil_div(n, V);
@@ -636,8 +907,10 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
   const double expect = (double)k * ((double)nblocks * V) / (double)n;
   const double want = expect + 6.0 * sqrt(expect) + 16.0;
   const uint32_t rank = want > 4.0e9 ? 0xffffffffu : (uint32_t)want;
-  launch_fill<uint32_t>(hist, 0u, kFineBins + 1, stream);
-  ZEN_LAUNCH_CHECK("sample: clear histogram");
+  if (!is_zero) {
+    launch_fill<uint32_t>(hist, 0u, kFineBins + 1, stream);
+    ZEN_LAUNCH_CHECK("sample: clear histogram");
+  }
   // every block must see fewer than 65536 sample elements (16-bit LDS counters)
   int64_t blocks = ceil_div(nblocks * V, 32768);
   if (blocks < 128) blocks = 128;
@@ -688,10 +961,13 @@ int topk_exact(const void *in, int dtype, int64_t n, const uint32_t *n_dev, int6
 }
 
 int topk_sampled_floor(const void *in, int dtype, int64_t n, int64_t k, uint32_t *thr_lo, void *scratch,
-                       hipStream_t stream) {
-  if (dtype == ZEN_BF16) return sample_launch(static_cast<const uint16_t *>(in), n, k, thr_lo, scratch, stream);
-  return sample_launch(static_cast<const uint32_t *>(in), n, k, thr_lo, scratch, stream);
+                       hipStream_t stream, bool scratch_is_zero) {
+  if (dtype == ZEN_BF16)
+    return sample_launch(static_cast<const uint16_t *>(in), n, k, thr_lo, scratch, stream, scratch_is_zero);
+  return sample_launch(static_cast<const uint32_t *>(in), n, k, thr_lo, scratch, stream, scratch_is_zero);
 }
+
+size_t sampled_floor_zero_bytes() { return (kFineBins + 1) * sizeof(uint32_t); }
 
 }  // namespace zen
 

@@ -1,0 +1,157 @@
+// Bucket slabs: the layout both fast paths (encode and merge) are built on.
+//
+// Keys that spread evenly over a range -- level-1 hash slots on the encode
+// side, hashed indices arriving at one destination on the merge side -- are
+// cut into `nbuckets` contiguous key ranges of equal width.  Every bucket owns
+// a slab of kSlabCap records in the workspace.  The producer kernel appends
+// records to the slabs in whatever order they turn up (one cursor per bucket,
+// reserved once per staged batch and bucket); afterwards one workgroup per
+// bucket sorts its slab inside LDS.  Buckets never straddle a partition
+// (nbuckets = partitions * buckets-per-partition), so bucket order is output
+// order.  A slab that overflows raises ZEN_STAT_RETRY and the caller falls
+// back to the general (radix sort) path.
+#pragma once
+
+#include "zen_common.h"
+
+namespace zen {
+
+constexpr uint32_t kRemovedBit = 1u << 31;  // in a sorted index word: the entry lost its level-1 slot
+constexpr uint32_t kIndexMask = kRemovedBit - 1u;
+
+constexpr int kSlabBlock = 512;                       // threads of a per-bucket workgroup
+constexpr int kSlabItems = 12;                        // records per thread
+constexpr int kSlabCap = kSlabBlock * kSlabItems;     // records per slab (6144)
+constexpr int kSlabSubs = 4096;                       // narrow key ranges inside a bucket (about one record each)
+constexpr int kSlabSubsPer = kSlabSubs / kSlabBlock;
+constexpr int kSlabGroupLimit = 1024;                 // bounds the rank loop on piled-up keys
+constexpr int kSlabMaxBuckets = 2048;
+constexpr int kSlabTarget = 3584;                     // records a bucket is sized for (leaves 40 % to spare)
+constexpr int kSlabMoveCap = 1024;                    // entries that may move into one bucket from elsewhere
+constexpr int kSlabSerialCap = 4096;                  // overflow entries per partition the fast path carries
+
+struct SlabGeom {
+  uint32_t m;         // keys are < m
+  uint32_t npp;       // keys per partition (m / partitions)
+  uint32_t bpp;       // buckets per partition
+  uint32_t bpp_mult;  // floor(bpp * 2^32 / npp)
+  uint32_t nbuckets;  // partitions * bpp
+  uint32_t sub_mult;  // floor(kSlabSubs * 2^32 / (widest bucket + 1)): key offset inside a bucket -> narrow range
+
+  __device__ inline uint32_t bucket_of(uint32_t key) const {
+    const uint32_t part = key / npp;
+    return part * bpp + __umulhi(key - part * npp, bpp_mult);
+  }
+  __device__ inline uint32_t first_key(uint32_t b) const {  // smallest key of bucket b
+    const uint32_t part = b / bpp, sb = b - part * bpp;
+    return part * npp + (uint32_t)((((uint64_t)sb << 32) + bpp_mult - 1) / bpp_mult);
+  }
+  __device__ inline uint32_t sub_of(uint32_t offset) const { return __umulhi(offset, sub_mult); }
+};
+
+// Host side: geometry for `partitions` partitions of a key space of m keys (m a
+// multiple of partitions) expected to hold about `expected` records.  Returns
+// false if the slab layout does not suit these sizes.
+inline bool slab_geometry(int64_t m, int partitions, int64_t expected, int target, SlabGeom *out) {
+  if (m < (1ll << 22) || m > 0x7fffffffll || partitions < 1 || partitions > kSlabMaxBuckets || m % partitions != 0 ||
+      expected < 1)
+    return false;
+  int64_t bpp = ceil_div(expected, (int64_t)target * partitions);
+  if (bpp < 1) bpp = 1;
+  if (bpp * partitions > kSlabMaxBuckets) bpp = kSlabMaxBuckets / partitions;
+  const int64_t nb = bpp * partitions;
+  if (expected / nb > (int64_t)kSlabCap * 3 / 4) return false;  // too many records per bucket
+  const int64_t npp = m / partitions;
+  if (npp / bpp < 4 * kSlabSubs) return false;                  // buckets narrower than their sub-ranges
+  SlabGeom g;
+  g.m = (uint32_t)m;
+  g.npp = (uint32_t)npp;
+  g.bpp = (uint32_t)bpp;
+  g.bpp_mult = (uint32_t)(((uint64_t)bpp << 32) / (uint64_t)npp);
+  g.nbuckets = (uint32_t)nb;
+  const uint64_t width = ((1ull << 32) + g.bpp_mult - 1) / g.bpp_mult + 1;  // keys per bucket, at most
+  g.sub_mult = (uint32_t)(((uint64_t)kSlabSubs << 32) / (width + 1));
+  *out = g;
+  return true;
+}
+
+// Shared memory of the in-LDS sort.
+struct SlabSortShared {
+  uint32_t key[kSlabCap];
+  uint32_t tie[kSlabCap];
+  uint32_t cnt[kSlabSubs + 1];
+  uint32_t scan[kSlabBlock / 64 + 1];
+  uint32_t bad;
+};
+
+// Ranks the live records of a workgroup by (key offset, tie), both unique as a
+// pair.  off[i] < bucket width.  The records are first grouped by narrow key
+// range with one LDS atomic each; inside its group every record counts the
+// records that precede it.  Returns false (for every thread) if a group is too
+// large for that; else rank[i] for live records and *n_out = number of live
+// records.  On return sh.key / sh.tie may be overwritten at once.
+__device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, const uint32_t (&off)[kSlabItems],
+                                 const uint32_t (&tie)[kSlabItems], uint32_t live, uint32_t (&rank)[kSlabItems],
+                                 uint32_t *n_out) {
+  for (int d = threadIdx.x; d <= kSlabSubs; d += kSlabBlock) sh.cnt[d] = 0;
+  if (threadIdx.x == 0) sh.bad = 0;
+  __syncthreads();
+  uint32_t sub[kSlabItems], at[kSlabItems];
+#pragma unroll
+  for (int i = 0; i < kSlabItems; ++i) {
+    sub[i] = at[i] = 0;
+    if (live & (1u << i)) {
+      sub[i] = geo.sub_of(off[i]);
+      at[i] = atomicAdd(&sh.cnt[sub[i]], 1u);
+    }
+  }
+  __syncthreads();
+  {
+    uint32_t c[kSlabSubsPer];
+    uint32_t sum = 0, big = 0;
+#pragma unroll
+    for (int e = 0; e < kSlabSubsPer; ++e) {
+      c[e] = sh.cnt[threadIdx.x * kSlabSubsPer + e];
+      sum += c[e];
+      big |= c[e] > (uint32_t)kSlabGroupLimit;
+    }
+    if (big) sh.bad = 1;
+    uint32_t total;
+    uint32_t running = block_exclusive_scan<uint32_t, kSlabBlock>(sum, sh.scan, &total);
+#pragma unroll
+    for (int e = 0; e < kSlabSubsPer; ++e) {
+      sh.cnt[threadIdx.x * kSlabSubsPer + e] = running;
+      running += c[e];
+    }
+    if (threadIdx.x == kSlabBlock - 1) sh.cnt[kSlabSubs] = running;
+  }
+  __syncthreads();
+  if (sh.bad) return false;
+#pragma unroll
+  for (int i = 0; i < kSlabItems; ++i) {
+    if (live & (1u << i)) {
+      const uint32_t p = sh.cnt[sub[i]] + at[i];
+      sh.key[p] = off[i];
+      sh.tie[p] = tie[i];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kSlabItems; ++i) {
+    rank[i] = 0;
+    if (live & (1u << i)) {
+      const uint32_t g0 = sh.cnt[sub[i]], g1 = sh.cnt[sub[i] + 1];
+      uint32_t less = 0;
+      for (uint32_t u = g0; u < g1; ++u) {
+        const uint32_t ku = sh.key[u];
+        less += (ku < off[i]) || (ku == off[i] && sh.tie[u] < tie[i]);
+      }
+      rank[i] = g0 + less;
+    }
+  }
+  *n_out = sh.cnt[kSlabSubs];
+  __syncthreads();
+  return true;
+}
+
+}  // namespace zen

@@ -1,0 +1,589 @@
+// Fused load balance on bucket slabs (the fast path of zen_load_balance).
+//
+// The reference inserts every selected index into an int32 table as large as
+// the gradient and then scans that table partition by partition
+// (functions_cuda_kernel.cu:97-167, tensor_load_balance.py:13-51).  Here the
+// candidates are appended to bucket slabs by the select kernel itself (a bucket
+// is a range of level-1 hash slots, zen_slab.h), and four short kernels finish
+// the job:
+//   k_slab_sort     one workgroup per bucket: applies the exact threshold, sorts
+//                   the bucket by (level-1 slot, index) inside LDS; in a run of
+//                   equal slots the first entry (smallest index) is the slot's
+//                   level-1 owner, the others lost level 1 and are logged;
+//   k_slab_chains   levels 2 and 3 for the losers through a small hash map,
+//                   with the reference's rule executed in ascending index order
+//                   (a slot belongs to the smallest index that ever probes it;
+//                   whoever takes a slot from a larger index continues that
+//                   index's probe sequence);
+//   k_slab_classify final slot of every logged entry, handed to the bucket that
+//                   slot lies in (or to the partition's serial list);
+//   k_slab_place    one workgroup per bucket: survivors and moved-in entries
+//                   merged by rank, written to the bucket's place in the
+//                   partition-major output; split sizes.
+#include "zen_balance.h"
+#include "zen_hashmap.h"
+#include "zen_slab.h"
+
+namespace zen {
+namespace {
+
+struct SlabTables {
+  uint32_t *cursor;     // [B] records appended by the select kernel
+  uint32_t *bucket_n;   // [B] selected records, sorted, in the slab
+  uint32_t *removed_n;  // [B] of which lost their level-1 slot
+  uint32_t *movein_n;   // [B] entries whose final slot lies in the bucket but whose level-1 slot does not own it
+  uint32_t *serial_n;   // [P] entries that found no slot
+  int32_t *slab_idx;    // [B * kSlabCap] index (sorted: | kRemovedBit)
+  void *slab_val;       // [B * kSlabCap]
+  uint32_t *slab_key;   // [B * kSlabCap] level-1 slot, ascending inside a slab after the sort
+  uint32_t *mv_key, *mv_idx, *mv_val;  // [B * kSlabMoveCap]
+  uint32_t *ser_idx;    // [P * kSlabSerialCap]
+  uint32_t *log_t, *log_v, *log_cell;  // [log_cap]
+  Counters *ctr;
+  uint32_t log_cap;
+};
+
+__device__ inline uint32_t level1_slot(const Probe &g, uint32_t t) { return (poly(t) + kSeed1) % g.m; }
+
+// ------------------------------------------------------------ sort a bucket
+
+template <typename S>
+__global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, Probe g, SlabTables tb,
+                                                          const uint32_t *__restrict__ filter,
+                                                          const S *__restrict__ dense, int32_t *status) {
+  __shared__ SlabSortShared sh;
+  __shared__ uint32_t s_lost, s_base;
+  const uint32_t b = blockIdx.x;
+  const size_t base = (size_t)b * kSlabCap;
+  uint32_t n_raw = tb.cursor[b];
+  if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the select kernel flagged the overflow
+  const uint32_t lo = geo.first_key(b);
+  const uint32_t thr = filter ? filter[0] : 0u;
+  S *slab_val = static_cast<S *>(tb.slab_val);
+  if (threadIdx.x == 0) s_lost = 0;
+  uint32_t off[kSlabItems], idx[kSlabItems], rank[kSlabItems];
+  S val[kSlabItems];
+  uint32_t live = 0;
+#pragma unroll
+  for (int i = 0; i < kSlabItems; ++i) {
+    const uint32_t j = threadIdx.x + i * kSlabBlock;
+    off[i] = idx[i] = 0;
+    val[i] = 0;
+    if (j < n_raw) {
+      idx[i] = (uint32_t)tb.slab_idx[base + j];
+      val[i] = slab_val[base + j];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kSlabItems; ++i) {
+    const uint32_t j = threadIdx.x + i * kSlabBlock;
+    // index 0 is never transmitted (0 is the table's empty marker, tensor_load_balance.py:31)
+    if (j < n_raw && idx[i] != 0 && (val[i] & KeyOf<S>::kMask) >= thr) {
+      off[i] = level1_slot(g, idx[i]) - lo;
+      live |= 1u << i;
+    }
+  }
+  uint32_t n = 0;
+  if (!slab_rank(sh, geo, off, idx, live, rank, &n)) {
+    if (threadIdx.x == 0) {
+      atomicOr(status, ZEN_STAT_RETRY);
+      tb.bucket_n[b] = 0;
+      tb.removed_n[b] = 0;
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < kSlabItems; ++i) {
+    if (live & (1u << i)) {
+      sh.key[rank[i]] = off[i];
+      sh.tie[rank[i]] = idx[i];
+      slab_val[base + rank[i]] = val[i];  // every thread has read its records: in place is safe
+    }
+  }
+  __syncthreads();
+  // In a run of equal slots the first entry has the smallest index: the slot's level-1 owner.  The others
+  // lost level 1.  Their places in the sorted slab are collected in sh.cnt (a bucket has at most kSlabSubs
+  // of them, else the call is declined).
+  for (uint32_t p = threadIdx.x; p < n; p += kSlabBlock) {
+    const uint32_t k = sh.key[p];
+    const bool lost = p > 0 && sh.key[p - 1] == k;
+    tb.slab_key[base + p] = k + lo;
+    tb.slab_idx[base + p] = (int32_t)(sh.tie[p] | (lost ? kRemovedBit : 0u));
+    if (lost) {
+      const uint32_t at = atomicAdd(&s_lost, 1u);
+      if (at < (uint32_t)kSlabSubs) sh.cnt[at] = p;
+    }
+  }
+  __syncthreads();
+  uint32_t lost_n = s_lost;
+  if (lost_n > (uint32_t)kSlabSubs) {
+    if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
+    lost_n = kSlabSubs;
+  }
+  if (threadIdx.x == 0) {
+    tb.bucket_n[b] = n;
+    tb.removed_n[b] = lost_n;
+    s_base = lost_n ? atomicAdd(&tb.ctr->losers, lost_n) : 0u;
+  }
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < lost_n; i += kSlabBlock) {
+    const uint32_t at = s_base + i;
+    const uint32_t t = sh.tie[sh.cnt[i]];
+    if (at < tb.log_cap) {
+      tb.log_t[at] = t;
+      tb.log_v[at] = (uint32_t)dense[t];
+    } else {
+      atomicOr(status, ZEN_STAT_RETRY);
+    }
+  }
+}
+
+// ------------------------------------------------------ levels 2 and 3
+
+// Smallest index whose level-1 slot is `slot` (kNone if nobody's), and where it sits.
+__device__ inline uint32_t slab_head(const SlabGeom &geo, const SlabTables &tb, uint32_t slot, size_t *pos_out,
+                                     uint32_t *bucket_out) {
+  const uint32_t b = geo.bucket_of(slot);
+  const uint32_t *keys = tb.slab_key + (size_t)b * kSlabCap;
+  const uint32_t n = tb.bucket_n[b];
+  const uint32_t p = lower_bound_u32(keys, n, slot);
+  if (p >= n || keys[p] != slot) return kNone;
+  *pos_out = (size_t)b * kSlabCap + p;
+  *bucket_out = b;
+  return (uint32_t)tb.slab_idx[*pos_out] & kIndexMask;
+}
+
+template <typename S>
+__global__ __launch_bounds__(256) void k_slab_chains(SlabGeom geo, Probe g, SlabTables tb, unsigned long long *cells,
+                                                     uint32_t log2, int32_t *status) {
+  Counters *ctr = tb.ctr;
+  uint32_t losers = ctr->losers;
+  if (losers > tb.log_cap) losers = tb.log_cap;
+  const S *slab_val = static_cast<const S *>(tb.slab_val);
+  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < losers; i += gridDim.x * 256u) {
+    uint32_t cur = tb.log_t[i];
+    int lv = 1;
+    bool full = false;
+    for (uint32_t steps = 0; lv < g.levels; ++steps) {
+      if (steps > kChainLimit) {
+        atomicOr(status, ZEN_STAT_INTERNAL);
+        break;
+      }
+      uint32_t part;
+      const uint32_t slot = probe_slot(g, cur, lv, &part);
+      size_t head_pos = 0;
+      uint32_t head_bucket = 0;
+      const uint32_t head = slab_head(geo, tb, slot, &head_pos, &head_bucket);
+      if (head < cur) {  // a smaller index probes this slot at level 1: cur moves on
+        ++lv;
+        continue;
+      }
+      const uint32_t old = map_min(cells, log2, slot, cur, ctr, &full);
+      if (full) {
+        atomicOr(status, ZEN_STAT_RETRY);
+        break;
+      }
+      if (old < cur) {  // a smaller index got here at level 2 or 3
+        ++lv;
+        continue;
+      }
+      if (old == kNone) {
+        // first level-2/3 prober of this slot: its level-1 owner (a larger index, if any) is pushed out
+        if (head == kNone) break;
+        atomicOr(reinterpret_cast<uint32_t *>(&tb.slab_idx[head_pos]), kRemovedBit);
+        atomicAdd(&tb.removed_n[head_bucket], 1u);
+        const uint32_t at = losers + atomicAdd(&ctr->displaced, 1u);
+        if (at < tb.log_cap) {
+          tb.log_t[at] = head;
+          tb.log_v[at] = (uint32_t)slab_val[head_pos];
+        } else {
+          atomicOr(status, ZEN_STAT_RETRY);
+        }
+        cur = head;
+        lv = 1;
+        continue;
+      }
+      if (old == cur) break;
+      // took the slot from a larger index that held it at its first level mapping here
+      int lw = 1;
+      while (lw < g.levels && probe_slot(g, old, lw, &part) != slot) ++lw;
+      cur = old;
+      lv = lw + 1;
+    }
+  }
+}
+
+// Final place of every logged entry: the level-2/3 slot it holds in the map, or its partition's serial list.
+__global__ __launch_bounds__(256) void k_slab_classify(SlabGeom geo, Probe g, SlabTables tb,
+                                                       const unsigned long long *__restrict__ cells, uint32_t log2,
+                                                       int64_t spp, int32_t *status) {
+  const Counters *ctr = tb.ctr;
+  uint32_t losers = ctr->losers;
+  if (losers > tb.log_cap) losers = tb.log_cap;
+  uint32_t total = losers + ctr->displaced;
+  if (total > tb.log_cap) total = tb.log_cap;
+  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+    const uint32_t t = tb.log_t[i];
+    uint32_t part = 0, cell = kNone, slot = kNone;
+    for (int lv = 1; lv < g.levels && slot == kNone; ++lv) {
+      const uint32_t s = probe_slot(g, t, lv, &part);
+      uint32_t at = 0;
+      if (map_find(cells, log2, s, &at) == t) {
+        slot = s;
+        cell = at;
+      }
+    }
+    tb.log_cell[i] = cell;
+    if (slot != kNone) {
+      const uint32_t b = geo.bucket_of(slot);
+      const uint32_t at = atomicAdd(&tb.movein_n[b], 1u);
+      if (at < (uint32_t)kSlabMoveCap) {
+        const size_t dst = (size_t)b * kSlabMoveCap + at;
+        tb.mv_key[dst] = slot;
+        tb.mv_idx[dst] = t;
+        tb.mv_val[dst] = tb.log_v[i];
+      } else {
+        atomicOr(status, ZEN_STAT_RETRY);
+      }
+    } else {
+      part = level1_slot(g, t) / g.npp;
+      const uint32_t at = atomicAdd(&tb.serial_n[part], 1u);
+      if (at < (uint32_t)kSlabSerialCap)
+        tb.ser_idx[(size_t)part * kSlabSerialCap + at] = t;
+      else  // more than the partition's serial region holds is an overflow; more than this path carries, a retry
+        atomicOr(status, (int64_t)at >= spp ? ZEN_STAT_SERIAL_OVERFLOW : ZEN_STAT_RETRY);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ place
+
+template <typename S>
+__global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTables tb, unsigned long long *cells,
+                                                           int partitions, int64_t spp,
+                                                           const S *__restrict__ dense, int32_t *__restrict__ out_idx,
+                                                           S *__restrict__ out_val, uint32_t capacity,
+                                                           int64_t *__restrict__ splits, int32_t *status) {
+  __shared__ uint32_t s_key[kSlabCap];   // sorted slots of the bucket; later the bucket's output indices
+  __shared__ uint32_t s_idx[kSlabCap];   // their indices (| kRemovedBit); later the output values
+  __shared__ uint32_t s_mk[kSlabMoveCap], s_mi[kSlabMoveCap], s_mv[kSlabMoveCap];
+  __shared__ uint32_t s_pref[kSlabMaxBuckets + 1];
+  __shared__ uint32_t s_tb[kSlabBlock];
+  __shared__ uint32_t s_scan[kSlabBlock / 64 + 1];
+  const uint32_t b = blockIdx.x;
+  const uint32_t B = geo.nbuckets;
+  const size_t base = (size_t)b * kSlabCap;
+  const S *slab_val = static_cast<const S *>(tb.slab_val);
+
+  // every occupied map cell ends with the index that finally holds its slot, and that index recorded the
+  // cell: clearing by cell number leaves the borrowed memory zero again
+  {
+    uint32_t losers = tb.ctr->losers;
+    if (losers > tb.log_cap) losers = tb.log_cap;
+    uint32_t total = losers + tb.ctr->displaced;
+    if (total > tb.log_cap) total = tb.log_cap;
+    for (uint32_t i = b * kSlabBlock + threadIdx.x; i < total; i += B * kSlabBlock) {
+      const uint32_t cell = tb.log_cell[i];
+      if (cell != kNone) cells[cell] = 0ull;
+    }
+  }
+
+  // where every bucket starts in the output: survivors + moved-in entries, the partition's serial entries
+  // behind its last bucket
+  {
+    constexpr int kPer = kSlabMaxBuckets / kSlabBlock;
+    uint32_t c[kPer];
+    uint32_t sum = 0;
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) {
+      const uint32_t x = threadIdx.x * kPer + e;
+      c[e] = 0;
+      if (x < B) {
+        uint32_t mv = tb.movein_n[x];
+        if (mv > (uint32_t)kSlabMoveCap) mv = kSlabMoveCap;
+        c[e] = tb.bucket_n[x] - tb.removed_n[x] + mv;
+        if (x % geo.bpp == geo.bpp - 1) {
+          uint32_t sn = tb.serial_n[x / geo.bpp];
+          if (sn > (uint32_t)kSlabSerialCap) sn = kSlabSerialCap;
+          c[e] += sn;
+        }
+      }
+      sum += c[e];
+    }
+    uint32_t total;
+    uint32_t running = block_exclusive_scan<uint32_t, kSlabBlock>(sum, s_scan, &total);
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) {
+      const uint32_t x = threadIdx.x * kPer + e;
+      if (x <= B) s_pref[x] = running;
+      running += c[e];
+    }
+    if (B == (uint32_t)kSlabMaxBuckets && threadIdx.x == kSlabBlock - 1) s_pref[B] = running;
+  }
+  const uint32_t n = tb.bucket_n[b];
+  uint32_t mv_n = tb.movein_n[b];
+  if (mv_n > (uint32_t)kSlabMoveCap) mv_n = kSlabMoveCap;
+  for (uint32_t p = threadIdx.x; p < n; p += kSlabBlock) {
+    s_key[p] = tb.slab_key[base + p];
+    s_idx[p] = (uint32_t)tb.slab_idx[base + p];
+  }
+  // moved-in entries ordered by slot (slots are distinct: each is owned by one index)
+  uint32_t mk[kSlabMoveCap / kSlabBlock], mi[kSlabMoveCap / kSlabBlock], mvv[kSlabMoveCap / kSlabBlock];
+#pragma unroll
+  for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
+    const uint32_t j = threadIdx.x + e * kSlabBlock;
+    mk[e] = mi[e] = mvv[e] = 0;
+    if (j < mv_n) {
+      mk[e] = tb.mv_key[(size_t)b * kSlabMoveCap + j];
+      mi[e] = tb.mv_idx[(size_t)b * kSlabMoveCap + j];
+      mvv[e] = tb.mv_val[(size_t)b * kSlabMoveCap + j];
+      s_mk[j] = mk[e];
+    }
+  }
+  __syncthreads();
+  const uint32_t out_base = s_pref[b];
+  const uint32_t out_n = s_pref[b + 1] - out_base;
+  {
+    uint32_t r[kSlabMoveCap / kSlabBlock];
+#pragma unroll
+    for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
+      r[e] = 0;
+      if (threadIdx.x + e * kSlabBlock < mv_n)
+        for (uint32_t u = 0; u < mv_n; ++u) r[e] += s_mk[u] < mk[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
+      if (threadIdx.x + e * kSlabBlock < mv_n) {
+        s_mk[r[e]] = mk[e];
+        s_mi[r[e]] = mi[e];
+        s_mv[r[e]] = mvv[e];
+      }
+    }
+  }
+  // survivors: thread t owns the sorted places [t * kSlabItems, (t + 1) * kSlabItems)
+  const uint32_t first = threadIdx.x * kSlabItems;
+  uint32_t flags = 0;
+#pragma unroll
+  for (int i = 0; i < kSlabItems; ++i)
+    if (first + i < n && !(s_idx[first + i] & kRemovedBit)) flags |= 1u << i;
+  uint32_t surv_total;
+  const uint32_t before = block_exclusive_scan<uint32_t, kSlabBlock>((uint32_t)__popc(flags), s_scan, &surv_total);
+  s_tb[threadIdx.x] = before;
+  __syncthreads();  // also: s_mk sorted
+  uint32_t place[kSlabItems], o_idx[kSlabItems];
+  S o_val[kSlabItems];
+  {
+    uint32_t run = before;
+#pragma unroll
+    for (int i = 0; i < kSlabItems; ++i) {
+      place[i] = kNone;
+      o_idx[i] = 0;
+      o_val[i] = 0;
+      if (flags & (1u << i)) {
+        place[i] = run + lower_bound_u32(s_mk, mv_n, s_key[first + i]);
+        o_idx[i] = s_idx[first + i];
+        o_val[i] = slab_val[base + first + i];
+        ++run;
+      }
+    }
+  }
+  // moved-in entry j: its rank among them plus the survivors whose slot is smaller
+  uint32_t mplace[kSlabMoveCap / kSlabBlock];
+#pragma unroll
+  for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
+    const uint32_t j = threadIdx.x + e * kSlabBlock;
+    mplace[e] = kNone;
+    if (j < mv_n) {
+      const uint32_t p0 = lower_bound_u32(s_key, n, s_mk[j]);
+      const uint32_t owner = p0 / kSlabItems;
+      uint32_t surv = owner < (uint32_t)kSlabBlock ? s_tb[owner] : surv_total;
+      for (uint32_t p = owner * kSlabItems; p < p0; ++p) surv += !(s_idx[p] & kRemovedBit);
+      mplace[e] = j + surv;
+      mi[e] = s_mi[j];
+      mvv[e] = s_mv[j];
+    }
+  }
+  __syncthreads();
+  // gather the bucket's output in LDS, then write it with consecutive lanes
+#pragma unroll
+  for (int i = 0; i < kSlabItems; ++i) {
+    if (place[i] != kNone && place[i] < (uint32_t)kSlabCap) {
+      s_key[place[i]] = o_idx[i];
+      s_idx[place[i]] = (uint32_t)o_val[i];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
+    if (mplace[e] != kNone && mplace[e] < (uint32_t)kSlabCap) {
+      s_key[mplace[e]] = mi[e];
+      s_idx[mplace[e]] = mvv[e];
+    }
+  }
+  __syncthreads();
+  const uint32_t part = b / geo.bpp;
+  const bool last_of_part = b % geo.bpp == geo.bpp - 1;
+  uint32_t serial = 0;
+  if (last_of_part) {
+    serial = tb.serial_n[part];
+    if (serial > (uint32_t)kSlabSerialCap) serial = kSlabSerialCap;
+  }
+  const uint32_t own_n = out_n - serial;  // survivors + moved-in
+  if (own_n > (uint32_t)kSlabCap) {       // cannot happen with the capacities above; never write past LDS
+    if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_INTERNAL);
+    return;
+  }
+  for (uint32_t i = threadIdx.x; i < own_n; i += kSlabBlock) {
+    const uint32_t pos = out_base + i;
+    if (pos < capacity) {
+      out_idx[pos] = (int32_t)s_key[i];
+      out_val[pos] = (S)s_idx[i];
+    }
+  }
+  if (serial) {
+    // the partition's overflow entries in ascending index order (the reference hands its tickets to
+    // ascending thread ids, functions_cuda_kernel.cu:107-108), behind everything that found a slot
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < serial; i += kSlabBlock) s_key[i] = tb.ser_idx[(size_t)part * kSlabSerialCap + i];
+    __syncthreads();
+    sort_network(s_key, serial);
+    for (uint32_t i = threadIdx.x; i < serial; i += kSlabBlock) {
+      const uint32_t pos = out_base + own_n + i;
+      if (pos < capacity) {
+        out_idx[pos] = (int32_t)s_key[i];
+        out_val[pos] = dense[s_key[i]];
+      }
+    }
+  }
+  if (b % geo.bpp == 0 && threadIdx.x == 0) {
+    const uint32_t lo = s_pref[b], hi = s_pref[b + geo.bpp];
+    splits[part] = (int64_t)(hi - lo);
+    if ((int64_t)tb.serial_n[part] > spp) atomicOr(status, ZEN_STAT_SERIAL_OVERFLOW);
+    if (hi > capacity) atomicOr(status, ZEN_STAT_CAPACITY);
+  }
+  (void)partitions;
+}
+
+struct SlabPlan {
+  SlabTables tb;
+  uint32_t *sample_hist;  // sampled floor histogram (+ finished-block count)
+  uint32_t *cand_hist;
+  uint32_t *ticket;
+  uint32_t *thr;          // [0..1] exact threshold + count, [2..3] sampled floor
+  void *zero_begin;
+  size_t zero_bytes;
+  size_t bytes;
+};
+
+SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dtype, int64_t list_cap) {
+  Carver cv(workspace);
+  SlabPlan p;
+  const size_t B = geo.nbuckets;
+  // everything that must be zero when the first kernel starts sits together: one fill
+  p.zero_begin = cv.base + cv.used;
+  p.sample_hist = cv.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
+  p.cand_hist = cv.take<uint32_t>((size_t)kCandHistWords);
+  p.ticket = cv.take<uint32_t>(4);
+  p.tb.cursor = cv.take<uint32_t>(B);
+  p.tb.movein_n = cv.take<uint32_t>(B);
+  p.tb.serial_n = cv.take<uint32_t>((size_t)partitions);
+  p.tb.ctr = cv.take<Counters>(1);
+  p.zero_bytes = (size_t)(cv.base + cv.used - static_cast<char *>(p.zero_begin));
+  p.thr = cv.take<uint32_t>(4);
+  p.tb.bucket_n = cv.take<uint32_t>(B);
+  p.tb.removed_n = cv.take<uint32_t>(B);
+  p.tb.slab_idx = cv.take<int32_t>(B * kSlabCap);
+  p.tb.slab_val = cv.take<char>(B * kSlabCap * (dtype == ZEN_BF16 ? 2 : 4));
+  p.tb.slab_key = cv.take<uint32_t>(B * kSlabCap);
+  p.tb.mv_key = cv.take<uint32_t>(B * kSlabMoveCap);
+  p.tb.mv_idx = cv.take<uint32_t>(B * kSlabMoveCap);
+  p.tb.mv_val = cv.take<uint32_t>(B * kSlabMoveCap);
+  p.tb.ser_idx = cv.take<uint32_t>((size_t)partitions * kSlabSerialCap);
+  p.tb.log_cap = (uint32_t)(list_cap / 4 + 1024);
+  p.tb.log_t = cv.take<uint32_t>(p.tb.log_cap);
+  p.tb.log_v = cv.take<uint32_t>(p.tb.log_cap);
+  p.tb.log_cell = cv.take<uint32_t>(p.tb.log_cap);
+  p.bytes = cv.used;
+  return p;
+}
+
+template <typename S>
+int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p, hipStream_t s) {
+  const uint32_t B = geo.nbuckets;
+  const uint32_t *filter = a.k > 0 ? p.thr : nullptr;
+  const S *dense = static_cast<const S *>(a.input);
+  {
+    ProfScope prof(kProfInsertList, s);
+    k_slab_sort<S><<<dim3(B), dim3(kSlabBlock), 0, s>>>(geo, a.g, p.tb, filter, dense, a.status);
+    ZEN_LAUNCH_CHECK("k_slab_sort");
+  }
+  {
+    ProfScope prof(kProfFinalKey, s);
+    k_slab_chains<S><<<dim3(256), dim3(256), 0, s>>>(geo, a.g, p.tb, a.hash, a.hash_log2, a.status);
+    ZEN_LAUNCH_CHECK("k_slab_chains");
+    k_slab_classify<<<dim3(256), dim3(256), 0, s>>>(geo, a.g, p.tb, a.hash, a.hash_log2, a.spp, a.status);
+    ZEN_LAUNCH_CHECK("k_slab_classify");
+  }
+  {
+    ProfScope prof(kProfGather, s);
+    k_slab_place<S><<<dim3(B), dim3(kSlabBlock), 0, s>>>(geo, p.tb, a.hash, a.partitions, a.spp, dense, a.out_idx,
+                                                         static_cast<S *>(a.out_val), (uint32_t)a.capacity, a.splits,
+                                                         a.status);
+    ZEN_LAUNCH_CHECK("k_slab_place");
+  }
+  return ZEN_OK;
+}
+
+}  // namespace
+
+bool slab_balance_fits(int64_t n, int64_t m, int partitions, int dtype, int64_t capacity, int64_t k, SlabGeom *geo) {
+  (void)n;
+  if (k > 0 && dtype != ZEN_BF16) return false;  // the candidate histogram resolves bf16 keys only
+  if (capacity > 0x1fffffffll) return false;
+  SlabGeom g;
+  if (!slab_geometry(m, partitions, capacity, kSlabTarget, &g)) return false;
+  if (geo) *geo = g;
+  return true;
+}
+
+size_t slab_balance_bytes(int64_t m, int partitions, int dtype, int64_t capacity) {
+  SlabGeom geo;
+  if (!slab_geometry(m, partitions, capacity, kSlabTarget, &geo)) return 0;
+  return plan_slab(nullptr, geo, partitions, dtype, list_capacity(capacity)).bytes;
+}
+
+int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
+  SlabGeom geo;
+  if (!slab_balance_fits(a.n, a.g.m, a.partitions, a.dtype, a.capacity, a.k, &geo))
+    return fail(ZEN_EINVAL, "slab_load_balance: sizes do not suit the slab layout");
+  const SlabPlan p = plan_slab(a.workspace, geo, a.partitions, a.dtype, list_capacity(a.capacity));
+  launch_fill<uint32_t>(static_cast<uint32_t *>(p.zero_begin), 0u, p.zero_bytes / sizeof(uint32_t), s);
+  ZEN_LAUNCH_CHECK("slab: clear counters");
+  ScatterArgs sc;
+  sc.in = a.input;
+  sc.dtype = a.dtype;
+  sc.n = a.n;
+  sc.thr = a.thr;
+  sc.geo = geo;
+  sc.cursor = p.tb.cursor;
+  sc.slab_idx = p.tb.slab_idx;
+  sc.slab_val = p.tb.slab_val;
+  sc.ticket = p.ticket;
+  sc.status = a.status;
+  int rc;
+  if (a.k > 0) {
+    // one pass: everything at or above a floor estimated from a sample goes to the slabs, the exact
+    // threshold is read off the candidates' histogram and applied when the buckets are sorted
+    if ((rc = topk_sampled_floor(a.input, a.dtype, a.n, a.k, p.thr + 2, p.sample_hist, s, true)) != ZEN_OK) return rc;
+    sc.thr = p.thr + 2;
+    sc.cand_hist = p.cand_hist;
+    sc.pick_k = a.k;
+    sc.pick_thr = p.thr;
+    sc.thr_copy = a.thr_out;
+  }
+  if ((rc = select_scatter(sc, s)) != ZEN_OK) return rc;
+  if (a.dtype == ZEN_BF16) return slab_launch<uint16_t>(a, geo, p, s);
+  return slab_launch<uint32_t>(a, geo, p, s);
+}
+
+}  // namespace zen
