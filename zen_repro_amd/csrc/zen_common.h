@@ -142,6 +142,10 @@ __device__ inline uint16_t f32_to_bf16_rne(float f) {
   return uint16_t(u >> 16);
 }
 
+// Waits until the global memory operations this wave has issued, stores and atomics without a return value
+// included, have been acknowledged by the place that carries them out.
+__device__ inline void wait_global_acks() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 __device__ inline int lane_id() { return int(__lane_id()); }
 
 __device__ inline uint64_t lanes_below() {  // mask of lanes with a smaller id

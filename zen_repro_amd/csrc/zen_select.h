@@ -89,19 +89,20 @@ constexpr int kCandRows = 8;   // partial candidate histograms (blocks spread ov
 constexpr int kCandHistWords = kCandRows * kCandBins + 1;
 
 // One pass over a dense tensor that appends every element with key >= max(thr[0], 1) (thr == nullptr: the
-// nonzero ones), as (index, value), to the bucket slab of its level-1 hash slot.  cursor[nbuckets], *ticket and
-// cand_hist must be zero on entry.  A slab that fills up raises ZEN_STAT_RETRY.  With cand_hist / pick_k /
-// pick_thr the exact k-th largest key is read off the candidates' histogram as in SelectArgs (and copied to
-// thr_copy if that is not null).
-struct ScatterArgs {
+// nonzero ones), as (index, value), to a list, in no particular order, by persistent workgroups.
+// *list_count, *ticket and cand_hist must be zero on entry; *list_count ends as the number found, which may
+// exceed `capacity` (the excess is dropped; callers compare).  With cand_hist / pick_k / pick_thr the exact
+// k-th largest key is read off the candidates' histogram as in SelectArgs (and copied to thr_copy if that
+// is not null).
+struct StageArgs {
   const void *in = nullptr;
   int dtype = ZEN_F32;
   int64_t n = 0;
   const uint32_t *thr = nullptr;
-  SlabGeom geo;
-  uint32_t *cursor = nullptr;      // [nbuckets] records appended per bucket (may exceed kSlabCap: then RETRY)
-  int32_t *slab_idx = nullptr;     // [nbuckets * kSlabCap]
-  void *slab_val = nullptr;        // [nbuckets * kSlabCap] elements of the tensor's type
+  uint32_t *list_count = nullptr;
+  int32_t *list_idx = nullptr;
+  void *list_val = nullptr;        // elements of the tensor's type
+  int64_t capacity = 0;            // < 2^32
   uint32_t *ticket = nullptr;
   uint32_t *cand_hist = nullptr;
   int64_t pick_k = 0;
@@ -109,6 +110,6 @@ struct ScatterArgs {
   uint32_t *thr_copy = nullptr;
   int32_t *status = nullptr;
 };
-int select_scatter(const ScatterArgs &a, hipStream_t stream);
+int select_stage_list(const StageArgs &a, hipStream_t stream);
 
 }  // namespace zen

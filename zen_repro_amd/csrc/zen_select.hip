@@ -3,6 +3,7 @@
 // (train.py:83), and the ordered single-pass compaction that turns a dense
 // tensor into ascending (index, value) lists (comm.py:47-50).
 #include <math.h>
+#include <stdlib.h>
 
 #include "zen_select.h"
 
@@ -128,6 +129,11 @@ __global__ __launch_bounds__(kHistBlock) void k_topk_pick(TopkState *st, uint32_
 constexpr int kFineBins = 32768;
 constexpr int kSampleBlock = 1024;
 
+// Device-wide atomics on one 128-byte line are carried out one after the other (about 10 ns each), and the
+// populated part of a magnitude histogram is a few hundred neighbouring bins.  So neighbouring bins are kept
+// 2 KiB apart in the global histogram.
+__device__ inline uint32_t fine_place(uint32_t bin) { return ((bin & 63u) << 9) | (bin >> 6); }
+
 // Run by one whole block once the histogram is complete: the lowest fine bin b
 // such that `rank` sample elements lie in bins >= b; floor_out[0] = lowest key
 // of that bin (0 if the sample is too small).
@@ -135,39 +141,39 @@ __device__ inline uint32_t load_fresh(const uint32_t *p) {  // written by other 
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Walks down from the highest populated bin (hist[kFineBins + 1]) in windows of one bin per thread, with
+// consecutive lanes on consecutive words (one workgroup fetching 32768 scattered words past the caches would
+// take tens of microseconds), until `rank` sample elements lie at or above a bin.
 __device__ inline void sample_pick_block(const uint32_t *hist, uint32_t rank, int key_shift, uint32_t *floor_out,
                                          uint32_t *smem) {
-  constexpr int kPer = kFineBins / kSampleBlock;
-  uint32_t c[kPer];
-  uint32_t mine = 0;
-#pragma unroll
-  for (int j = 0; j < kPer; ++j) {
-    c[j] = load_fresh(&hist[kFineBins - 1 - (threadIdx.x * kPer + j)]);
-    mine += c[j];
+  int base = (int)load_fresh(&hist[kFineBins + 1]);
+  if (base > kFineBins - 1) base = kFineBins - 1;
+  uint32_t cum = 0;
+  for (;; base -= kSampleBlock) {
+    const int bin = base - (int)threadIdx.x;
+    const uint32_t c = bin >= 0 ? load_fresh(&hist[fine_place((uint32_t)bin)]) : 0u;
+    uint32_t total;
+    const uint32_t above = cum + block_exclusive_scan<uint32_t, kSampleBlock>(c, smem, &total);
+    if (above < rank && rank <= above + c) floor_out[0] = (uint32_t)bin << key_shift;
+    cum += total;
+    if (cum >= rank) return;
+    if (base < kSampleBlock) break;
   }
-  uint32_t total;
-  uint32_t above = block_exclusive_scan<uint32_t, kSampleBlock>(mine, smem, &total);
-  if (total < rank) {
-    if (threadIdx.x == 0) floor_out[0] = 0;
-  } else {
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-      if (above < rank && rank <= above + c[j]) floor_out[0] = (uint32_t)(kFineBins - 1 - (threadIdx.x * kPer + j)) << key_shift;
-      above += c[j];
-    }
-  }
+  if (threadIdx.x == 0) floor_out[0] = 0;  // the sample is too small
 }
 
 template <typename S, bool ALIGNED>
 __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restrict__ in, int64_t n, int block_log2,
                                                               uint32_t *__restrict__ hist, uint32_t rank,
-                                                              uint32_t *floor_out) {
+                                                              uint32_t *floor_out, bool fused) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kShift = KeyOf<S>::kBits - 15;
-  __shared__ uint32_t bins[kFineBins / 2];
+  // one pad word per 32: the flush below reads 16 consecutive words per thread, which would otherwise put
+  // all lanes of a wave on two LDS banks
+  __shared__ uint32_t bins[kFineBins / 2 + kFineBins / 64];
   __shared__ uint32_t smem[kSampleBlock / 64 + 1];
   __shared__ bool s_last;
-  for (int i = threadIdx.x; i < kFineBins / 2; i += kSampleBlock) bins[i] = 0;
+  for (int i = threadIdx.x; i < kFineBins / 2 + kFineBins / 64; i += kSampleBlock) bins[i] = 0;
   __syncthreads();
   const int64_t nvec = (n + V - 1) / V;
   const int64_t nblocks = (nvec + (1ll << block_log2) - 1) >> block_log2;
@@ -181,48 +187,98 @@ __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restric
     for (int i = 0; i < V; ++i) {
       if (i < live) {
         const uint32_t bin = (e[i] & KeyOf<S>::kMask) >> kShift;
-        atomicAdd(&bins[bin >> 1], 1u << (16 * (bin & 1u)));
+        atomicAdd(&bins[(bin >> 1) + (bin >> 6)], 1u << (16 * (bin & 1u)));
       }
     }
   }
   __syncthreads();
-  uint32_t landed = 0;
-  for (int i = threadIdx.x; i < kFineBins / 2; i += kSampleBlock) {
-    const uint32_t c = bins[i];
-    if (c & 0xffffu) landed += atomicAdd(&hist[2 * i], c & 0xffffu);
-    if (c >> 16) landed += atomicAdd(&hist[2 * i + 1], c >> 16);
+  // Only the top of the histogram matters (the rank looked for is a small fraction of the sample), and a
+  // global atomic per populated bin and block is what this kernel would spend its time on.  So a block adds
+  // its bins from the top down only until it has added 16 times its share of the rank: counts further down
+  // stay too low, which can only make the floor lower (more candidates), never higher.
+  {
+    constexpr int kWords = kFineBins / 2 / kSampleBlock;
+    const uint64_t lim64 = 16ull * rank / gridDim.x + 1024ull;
+    const uint32_t limit = lim64 > 0xffffffffull ? 0xffffffffu : (uint32_t)lim64;
+    uint32_t c[kWords];
+    uint32_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < kWords; ++j) {
+      const int w = kFineBins / 2 - 1 - (threadIdx.x * kWords + j);
+      c[j] = bins[w + (w >> 5)];
+      mine += (c[j] & 0xffffu) + (c[j] >> 16);
+    }
+    uint32_t total;
+    uint32_t above = block_exclusive_scan<uint32_t, kSampleBlock>(mine, smem, &total);
+    // the highest populated bin of the block belongs to the first thread that has anything
+    if (mine && above == 0) {
+      int top = 0;
+#pragma unroll
+      for (int j = kWords - 1; j >= 0; --j) {
+        const int w = kFineBins / 2 - 1 - (threadIdx.x * kWords + j);
+        if (c[j] & 0xffffu) top = 2 * w;
+        if (c[j] >> 16) top = 2 * w + 1;
+      }
+      atomicMax(&hist[kFineBins + 1], (uint32_t)top);
+    }
+#pragma unroll
+    for (int j = 0; j < kWords; ++j) {
+      const int w = kFineBins / 2 - 1 - (threadIdx.x * kWords + j);
+      const uint32_t hi = c[j] >> 16, lo = c[j] & 0xffffu;
+      if (hi && above < limit) atomicAdd(&hist[fine_place(2 * w + 1)], hi);
+      above += hi;
+      if (lo && above < limit) atomicAdd(&hist[fine_place(2 * w)], lo);
+      above += lo;
+    }
   }
   // The block that finishes last reads the threshold off the complete histogram (hist[kFineBins] counts
-  // finished blocks).  No fence: every add above has returned its old value, so it has been carried out
-  // where atomics are carried out, before this block's count goes up; the reader loads from that place.
-  // (A device-wide fence in every block would write back and invalidate the caches each time.)
-  if (__syncthreads_or(landed == 0xffffffffu)) return;  // never true: keeps the returns alive
+  // finished blocks).  The adds above return nothing, so they are all in flight together.  They are carried
+  // out where device-wide atomics are carried out; every wave waits until its own have been acknowledged
+  // (a device-scope fence would also write the whole L2 back, once per wave) before this block's count goes
+  // up, and the reader loads from that same place (load_fresh).
+  wait_global_acks();
+  __syncthreads();
   if (threadIdx.x == 0) s_last = atomicAdd(&hist[kFineBins], 1u) == gridDim.x - 1;
   __syncthreads();
   if (!s_last) return;
-  sample_pick_block(hist, rank, kShift, floor_out, smem);
+  if (fused) sample_pick_block(hist, rank, kShift, floor_out, smem);
 }
 
-// Run by one whole block (kSelBlock threads) over the complete candidate
+__global__ __launch_bounds__(kSampleBlock) void k_sample_pick(const uint32_t *hist, uint32_t rank, int key_shift,
+                                                              uint32_t *floor_out) {
+  __shared__ uint32_t smem[kSampleBlock / 64 + 1];
+  sample_pick_block(hist, rank, key_shift, floor_out, smem);
+}
+
+// Run by one whole block (BLOCK threads) over the complete candidate
 // histogram (bin = min((key - floor) >> shift, kCandBins-1), kCandRows partial
 // rows): the exact k-th largest key when the bins are single keys (shift 0),
 // else the lowest key of its bin.  thr_out = (key, number of candidates >=
 // key).  Too few candidates, or the k-th lies in the clipped last bin:
 // ZEN_STAT_RETRY.
+// Place of a candidate bin inside its row of the global histogram: neighbours 256 bytes apart (see fine_place).
+__device__ inline uint32_t cand_place(uint32_t bin) { return ((bin & 31u) << 6) | (bin >> 5); }
+__device__ inline uint32_t cand_bin_at(uint32_t place) { return ((place & 63u) << 5) | (place >> 6); }
+
 template <int BLOCK>
 __device__ inline void cand_pick_block(const uint32_t *hist, uint32_t base, uint32_t k, int shift,
-                                       uint32_t *thr_out, int32_t *status, uint32_t *smem) {
+                                       uint32_t *thr_out, int32_t *status, uint32_t *smem, uint32_t *s_sum) {
   constexpr int kPer = kCandBins / BLOCK;
+  // the rows are summed into s_sum (kCandBins words of LDS) with consecutive lanes on consecutive words
+  __syncthreads();
+  for (int i = threadIdx.x; i < kCandBins; i += BLOCK) {
+    uint32_t sum = 0;
+#pragma unroll
+    for (int row = 0; row < kCandRows; ++row) sum += load_fresh(&hist[row * kCandBins + i]);
+    s_sum[cand_bin_at((uint32_t)i)] = sum;
+  }
+  __syncthreads();
   uint32_t c[kPer];
   uint32_t mine = 0;
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
-    const int bin = kCandBins - 1 - (threadIdx.x * kPer + j);
-    uint32_t sum = 0;
-#pragma unroll
-    for (int row = 0; row < kCandRows; ++row) sum += load_fresh(&hist[row * kCandBins + bin]);
-    c[j] = sum;
-    mine += sum;
+    c[j] = s_sum[kCandBins - 1 - (threadIdx.x * kPer + j)];
+    mine += c[j];
   }
   uint32_t total;
   uint32_t above = block_exclusive_scan<uint32_t, BLOCK>(mine, smem, &total);
@@ -508,23 +564,23 @@ __global__ __launch_bounds__(kSelBlock) void k_select_compact(
     // spread over kCandRows partial histograms: fewer blocks meet on one counter
     __syncthreads();
     uint32_t *row = cand_hist + (size_t)(blockIdx.x % kCandRows) * kCandBins;
-    uint32_t landed = 0;
     for (int i = threadIdx.x; i < kCandBins; i += kSelBlock) {
       const uint32_t c = s_hist[i];
-      if (c) landed += atomicAdd(&row[i], c);
+      if (c) atomicAdd(&row[cand_place((uint32_t)i)], c);  // nothing returned: the adds are in flight together
     }
     if (pick_thr) {
       // The block that finishes last reads the exact threshold off the complete histogram
-      // (cand_hist[kCandRows * kCandBins] counts finished blocks).  No fence: the adds above have returned,
-      // so they have been carried out before this block's count goes up, and the reader loads from the
-      // place where atomics are carried out.
+      // (cand_hist[kCandRows * kCandBins] counts finished blocks).
       __shared__ bool s_last;
-      if (__syncthreads_or(landed == 0xffffffffu)) return;  // never true: keeps the returns alive
+      // the adds are carried out (where device-wide atomics are) before the count goes up; no device-scope
+      // fence: that would write the L2 back once per wave
+      wait_global_acks();
+      __syncthreads();
       if (threadIdx.x == 0) s_last = atomicAdd(&cand_hist[kCandRows * kCandBins], 1u) == (uint32_t)ntiles - 1u;
       __syncthreads();
       if (s_last) {
         cand_pick_block<kSelBlock>(cand_hist, floor_key, pick_k, KeyOf<S>::kBits == 15 ? 0 : 16, pick_thr, status,
-                                   reinterpret_cast<uint32_t *>(st_idx));
+                                   reinterpret_cast<uint32_t *>(st_idx), s_hist);
       }
     }
   }
@@ -584,7 +640,7 @@ int select_compact(const SelectArgs &a, hipStream_t stream) {
   return a.idx64 ? select_launch<uint32_t, int64_t>(a, stream) : select_launch<uint32_t, int32_t>(a, stream);
 }
 
-// ------------------------------------------- compaction into bucket slabs
+// ------------------------------------------- compaction in no particular order
 //
 // The fused encode does not need its candidates in any order: they are sorted
 // by hash slot afterwards.  So this kernel runs as a few persistent workgroups
@@ -592,17 +648,15 @@ int select_compact(const SelectArgs &a, hipStream_t stream) {
 // (the next sub-tile is already in flight while the current one is examined),
 // needs one barrier per sub-tile (the wave totals are double buffered), and
 // stages candidates in LDS until kScatStage of them are there.  A full stage
-// is flushed: every entry's bucket (range of its level-1 hash slot) is counted
-// in LDS, a range in each bucket's slab is reserved with one atomic per bucket
-// and flush, and the entries are written there.  The candidate histogram is
-// taken at flush time.
+// is flushed to the output list with one reservation and coalesced stores; the
+// candidate histogram is taken at flush time.
 
 constexpr int kScatStage = 4096;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename S, bool ALIGNED>
-__device__ inline void scatter_load(const S *__restrict__ in, int64_t n, int64_t sub_base, uint4 (&q)[kSelVecs]) {
+__device__ inline void stage_load(const S *__restrict__ in, int64_t n, int64_t sub_base, uint4 (&q)[kSelVecs]) {
   constexpr int V = VecOf<S>::kN;
 #pragma unroll
   for (int j = 0; j < kSelVecs; ++j) {
@@ -644,53 +698,34 @@ __device__ inline uint32_t pick_elem<uint32_t>(const uint4 (&q)[kSelVecs], int o
   return pick_word(q, off);
 }
 
-// Called by the whole block after a barrier made the staged entries visible.
-// Nothing is kept in registers between the counting pass and the writing pass
-// (an entry's bucket is computed again): this runs rarely, and the streaming
-// loop around it should not pay for its registers.
+// Called by the whole block after a barrier made the staged entries visible:
+// one reservation in the output list, consecutive lanes write consecutive entries.
 template <typename S>
-__device__ __noinline__ void scatter_flush(uint32_t count, const int32_t *st_idx, const S *st_val, uint32_t *s_bcnt,
-                                           uint32_t *s_hist, uint32_t floor_key, const SlabGeom &geo,
-                                           uint32_t *cursor, int32_t *__restrict__ slab_idx,
-                                           S *__restrict__ slab_val, int32_t *status) {
-  for (uint32_t b = threadIdx.x; b < geo.nbuckets; b += kSelBlock) s_bcnt[b] = 0;
+__device__ inline void stage_flush(uint32_t count, const int32_t *st_idx, const S *st_val, uint32_t *s_base,
+                                   uint32_t *s_hist, uint32_t floor_key, uint32_t *list_count,
+                                   int32_t *__restrict__ list_idx, S *__restrict__ list_val, uint32_t capacity) {
+  if (threadIdx.x == 0) *s_base = atomicAdd(list_count, count);
   __syncthreads();
+  const uint32_t base = *s_base;
   for (uint32_t e = threadIdx.x; e < count; e += kSelBlock) {
-    const uint32_t t = (uint32_t)st_idx[e];
-    atomicAdd(&s_bcnt[geo.bucket_of((poly(t) + kSeed1) % geo.m)], 1u);
+    const S v = st_val[e];
+    if (base + e < capacity) {
+      list_idx[base + e] = st_idx[e];
+      list_val[base + e] = v;
+    }
     if (s_hist) {
-      const uint32_t bin = ((st_val[e] & KeyOf<S>::kMask) - floor_key) >> (sizeof(S) == 2 ? 0 : 16);
+      const uint32_t bin = ((v & KeyOf<S>::kMask) - floor_key) >> (sizeof(S) == 2 ? 0 : 16);
       atomicAdd(&s_hist[bin < (uint32_t)kCandBins - 1u ? bin : (uint32_t)kCandBins - 1u], 1u);
-    }
-  }
-  __syncthreads();
-  for (uint32_t b = threadIdx.x; b < geo.nbuckets; b += kSelBlock) {
-    const uint32_t c = s_bcnt[b];
-    if (c) {
-      const uint32_t base = atomicAdd(&cursor[b], c);
-      if (base + c > (uint32_t)kSlabCap) atomicOr(status, ZEN_STAT_RETRY);
-      s_bcnt[b] = base;  // from here on: the next free place in the bucket's slab
-    }
-  }
-  __syncthreads();
-  for (uint32_t e = threadIdx.x; e < count; e += kSelBlock) {
-    const uint32_t t = (uint32_t)st_idx[e];
-    const uint32_t b = geo.bucket_of((poly(t) + kSeed1) % geo.m);
-    const uint32_t pos = atomicAdd(&s_bcnt[b], 1u);
-    if (pos < (uint32_t)kSlabCap) {
-      const size_t dst = (size_t)b * kSlabCap + pos;
-      slab_idx[dst] = (int32_t)t;
-      slab_val[dst] = st_val[e];
     }
   }
   __syncthreads();
 }
 
 template <typename S, bool ALIGNED>
-__global__ __launch_bounds__(kSelBlock, 3) void k_select_scatter(
-    const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, SlabGeom geo, uint32_t *cursor,
-    int32_t *__restrict__ slab_idx, S *__restrict__ slab_val, uint32_t *ticket, int ntiles, int subs,
-    uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *thr_copy, int32_t *status) {
+__global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
+    const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, uint32_t *list_count,
+    int32_t *__restrict__ list_idx, S *__restrict__ list_val, uint32_t capacity, uint32_t *ticket, int ntiles,
+    int subs, uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *thr_copy, int32_t *status) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kSub = kSelBlock * kSelVecs * V;
   constexpr int kWaves = kSelBlock / 64;
@@ -698,7 +733,8 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_scatter(
   __shared__ int s_next[2];
   __shared__ int32_t st_idx[kScatStage];
   __shared__ S st_val[kScatStage];
-  __shared__ uint32_t s_bcnt[kSlabMaxBuckets];
+  __shared__ uint32_t s_base;
+  __shared__ uint32_t s_pick[kSelBlock / 64 + 1];
   __shared__ uint32_t s_hist[kCandBins];
   uint32_t *hist = cand_hist ? s_hist : nullptr;
   if (hist)
@@ -729,10 +765,10 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_scatter(
     __syncthreads();
     // what comes next: the following sub-tile of this tile, or the first one of the next tile
     if (sub + 1 < subs) {
-      scatter_load<S, ALIGNED>(in, n, sub_base + kSub, nxt);
+      stage_load<S, ALIGNED>(in, n, sub_base + kSub, nxt);
     } else {
       next_tile = s_next[turn & 1];
-      if (next_tile < ntiles) scatter_load<S, ALIGNED>(in, n, (int64_t)next_tile * subs * kSub, nxt);
+      if (next_tile < ntiles) stage_load<S, ALIGNED>(in, n, (int64_t)next_tile * subs * kSub, nxt);
     }
     uint32_t before = incl - cnt, total = 0;
 #pragma unroll
@@ -764,13 +800,13 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_scatter(
       done += take;
       if (count < (uint32_t)kScatStage) break;
       __syncthreads();
-      scatter_flush<S>(count, st_idx, st_val, s_bcnt, hist, floor_key, geo, cursor, slab_idx, slab_val, status);
+      stage_flush<S>(count, st_idx, st_val, &s_base, hist, floor_key, list_count, list_idx, list_val, capacity);
       count = 0;
       if (done == total) break;
     }
   };
 
-  if (tile < ntiles) scatter_load<S, ALIGNED>(in, n, (int64_t)tile * subs * kSub, qa);
+  if (tile < ntiles) stage_load<S, ALIGNED>(in, n, (int64_t)tile * subs * kSub, qa);
   while (tile < ntiles) {
     if (threadIdx.x == 0) s_next[turn & 1] = (int)gridDim.x + (int)atomicAdd(ticket, 1u);
     const int64_t tile_base = (int64_t)tile * subs * kSub;
@@ -785,25 +821,26 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_scatter(
     ++turn;
   }
   __syncthreads();
-  if (count) scatter_flush<S>(count, st_idx, st_val, s_bcnt, hist, floor_key, geo, cursor, slab_idx, slab_val, status);
+  if (count) stage_flush<S>(count, st_idx, st_val, &s_base, hist, floor_key, list_count, list_idx, list_val, capacity);
   if (hist) {
     __syncthreads();
     uint32_t *row = cand_hist + (size_t)(blockIdx.x % kCandRows) * kCandBins;
-    uint32_t landed = 0;
     for (int i = threadIdx.x; i < kCandBins; i += kSelBlock) {
       const uint32_t c = s_hist[i];
-      if (c) landed += atomicAdd(&row[i], c);
+      if (c) atomicAdd(&row[cand_place((uint32_t)i)], c);  // nothing returned: the adds are in flight together
     }
     if (pick_thr) {
-      // the block that finishes last reads the exact threshold off the complete histogram (the adds above
-      // have returned, so they are carried out before this block's count goes up)
+      // the block that finishes last reads the exact threshold off the complete histogram
       __shared__ bool s_last;
-      if (__syncthreads_or(landed == 0xffffffffu)) return;  // never true: keeps the returns alive
+      // the adds are carried out (where device-wide atomics are) before the count goes up; no device-scope
+      // fence: that would write the L2 back once per wave
+      wait_global_acks();
+      __syncthreads();
       if (threadIdx.x == 0) s_last = atomicAdd(&cand_hist[kCandRows * kCandBins], 1u) == gridDim.x - 1u;
       __syncthreads();
       if (s_last) {
         cand_pick_block<kSelBlock>(cand_hist, floor_key, pick_k, KeyOf<S>::kBits == 15 ? 0 : 16, pick_thr, status,
-                                   s_bcnt);
+                                   s_pick, s_hist);
         __syncthreads();
         if (thr_copy && threadIdx.x < 2)
           thr_copy[threadIdx.x] = __hip_atomic_load(&pick_thr[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -826,32 +863,32 @@ static int device_cus() {
 }
 
 template <typename S>
-static int scatter_launch(const ScatterArgs &a, hipStream_t stream) {
+static int stage_launch(const StageArgs &a, hipStream_t stream) {
   constexpr int V = VecOf<S>::kN;
   const int subs = select_subs(a.n, a.dtype);
   const int64_t tile = (int64_t)kSelBlock * kSelVecs * V * subs;
   const int64_t ntiles = ceil_div(a.n, tile);
-  if (ntiles > 0x3fffffff) return fail(ZEN_EINVAL, "select_scatter: too many tiles");
+  if (ntiles > 0x3fffffff) return fail(ZEN_EINVAL, "select_stage: too many tiles");
   int64_t blocks = (int64_t)device_cus() * 3;
   if (blocks > ntiles) blocks = ntiles;
   const S *in = static_cast<const S *>(a.in);
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
   ProfScope prof(kProfSelectCompact, stream);
   if (aligned)
-    k_select_scatter<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
-        in, a.n, a.thr, a.geo, a.cursor, a.slab_idx, static_cast<S *>(a.slab_val), a.ticket, (int)ntiles, subs,
-        a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
+    k_select_stage<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
+        in, a.n, a.thr, a.list_count, a.list_idx, static_cast<S *>(a.list_val), (uint32_t)a.capacity, a.ticket,
+        (int)ntiles, subs, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
   else
-    k_select_scatter<S, false><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
-        in, a.n, a.thr, a.geo, a.cursor, a.slab_idx, static_cast<S *>(a.slab_val), a.ticket, (int)ntiles, subs,
-        a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
-  ZEN_LAUNCH_CHECK("k_select_scatter");
+    k_select_stage<S, false><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
+        in, a.n, a.thr, a.list_count, a.list_idx, static_cast<S *>(a.list_val), (uint32_t)a.capacity, a.ticket,
+        (int)ntiles, subs, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
+  ZEN_LAUNCH_CHECK("k_select_stage");
   return ZEN_OK;
 }
 
-int select_scatter(const ScatterArgs &a, hipStream_t stream) {
-  if (a.dtype == ZEN_BF16) return scatter_launch<uint16_t>(a, stream);
-  return scatter_launch<uint32_t>(a, stream);
+int select_stage_list(const StageArgs &a, hipStream_t stream) {
+  if (a.dtype == ZEN_BF16) return stage_launch<uint16_t>(a, stream);
+  return stage_launch<uint32_t>(a, stream);
 }
 
 namespace {
@@ -908,22 +945,27 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
   const double want = expect + 6.0 * sqrt(expect) + 16.0;
   const uint32_t rank = want > 4.0e9 ? 0xffffffffu : (uint32_t)want;
   if (!is_zero) {
-    launch_fill<uint32_t>(hist, 0u, kFineBins + 1, stream);
+    launch_fill<uint32_t>(hist, 0u, kFineBins + 2, stream);
     ZEN_LAUNCH_CHECK("sample: clear histogram");
   }
   // every block must see fewer than 65536 sample elements (16-bit LDS counters)
   int64_t blocks = ceil_div(nblocks * V, 32768);
   if (blocks < 128) blocks = 128;
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+  const bool fused = getenv("ZSPLIT") == nullptr;
   {
     ProfScope prof(kProfTopkHist, stream);
     if (aligned)
       k_sample_hist<S, true><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist, rank,
-                                                                                        thr_lo);
+                                                                                        thr_lo, fused);
     else
       k_sample_hist<S, false><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist,
-                                                                                         rank, thr_lo);
+                                                                                         rank, thr_lo, fused);
     ZEN_LAUNCH_CHECK("k_sample_hist");
+    if (!fused) {
+      k_sample_pick<<<dim3(1), dim3(kSampleBlock), 0, stream>>>(hist, rank, KeyOf<S>::kBits - 15, thr_lo);
+      ZEN_LAUNCH_CHECK("k_sample_pick");
+    }
   }
   return ZEN_OK;
 }
@@ -949,7 +991,7 @@ int compress_launch(const S *in, int64_t n, const uint32_t *thr, S *out, hipStre
 
 size_t topk_scratch_bytes() {
   const size_t exact = align_up(sizeof(TopkState), 256) + align_up(kHistBins * sizeof(uint32_t), 256);
-  const size_t sampled = align_up((kFineBins + 1) * sizeof(uint32_t), 256);
+  const size_t sampled = align_up((kFineBins + 2) * sizeof(uint32_t), 256);
   return exact > sampled ? exact : sampled;
 }
 
@@ -967,7 +1009,7 @@ int topk_sampled_floor(const void *in, int dtype, int64_t n, int64_t k, uint32_t
   return sample_launch(static_cast<const uint32_t *>(in), n, k, thr_lo, scratch, stream, scratch_is_zero);
 }
 
-size_t sampled_floor_zero_bytes() { return (kFineBins + 1) * sizeof(uint32_t); }
+size_t sampled_floor_zero_bytes() { return (kFineBins + 2) * sizeof(uint32_t); }
 
 }  // namespace zen
 

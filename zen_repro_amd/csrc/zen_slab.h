@@ -12,6 +12,8 @@
 // back to the general (radix sort) path.
 #pragma once
 
+#include <math.h>
+
 #include "zen_common.h"
 
 namespace zen {
@@ -37,10 +39,31 @@ struct SlabGeom {
   uint32_t bpp_mult;  // floor(bpp * 2^32 / npp)
   uint32_t nbuckets;  // partitions * bpp
   uint32_t sub_mult;  // floor(kSlabSubs * 2^32 / (widest bucket + 1)): key offset inside a bucket -> narrow range
+  float inv_m;        // (1 / m)(1 - 2^-20), rounded down
+  float inv_npp;      // the same for npp
 
+  // x / d for x < 2^32 and quotients below 2^11, without the long integer division sequence.  `inv` is
+  // (1 / d)(1 - 2^-20): the two roundings of the float estimate (each at most 2^-24, relative) cannot lift it
+  // above x / d, and it falls short by less than 2^11 * 2^-19: it is the quotient or one less.
+  __device__ static inline uint32_t div_small(uint32_t x, uint32_t d, float inv, uint32_t *rem) {
+    uint32_t q = (uint32_t)((float)x * inv);
+    uint32_t r = x - q * d;
+    if (r >= d) {
+      r -= d;
+      ++q;
+    }
+    *rem = r;
+    return q;
+  }
+  __device__ inline uint32_t mod_m(uint32_t h) const {  // h % m
+    uint32_t r;
+    div_small(h, m, inv_m, &r);
+    return r;
+  }
   __device__ inline uint32_t bucket_of(uint32_t key) const {
-    const uint32_t part = key / npp;
-    return part * bpp + __umulhi(key - part * npp, bpp_mult);
+    uint32_t local;
+    const uint32_t part = div_small(key, npp, inv_npp, &local);
+    return part * bpp + __umulhi(local, bpp_mult);
   }
   __device__ inline uint32_t first_key(uint32_t b) const {  // smallest key of bucket b
     const uint32_t part = b / bpp, sb = b - part * bpp;
@@ -52,6 +75,13 @@ struct SlabGeom {
 // Host side: geometry for `partitions` partitions of a key space of m keys (m a
 // multiple of partitions) expected to hold about `expected` records.  Returns
 // false if the slab layout does not suit these sizes.
+inline float slab_inverse_below(uint32_t d) {
+  const double want = (1.0 / (double)d) * (1.0 - 1.0 / 1048576.0);
+  float f = (float)want;
+  while ((double)f > want) f = nextafterf(f, 0.0f);
+  return f;
+}
+
 inline bool slab_geometry(int64_t m, int partitions, int64_t expected, int target, SlabGeom *out) {
   if (m < (1ll << 22) || m > 0x7fffffffll || partitions < 1 || partitions > kSlabMaxBuckets || m % partitions != 0 ||
       expected < 1)
@@ -71,6 +101,8 @@ inline bool slab_geometry(int64_t m, int partitions, int64_t expected, int targe
   g.nbuckets = (uint32_t)nb;
   const uint64_t width = ((1ull << 32) + g.bpp_mult - 1) / g.bpp_mult + 1;  // keys per bucket, at most
   g.sub_mult = (uint32_t)(((uint64_t)kSlabSubs << 32) / (width + 1));
+  g.inv_m = slab_inverse_below(g.m);
+  g.inv_npp = slab_inverse_below(g.npp);
   *out = g;
   return true;
 }

@@ -3,9 +3,10 @@
 // The reference inserts every selected index into an int32 table as large as
 // the gradient and then scans that table partition by partition
 // (functions_cuda_kernel.cu:97-167, tensor_load_balance.py:13-51).  Here the
-// candidates are appended to bucket slabs by the select kernel itself (a bucket
-// is a range of level-1 hash slots, zen_slab.h), and four short kernels finish
-// the job:
+// select kernel leaves its candidates in one unordered list, and five short
+// kernels finish the job (a bucket is a range of level-1 hash slots, zen_slab.h):
+//   k_feed_*        the list, filtered by the exact threshold, goes to the bucket
+//                   slabs (count, scan, write);
 //   k_slab_sort     one workgroup per bucket: applies the exact threshold, sorts
 //                   the bucket by (level-1 slot, index) inside LDS; in a run of
 //                   equal slots the first entry (smallest index) is the slot's
@@ -28,7 +29,7 @@ namespace zen {
 namespace {
 
 struct SlabTables {
-  uint32_t *cursor;     // [B] records appended by the select kernel
+  uint32_t *cursor;     // [B] records in the bucket's slab
   uint32_t *bucket_n;   // [B] selected records, sorted, in the slab
   uint32_t *removed_n;  // [B] of which lost their level-1 slot
   uint32_t *movein_n;   // [B] entries whose final slot lies in the bucket but whose level-1 slot does not own it
@@ -45,20 +46,214 @@ struct SlabTables {
 
 __device__ inline uint32_t level1_slot(const Probe &g, uint32_t t) { return (poly(t) + kSeed1) % g.m; }
 
+// ------------------------------------------------- list -> bucket slabs
+
+constexpr int kFeedItems = 12;
+constexpr int kFeedBatch = kSlabBlock * kFeedItems;  // list entries per workgroup
+constexpr int kScanChunks = 16;
+
+// The select kernel left its candidates in one list, in no particular order.  Three kernels move them to the
+// bucket slabs without a single global atomic (a reservation per bucket and batch would be a million
+// device-wide atomics): every workgroup counts its batch of the list per bucket (k_feed_count), a scan over
+// the batches turns the counts of a bucket into the places where each batch's run starts in the bucket's slab
+// (k_feed_scan), and every workgroup orders its batch by bucket in LDS and writes the runs (k_feed_write).
+// Index 0 (never transmitted: 0 is the table's empty marker, tensor_load_balance.py:31) and whatever the exact
+// threshold excludes are dropped on the way.
+
+__device__ inline uint32_t feed_count(const uint32_t *list_count, uint32_t list_cap) {
+  const uint32_t c = *list_count;
+  return c < list_cap ? c : list_cap;
+}
+
+constexpr uint32_t kNoSlot = 0xffffffffu;  // list_key of an entry that is not selected
+
+// Counts the batch per bucket and leaves every entry's level-1 slot in list_key (kNoSlot: not selected), so
+// that nobody has to hash again.
+template <typename S>
+__global__ __launch_bounds__(kSlabBlock) void k_feed_count(SlabGeom geo, const uint32_t *__restrict__ list_count,
+                                                           uint32_t list_cap, const int32_t *__restrict__ list_idx,
+                                                           const S *__restrict__ list_val,
+                                                           const uint32_t *__restrict__ filter,
+                                                           uint32_t *__restrict__ list_key, uint32_t row_words,
+                                                           uint32_t *__restrict__ hist, int32_t *status) {
+  __shared__ uint32_t s_cnt[kSlabMaxBuckets];
+  if (*list_count > list_cap && blockIdx.x == 0 && threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);  // entries lost
+  const uint32_t count = feed_count(list_count, list_cap);
+  const uint32_t batch = blockIdx.x * (uint32_t)kFeedBatch;
+  if (batch >= count) return;
+  for (uint32_t b = threadIdx.x; b < row_words; b += kSlabBlock) s_cnt[b] = 0;
+  __syncthreads();
+  const uint32_t thr = filter ? filter[0] : 0u;
+  uint32_t t[kFeedItems];
+  S v[kFeedItems];
+#pragma unroll
+  for (int i = 0; i < kFeedItems; ++i) {
+    const uint32_t e = batch + threadIdx.x + i * kSlabBlock;
+    t[i] = 0;
+    v[i] = 0;
+    if (e < count) {
+      t[i] = (uint32_t)list_idx[e];
+      v[i] = list_val[e];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kFeedItems; ++i) {
+    const uint32_t e = batch + threadIdx.x + i * kSlabBlock;
+    uint32_t slot = kNoSlot;
+    if (t[i] != 0 && (v[i] & KeyOf<S>::kMask) >= thr) {
+      slot = geo.mod_m(poly(t[i]) + kSeed1);
+      atomicAdd(&s_cnt[geo.bucket_of(slot)], 1u);
+    }
+    if (e < count) list_key[e] = slot;
+  }
+  __syncthreads();
+  uint32_t *row = hist + (size_t)blockIdx.x * row_words;
+  for (uint32_t b = threadIdx.x; b < row_words; b += kSlabBlock) row[b] = s_cnt[b];
+}
+
+// Workgroup = 64 buckets x kScanChunks ranges of batches.  hist[batch][bucket] becomes the number of the
+// bucket's entries in earlier batches; cursor[bucket] = the bucket's total.
+__global__ __launch_bounds__(64 * kScanChunks) void k_feed_scan(const uint32_t *__restrict__ list_count,
+                                                                uint32_t list_cap, uint32_t nbuckets,
+                                                                uint32_t row_words, uint32_t *__restrict__ hist,
+                                                                uint32_t *__restrict__ cursor, int32_t *status) {
+  __shared__ uint32_t s_sum[kScanChunks][64];
+  const uint32_t count = feed_count(list_count, list_cap);
+  const uint32_t batches = (count + kFeedBatch - 1) / kFeedBatch;
+  const uint32_t b = blockIdx.x * 64u + (threadIdx.x & 63u);
+  const uint32_t chunk = threadIdx.x >> 6;
+  const uint32_t per = (batches + kScanChunks - 1) / kScanChunks;
+  const uint32_t r0 = chunk * per < batches ? chunk * per : batches;
+  const uint32_t r1 = r0 + per < batches ? r0 + per : batches;
+  uint32_t sum = 0;
+  if (b < row_words)
+    for (uint32_t r = r0; r < r1; ++r) sum += hist[(size_t)r * row_words + b];
+  s_sum[chunk][threadIdx.x & 63u] = sum;
+  __syncthreads();
+  uint32_t running = 0, total = 0;
+#pragma unroll
+  for (int c = 0; c < kScanChunks; ++c) {
+    const uint32_t x = s_sum[c][threadIdx.x & 63u];
+    if ((uint32_t)c < chunk) running += x;
+    total += x;
+  }
+  if (b < row_words)
+    for (uint32_t r = r0; r < r1; ++r) {
+      const uint32_t x = hist[(size_t)r * row_words + b];
+      hist[(size_t)r * row_words + b] = running;
+      running += x;
+    }
+  if (chunk == 0 && b < nbuckets) {
+    cursor[b] = total;
+    if (total > (uint32_t)kSlabCap) atomicOr(status, ZEN_STAT_RETRY);
+  }
+}
+
+template <typename S>
+__global__ __launch_bounds__(kSlabBlock) void k_feed_write(SlabGeom geo, SlabTables tb,
+                                                           const uint32_t *__restrict__ list_count, uint32_t list_cap,
+                                                           const int32_t *__restrict__ list_idx,
+                                                           const S *__restrict__ list_val,
+                                                           const uint32_t *__restrict__ list_key, uint32_t row_words,
+                                                           const uint32_t *__restrict__ hist) {
+  __shared__ uint32_t s_cnt[kSlabMaxBuckets];     // entries of the batch per bucket, then where the bucket's run
+                                                  // starts in the slab minus where it starts in the batch
+  __shared__ uint32_t s_start[kSlabMaxBuckets];   // where the bucket's run starts in the ordered batch
+  __shared__ uint32_t s_t[kFeedBatch];
+  __shared__ uint32_t s_k[kFeedBatch];
+  __shared__ S s_v[kFeedBatch];
+  __shared__ uint16_t s_b[kFeedBatch];
+  __shared__ uint32_t s_scan[kSlabBlock / 64 + 1];
+  const uint32_t count = feed_count(list_count, list_cap);
+  const uint32_t batch = blockIdx.x * (uint32_t)kFeedBatch;
+  if (batch >= count) return;
+  S *slab_val = static_cast<S *>(tb.slab_val);
+  for (uint32_t b = threadIdx.x; b < (uint32_t)kSlabMaxBuckets; b += kSlabBlock) s_cnt[b] = 0;
+  __syncthreads();
+  uint32_t t[kFeedItems], key[kFeedItems], bucket[kFeedItems], rank[kFeedItems];
+  S v[kFeedItems];
+#pragma unroll
+  for (int i = 0; i < kFeedItems; ++i) {
+    const uint32_t e = batch + threadIdx.x + i * kSlabBlock;
+    t[i] = 0;
+    v[i] = 0;
+    key[i] = kNoSlot;
+    if (e < count) {
+      key[i] = list_key[e];
+      t[i] = (uint32_t)list_idx[e];
+      v[i] = list_val[e];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kFeedItems; ++i) {
+    bucket[i] = rank[i] = 0;
+    if (key[i] != kNoSlot) {
+      bucket[i] = geo.bucket_of(key[i]);
+      rank[i] = atomicAdd(&s_cnt[bucket[i]], 1u);
+    }
+  }
+  __syncthreads();
+  uint32_t batch_live;
+  {
+    // thread owns kPer consecutive buckets: where their runs start in the ordered batch and in the slabs
+    constexpr int kPer = kSlabMaxBuckets / kSlabBlock;
+    const uint32_t *row = hist + (size_t)blockIdx.x * row_words;
+    uint32_t c[kPer], base[kPer];
+    uint32_t sum = 0;
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) {
+      const uint32_t b = threadIdx.x * kPer + e;
+      c[e] = s_cnt[b];
+      base[e] = b < row_words ? row[b] : 0u;
+      sum += c[e];
+    }
+    uint32_t running = block_exclusive_scan<uint32_t, kSlabBlock>(sum, s_scan, &batch_live);
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) {
+      const uint32_t b = threadIdx.x * kPer + e;
+      s_start[b] = running;
+      s_cnt[b] = base[e] - running;  // slab position = this + position in the ordered batch (mod 2^32)
+      running += c[e];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kFeedItems; ++i) {
+    if (key[i] != kNoSlot) {
+      const uint32_t p = s_start[bucket[i]] + rank[i];
+      s_t[p] = t[i];
+      s_k[p] = key[i];
+      s_v[p] = v[i];
+      s_b[p] = (uint16_t)bucket[i];
+    }
+  }
+  __syncthreads();
+  // consecutive lanes write consecutive places of a run
+  for (uint32_t e = threadIdx.x; e < batch_live; e += kSlabBlock) {
+    const uint32_t b = s_b[e];
+    const uint32_t pos = s_cnt[b] + e;
+    if (pos < (uint32_t)kSlabCap) {  // a slab that overflows was flagged by the scan
+      const size_t dst = (size_t)b * kSlabCap + pos;
+      tb.slab_idx[dst] = (int32_t)s_t[e];
+      tb.slab_key[dst] = s_k[e];
+      slab_val[dst] = s_v[e];
+    }
+  }
+}
+
 // ------------------------------------------------------------ sort a bucket
 
 template <typename S>
-__global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, Probe g, SlabTables tb,
-                                                          const uint32_t *__restrict__ filter,
-                                                          const S *__restrict__ dense, int32_t *status) {
+__global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTables tb, const S *__restrict__ dense,
+                                                          int32_t *status) {
   __shared__ SlabSortShared sh;
+  __shared__ S s_val[kSlabCap];
   __shared__ uint32_t s_lost, s_base;
   const uint32_t b = blockIdx.x;
   const size_t base = (size_t)b * kSlabCap;
   uint32_t n_raw = tb.cursor[b];
-  if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the select kernel flagged the overflow
+  if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the scan flagged the overflow
   const uint32_t lo = geo.first_key(b);
-  const uint32_t thr = filter ? filter[0] : 0u;
   S *slab_val = static_cast<S *>(tb.slab_val);
   if (threadIdx.x == 0) s_lost = 0;
   uint32_t off[kSlabItems], idx[kSlabItems], rank[kSlabItems];
@@ -70,16 +265,9 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, Probe g,
     off[i] = idx[i] = 0;
     val[i] = 0;
     if (j < n_raw) {
+      off[i] = tb.slab_key[base + j] - lo;
       idx[i] = (uint32_t)tb.slab_idx[base + j];
       val[i] = slab_val[base + j];
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < kSlabItems; ++i) {
-    const uint32_t j = threadIdx.x + i * kSlabBlock;
-    // index 0 is never transmitted (0 is the table's empty marker, tensor_load_balance.py:31)
-    if (j < n_raw && idx[i] != 0 && (val[i] & KeyOf<S>::kMask) >= thr) {
-      off[i] = level1_slot(g, idx[i]) - lo;
       live |= 1u << i;
     }
   }
@@ -97,7 +285,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, Probe g,
     if (live & (1u << i)) {
       sh.key[rank[i]] = off[i];
       sh.tie[rank[i]] = idx[i];
-      slab_val[base + rank[i]] = val[i];  // every thread has read its records: in place is safe
+      s_val[rank[i]] = val[i];
     }
   }
   __syncthreads();
@@ -109,6 +297,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, Probe g,
     const bool lost = p > 0 && sh.key[p - 1] == k;
     tb.slab_key[base + p] = k + lo;
     tb.slab_idx[base + p] = (int32_t)(sh.tie[p] | (lost ? kRemovedBit : 0u));
+    slab_val[base + p] = s_val[p];  // every thread has read its records: in place is safe
     if (lost) {
       const uint32_t at = atomicAdd(&s_lost, 1u);
       if (at < (uint32_t)kSlabSubs) sh.cnt[at] = p;
@@ -469,6 +658,13 @@ struct SlabPlan {
   uint32_t *sample_hist;  // sampled floor histogram (+ finished-block count)
   uint32_t *cand_hist;
   uint32_t *ticket;
+  uint32_t *list_count;   // candidates the select kernel found
+  int32_t *list_idx;      // [list_cap] the candidates, in no particular order
+  void *list_val;
+  uint32_t *list_key;     // [list_cap] level-1 slot of every selected candidate
+  uint32_t list_cap;
+  uint32_t *feed_hist;    // [batches of the list][row_words] per-batch bucket counts, then run starts
+  uint32_t row_words;
   uint32_t *thr;          // [0..1] exact threshold + count, [2..3] sampled floor
   void *zero_begin;
   size_t zero_bytes;
@@ -484,12 +680,19 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.sample_hist = cv.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
   p.cand_hist = cv.take<uint32_t>((size_t)kCandHistWords);
   p.ticket = cv.take<uint32_t>(4);
+  p.list_count = cv.take<uint32_t>(4);
   p.tb.cursor = cv.take<uint32_t>(B);
   p.tb.movein_n = cv.take<uint32_t>(B);
   p.tb.serial_n = cv.take<uint32_t>((size_t)partitions);
   p.tb.ctr = cv.take<Counters>(1);
   p.zero_bytes = (size_t)(cv.base + cv.used - static_cast<char *>(p.zero_begin));
   p.thr = cv.take<uint32_t>(4);
+  p.list_cap = (uint32_t)list_cap;
+  p.list_idx = cv.take<int32_t>((size_t)list_cap);
+  p.list_val = cv.take<char>((size_t)list_cap * (dtype == ZEN_BF16 ? 2 : 4));
+  p.list_key = cv.take<uint32_t>((size_t)list_cap);
+  p.row_words = (uint32_t)((B + 63) / 64 * 64);
+  p.feed_hist = cv.take<uint32_t>((size_t)ceil_div(list_cap, kFeedBatch) * p.row_words);
   p.tb.bucket_n = cv.take<uint32_t>(B);
   p.tb.removed_n = cv.take<uint32_t>(B);
   p.tb.slab_idx = cv.take<int32_t>(B * kSlabCap);
@@ -514,7 +717,18 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
   const S *dense = static_cast<const S *>(a.input);
   {
     ProfScope prof(kProfInsertList, s);
-    k_slab_sort<S><<<dim3(B), dim3(kSlabBlock), 0, s>>>(geo, a.g, p.tb, filter, dense, a.status);
+    const unsigned batches = (unsigned)ceil_div((int64_t)p.list_cap, kFeedBatch);
+    const S *list_val = static_cast<const S *>(p.list_val);
+    k_feed_count<S><<<dim3(batches), dim3(kSlabBlock), 0, s>>>(geo, p.list_count, p.list_cap, p.list_idx, list_val,
+                                                                filter, p.list_key, p.row_words, p.feed_hist, a.status);
+    ZEN_LAUNCH_CHECK("k_feed_count");
+    k_feed_scan<<<dim3(p.row_words / 64), dim3(64 * kScanChunks), 0, s>>>(p.list_count, p.list_cap, B, p.row_words,
+                                                                           p.feed_hist, p.tb.cursor, a.status);
+    ZEN_LAUNCH_CHECK("k_feed_scan");
+    k_feed_write<S><<<dim3(batches), dim3(kSlabBlock), 0, s>>>(geo, p.tb, p.list_count, p.list_cap, p.list_idx,
+                                                                list_val, p.list_key, p.row_words, p.feed_hist);
+    ZEN_LAUNCH_CHECK("k_feed_write");
+    k_slab_sort<S><<<dim3(B), dim3(kSlabBlock), 0, s>>>(geo, p.tb, dense, a.status);
     ZEN_LAUNCH_CHECK("k_slab_sort");
   }
   {
@@ -559,15 +773,15 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
   const SlabPlan p = plan_slab(a.workspace, geo, a.partitions, a.dtype, list_capacity(a.capacity));
   launch_fill<uint32_t>(static_cast<uint32_t *>(p.zero_begin), 0u, p.zero_bytes / sizeof(uint32_t), s);
   ZEN_LAUNCH_CHECK("slab: clear counters");
-  ScatterArgs sc;
+  StageArgs sc;
   sc.in = a.input;
   sc.dtype = a.dtype;
   sc.n = a.n;
   sc.thr = a.thr;
-  sc.geo = geo;
-  sc.cursor = p.tb.cursor;
-  sc.slab_idx = p.tb.slab_idx;
-  sc.slab_val = p.tb.slab_val;
+  sc.list_count = p.list_count;
+  sc.list_idx = p.list_idx;
+  sc.list_val = p.list_val;
+  sc.capacity = p.list_cap;
   sc.ticket = p.ticket;
   sc.status = a.status;
   int rc;
@@ -581,7 +795,7 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
     sc.pick_thr = p.thr;
     sc.thr_copy = a.thr_out;
   }
-  if ((rc = select_scatter(sc, s)) != ZEN_OK) return rc;
+  if ((rc = select_stage_list(sc, s)) != ZEN_OK) return rc;
   if (a.dtype == ZEN_BF16) return slab_launch<uint16_t>(a, geo, p, s);
   return slab_launch<uint32_t>(a, geo, p, s);
 }
