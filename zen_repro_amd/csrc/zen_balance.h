@@ -50,6 +50,15 @@ __device__ inline uint32_t lower_bound_u32(const uint32_t *a, uint32_t n, uint32
 }
 
 
+__device__ inline uint32_t upper_bound_u32(const uint32_t *a, uint32_t n, uint32_t x) {  // entries <= x
+  uint32_t lo = 0, hi = n;
+  while (lo < hi) {
+    const uint32_t mid = lo + ((hi - lo) >> 1);
+    if (a[mid] <= x) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
 // Room for the candidates of a sampled top-k (the selected plus those between
 // the sampled floor and the exact threshold).
 inline int64_t list_capacity(int64_t capacity) { return capacity + capacity / 2 + 4096; }

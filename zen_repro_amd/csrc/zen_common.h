@@ -146,6 +146,12 @@ __device__ inline uint16_t f32_to_bf16_rne(float f) {
 // included, have been acknowledged by the place that carries them out.
 __device__ inline void wait_global_acks() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// Reads a word that other workgroups of the running kernel have changed with device-wide atomics, from the
+// place where those are carried out (not from this compute unit's caches).
+__device__ inline uint32_t load_fresh(const uint32_t *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ inline int lane_id() { return int(__lane_id()); }
 
 __device__ inline uint64_t lanes_below() {  // mask of lanes with a smaller id

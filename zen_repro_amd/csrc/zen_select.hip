@@ -137,9 +137,6 @@ __device__ inline uint32_t fine_place(uint32_t bin) { return ((bin & 63u) << 9) 
 // Run by one whole block once the histogram is complete: the lowest fine bin b
 // such that `rank` sample elements lie in bins >= b; floor_out[0] = lowest key
 // of that bin (0 if the sample is too small).
-__device__ inline uint32_t load_fresh(const uint32_t *p) {  // written by other blocks' atomics: read at L2
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 // Walks down from the highest populated bin (hist[kFineBins + 1]) in windows of one bin per thread, with
 // consecutive lanes on consecutive words (one workgroup fetching 32768 scattered words past the caches would

@@ -107,6 +107,13 @@ inline bool slab_geometry(int64_t m, int partitions, int64_t expected, int targe
   return true;
 }
 
+// Where the counter of narrow range s lives in SlabSortShared::cnt: a thread owns kSlabSubsPer consecutive
+// ranges during the prefix step, and this keeps the lanes of a wave on different LDS banks while they walk
+// through their ranges.  Range kSlabSubs (the end marker) stays at index kSlabSubs.
+__device__ inline uint32_t sub_place(uint32_t s) {
+  return s < (uint32_t)kSlabSubs ? (s % kSlabSubsPer) * kSlabBlock + s / kSlabSubsPer : s;
+}
+
 // Shared memory of the in-LDS sort.
 struct SlabSortShared {
   uint32_t key[kSlabCap];
@@ -134,7 +141,7 @@ __device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, const 
     sub[i] = at[i] = 0;
     if (live & (1u << i)) {
       sub[i] = geo.sub_of(off[i]);
-      at[i] = atomicAdd(&sh.cnt[sub[i]], 1u);
+      at[i] = atomicAdd(&sh.cnt[sub_place(sub[i])], 1u);
     }
   }
   __syncthreads();
@@ -143,7 +150,7 @@ __device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, const 
     uint32_t sum = 0, big = 0;
 #pragma unroll
     for (int e = 0; e < kSlabSubsPer; ++e) {
-      c[e] = sh.cnt[threadIdx.x * kSlabSubsPer + e];
+      c[e] = sh.cnt[e * kSlabBlock + threadIdx.x];
       sum += c[e];
       big |= c[e] > (uint32_t)kSlabGroupLimit;
     }
@@ -152,7 +159,7 @@ __device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, const 
     uint32_t running = block_exclusive_scan<uint32_t, kSlabBlock>(sum, sh.scan, &total);
 #pragma unroll
     for (int e = 0; e < kSlabSubsPer; ++e) {
-      sh.cnt[threadIdx.x * kSlabSubsPer + e] = running;
+      sh.cnt[e * kSlabBlock + threadIdx.x] = running;
       running += c[e];
     }
     if (threadIdx.x == kSlabBlock - 1) sh.cnt[kSlabSubs] = running;
@@ -162,7 +169,7 @@ __device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, const 
 #pragma unroll
   for (int i = 0; i < kSlabItems; ++i) {
     if (live & (1u << i)) {
-      const uint32_t p = sh.cnt[sub[i]] + at[i];
+      const uint32_t p = sh.cnt[sub_place(sub[i])] + at[i];
       sh.key[p] = off[i];
       sh.tie[p] = tie[i];
     }
@@ -172,7 +179,7 @@ __device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, const 
   for (int i = 0; i < kSlabItems; ++i) {
     rank[i] = 0;
     if (live & (1u << i)) {
-      const uint32_t g0 = sh.cnt[sub[i]], g1 = sh.cnt[sub[i] + 1];
+      const uint32_t g0 = sh.cnt[sub_place(sub[i])], g1 = sh.cnt[sub_place(sub[i] + 1)];
       uint32_t less = 0;
       for (uint32_t u = g0; u < g1; ++u) {
         const uint32_t ku = sh.key[u];

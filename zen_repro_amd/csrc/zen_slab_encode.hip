@@ -30,16 +30,20 @@ namespace {
 
 struct SlabTables {
   uint32_t *cursor;     // [B] records in the bucket's slab
+  uint32_t *bucket_lo;  // [B] smallest level-1 slot of the bucket
   uint32_t *bucket_n;   // [B] selected records, sorted, in the slab
   uint32_t *removed_n;  // [B] of which lost their level-1 slot
   uint32_t *movein_n;   // [B] entries whose final slot lies in the bucket but whose level-1 slot does not own it
   uint32_t *serial_n;   // [P] entries that found no slot
-  int32_t *slab_idx;    // [B * kSlabCap] index (sorted: | kRemovedBit)
-  void *slab_val;       // [B * kSlabCap]
-  uint32_t *slab_key;   // [B * kSlabCap] level-1 slot, ascending inside a slab after the sort
+  uint4 *slab_rec;      // [B * kSlabCap] records as they arrive: (level-1 slot, index, value, 0)
+  int32_t *slab_idx;    // [B * kSlabCap] after the sort: index | kRemovedBit
+  void *slab_val;       // [B * kSlabCap] after the sort: value
+  uint32_t *slab_key;   // [B * kSlabCap] after the sort: level-1 slot, ascending inside a slab
   uint32_t *mv_key, *mv_idx, *mv_val;  // [B * kSlabMoveCap]
   uint32_t *ser_idx;    // [P * kSlabSerialCap]
   uint32_t *log_t, *log_v, *log_cell;  // [log_cap]
+  uint32_t *out_start;  // [B + 1] where every bucket starts in the output
+  uint32_t *done;       // [1] workgroups of k_slab_classify that have finished
   Counters *ctr;
   uint32_t log_cap;
 };
@@ -48,9 +52,9 @@ __device__ inline uint32_t level1_slot(const Probe &g, uint32_t t) { return (pol
 
 // ------------------------------------------------- list -> bucket slabs
 
-constexpr int kFeedItems = 12;
+constexpr int kFeedItems = 8;
 constexpr int kFeedBatch = kSlabBlock * kFeedItems;  // list entries per workgroup
-constexpr int kScanChunks = 16;
+constexpr int kScanChunks = 64;
 
 // The select kernel left its candidates in one list, in no particular order.  Three kernels move them to the
 // bucket slabs without a single global atomic (a reservation per bucket and batch would be a million
@@ -111,29 +115,32 @@ __global__ __launch_bounds__(kSlabBlock) void k_feed_count(SlabGeom geo, const u
   for (uint32_t b = threadIdx.x; b < row_words; b += kSlabBlock) row[b] = s_cnt[b];
 }
 
-// Workgroup = 64 buckets x kScanChunks ranges of batches.  hist[batch][bucket] becomes the number of the
+// Workgroup = kScanCols buckets x kScanChunks ranges of batches.  hist[batch][bucket] becomes the number of the
 // bucket's entries in earlier batches; cursor[bucket] = the bucket's total.
-__global__ __launch_bounds__(64 * kScanChunks) void k_feed_scan(const uint32_t *__restrict__ list_count,
-                                                                uint32_t list_cap, uint32_t nbuckets,
-                                                                uint32_t row_words, uint32_t *__restrict__ hist,
-                                                                uint32_t *__restrict__ cursor, int32_t *status) {
-  __shared__ uint32_t s_sum[kScanChunks][64];
+constexpr int kScanCols = 16;
+__global__ __launch_bounds__(kScanCols * kScanChunks) void k_feed_scan(SlabGeom geo,
+                                                                       const uint32_t *__restrict__ list_count,
+                                                                       uint32_t list_cap, uint32_t nbuckets,
+                                                                       uint32_t row_words, uint32_t *__restrict__ hist,
+                                                                       uint32_t *__restrict__ cursor,
+                                                                       uint32_t *__restrict__ bucket_lo,
+                                                                       int32_t *status) {
+  __shared__ uint32_t s_sum[kScanChunks][kScanCols];
   const uint32_t count = feed_count(list_count, list_cap);
   const uint32_t batches = (count + kFeedBatch - 1) / kFeedBatch;
-  const uint32_t b = blockIdx.x * 64u + (threadIdx.x & 63u);
-  const uint32_t chunk = threadIdx.x >> 6;
+  const uint32_t col = threadIdx.x % kScanCols, chunk = threadIdx.x / kScanCols;
+  const uint32_t b = blockIdx.x * kScanCols + col;
   const uint32_t per = (batches + kScanChunks - 1) / kScanChunks;
   const uint32_t r0 = chunk * per < batches ? chunk * per : batches;
   const uint32_t r1 = r0 + per < batches ? r0 + per : batches;
   uint32_t sum = 0;
   if (b < row_words)
     for (uint32_t r = r0; r < r1; ++r) sum += hist[(size_t)r * row_words + b];
-  s_sum[chunk][threadIdx.x & 63u] = sum;
+  s_sum[chunk][col] = sum;
   __syncthreads();
   uint32_t running = 0, total = 0;
-#pragma unroll
   for (int c = 0; c < kScanChunks; ++c) {
-    const uint32_t x = s_sum[c][threadIdx.x & 63u];
+    const uint32_t x = s_sum[c][col];
     if ((uint32_t)c < chunk) running += x;
     total += x;
   }
@@ -145,10 +152,15 @@ __global__ __launch_bounds__(64 * kScanChunks) void k_feed_scan(const uint32_t *
     }
   if (chunk == 0 && b < nbuckets) {
     cursor[b] = total;
+    bucket_lo[b] = geo.first_key(b);  // a 64-bit division: once per bucket here, not once per thread later
     if (total > (uint32_t)kSlabCap) atomicOr(status, ZEN_STAT_RETRY);
   }
 }
 
+// Every selected entry of the batch goes to its bucket's slab as one 16-byte record.  Scattered stores cost
+// one memory request each whatever their size (about 80 G requests/s on this part), so the batch is first
+// ordered by bucket in LDS: the records of a bucket then leave as one run, a few requests instead of one per
+// record.  A run's place in the slab comes from the scan.
 template <typename S>
 __global__ __launch_bounds__(kSlabBlock) void k_feed_write(SlabGeom geo, SlabTables tb,
                                                            const uint32_t *__restrict__ list_count, uint32_t list_cap,
@@ -156,19 +168,27 @@ __global__ __launch_bounds__(kSlabBlock) void k_feed_write(SlabGeom geo, SlabTab
                                                            const S *__restrict__ list_val,
                                                            const uint32_t *__restrict__ list_key, uint32_t row_words,
                                                            const uint32_t *__restrict__ hist) {
-  __shared__ uint32_t s_cnt[kSlabMaxBuckets];     // entries of the batch per bucket, then where the bucket's run
-                                                  // starts in the slab minus where it starts in the batch
-  __shared__ uint32_t s_start[kSlabMaxBuckets];   // where the bucket's run starts in the ordered batch
-  __shared__ uint32_t s_t[kFeedBatch];
-  __shared__ uint32_t s_k[kFeedBatch];
-  __shared__ S s_v[kFeedBatch];
-  __shared__ uint16_t s_b[kFeedBatch];
+  // entries of the batch per bucket; then (where the bucket's run starts in the ordered batch) << 13 | (where it
+  // starts in the slab).  One array, so that two workgroups fit into a compute unit's LDS.
+  __shared__ uint32_t s_cnt[kSlabMaxBuckets];
+  __shared__ uint4 s_rec[kFeedBatch];  // the ordered batch; .w = bucket << 13 | place in the slab
   __shared__ uint32_t s_scan[kSlabBlock / 64 + 1];
+  static_assert(kSlabCap <= (1 << 13) && kFeedBatch < (1 << 13) && kSlabMaxBuckets <= (1 << 11), "packed fields");
   const uint32_t count = feed_count(list_count, list_cap);
   const uint32_t batch = blockIdx.x * (uint32_t)kFeedBatch;
   if (batch >= count) return;
-  S *slab_val = static_cast<S *>(tb.slab_val);
   for (uint32_t b = threadIdx.x; b < (uint32_t)kSlabMaxBuckets; b += kSlabBlock) s_cnt[b] = 0;
+  // where the runs of this thread's buckets start in the slabs: asked for now, needed after the counting
+  constexpr int kPer = kSlabMaxBuckets / kSlabBlock;
+  uint32_t base[kPer];
+  {
+    const uint32_t *row = hist + (size_t)blockIdx.x * row_words;
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) {
+      const uint32_t b = threadIdx.x * kPer + e;
+      base[e] = b < row_words ? row[b] : 0u;
+    }
+  }
   __syncthreads();
   uint32_t t[kFeedItems], key[kFeedItems], bucket[kFeedItems], rank[kFeedItems];
   S v[kFeedItems];
@@ -195,24 +215,20 @@ __global__ __launch_bounds__(kSlabBlock) void k_feed_write(SlabGeom geo, SlabTab
   __syncthreads();
   uint32_t batch_live;
   {
-    // thread owns kPer consecutive buckets: where their runs start in the ordered batch and in the slabs
-    constexpr int kPer = kSlabMaxBuckets / kSlabBlock;
-    const uint32_t *row = hist + (size_t)blockIdx.x * row_words;
-    uint32_t c[kPer], base[kPer];
+    // thread owns kPer consecutive buckets: one exclusive prefix over the buckets gives every bucket's run a
+    // place in the ordered batch
+    uint32_t c[kPer];
     uint32_t sum = 0;
 #pragma unroll
     for (int e = 0; e < kPer; ++e) {
-      const uint32_t b = threadIdx.x * kPer + e;
-      c[e] = s_cnt[b];
-      base[e] = b < row_words ? row[b] : 0u;
+      c[e] = s_cnt[threadIdx.x * kPer + e];
       sum += c[e];
     }
     uint32_t running = block_exclusive_scan<uint32_t, kSlabBlock>(sum, s_scan, &batch_live);
 #pragma unroll
     for (int e = 0; e < kPer; ++e) {
-      const uint32_t b = threadIdx.x * kPer + e;
-      s_start[b] = running;
-      s_cnt[b] = base[e] - running;  // slab position = this + position in the ordered batch (mod 2^32)
+      // a run that starts past the slab's end (overflow, flagged by the scan) is clipped to the end
+      s_cnt[threadIdx.x * kPer + e] = (running << 13) | (base[e] < (uint32_t)kSlabCap ? base[e] : (uint32_t)kSlabCap);
       running += c[e];
     }
   }
@@ -220,24 +236,19 @@ __global__ __launch_bounds__(kSlabBlock) void k_feed_write(SlabGeom geo, SlabTab
 #pragma unroll
   for (int i = 0; i < kFeedItems; ++i) {
     if (key[i] != kNoSlot) {
-      const uint32_t p = s_start[bucket[i]] + rank[i];
-      s_t[p] = t[i];
-      s_k[p] = key[i];
-      s_v[p] = v[i];
-      s_b[p] = (uint16_t)bucket[i];
+      const uint32_t sb = s_cnt[bucket[i]];
+      uint32_t pos = (sb & 8191u) + rank[i];
+      if (pos > 8191u) pos = 8191u;  // beyond the slab anyway: dropped below, must not spill into the bucket field
+      s_rec[(sb >> 13) + rank[i]] = make_uint4(key[i], t[i], (uint32_t)v[i], (bucket[i] << 13) | pos);
     }
   }
   __syncthreads();
-  // consecutive lanes write consecutive places of a run
+  // consecutive lanes write consecutive records of a run
   for (uint32_t e = threadIdx.x; e < batch_live; e += kSlabBlock) {
-    const uint32_t b = s_b[e];
-    const uint32_t pos = s_cnt[b] + e;
-    if (pos < (uint32_t)kSlabCap) {  // a slab that overflows was flagged by the scan
-      const size_t dst = (size_t)b * kSlabCap + pos;
-      tb.slab_idx[dst] = (int32_t)s_t[e];
-      tb.slab_key[dst] = s_k[e];
-      slab_val[dst] = s_v[e];
-    }
+    uint4 rec = s_rec[e];
+    const uint32_t b = rec.w >> 13, pos = rec.w & 8191u;
+    rec.w = 0;
+    if (pos < (uint32_t)kSlabCap) tb.slab_rec[(size_t)b * kSlabCap + pos] = rec;
   }
 }
 
@@ -253,7 +264,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
   const size_t base = (size_t)b * kSlabCap;
   uint32_t n_raw = tb.cursor[b];
   if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the scan flagged the overflow
-  const uint32_t lo = geo.first_key(b);
+  const uint32_t lo = tb.bucket_lo[b];
   S *slab_val = static_cast<S *>(tb.slab_val);
   if (threadIdx.x == 0) s_lost = 0;
   uint32_t off[kSlabItems], idx[kSlabItems], rank[kSlabItems];
@@ -265,9 +276,10 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
     off[i] = idx[i] = 0;
     val[i] = 0;
     if (j < n_raw) {
-      off[i] = tb.slab_key[base + j] - lo;
-      idx[i] = (uint32_t)tb.slab_idx[base + j];
-      val[i] = slab_val[base + j];
+      const uint4 rec = tb.slab_rec[base + j];
+      off[i] = rec.x - lo;
+      idx[i] = rec.y;
+      val[i] = (S)rec.z;
       live |= 1u << i;
     }
   }
@@ -317,10 +329,10 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
   __syncthreads();
   for (uint32_t i = threadIdx.x; i < lost_n; i += kSlabBlock) {
     const uint32_t at = s_base + i;
-    const uint32_t t = sh.tie[sh.cnt[i]];
+    const uint32_t p = sh.cnt[i];
     if (at < tb.log_cap) {
-      tb.log_t[at] = t;
-      tb.log_v[at] = (uint32_t)dense[t];
+      tb.log_t[at] = sh.tie[p];
+      tb.log_v[at] = (uint32_t)s_val[p];
     } else {
       atomicOr(status, ZEN_STAT_RETRY);
     }
@@ -402,16 +414,53 @@ __global__ __launch_bounds__(256) void k_slab_chains(SlabGeom geo, Probe g, Slab
   }
 }
 
+// Where every bucket starts in the output: survivors + moved-in entries, the partition's serial entries
+// behind its last bucket.  Run by one workgroup of kSlabBlock threads once all counts are final.
+__device__ inline void slab_output_starts(const SlabGeom &geo, const SlabTables &tb, uint32_t *s_scan) {
+  constexpr int kPer = kSlabMaxBuckets / kSlabBlock;
+  const uint32_t B = geo.nbuckets;
+  uint32_t c[kPer];
+  uint32_t sum = 0;
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) {
+    const uint32_t x = threadIdx.x * kPer + e;
+    c[e] = 0;
+    if (x < B) {
+      uint32_t mv = load_fresh(&tb.movein_n[x]);
+      if (mv > (uint32_t)kSlabMoveCap) mv = kSlabMoveCap;
+      c[e] = tb.bucket_n[x] - load_fresh(&tb.removed_n[x]) + mv;
+      if (x % geo.bpp == geo.bpp - 1) {
+        uint32_t sn = load_fresh(&tb.serial_n[x / geo.bpp]);
+        if (sn > (uint32_t)kSlabSerialCap) sn = kSlabSerialCap;
+        c[e] += sn;
+      }
+    }
+    sum += c[e];
+  }
+  uint32_t total;
+  uint32_t running = block_exclusive_scan<uint32_t, kSlabBlock>(sum, s_scan, &total);
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) {
+    const uint32_t x = threadIdx.x * kPer + e;
+    if (x <= B) tb.out_start[x] = running;
+    running += c[e];
+  }
+  if (B == (uint32_t)kSlabMaxBuckets && threadIdx.x == kSlabBlock - 1) tb.out_start[B] = running;
+}
+
 // Final place of every logged entry: the level-2/3 slot it holds in the map, or its partition's serial list.
-__global__ __launch_bounds__(256) void k_slab_classify(SlabGeom geo, Probe g, SlabTables tb,
-                                                       const unsigned long long *__restrict__ cells, uint32_t log2,
-                                                       int64_t spp, int32_t *status) {
+// The workgroup that finishes last then knows every count and lays out the output.
+__global__ __launch_bounds__(kSlabBlock) void k_slab_classify(SlabGeom geo, Probe g, SlabTables tb,
+                                                              const unsigned long long *__restrict__ cells,
+                                                              uint32_t log2, int64_t spp, int32_t *status) {
+  __shared__ uint32_t s_scan[kSlabBlock / 64 + 1];
+  __shared__ bool s_last;
   const Counters *ctr = tb.ctr;
   uint32_t losers = ctr->losers;
   if (losers > tb.log_cap) losers = tb.log_cap;
   uint32_t total = losers + ctr->displaced;
   if (total > tb.log_cap) total = tb.log_cap;
-  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+  for (uint32_t i = blockIdx.x * kSlabBlock + threadIdx.x; i < total; i += gridDim.x * kSlabBlock) {
     const uint32_t t = tb.log_t[i];
     uint32_t part = 0, cell = kNone, slot = kNone;
     for (int lv = 1; lv < g.levels && slot == kNone; ++lv) {
@@ -443,26 +492,61 @@ __global__ __launch_bounds__(256) void k_slab_classify(SlabGeom geo, Probe g, Sl
         atomicOr(status, (int64_t)at >= spp ? ZEN_STAT_SERIAL_OVERFLOW : ZEN_STAT_RETRY);
     }
   }
+  // the counters above were raised with atomics that returned (movein_n, serial_n): they have been carried out
+  __syncthreads();
+  if (threadIdx.x == 0) s_last = atomicAdd(tb.done, 1u) == gridDim.x - 1u;
+  __syncthreads();
+  if (s_last) slab_output_starts(geo, tb, s_scan);
 }
 
 // ------------------------------------------------------------------ place
 
+constexpr int kPlaceRemoved = 1024;  // removed entries per bucket the place kernel keeps track of
+
+// Ranks the n (distinct) words of `a` in LDS: on return a is ascending.  Called by the whole workgroup; n is
+// small in practice (a handful), at most kSlabMoveCap.
+__device__ inline void sort_small(uint32_t *a, uint32_t n) {
+  constexpr int kPer = kSlabMoveCap / kSlabBlock;
+  uint32_t x[kPer], r[kPer];
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) {
+    const uint32_t j = threadIdx.x + e * kSlabBlock;
+    x[e] = j < n ? a[j] : 0u;
+    r[e] = 0;
+    if (j < n)
+      for (uint32_t u = 0; u < n; ++u) r[e] += a[u] < x[e];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < kPer; ++e)
+    if (threadIdx.x + e * kSlabBlock < n) a[r[e]] = x[e];
+  __syncthreads();
+}
+
+// The sorted slab of a bucket is almost its part of the output already: the entries that lost their slot
+// (a handful) drop out and the entries that moved in from elsewhere (another handful) slip in between.  So
+// an entry at sorted place p goes to
+//     bucket start + p - (removed entries before p) + (moved-in entries whose slot is smaller),
+// both counts being searches in two short sorted lists; consecutive lanes read consecutive entries and write
+// (almost) consecutive places, and nothing but the bucket's slots passes through LDS.
 template <typename S>
 __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTables tb, unsigned long long *cells,
                                                            int partitions, int64_t spp,
                                                            const S *__restrict__ dense, int32_t *__restrict__ out_idx,
                                                            S *__restrict__ out_val, uint32_t capacity,
                                                            int64_t *__restrict__ splits, int32_t *status) {
-  __shared__ uint32_t s_key[kSlabCap];   // sorted slots of the bucket; later the bucket's output indices
-  __shared__ uint32_t s_idx[kSlabCap];   // their indices (| kRemovedBit); later the output values
-  __shared__ uint32_t s_mk[kSlabMoveCap], s_mi[kSlabMoveCap], s_mv[kSlabMoveCap];
-  __shared__ uint32_t s_pref[kSlabMaxBuckets + 1];
-  __shared__ uint32_t s_tb[kSlabBlock];
-  __shared__ uint32_t s_scan[kSlabBlock / 64 + 1];
+  __shared__ uint32_t s_key[kSlabCap];                 // sorted slots of the bucket
+  __shared__ uint32_t s_mk[kSlabMoveCap];              // slots of the moved-in entries, ascending
+  __shared__ uint32_t s_mp[kSlabMoveCap];              // sorted place in front of which each of them slips in
+  __shared__ uint32_t s_rm[kPlaceRemoved];             // sorted places of the removed entries, ascending
+  __shared__ int32_t s_delta[kSlabCap / 64];           // per 64 sorted places: how far their entries move
+  __shared__ uint32_t s_nrm;
+  constexpr int32_t kNoDelta = INT32_MIN;              // the stretch has no common amount
   const uint32_t b = blockIdx.x;
   const uint32_t B = geo.nbuckets;
   const size_t base = (size_t)b * kSlabCap;
   const S *slab_val = static_cast<const S *>(tb.slab_val);
+  if (threadIdx.x == 0) s_nrm = 0;
 
   // every occupied map cell ends with the index that finally holds its slot, and that index recorded the
   // cell: clearing by cell number leaves the borrowed memory zero again
@@ -477,139 +561,106 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
     }
   }
 
-  // where every bucket starts in the output: survivors + moved-in entries, the partition's serial entries
-  // behind its last bucket
-  {
-    constexpr int kPer = kSlabMaxBuckets / kSlabBlock;
-    uint32_t c[kPer];
-    uint32_t sum = 0;
-#pragma unroll
-    for (int e = 0; e < kPer; ++e) {
-      const uint32_t x = threadIdx.x * kPer + e;
-      c[e] = 0;
-      if (x < B) {
-        uint32_t mv = tb.movein_n[x];
-        if (mv > (uint32_t)kSlabMoveCap) mv = kSlabMoveCap;
-        c[e] = tb.bucket_n[x] - tb.removed_n[x] + mv;
-        if (x % geo.bpp == geo.bpp - 1) {
-          uint32_t sn = tb.serial_n[x / geo.bpp];
-          if (sn > (uint32_t)kSlabSerialCap) sn = kSlabSerialCap;
-          c[e] += sn;
-        }
-      }
-      sum += c[e];
-    }
-    uint32_t total;
-    uint32_t running = block_exclusive_scan<uint32_t, kSlabBlock>(sum, s_scan, &total);
-#pragma unroll
-    for (int e = 0; e < kPer; ++e) {
-      const uint32_t x = threadIdx.x * kPer + e;
-      if (x <= B) s_pref[x] = running;
-      running += c[e];
-    }
-    if (B == (uint32_t)kSlabMaxBuckets && threadIdx.x == kSlabBlock - 1) s_pref[B] = running;
-  }
   const uint32_t n = tb.bucket_n[b];
   uint32_t mv_n = tb.movein_n[b];
   if (mv_n > (uint32_t)kSlabMoveCap) mv_n = kSlabMoveCap;
-  for (uint32_t p = threadIdx.x; p < n; p += kSlabBlock) {
-    s_key[p] = tb.slab_key[base + p];
-    s_idx[p] = (uint32_t)tb.slab_idx[base + p];
-  }
-  // moved-in entries ordered by slot (slots are distinct: each is owned by one index)
-  uint32_t mk[kSlabMoveCap / kSlabBlock], mi[kSlabMoveCap / kSlabBlock], mvv[kSlabMoveCap / kSlabBlock];
-#pragma unroll
-  for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
-    const uint32_t j = threadIdx.x + e * kSlabBlock;
-    mk[e] = mi[e] = mvv[e] = 0;
-    if (j < mv_n) {
-      mk[e] = tb.mv_key[(size_t)b * kSlabMoveCap + j];
-      mi[e] = tb.mv_idx[(size_t)b * kSlabMoveCap + j];
-      mvv[e] = tb.mv_val[(size_t)b * kSlabMoveCap + j];
-      s_mk[j] = mk[e];
-    }
-  }
-  __syncthreads();
-  const uint32_t out_base = s_pref[b];
-  const uint32_t out_n = s_pref[b + 1] - out_base;
-  {
-    uint32_t r[kSlabMoveCap / kSlabBlock];
-#pragma unroll
-    for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
-      r[e] = 0;
-      if (threadIdx.x + e * kSlabBlock < mv_n)
-        for (uint32_t u = 0; u < mv_n; ++u) r[e] += s_mk[u] < mk[e];
-    }
-    __syncthreads();
-#pragma unroll
-    for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
-      if (threadIdx.x + e * kSlabBlock < mv_n) {
-        s_mk[r[e]] = mk[e];
-        s_mi[r[e]] = mi[e];
-        s_mv[r[e]] = mvv[e];
-      }
-    }
-  }
-  // survivors: thread t owns the sorted places [t * kSlabItems, (t + 1) * kSlabItems)
-  const uint32_t first = threadIdx.x * kSlabItems;
-  uint32_t flags = 0;
-#pragma unroll
-  for (int i = 0; i < kSlabItems; ++i)
-    if (first + i < n && !(s_idx[first + i] & kRemovedBit)) flags |= 1u << i;
-  uint32_t surv_total;
-  const uint32_t before = block_exclusive_scan<uint32_t, kSlabBlock>((uint32_t)__popc(flags), s_scan, &surv_total);
-  s_tb[threadIdx.x] = before;
-  __syncthreads();  // also: s_mk sorted
-  uint32_t place[kSlabItems], o_idx[kSlabItems];
-  S o_val[kSlabItems];
-  {
-    uint32_t run = before;
-#pragma unroll
-    for (int i = 0; i < kSlabItems; ++i) {
-      place[i] = kNone;
-      o_idx[i] = 0;
-      o_val[i] = 0;
-      if (flags & (1u << i)) {
-        place[i] = run + lower_bound_u32(s_mk, mv_n, s_key[first + i]);
-        o_idx[i] = s_idx[first + i];
-        o_val[i] = slab_val[base + first + i];
-        ++run;
-      }
-    }
-  }
-  // moved-in entry j: its rank among them plus the survivors whose slot is smaller
-  uint32_t mplace[kSlabMoveCap / kSlabBlock];
-#pragma unroll
-  for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
-    const uint32_t j = threadIdx.x + e * kSlabBlock;
-    mplace[e] = kNone;
-    if (j < mv_n) {
-      const uint32_t p0 = lower_bound_u32(s_key, n, s_mk[j]);
-      const uint32_t owner = p0 / kSlabItems;
-      uint32_t surv = owner < (uint32_t)kSlabBlock ? s_tb[owner] : surv_total;
-      for (uint32_t p = owner * kSlabItems; p < p0; ++p) surv += !(s_idx[p] & kRemovedBit);
-      mplace[e] = j + surv;
-      mi[e] = s_mi[j];
-      mvv[e] = s_mv[j];
-    }
-  }
-  __syncthreads();
-  // gather the bucket's output in LDS, then write it with consecutive lanes
+  // the thread's entries (sorted places threadIdx.x + i * kSlabBlock) stay in registers; the slots go to LDS
+  // for the searches, the places of removed entries are collected
+  uint32_t idx[kSlabItems];
+  S val[kSlabItems];
 #pragma unroll
   for (int i = 0; i < kSlabItems; ++i) {
-    if (place[i] != kNone && place[i] < (uint32_t)kSlabCap) {
-      s_key[place[i]] = o_idx[i];
-      s_idx[place[i]] = (uint32_t)o_val[i];
+    const uint32_t p = threadIdx.x + i * kSlabBlock;
+    idx[i] = kRemovedBit;
+    val[i] = 0;
+    if (p < n) {
+      s_key[p] = tb.slab_key[base + p];
+      idx[i] = (uint32_t)tb.slab_idx[base + p];
+      val[i] = slab_val[base + p];
     }
   }
+  for (uint32_t j = threadIdx.x; j < mv_n; j += kSlabBlock) s_mk[j] = tb.mv_key[(size_t)b * kSlabMoveCap + j];
+  __syncthreads();  // s_nrm is zero, s_key and s_mk are there
 #pragma unroll
-  for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
-    if (mplace[e] != kNone && mplace[e] < (uint32_t)kSlabCap) {
-      s_key[mplace[e]] = mi[e];
-      s_idx[mplace[e]] = mvv[e];
+  for (int i = 0; i < kSlabItems; ++i) {
+    const uint32_t p = threadIdx.x + i * kSlabBlock;
+    if (p < n && (idx[i] & kRemovedBit)) {
+      const uint32_t at = atomicAdd(&s_nrm, 1u);
+      if (at < (uint32_t)kPlaceRemoved) s_rm[at] = p;
     }
   }
   __syncthreads();
+  uint32_t rm_n = s_nrm;
+  if (rm_n > (uint32_t)kPlaceRemoved) {  // more collisions than this path carries
+    if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
+    return;
+  }
+  if (rm_n > 1) sort_small(s_rm, rm_n);
+  // moved-in entry j: its slot's rank among the moved-in slots (they are distinct: a slot has one owner), and
+  // the sorted place in front of which it slips in
+  uint32_t mj[kSlabMoveCap / kSlabBlock], mplace[kSlabMoveCap / kSlabBlock];
+#pragma unroll
+  for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
+    const uint32_t j = threadIdx.x + e * kSlabBlock;
+    mj[e] = mplace[e] = 0;
+    if (j < mv_n) {
+      const uint32_t k = s_mk[j];
+      uint32_t r = 0;
+      for (uint32_t u = 0; u < mv_n; ++u) r += s_mk[u] < k;
+      mj[e] = r;
+      mplace[e] = lower_bound_u32(s_key, n, k);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e)
+    if (threadIdx.x + e * kSlabBlock < mv_n) s_mp[mj[e]] = mplace[e];
+  __syncthreads();
+  const uint32_t out_base = tb.out_start[b];
+  const uint32_t out_n = tb.out_start[b + 1] - out_base;
+  // Most stretches of 64 consecutive sorted places contain neither a removed entry nor the place where a
+  // moved-in entry slips in: all their entries move by the same amount, found once per stretch.
+  for (uint32_t c = threadIdx.x; c * 64u < n; c += kSlabBlock) {
+    const uint32_t p0 = c * 64u, p1 = p0 + 63u < n ? p0 + 63u : n - 1u;
+    uint32_t mv0 = 0, mv1 = 0, r0 = 0, r1 = 0;
+    if (mv_n) {
+      mv0 = upper_bound_u32(s_mp, mv_n, p0);
+      mv1 = upper_bound_u32(s_mp, mv_n, p1);
+    }
+    if (rm_n) {
+      r0 = lower_bound_u32(s_rm, rm_n, p0);
+      r1 = lower_bound_u32(s_rm, rm_n, p1);
+    }
+    s_delta[c] = (mv0 == mv1 && r0 == r1) ? (int32_t)(mv0 - r0) : kNoDelta;
+  }
+  __syncthreads();
+  // survivors
+#pragma unroll
+  for (int i = 0; i < kSlabItems; ++i) {
+    const uint32_t p = threadIdx.x + i * kSlabBlock;
+    if (p < n && !(idx[i] & kRemovedBit)) {
+      int32_t delta = s_delta[p >> 6];
+      if (delta == kNoDelta)
+        delta = (int32_t)((mv_n ? upper_bound_u32(s_mp, mv_n, p) : 0u) - (rm_n ? lower_bound_u32(s_rm, rm_n, p) : 0u));
+      const uint32_t pos = out_base + p + (uint32_t)delta;
+      if (pos < capacity) {
+        out_idx[pos] = (int32_t)idx[i];
+        out_val[pos] = val[i];
+      }
+    }
+  }
+  // moved-in entries
+#pragma unroll
+  for (int e = 0; e < kSlabMoveCap / kSlabBlock; ++e) {
+    const uint32_t j = threadIdx.x + e * kSlabBlock;
+    if (j < mv_n) {
+      const uint32_t pos = out_base + mplace[e] + mj[e] - (rm_n ? lower_bound_u32(s_rm, rm_n, mplace[e]) : 0u);
+      if (pos < capacity) {
+        out_idx[pos] = (int32_t)tb.mv_idx[(size_t)b * kSlabMoveCap + j];
+        out_val[pos] = (S)tb.mv_val[(size_t)b * kSlabMoveCap + j];
+      }
+    }
+  }
   const uint32_t part = b / geo.bpp;
   const bool last_of_part = b % geo.bpp == geo.bpp - 1;
   uint32_t serial = 0;
@@ -618,17 +669,6 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
     if (serial > (uint32_t)kSlabSerialCap) serial = kSlabSerialCap;
   }
   const uint32_t own_n = out_n - serial;  // survivors + moved-in
-  if (own_n > (uint32_t)kSlabCap) {       // cannot happen with the capacities above; never write past LDS
-    if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_INTERNAL);
-    return;
-  }
-  for (uint32_t i = threadIdx.x; i < own_n; i += kSlabBlock) {
-    const uint32_t pos = out_base + i;
-    if (pos < capacity) {
-      out_idx[pos] = (int32_t)s_key[i];
-      out_val[pos] = (S)s_idx[i];
-    }
-  }
   if (serial) {
     // the partition's overflow entries in ascending index order (the reference hands its tickets to
     // ascending thread ids, functions_cuda_kernel.cu:107-108), behind everything that found a slot
@@ -645,7 +685,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
     }
   }
   if (b % geo.bpp == 0 && threadIdx.x == 0) {
-    const uint32_t lo = s_pref[b], hi = s_pref[b + geo.bpp];
+    const uint32_t lo = tb.out_start[b], hi = tb.out_start[b + geo.bpp];
     splits[part] = (int64_t)(hi - lo);
     if ((int64_t)tb.serial_n[part] > spp) atomicOr(status, ZEN_STAT_SERIAL_OVERFLOW);
     if (hi > capacity) atomicOr(status, ZEN_STAT_CAPACITY);
@@ -685,6 +725,7 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.tb.movein_n = cv.take<uint32_t>(B);
   p.tb.serial_n = cv.take<uint32_t>((size_t)partitions);
   p.tb.ctr = cv.take<Counters>(1);
+  p.tb.done = cv.take<uint32_t>(1);
   p.zero_bytes = (size_t)(cv.base + cv.used - static_cast<char *>(p.zero_begin));
   p.thr = cv.take<uint32_t>(4);
   p.list_cap = (uint32_t)list_cap;
@@ -693,8 +734,11 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.list_key = cv.take<uint32_t>((size_t)list_cap);
   p.row_words = (uint32_t)((B + 63) / 64 * 64);
   p.feed_hist = cv.take<uint32_t>((size_t)ceil_div(list_cap, kFeedBatch) * p.row_words);
+  p.tb.bucket_lo = cv.take<uint32_t>(B);
+  p.tb.out_start = cv.take<uint32_t>(B + 1);
   p.tb.bucket_n = cv.take<uint32_t>(B);
   p.tb.removed_n = cv.take<uint32_t>(B);
+  p.tb.slab_rec = cv.take<uint4>(B * kSlabCap);
   p.tb.slab_idx = cv.take<int32_t>(B * kSlabCap);
   p.tb.slab_val = cv.take<char>(B * kSlabCap * (dtype == ZEN_BF16 ? 2 : 4));
   p.tb.slab_key = cv.take<uint32_t>(B * kSlabCap);
@@ -722,8 +766,8 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
     k_feed_count<S><<<dim3(batches), dim3(kSlabBlock), 0, s>>>(geo, p.list_count, p.list_cap, p.list_idx, list_val,
                                                                 filter, p.list_key, p.row_words, p.feed_hist, a.status);
     ZEN_LAUNCH_CHECK("k_feed_count");
-    k_feed_scan<<<dim3(p.row_words / 64), dim3(64 * kScanChunks), 0, s>>>(p.list_count, p.list_cap, B, p.row_words,
-                                                                           p.feed_hist, p.tb.cursor, a.status);
+    k_feed_scan<<<dim3(p.row_words / kScanCols), dim3(kScanCols * kScanChunks), 0, s>>>(
+        geo, p.list_count, p.list_cap, B, p.row_words, p.feed_hist, p.tb.cursor, p.tb.bucket_lo, a.status);
     ZEN_LAUNCH_CHECK("k_feed_scan");
     k_feed_write<S><<<dim3(batches), dim3(kSlabBlock), 0, s>>>(geo, p.tb, p.list_count, p.list_cap, p.list_idx,
                                                                 list_val, p.list_key, p.row_words, p.feed_hist);
@@ -735,7 +779,7 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
     ProfScope prof(kProfFinalKey, s);
     k_slab_chains<S><<<dim3(256), dim3(256), 0, s>>>(geo, a.g, p.tb, a.hash, a.hash_log2, a.status);
     ZEN_LAUNCH_CHECK("k_slab_chains");
-    k_slab_classify<<<dim3(256), dim3(256), 0, s>>>(geo, a.g, p.tb, a.hash, a.hash_log2, a.spp, a.status);
+    k_slab_classify<<<dim3(128), dim3(kSlabBlock), 0, s>>>(geo, a.g, p.tb, a.hash, a.hash_log2, a.spp, a.status);
     ZEN_LAUNCH_CHECK("k_slab_classify");
   }
   {
