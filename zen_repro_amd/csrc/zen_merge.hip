@@ -5,6 +5,8 @@
 // (the order a sequential scatter_add_ uses, so the result is reproducible),
 // zero sums are dropped and the survivors leave in ascending index order.
 #include "zen_common.h"
+#include "zen_slab.h"
+#include "zen_slab_feed.h"
 
 namespace zen {
 namespace {
@@ -135,6 +137,243 @@ __global__ __launch_bounds__(256) void k_scatter_dense<uint16_t>(const int32_t *
   if (i < *count) dense[idx[i]] = f32_to_bf16_rne(sum[i]);
 }
 
+// ---------------------------------------------------------- merge on bucket slabs
+//
+// The indices a destination receives were assigned to it by a hash, so they spread evenly over [0, dense_n):
+// the entries go to bucket slabs by index range (zen_slab_feed.h) as (index, arrival number, value) records,
+// and one workgroup per bucket sorts its slab by (index, arrival number) inside LDS (one word per record), sums every run of equal
+// indices in arrival order, drops zero sums and writes what is left at the place the buckets before it
+// leave off (every bucket publishes how much it keeps and adds up what the earlier ones published).
+
+constexpr int kMergeTarget = 3072;   // records a bucket is sized for: duplicates make the buckets less even
+constexpr int kMergeItems = 13;      // sorted records per thread while summing (odd: no LDS bank conflicts)
+static_assert(kSlabBlock * kMergeItems >= kSlabCap, "every sorted place needs an owner");
+
+template <typename I>
+struct MergeCountSrc {
+  const I *idx;
+  uint32_t dense_n;
+  int32_t *status;
+  __device__ inline uint32_t key(uint32_t e) const {
+    const I k = idx[e];
+    if (k >= 0 && (uint64_t)k < (uint64_t)dense_n) return (uint32_t)k;
+    atomicOr(status, ZEN_STAT_BAD_INDEX);  // skipped, like everything behind the good ones in the general path
+    return kNoSlot;
+  }
+};
+template <typename I, typename S>
+struct MergeWriteSrc {
+  const I *idx;
+  const S *val;
+  uint32_t dense_n;
+  __device__ inline void rec(uint32_t e, uint32_t *key, uint32_t *a, uint32_t *b) const {
+    const I k = idx[e];
+    *key = (k >= 0 && (uint64_t)k < (uint64_t)dense_n) ? (uint32_t)k : kNoSlot;
+    *a = e;
+    *b = __float_as_uint(KeyOf<S>::to_f32(val[e]));
+  }
+};
+
+template <typename I>
+__global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const uint32_t *__restrict__ cursor,
+                                                             const uint32_t *__restrict__ bucket_lo,
+                                                             const uint4 *__restrict__ slab_rec,
+                                                             I *__restrict__ out_idx, float *__restrict__ out_val,
+                                                             int64_t capacity, ScanState st, int tie_bits,
+                                                             int64_t *out_count, int32_t *status) {
+  __shared__ SlabSortShared sh;
+  __shared__ uint64_t s_scan64[kSlabBlock / 64 + 1];
+  __shared__ int s_tile;
+  if (threadIdx.x == 0) s_tile = (int)atomicAdd(st.ticket, 1u);
+  __syncthreads();
+  const int b = s_tile;  // buckets are taken in order, so every earlier bucket already runs
+  const int nb = (int)geo.nbuckets;
+  if (b >= nb) return;
+  const size_t base = (size_t)b * kSlabCap;
+  uint32_t n_raw = cursor[b];
+  if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the scan flagged the overflow
+  const uint32_t lo = bucket_lo[b];
+  uint32_t off[kSlabItems], arr[kSlabItems], val[kSlabItems], rank[kSlabItems];
+  uint32_t live = 0;
+#pragma unroll
+  for (int i = 0; i < kSlabItems; ++i) {
+    const uint32_t j = threadIdx.x + i * kSlabBlock;
+    off[i] = arr[i] = val[i] = 0;
+    if (j < n_raw) {
+      const uint4 rec = slab_rec[base + j];
+      off[i] = rec.x - lo;
+      arr[i] = rec.y;
+      val[i] = rec.z;
+      live |= 1u << i;
+    }
+  }
+  uint32_t n = 0;
+  const bool ranked = slab_rank(sh, geo, tie_bits, off, arr, live, rank, &n);
+  if (!ranked) {
+    if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
+    n = 0;  // the bucket contributes nothing; the prefix protocol still gets its (empty) tile
+  } else {
+#pragma unroll
+    for (int i = 0; i < kSlabItems; ++i) {
+      if (live & (1u << i)) {
+        sh.key[rank[i]] = off[i];
+        sh.tie[rank[i]] = val[i];  // the arrival numbers have done their work: their place takes the values
+      }
+    }
+  }
+  __syncthreads();
+  // Thread t owns the sorted places [t * kMergeItems, (t + 1) * kMergeItems).  It walks once from its first
+  // place to the end of the last run that starts in its range, summing every run that starts there in arrival
+  // order from +0 (like the dense tensor of comm.py:35), and leaves each sum in the value word of the run's
+  // head.  (One walk: a loop per run would cost every lane of a wave the longest run of any lane, each time.)
+  // A run's words are read by the thread of its head only, so the sums can be written in place.
+  const uint32_t first = threadIdx.x * kMergeItems;
+  if (first < n) {
+    const uint32_t end = first + kMergeItems < n ? first + kMergeItems : n;
+    uint32_t cur = first > 0 ? sh.key[first - 1] : 0xffffffffu;  // index of the run the walk is in
+    uint32_t head = 0xffffffffu;                                  // place of its head if it started in the range
+    float acc = 0.0f;
+    for (uint32_t u = first; u < n; ++u) {
+      const uint32_t ku = sh.key[u];
+      if (ku != cur) {
+        if (head != 0xffffffffu) sh.tie[head] = __float_as_uint(acc);
+        if (u >= end) {
+          head = 0xffffffffu;
+          break;
+        }
+        cur = ku;
+        head = u;
+        acc = 0.0f;
+      }
+      if (head != 0xffffffffu) acc += __uint_as_float(sh.tie[u]);
+    }
+    if (head != 0xffffffffu) sh.tie[head] = __float_as_uint(acc);  // the bucket's last run
+  }
+  __syncthreads();
+  uint32_t k[kMergeItems];
+  float sum[kMergeItems];
+  uint32_t keep = 0;
+  uint32_t prev = first > 0 && first <= n ? sh.key[first - 1] : 0xffffffffu;
+#pragma unroll
+  for (int q = 0; q < kMergeItems; ++q) {
+    const uint32_t p = first + q;
+    k[q] = 0;
+    sum[q] = 0.0f;
+    if (p < n) {
+      k[q] = sh.key[p];
+      const bool is_head = p == 0 || k[q] != prev;
+      prev = k[q];
+      sum[q] = __uint_as_float(sh.tie[p]);
+      if (is_head && sum[q] != 0.0f) keep |= 1u << q;  // torch.nonzero keeps NaN, drops +-0
+    }
+  }
+  uint32_t total;
+  const uint32_t before = block_exclusive_scan<uint32_t, kSlabBlock>((uint32_t)__popc(keep), sh.scan, &total);
+  // where this bucket's output starts: the sum of what all earlier buckets keep.  Every thread waits for a
+  // few of them (bounded), nobody waits for a chain of prefixes.
+  if (threadIdx.x == 0) desc_store(&st.desc[b], kDescAggregate | total);
+  uint64_t mine = 0;
+  bool gave_up = false;
+  for (int p = (int)threadIdx.x; p < b; p += kSlabBlock) {
+    uint64_t d = desc_load(&st.desc[p]);
+    uint32_t spins = 0;
+    while ((d >> 62) == 0) {
+      if (++spins > kSpinLimit) {
+        gave_up = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+      d = desc_load(&st.desc[p]);
+    }
+    mine += d & kDescValue;
+  }
+  if (gave_up) atomicOr(status, ZEN_STAT_INTERNAL);
+  uint64_t all_before;
+  block_exclusive_scan<uint64_t, kSlabBlock>(mine, s_scan64, &all_before);
+  const uint64_t tile_start = all_before;
+  if (b == nb - 1 && threadIdx.x == 0) {
+    const uint64_t all = tile_start + total;
+    *out_count = (int64_t)all;
+    if (all > (uint64_t)capacity) atomicOr(status, ZEN_STAT_CAPACITY);
+  }
+  // gather what is kept in LDS (everybody is past reading the sorted bucket: the scans synchronised), then
+  // write it with consecutive lanes
+  uint32_t li = before;
+#pragma unroll
+  for (int q = 0; q < kMergeItems; ++q) {
+    if (keep & (1u << q)) {
+      sh.key[li] = k[q] + lo;
+      sh.tie[li] = __float_as_uint(sum[q]);
+      ++li;
+    }
+  }
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < total; i += kSlabBlock) {
+    const uint64_t pos = tile_start + i;
+    if (pos < (uint64_t)capacity) {
+      out_idx[pos] = (I)sh.key[i];
+      out_val[pos] = __uint_as_float(sh.tie[i]);
+    }
+  }
+}
+
+struct SlabMergePlan {
+  unsigned long long *scan;  // prefix state over the buckets (zeroed before use)
+  uint32_t *cursor, *bucket_lo, *hist;
+  uint4 *slab_rec;
+  size_t zero_bytes;
+  size_t bytes;
+};
+
+SlabMergePlan plan_slab_merge(void *workspace, const SlabGeom &geo, int64_t r) {
+  Carver cv(workspace);
+  SlabMergePlan p;
+  const size_t B = geo.nbuckets;
+  p.scan = cv.take<unsigned long long>(scan_words((int64_t)B));
+  p.zero_bytes = cv.used;
+  p.cursor = cv.take<uint32_t>(B);
+  p.bucket_lo = cv.take<uint32_t>(B);
+  p.hist = cv.take<uint32_t>((size_t)feed_batches(r) * feed_row_words((uint32_t)B));
+  p.slab_rec = cv.take<uint4>(B * kSlabCap);
+  p.bytes = cv.used;
+  return p;
+}
+
+bool slab_merge_fits(int64_t r, int64_t dense_n, SlabGeom *geo) {
+  SlabGeom g;
+  if (r < (1 << 15) || r > 0x7ffffffell || !slab_geometry(dense_n, 1, r, kMergeTarget, &g)) return false;
+  if (g.sub_shift + ceil_log2_u64((uint64_t)r) > 32) return false;  // (index inside a narrow range, arrival number) must fit a word
+  if (geo) *geo = g;
+  return true;
+}
+
+template <typename I, typename S>
+int slab_merge_launch(const SlabGeom &geo, const I *idx, const S *val, int64_t r, int64_t dense_n, void *out_idx,
+                      int idx64_out, float *out_val, int64_t capacity, int64_t *out_count, void *workspace,
+                      int32_t *status, hipStream_t s) {
+  const SlabMergePlan p = plan_slab_merge(workspace, geo, r);
+  launch_fill<unsigned long long>(p.scan, 0ull, p.zero_bytes / sizeof(unsigned long long), s);
+  ZEN_LAUNCH_CHECK("merge: clear prefix state");
+  {
+    ProfScope prof(kProfMergePrep, s);
+    const MergeCountSrc<I> csrc{idx, (uint32_t)dense_n, status};
+    const MergeWriteSrc<I, S> wsrc{idx, val, (uint32_t)dense_n};
+    const int rc = feed_slabs(geo, csrc, wsrc, nullptr, r, p.hist, p.cursor, p.bucket_lo, p.slab_rec, status, s);
+    if (rc != ZEN_OK) return rc;
+  }
+  const ScanState st = scan_state(p.scan, (int64_t)geo.nbuckets);
+  const int tie_bits = ceil_log2_u64((uint64_t)r);  // arrival numbers are < r
+  ProfScope prof(kProfMergeReduce, s);
+  if (idx64_out)
+    k_merge_bucket<int64_t><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
+        geo, p.cursor, p.bucket_lo, p.slab_rec, static_cast<int64_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
+  else
+    k_merge_bucket<int32_t><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
+        geo, p.cursor, p.bucket_lo, p.slab_rec, static_cast<int32_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
+  ZEN_LAUNCH_CHECK("k_merge_bucket");
+  return ZEN_OK;
+}
+
 struct MergePlan {
   uint32_t *keys, *tmp_v, *sort_k, *sort_v;
   void *scan;  // prefix state of the reduce kernel
@@ -147,7 +386,6 @@ MergePlan plan_merge(void *workspace, int64_t r, int64_t dense_n) {
   Carver cv(workspace);
   MergePlan p;
   const size_t cap = (size_t)(r > 0 ? r : 1);
-  (void)dense_n;
   p.keys = cv.take<uint32_t>(cap);
   p.tmp_v = cv.take<uint32_t>(cap);
   p.sort_k = cv.take<uint32_t>(cap);
@@ -156,6 +394,11 @@ MergePlan plan_merge(void *workspace, int64_t r, int64_t dense_n) {
   p.scan = cv.take<unsigned long long>(scan_words(p.ntiles));
   p.sort_scratch = cv.take<char>(sort_scratch_bytes((int64_t)cap));
   p.bytes = cv.used;
+  SlabGeom geo;
+  if (slab_merge_fits(r, dense_n, &geo)) {
+    const size_t slabs = plan_slab_merge(nullptr, geo, r).bytes;
+    if (slabs > p.bytes) p.bytes = slabs;
+  }
   return p;
 }
 
@@ -163,6 +406,14 @@ template <typename S>
 int merge_launch(const void *idx, int idx64_in, const S *val, int64_t r, int64_t dense_n, void *out_idx,
                  int idx64_out, float *out_val, int64_t capacity, int64_t *out_count, int mode, void *workspace,
                  int32_t *status, hipStream_t s) {
+  SlabGeom geo;
+  if (mode == ZEN_MODE_FAST && slab_merge_fits(r, dense_n, &geo)) {
+    if (idx64_in)
+      return slab_merge_launch(geo, static_cast<const int64_t *>(idx), val, r, dense_n, out_idx, idx64_out, out_val,
+                               capacity, out_count, workspace, status, s);
+    return slab_merge_launch(geo, static_cast<const int32_t *>(idx), val, r, dense_n, out_idx, idx64_out, out_val,
+                             capacity, out_count, workspace, status, s);
+  }
   MergePlan p = plan_merge(workspace, r, dense_n);
   const unsigned blocks = (unsigned)ceil_div(r, 256);
   launch_fill<unsigned long long>(static_cast<unsigned long long *>(p.scan), 0ull, scan_words(p.ntiles), s);

@@ -38,7 +38,7 @@ struct SlabGeom {
   uint32_t bpp;       // buckets per partition
   uint32_t bpp_mult;  // floor(bpp * 2^32 / npp)
   uint32_t nbuckets;  // partitions * bpp
-  uint32_t sub_mult;  // floor(kSlabSubs * 2^32 / (widest bucket + 1)): key offset inside a bucket -> narrow range
+  int sub_shift;      // key offset inside a bucket >> sub_shift = narrow range (fewer than kSlabSubs of them)
   float inv_m;        // (1 / m)(1 - 2^-20), rounded down
   float inv_npp;      // the same for npp
 
@@ -69,7 +69,6 @@ struct SlabGeom {
     const uint32_t part = b / bpp, sb = b - part * bpp;
     return part * npp + (uint32_t)((((uint64_t)sb << 32) + bpp_mult - 1) / bpp_mult);
   }
-  __device__ inline uint32_t sub_of(uint32_t offset) const { return __umulhi(offset, sub_mult); }
 };
 
 // Host side: geometry for `partitions` partitions of a key space of m keys (m a
@@ -100,7 +99,8 @@ inline bool slab_geometry(int64_t m, int partitions, int64_t expected, int targe
   g.bpp_mult = (uint32_t)(((uint64_t)bpp << 32) / (uint64_t)npp);
   g.nbuckets = (uint32_t)nb;
   const uint64_t width = ((1ull << 32) + g.bpp_mult - 1) / g.bpp_mult + 1;  // keys per bucket, at most
-  g.sub_mult = (uint32_t)(((uint64_t)kSlabSubs << 32) / (width + 1));
+  g.sub_shift = 0;
+  while ((width >> g.sub_shift) >= (uint64_t)kSlabSubs) ++g.sub_shift;
   g.inv_m = slab_inverse_below(g.m);
   g.inv_npp = slab_inverse_below(g.npp);
   *out = g;
@@ -123,24 +123,25 @@ struct SlabSortShared {
   uint32_t bad;
 };
 
-// Ranks the live records of a workgroup by (key offset, tie), both unique as a
-// pair.  off[i] < bucket width.  The records are first grouped by narrow key
-// range with one LDS atomic each; inside its group every record counts the
-// records that precede it.  Returns false (for every thread) if a group is too
-// large for that; else rank[i] for live records and *n_out = number of live
-// records.  On return sh.key / sh.tie may be overwritten at once.
-__device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, const uint32_t (&off)[kSlabItems],
-                                 const uint32_t (&tie)[kSlabItems], uint32_t live, uint32_t (&rank)[kSlabItems],
-                                 uint32_t *n_out) {
+// Ranks the live records of a workgroup by (key offset, tie); tie < 2^tie_bits, the pair unique, and
+// geo.sub_shift + tie_bits <= 32.  off[i] < bucket width.  The records are first grouped by narrow key range
+// with one LDS atomic each; a record is then one word, (offset inside the range) << tie_bits | tie, and
+// inside its group every record counts the words smaller than its own.  Returns false (for every thread) if a
+// group is too large for that; else rank[i] for live records and *n_out = number of live records.  On return
+// sh.key / sh.tie may be overwritten at once (sh.tie is not touched at all).
+__device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, int tie_bits,
+                                 const uint32_t (&off)[kSlabItems], const uint32_t (&tie)[kSlabItems], uint32_t live,
+                                 uint32_t (&rank)[kSlabItems], uint32_t *n_out) {
   for (int d = threadIdx.x; d <= kSlabSubs; d += kSlabBlock) sh.cnt[d] = 0;
   if (threadIdx.x == 0) sh.bad = 0;
   __syncthreads();
+  const uint32_t low_mask = (1u << geo.sub_shift) - 1u;
   uint32_t sub[kSlabItems], at[kSlabItems];
 #pragma unroll
   for (int i = 0; i < kSlabItems; ++i) {
     sub[i] = at[i] = 0;
     if (live & (1u << i)) {
-      sub[i] = geo.sub_of(off[i]);
+      sub[i] = off[i] >> geo.sub_shift;
       at[i] = atomicAdd(&sh.cnt[sub_place(sub[i])], 1u);
     }
   }
@@ -166,12 +167,14 @@ __device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, const 
   }
   __syncthreads();
   if (sh.bad) return false;
+  uint32_t g0[kSlabItems], word[kSlabItems];
 #pragma unroll
   for (int i = 0; i < kSlabItems; ++i) {
+    g0[i] = word[i] = 0;
     if (live & (1u << i)) {
-      const uint32_t p = sh.cnt[sub_place(sub[i])] + at[i];
-      sh.key[p] = off[i];
-      sh.tie[p] = tie[i];
+      g0[i] = sh.cnt[sub_place(sub[i])];
+      word[i] = ((off[i] & low_mask) << tie_bits) | tie[i];
+      sh.key[g0[i] + at[i]] = word[i];
     }
   }
   __syncthreads();
@@ -179,13 +182,10 @@ __device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, const 
   for (int i = 0; i < kSlabItems; ++i) {
     rank[i] = 0;
     if (live & (1u << i)) {
-      const uint32_t g0 = sh.cnt[sub_place(sub[i])], g1 = sh.cnt[sub_place(sub[i] + 1)];
+      const uint32_t g1 = sh.cnt[sub_place(sub[i] + 1)];
       uint32_t less = 0;
-      for (uint32_t u = g0; u < g1; ++u) {
-        const uint32_t ku = sh.key[u];
-        less += (ku < off[i]) || (ku == off[i] && sh.tie[u] < tie[i]);
-      }
-      rank[i] = g0 + less;
+      for (uint32_t u = g0[i]; u < g1; ++u) less += sh.key[u] < word[i];
+      rank[i] = g0[i] + less;
     }
   }
   *n_out = sh.cnt[kSlabSubs];

@@ -24,6 +24,7 @@
 #include "zen_balance.h"
 #include "zen_hashmap.h"
 #include "zen_slab.h"
+#include "zen_slab_feed.h"
 
 namespace zen {
 namespace {
@@ -52,72 +53,8 @@ __device__ inline uint32_t level1_slot(const Probe &g, uint32_t t) { return (pol
 
 // ------------------------------------------------- list -> bucket slabs
 
-constexpr int kFeedItems = 8;
-constexpr int kFeedBatch = kSlabBlock * kFeedItems;  // list entries per workgroup
-constexpr int kScanChunks = 64;
+}  // namespace
 
-// The select kernel left its candidates in one list, in no particular order.  Three kernels move them to the
-// bucket slabs without a single global atomic (a reservation per bucket and batch would be a million
-// device-wide atomics): every workgroup counts its batch of the list per bucket (k_feed_count), a scan over
-// the batches turns the counts of a bucket into the places where each batch's run starts in the bucket's slab
-// (k_feed_scan), and every workgroup orders its batch by bucket in LDS and writes the runs (k_feed_write).
-// Index 0 (never transmitted: 0 is the table's empty marker, tensor_load_balance.py:31) and whatever the exact
-// threshold excludes are dropped on the way.
-
-__device__ inline uint32_t feed_count(const uint32_t *list_count, uint32_t list_cap) {
-  const uint32_t c = *list_count;
-  return c < list_cap ? c : list_cap;
-}
-
-constexpr uint32_t kNoSlot = 0xffffffffu;  // list_key of an entry that is not selected
-
-// Counts the batch per bucket and leaves every entry's level-1 slot in list_key (kNoSlot: not selected), so
-// that nobody has to hash again.
-template <typename S>
-__global__ __launch_bounds__(kSlabBlock) void k_feed_count(SlabGeom geo, const uint32_t *__restrict__ list_count,
-                                                           uint32_t list_cap, const int32_t *__restrict__ list_idx,
-                                                           const S *__restrict__ list_val,
-                                                           const uint32_t *__restrict__ filter,
-                                                           uint32_t *__restrict__ list_key, uint32_t row_words,
-                                                           uint32_t *__restrict__ hist, int32_t *status) {
-  __shared__ uint32_t s_cnt[kSlabMaxBuckets];
-  if (*list_count > list_cap && blockIdx.x == 0 && threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);  // entries lost
-  const uint32_t count = feed_count(list_count, list_cap);
-  const uint32_t batch = blockIdx.x * (uint32_t)kFeedBatch;
-  if (batch >= count) return;
-  for (uint32_t b = threadIdx.x; b < row_words; b += kSlabBlock) s_cnt[b] = 0;
-  __syncthreads();
-  const uint32_t thr = filter ? filter[0] : 0u;
-  uint32_t t[kFeedItems];
-  S v[kFeedItems];
-#pragma unroll
-  for (int i = 0; i < kFeedItems; ++i) {
-    const uint32_t e = batch + threadIdx.x + i * kSlabBlock;
-    t[i] = 0;
-    v[i] = 0;
-    if (e < count) {
-      t[i] = (uint32_t)list_idx[e];
-      v[i] = list_val[e];
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < kFeedItems; ++i) {
-    const uint32_t e = batch + threadIdx.x + i * kSlabBlock;
-    uint32_t slot = kNoSlot;
-    if (t[i] != 0 && (v[i] & KeyOf<S>::kMask) >= thr) {
-      slot = geo.mod_m(poly(t[i]) + kSeed1);
-      atomicAdd(&s_cnt[geo.bucket_of(slot)], 1u);
-    }
-    if (e < count) list_key[e] = slot;
-  }
-  __syncthreads();
-  uint32_t *row = hist + (size_t)blockIdx.x * row_words;
-  for (uint32_t b = threadIdx.x; b < row_words; b += kSlabBlock) row[b] = s_cnt[b];
-}
-
-// Workgroup = kScanCols buckets x kScanChunks ranges of batches.  hist[batch][bucket] becomes the number of the
-// bucket's entries in earlier batches; cursor[bucket] = the bucket's total.
-constexpr int kScanCols = 16;
 __global__ __launch_bounds__(kScanCols * kScanChunks) void k_feed_scan(SlabGeom geo,
                                                                        const uint32_t *__restrict__ list_count,
                                                                        uint32_t list_cap, uint32_t nbuckets,
@@ -157,100 +94,38 @@ __global__ __launch_bounds__(kScanCols * kScanChunks) void k_feed_scan(SlabGeom 
   }
 }
 
-// Every selected entry of the batch goes to its bucket's slab as one 16-byte record.  Scattered stores cost
-// one memory request each whatever their size (about 80 G requests/s on this part), so the batch is first
-// ordered by bucket in LDS: the records of a bucket then leave as one run, a few requests instead of one per
-// record.  A run's place in the slab comes from the scan.
+namespace {
+
+// The select kernel left its candidates in one list, in no particular order.  On the way to the slabs index 0
+// (never transmitted: 0 is the table's empty marker, tensor_load_balance.py:31) and whatever the exact
+// threshold excludes are dropped; every kept entry's level-1 slot is computed once, in the counting pass, and
+// kept in list_key for the writing pass.
 template <typename S>
-__global__ __launch_bounds__(kSlabBlock) void k_feed_write(SlabGeom geo, SlabTables tb,
-                                                           const uint32_t *__restrict__ list_count, uint32_t list_cap,
-                                                           const int32_t *__restrict__ list_idx,
-                                                           const S *__restrict__ list_val,
-                                                           const uint32_t *__restrict__ list_key, uint32_t row_words,
-                                                           const uint32_t *__restrict__ hist) {
-  // entries of the batch per bucket; then (where the bucket's run starts in the ordered batch) << 13 | (where it
-  // starts in the slab).  One array, so that two workgroups fit into a compute unit's LDS.
-  __shared__ uint32_t s_cnt[kSlabMaxBuckets];
-  __shared__ uint4 s_rec[kFeedBatch];  // the ordered batch; .w = bucket << 13 | place in the slab
-  __shared__ uint32_t s_scan[kSlabBlock / 64 + 1];
-  static_assert(kSlabCap <= (1 << 13) && kFeedBatch < (1 << 13) && kSlabMaxBuckets <= (1 << 11), "packed fields");
-  const uint32_t count = feed_count(list_count, list_cap);
-  const uint32_t batch = blockIdx.x * (uint32_t)kFeedBatch;
-  if (batch >= count) return;
-  for (uint32_t b = threadIdx.x; b < (uint32_t)kSlabMaxBuckets; b += kSlabBlock) s_cnt[b] = 0;
-  // where the runs of this thread's buckets start in the slabs: asked for now, needed after the counting
-  constexpr int kPer = kSlabMaxBuckets / kSlabBlock;
-  uint32_t base[kPer];
-  {
-    const uint32_t *row = hist + (size_t)blockIdx.x * row_words;
-#pragma unroll
-    for (int e = 0; e < kPer; ++e) {
-      const uint32_t b = threadIdx.x * kPer + e;
-      base[e] = b < row_words ? row[b] : 0u;
-    }
+struct EncodeCountSrc {
+  SlabGeom geo;
+  const int32_t *list_idx;
+  const S *list_val;
+  const uint32_t *filter;  // optional exact threshold
+  uint32_t *list_key;
+  __device__ inline uint32_t key(uint32_t e) const {
+    const uint32_t t = (uint32_t)list_idx[e];
+    uint32_t slot = kNoSlot;
+    if (t != 0 && (list_val[e] & KeyOf<S>::kMask) >= (filter ? filter[0] : 0u)) slot = geo.mod_m(poly(t) + kSeed1);
+    list_key[e] = slot;
+    return slot;
   }
-  __syncthreads();
-  uint32_t t[kFeedItems], key[kFeedItems], bucket[kFeedItems], rank[kFeedItems];
-  S v[kFeedItems];
-#pragma unroll
-  for (int i = 0; i < kFeedItems; ++i) {
-    const uint32_t e = batch + threadIdx.x + i * kSlabBlock;
-    t[i] = 0;
-    v[i] = 0;
-    key[i] = kNoSlot;
-    if (e < count) {
-      key[i] = list_key[e];
-      t[i] = (uint32_t)list_idx[e];
-      v[i] = list_val[e];
-    }
+};
+template <typename S>
+struct EncodeWriteSrc {
+  const int32_t *list_idx;
+  const S *list_val;
+  const uint32_t *list_key;
+  __device__ inline void rec(uint32_t e, uint32_t *key, uint32_t *a, uint32_t *b) const {
+    *key = list_key[e];
+    *a = (uint32_t)list_idx[e];
+    *b = (uint32_t)list_val[e];
   }
-#pragma unroll
-  for (int i = 0; i < kFeedItems; ++i) {
-    bucket[i] = rank[i] = 0;
-    if (key[i] != kNoSlot) {
-      bucket[i] = geo.bucket_of(key[i]);
-      rank[i] = atomicAdd(&s_cnt[bucket[i]], 1u);
-    }
-  }
-  __syncthreads();
-  uint32_t batch_live;
-  {
-    // thread owns kPer consecutive buckets: one exclusive prefix over the buckets gives every bucket's run a
-    // place in the ordered batch
-    uint32_t c[kPer];
-    uint32_t sum = 0;
-#pragma unroll
-    for (int e = 0; e < kPer; ++e) {
-      c[e] = s_cnt[threadIdx.x * kPer + e];
-      sum += c[e];
-    }
-    uint32_t running = block_exclusive_scan<uint32_t, kSlabBlock>(sum, s_scan, &batch_live);
-#pragma unroll
-    for (int e = 0; e < kPer; ++e) {
-      // a run that starts past the slab's end (overflow, flagged by the scan) is clipped to the end
-      s_cnt[threadIdx.x * kPer + e] = (running << 13) | (base[e] < (uint32_t)kSlabCap ? base[e] : (uint32_t)kSlabCap);
-      running += c[e];
-    }
-  }
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < kFeedItems; ++i) {
-    if (key[i] != kNoSlot) {
-      const uint32_t sb = s_cnt[bucket[i]];
-      uint32_t pos = (sb & 8191u) + rank[i];
-      if (pos > 8191u) pos = 8191u;  // beyond the slab anyway: dropped below, must not spill into the bucket field
-      s_rec[(sb >> 13) + rank[i]] = make_uint4(key[i], t[i], (uint32_t)v[i], (bucket[i] << 13) | pos);
-    }
-  }
-  __syncthreads();
-  // consecutive lanes write consecutive records of a run
-  for (uint32_t e = threadIdx.x; e < batch_live; e += kSlabBlock) {
-    uint4 rec = s_rec[e];
-    const uint32_t b = rec.w >> 13, pos = rec.w & 8191u;
-    rec.w = 0;
-    if (pos < (uint32_t)kSlabCap) tb.slab_rec[(size_t)b * kSlabCap + pos] = rec;
-  }
-}
+};
 
 // ------------------------------------------------------------ sort a bucket
 
@@ -267,24 +142,28 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
   const uint32_t lo = tb.bucket_lo[b];
   S *slab_val = static_cast<S *>(tb.slab_val);
   if (threadIdx.x == 0) s_lost = 0;
-  uint32_t off[kSlabItems], idx[kSlabItems], rank[kSlabItems];
+  uint32_t off[kSlabItems], idx[kSlabItems], pos[kSlabItems], rank[kSlabItems];
   S val[kSlabItems];
   uint32_t live = 0;
 #pragma unroll
   for (int i = 0; i < kSlabItems; ++i) {
     const uint32_t j = threadIdx.x + i * kSlabBlock;
-    off[i] = idx[i] = 0;
+    off[i] = idx[i] = pos[i] = 0;
     val[i] = 0;
     if (j < n_raw) {
       const uint4 rec = tb.slab_rec[base + j];
       off[i] = rec.x - lo;
       idx[i] = rec.y;
       val[i] = (S)rec.z;
+      pos[i] = j;
       live |= 1u << i;
     }
   }
+  // ties between equal slots are broken by the record's place in the slab (13 bits, so a record is one word
+  // while it is ranked); the runs of equal slots, few and short, are put right afterwards
+  static_assert(kSlabCap <= (1 << 13), "slab places in 13 bits");
   uint32_t n = 0;
-  if (!slab_rank(sh, geo, off, idx, live, rank, &n)) {
+  if (!slab_rank(sh, geo, 13, off, pos, live, rank, &n)) {
     if (threadIdx.x == 0) {
       atomicOr(status, ZEN_STAT_RETRY);
       tb.bucket_n[b] = 0;
@@ -298,6 +177,24 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
       sh.key[rank[i]] = off[i];
       sh.tie[rank[i]] = idx[i];
       s_val[rank[i]] = val[i];
+    }
+  }
+  __syncthreads();
+  // a run of equal slots gets its smallest index in front (the thread at the run's first place does it)
+  for (uint32_t p = threadIdx.x; p + 1 < n; p += kSlabBlock) {
+    const uint32_t k = sh.key[p];
+    if (sh.key[p + 1] == k && (p == 0 || sh.key[p - 1] != k)) {
+      uint32_t best = p;
+      for (uint32_t u = p + 1; u < n && sh.key[u] == k; ++u)
+        if (sh.tie[u] < sh.tie[best]) best = u;
+      if (best != p) {
+        const uint32_t ti = sh.tie[p];
+        const S tv = s_val[p];
+        sh.tie[p] = sh.tie[best];
+        s_val[p] = s_val[best];
+        sh.tie[best] = ti;
+        s_val[best] = tv;
+      }
     }
   }
   __syncthreads();
@@ -703,8 +600,7 @@ struct SlabPlan {
   void *list_val;
   uint32_t *list_key;     // [list_cap] level-1 slot of every selected candidate
   uint32_t list_cap;
-  uint32_t *feed_hist;    // [batches of the list][row_words] per-batch bucket counts, then run starts
-  uint32_t row_words;
+  uint32_t *feed_hist;    // per-batch bucket counts, then run starts (zen_slab_feed.h)
   uint32_t *thr;          // [0..1] exact threshold + count, [2..3] sampled floor
   void *zero_begin;
   size_t zero_bytes;
@@ -732,8 +628,7 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.list_idx = cv.take<int32_t>((size_t)list_cap);
   p.list_val = cv.take<char>((size_t)list_cap * (dtype == ZEN_BF16 ? 2 : 4));
   p.list_key = cv.take<uint32_t>((size_t)list_cap);
-  p.row_words = (uint32_t)((B + 63) / 64 * 64);
-  p.feed_hist = cv.take<uint32_t>((size_t)ceil_div(list_cap, kFeedBatch) * p.row_words);
+  p.feed_hist = cv.take<uint32_t>((size_t)feed_batches(list_cap) * feed_row_words((uint32_t)B));
   p.tb.bucket_lo = cv.take<uint32_t>(B);
   p.tb.out_start = cv.take<uint32_t>(B + 1);
   p.tb.bucket_n = cv.take<uint32_t>(B);
@@ -761,17 +656,12 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
   const S *dense = static_cast<const S *>(a.input);
   {
     ProfScope prof(kProfInsertList, s);
-    const unsigned batches = (unsigned)ceil_div((int64_t)p.list_cap, kFeedBatch);
     const S *list_val = static_cast<const S *>(p.list_val);
-    k_feed_count<S><<<dim3(batches), dim3(kSlabBlock), 0, s>>>(geo, p.list_count, p.list_cap, p.list_idx, list_val,
-                                                                filter, p.list_key, p.row_words, p.feed_hist, a.status);
-    ZEN_LAUNCH_CHECK("k_feed_count");
-    k_feed_scan<<<dim3(p.row_words / kScanCols), dim3(kScanCols * kScanChunks), 0, s>>>(
-        geo, p.list_count, p.list_cap, B, p.row_words, p.feed_hist, p.tb.cursor, p.tb.bucket_lo, a.status);
-    ZEN_LAUNCH_CHECK("k_feed_scan");
-    k_feed_write<S><<<dim3(batches), dim3(kSlabBlock), 0, s>>>(geo, p.tb, p.list_count, p.list_cap, p.list_idx,
-                                                                list_val, p.list_key, p.row_words, p.feed_hist);
-    ZEN_LAUNCH_CHECK("k_feed_write");
+    const EncodeCountSrc<S> csrc{geo, p.list_idx, list_val, filter, p.list_key};
+    const EncodeWriteSrc<S> wsrc{p.list_idx, list_val, p.list_key};
+    const int rc = feed_slabs(geo, csrc, wsrc, p.list_count, p.list_cap, p.feed_hist, p.tb.cursor, p.tb.bucket_lo,
+                              p.tb.slab_rec, a.status, s);
+    if (rc != ZEN_OK) return rc;
     k_slab_sort<S><<<dim3(B), dim3(kSlabBlock), 0, s>>>(geo, p.tb, dense, a.status);
     ZEN_LAUNCH_CHECK("k_slab_sort");
   }
