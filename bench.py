@@ -35,6 +35,9 @@ def parse():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run five device copies of 1 GiB and exit (scale for hardware byte counters)")
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
+    ap.add_argument("--depth", type=int, default=2,
+                    help="gradient buckets in flight: step i+1 is enqueued on its own streams next to step i "
+                         "(1 = a step starts when the previous one has finished)")
     ap.add_argument("--no-kernel-timing", action="store_true",
                     help="leave the HIP-event kernel timers off during the timed region")
     return ap.parse_args()
@@ -112,41 +115,56 @@ def main():
     idx_l, val_l, flat_idx, flat_val = workloads.peer_payloads(cfg, per_peer, device=dev, seed=1)
     received = flat_idx.numel()
 
-    # The merge of the received payloads does not depend on this rank's own
-    # encode, so it runs on a second stream and fills the gaps the short
-    # kernels of either side leave (both streams at default priority).
+    # The merge of the received payloads does not depend on this rank's own encode, so it runs on a second
+    # stream.  A training step hands over one gradient bucket after the other (train.py:167-185 is called
+    # per bucket), and nothing in bucket i+1 depends on bucket i: with --depth 2 consecutive steps alternate
+    # between two sets of streams, workspaces and tables ("slots"), so the long, memory-bound select of one
+    # step runs next to the short, latency-bound kernels of the other.  All streams have default priority.
+    depth = 1 if args.one_stream else max(1, args.depth)
     main = torch.cuda.current_stream(dev)
-    side = None if args.one_stream else torch.cuda.Stream(device=dev)
+    enc_streams = [main] + [torch.cuda.Stream(device=dev) for _ in range(depth - 1)]
+    mrg_streams = [None if args.one_stream else torch.cuda.Stream(device=dev) for _ in range(depth)]
 
-    def step():
-        if side is not None:
-            side.wait_stream(main)
-        enc = tp.load_balance_flat(grad, None, capacity, k=cfg.k)  # enqueued first: its long kernel starts at once
-        if side is None:
-            mrg = lba.merge_sparse_flat(flat_idx, flat_val, n, capacity=received)
-        else:
-            with torch.cuda.stream(side):
-                mrg = lba.merge_sparse_flat(flat_idx, flat_val, n, capacity=received)
-            main.wait_stream(side)
+    def step(i):
+        slot = i % depth
+        es, ms_ = enc_streams[slot], mrg_streams[slot]
+        with torch.cuda.stream(es):
+            enc = tp.load_balance_flat(grad, None, capacity, k=cfg.k, slot=slot)
+        with torch.cuda.stream(ms_ if ms_ is not None else es):
+            mrg = lba.merge_sparse_flat(flat_idx, flat_val, n, capacity=received, slot=slot)
         return enc, mrg
 
-    for _ in range(args.warmup):
-        out = step()
+    def run(count):
+        outs = []
+        for s_ in enc_streams[1:] + [m for m in mrg_streams if m is not None]:
+            s_.wait_stream(main)  # the inputs were produced on the main stream
+        for i in range(count):
+            outs.append(step(i))
+        for s_ in enc_streams[1:] + [m for m in mrg_streams if m is not None]:
+            main.wait_stream(s_)
+        return outs
+
+    run(args.warmup)
     torch.cuda.synchronize()
     if not args.no_kernel_timing:
         _lib.profile_enable(True)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out = step()
+    outs = run(args.steps)
+    t_enq = time.perf_counter()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     kernels = {} if args.no_kernel_timing else _lib.profile_read()
     _lib.profile_enable(False)
 
-    (o_idx, o_val, splits, st_enc), (m_idx, m_val, m_count, st_mrg) = out
+    (o_idx, o_val, splits, st_enc), (m_idx, m_val, m_count, st_mrg) = outs[-1]
     nnz = int(splits.sum())
     merged = int(m_count)
-    flags = int(st_enc) | int(st_mrg)
+    flags = 0
+    for enc, mrg in outs:  # every step of the timed region must have gone through cleanly and agree
+        flags |= int(enc[3]) | int(mrg[3])
+        if int(enc[2].sum()) != nnz or int(mrg[2]) != merged:
+            print("bench.py: steps disagree on their result sizes", file=sys.stderr)
+            sys.exit(1)
     if flags:
         print("bench.py: device status " + _lib.describe_status(flags), file=sys.stderr)
         sys.exit(1)
@@ -190,9 +208,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{cfg.name}: {cfg.note}", "elements": n, "partitions": P, "k": cfg.k,
                    "selected": nnz, "received": received, "merged": merged, "peers": cfg.peers,
-                   "overlap": cfg.overlap, "shrink": args.shrink},
+                   "overlap": cfg.overlap, "shrink": args.shrink, "steps_in_flight": depth},
         "path_algorithmic_GBps": round(b_alg / (ms * 1e-3) / 1e9, 2),
         "path_frac_of_hbm_peak": round(b_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "host_enqueue_ms_per_step": round((t_enq - t0) * 1e3 / args.steps, 4),
         "stage_ms_per_step": stage_ms,
         "roofline": roofline,
         "cpu_baseline": None,

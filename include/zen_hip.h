@@ -165,6 +165,14 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m,
                      void *workspace, size_t workspace_bytes,
                      int32_t *status, void *stream);
 
+/*
+ * Which implementation a zen_load_balance call with these sizes takes: 0 = owner table (the general
+ * mode), 1 = sort-based owner resolution, 2 = bucket slabs (large inputs whose expected output is a small
+ * fraction of the table: one streaming pass, then per-bucket sorts inside LDS).  No counterpart in the
+ * reference; tests and benchmarks use it to know what they measured.
+ */
+int zen_load_balance_path(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions, int64_t k, int mode);
+
 /* ----------------------------------------------------------------- merge */
 
 /*
@@ -177,6 +185,8 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m,
  * `mode` is ZEN_MODE_FAST or ZEN_MODE_GENERAL; both give identical results.
  */
 size_t zen_merge_workspace(int64_t r, int64_t dense_n);
+/* 0 = radix sort (general mode), 1 = one bucket pass + per-range sorts, 2 = bucket slabs; see zen_load_balance_path */
+int zen_merge_path(int64_t r, int64_t dense_n, int mode);
 int zen_merge(const void *idx, int idx64_in, const void *val, int dtype,
               int64_t r, int64_t dense_n,
               void *out_idx, int idx64_out, float *out_val, int64_t capacity,

@@ -1,0 +1,232 @@
+"""Parity of the bucket-slab fast paths (large inputs) against the CPU oracle:
+load balance with many collisions (levels 2 and 3, serial entries, declined
+calls that fall back to the general mode), merge with heavy duplication, bad
+indices and 64-bit indices, and calls in flight on two streams with their own
+slots.  Every test first checks through zen_*_path that the sizes really take
+the slab path.  Bar: bit-exact, as in test_gpu_parity.py."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import make_grad, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+SLAB = 2
+
+
+@pytest.fixture(scope="module")
+def zen():
+    import zen_repro_amd
+    from zen_repro_amd import _lib
+
+    _lib.lib()
+    assert torch.cuda.is_available()
+    return zen_repro_amd
+
+
+def lb_path(zen, n, P, dtype, capacity, k=0, mode=0, scale=1):
+    from zen_repro_amd import _lib
+
+    m = int(n * scale // P * P)
+    return _lib.lib().zen_load_balance_path(n, m, 1 if dtype == "bf16" else 0, capacity, P, k, mode)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("n,P,density,rehash", [
+    ((1 << 23), 16, 0.15, 3),        # 15 % of the slots taken: thousands of level-2/3 moves per partition
+    ((1 << 23), 16, 0.15, 2),        # two levels: serial entries in every partition
+    ((1 << 23) + 4096, 8, 0.05, 3),  # table size not a power of two
+    ((1 << 24), 64, 0.01, 3),
+    (6000000, 3, 0.02, 3),           # partitions not a power of two, odd bucket widths
+])
+def test_slab_load_balance_bit_exact(zen, oracle, n, P, density, rehash, dtype):
+    from zen_repro_amd import _lib
+
+    n = n // P * P
+    g = make_grad(oracle, n, density, dtype, seed=n ^ (P * 131) ^ rehash)
+    g[0] = 0x3F80 if dtype == "bf16" else 1.0  # index 0 holds a value and is never transmitted
+    idx_o, val_o, splits_o, st_o = oracle.load_balance(g, P, 1, rehash)
+    assert st_o == 0
+    capacity = int(len(idx_o) * 1.1) + 1024
+    assert lb_path(zen, n, P, dtype, capacity) == SLAB
+    tp = zen.TensorPartition(P, 1, rehash)
+    d = to_dev(g)
+    for rep in range(2):  # the second call finds the borrowed table zero again
+        oi, ov, splits, status = tp.load_balance_flat(d, capacity=capacity, mode=_lib.MODE_FAST)
+        assert status.item() == 0
+        assert np.array_equal(to_np(splits), splits_o)
+        total = int(splits_o.sum())
+        assert np.array_equal(to_np(oi)[:total], idx_o)
+        assert np.array_equal(to_np(ov)[:total], val_o)
+    m, _ = oracle.table_sizes(n, P, 1)
+    assert not tp._table(d.device, m).any()
+
+
+def test_slab_load_balance_declines_and_general_mode_takes_over(zen, oracle):
+    """One rehash level at 15 % load sends every level-1 loser to the serial
+    lists: far more than the slab path carries per partition.  It must say so
+    (RETRY), and the reference-shaped call must come back with the right
+    answer from the general mode."""
+    from zen_repro_amd import _lib
+
+    n, P = (1 << 23) + 16000, 16  # not a power of two: about 8000 level-1 losers per partition
+    g = make_grad(oracle, n, 0.15, "bf16", seed=99)
+    idx_o, val_o, splits_o, st_o = oracle.load_balance(g, P, 1, 1)
+    assert st_o == 0
+    capacity = int(len(idx_o) * 1.1) + 1024
+    assert lb_path(zen, n, P, "bf16", capacity) == SLAB
+    tp = zen.TensorPartition(P, 1, 1)
+    d = to_dev(g)
+    _, _, _, status = tp.load_balance_flat(d, capacity=capacity, mode=_lib.MODE_FAST)
+    assert status.item() & _lib.STAT_RETRY
+    tp._table(d.device, n).zero_()
+    indices, values, splits = tp.load_balance(d, capacity=capacity)
+    assert np.array_equal(to_np(splits), splits_o)
+    assert np.array_equal(np.concatenate([to_np(i) for i in indices]), idx_o)
+    assert np.array_equal(np.concatenate([to_np(v) for v in values]), val_o)
+
+
+def test_slab_load_balance_too_many_candidates_declines(zen, oracle):
+    """A capacity far below what is selected: the candidate list overflows, the
+    call declines instead of writing out of bounds."""
+    from zen_repro_amd import _lib
+
+    n, P = 1 << 23, 8
+    g = make_grad(oracle, n, 0.05, "f32", seed=5)
+    capacity = 1 << 16  # about a sixth of the nonzeros
+    assert lb_path(zen, n, P, "f32", capacity) == SLAB
+    tp = zen.TensorPartition(P, 1, 3)
+    _, _, _, status = tp.load_balance_flat(to_dev(g), capacity=capacity, mode=_lib.MODE_FAST)
+    assert status.item() & (_lib.STAT_RETRY | _lib.STAT_CAPACITY)
+
+
+def test_slab_load_balance_threshold_given(zen, oracle):
+    """Selection by a threshold the caller computed (topk_threshold) instead of k."""
+    from zen_repro_amd import _lib
+
+    n, P = 1 << 24, 16
+    rng = np.random.default_rng(8)
+    g = oracle.f32_to_bf16_bits((rng.standard_normal(n) * 1e-3).astype(np.float32))
+    k = n // 100
+    key = oracle.kth_key(g, k)
+    masked, kept = oracle.mask_dense(g, key)
+    idx_o, val_o, splits_o, _ = oracle.load_balance(masked, P, 1, 3)
+    d = to_dev(g)
+    thr = zen.topk_threshold(d, k)
+    capacity = kept + 4096
+    assert lb_path(zen, n, P, "bf16", capacity) == SLAB
+    tp = zen.TensorPartition(P, 1, 3)
+    oi, ov, splits, status = tp.load_balance_flat(d, thr=thr, capacity=capacity)
+    assert status.item() == 0 and np.array_equal(to_np(splits), splits_o)
+    assert np.array_equal(to_np(oi)[:kept], idx_o) and np.array_equal(to_np(ov)[:kept], val_o)
+
+
+def test_two_slots_in_flight_give_the_same_answer(zen, oracle):
+    """Two encodes and two merges enqueued on four streams, each pair with its
+    own slot (workspace and table): same bytes as one call alone."""
+    n, P = 1 << 24, 16
+    rng = np.random.default_rng(21)
+    g = oracle.f32_to_bf16_bits((rng.standard_normal(n) * 1e-3).astype(np.float32))
+    d = to_dev(g)
+    k = n // 200
+    capacity = int(1.3 * k) + 4096
+    assert lb_path(zen, n, P, "bf16", capacity, k=k) == SLAB
+    tp = zen.TensorPartition(P, 1, 3)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P), None, None)
+    mi = to_dev(rng.integers(1, n, 400000).astype(np.int32))
+    mv = to_dev((rng.standard_normal(400000) * 1e-3).astype(np.float32))
+    ref = tp.load_balance_flat(d, capacity=capacity, k=k)
+    ref_m = lba.merge_sparse_flat(mi, mv, n)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    outs = []
+    for rep in range(3):
+        for slot in range(2):
+            with torch.cuda.stream(streams[slot]):
+                outs.append(("e", tp.load_balance_flat(d, capacity=capacity, k=k, slot=slot)))
+            with torch.cuda.stream(streams[2 + slot]):
+                outs.append(("m", lba.merge_sparse_flat(mi, mv, n, slot=slot)))
+    torch.cuda.synchronize()
+    total = int(ref[2].sum())
+    for kind, o in outs:
+        if kind == "e":
+            assert o[3].item() == 0 and torch.equal(o[2], ref[2])
+            assert torch.equal(o[0][:total], ref[0][:total]) and torch.equal(o[1][:total], ref[1][:total])
+        else:
+            cnt = int(ref_m[2])
+            assert o[3].item() == 0 and int(o[2]) == cnt
+            assert torch.equal(o[0][:cnt], ref_m[0][:cnt]) and torch.equal(o[1][:cnt], ref_m[1][:cnt])
+
+
+# ------------------------------------------------------------------ merge
+
+
+def payloads(oracle, rng, n, peers, per_peer, overlap, dtype):
+    pool = rng.choice(n, max(1, int(per_peer * overlap) * 2), replace=False)
+    idx, val = [], []
+    for _ in range(peers):
+        shared = rng.choice(pool, int(per_peer * overlap), replace=False) if overlap > 0 else np.empty(0, np.int64)
+        own = rng.integers(0, n, per_peer - len(shared))
+        i = np.concatenate([shared, own])
+        rng.shuffle(i)
+        v = (rng.standard_normal(len(i)) * 1e-3).astype(np.float32)
+        idx.append(i)
+        val.append(oracle.f32_to_bf16_bits(v) if dtype == "bf16" else v)
+    return np.concatenate(idx), np.concatenate(val)
+
+
+@pytest.mark.parametrize("idx64", [False, True])
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("n,peers,per_peer,overlap", [
+    (1 << 24, 16, 20000, 0.3),
+    (50000000, 64, 4000, 0.5),   # every shared index arrives 64 times
+    ((1 << 23) + 12345, 4, 30000, 0.0),
+])
+def test_slab_merge_bit_exact(zen, oracle, n, peers, per_peer, overlap, dtype, idx64):
+    from zen_repro_amd import _lib
+
+    rng = np.random.default_rng(n % 1000 + peers)
+    ci, cv = payloads(oracle, rng, n, peers, per_peer, overlap, dtype)
+    ci = ci.astype(np.int64 if idx64 else np.int32)
+    assert _lib.lib().zen_merge_path(len(ci), n, _lib.MODE_FAST) == SLAB
+    want_i, want_v = oracle.merge_sparse(ci, cv, n)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(peers), None, None)
+    gi, gv, cnt, st = lba.merge_sparse_flat(to_dev(ci), to_dev(cv), n, idx64=idx64, mode=_lib.MODE_FAST)
+    assert st.item() == 0 and cnt.item() == len(want_i)
+    assert np.array_equal(to_np(gi)[:len(want_i)], want_i.astype(np.int64 if idx64 else np.int32))
+    # same adds in the same order as a sequential scatter_add_: bit-exact
+    assert np.array_equal(to_np(gv)[:len(want_i)].view(np.uint32), want_v.view(np.uint32))
+    # and the dense form of the same merge
+    dense = lba.decode_sparse_tensors(to_dev(ci), to_dev(cv), n)
+    f32 = oracle.decode(ci, cv, n, "f32acc")
+    assert np.array_equal(to_np(dense), oracle.f32_to_bf16_bits(f32) if dtype == "bf16" else f32)
+
+
+def test_slab_merge_bad_indices_cancellation_and_pile_up(zen, oracle):
+    from zen_repro_amd import _lib
+
+    n = 1 << 24
+    rng = np.random.default_rng(17)
+    idx = rng.integers(0, n, 200000).astype(np.int64)
+    val = (rng.standard_normal(len(idx)) * 1e-3).astype(np.float32)
+    idx[1000:1100] = idx[0:100]          # pairs that cancel exactly
+    val[1000:1100] = -val[0:100]
+    idx[5000] = -7                        # out of range on both sides
+    idx[5001] = n
+    assert _lib.lib().zen_merge_path(len(idx), n, _lib.MODE_FAST) == SLAB
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(4), None, None)
+    gi, gv, cnt, st = lba.merge_sparse_flat(to_dev(idx), to_dev(val), n, idx64=True, mode=_lib.MODE_FAST)
+    assert st.item() == _lib.STAT_BAD_INDEX
+    good = (idx >= 0) & (idx < n)
+    wi, wv = oracle.merge_sparse(idx[good], val[good], n)
+    assert cnt.item() == len(wi)
+    assert np.array_equal(to_np(gi)[:len(wi)], wi) and np.array_equal(to_np(gv)[:len(wi)].view(np.uint32), wv.view(np.uint32))
+    # one index received 50000 times: the slab path declines, the general mode answers
+    idx2 = np.concatenate([np.full(50000, 4242), rng.integers(0, n, 100000)]).astype(np.int32)
+    val2 = (rng.standard_normal(len(idx2)) * 1e-3).astype(np.float32)
+    _, _, _, st2 = lba.merge_sparse_flat(to_dev(idx2), to_dev(val2), n, mode=_lib.MODE_FAST)
+    assert st2.item() & _lib.STAT_RETRY
+    gi2, gv2 = lba.merge_sparse(to_dev(idx2), to_dev(val2), n)
+    wi2, wv2 = oracle.merge_sparse(idx2, val2, n)
+    assert np.array_equal(to_np(gi2), wi2) and np.array_equal(to_np(gv2).view(np.uint32), wv2.view(np.uint32))

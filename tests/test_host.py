@@ -44,6 +44,20 @@ def test_workspace_queries_are_host_only(L):
     assert L.zen_decode_dense_workspace(1000, 5000) > L.zen_merge_workspace(1000, 5000)
 
 
+def test_path_selection_is_host_only(L):
+    """Which implementation a call takes depends on sizes alone."""
+    # c3: 743 M bf16 elements, top 0.5 %, 16 partitions -> bucket slabs; fp32 top-k is not on that path
+    assert L.zen_load_balance_path(743440384, 743440384, 1, 4650000, 16, 3717201, 0) == 2
+    assert L.zen_load_balance_path(743440384, 743440384, 0, 4650000, 16, 3717201, 0) == 1
+    assert L.zen_load_balance_path(743440384, 743440384, 0, 4650000, 16, 0, 0) == 2
+    assert L.zen_load_balance_path(743440384, 743440384, 1, 4650000, 16, 3717201, 1) == 0   # general mode
+    assert L.zen_load_balance_path(1 << 20, 1 << 20, 1, 1 << 14, 4, 0, 0) == 1             # small table
+    assert L.zen_load_balance_path(1 << 24, 1 << 24, 1, 1 << 24, 16, 0, 0) == 1            # capacity = everything
+    assert L.zen_merge_path(3717200, 743440384, 0) == 2
+    assert L.zen_merge_path(3717200, 743440384, 1) == 0
+    assert L.zen_merge_path(1000, 1 << 20, 0) == 0
+
+
 def test_bad_arguments_are_rejected_on_the_host(L):
     from zen_repro_amd import _lib
 

@@ -51,7 +51,9 @@ def lib():
         "zen_select": (i32, [vp, i32, i64, vp, vp, i32, vp, i64, vp, vp, sz, vp, vp]),
         "zen_load_balance_workspace": (sz, [i64, i64, i32, i64, i32]),
         "zen_load_balance": (i32, [vp, i32, i64, i64, i32, i32, vp, i64, vp, vp, vp, i64, vp, vp, i32, vp, sz, vp, vp]),
+        "zen_load_balance_path": (i32, [i64, i64, i32, i64, i32, i64, i32]),
         "zen_merge_workspace": (sz, [i64, i64]),
+        "zen_merge_path": (i32, [i64, i64, i32]),
         "zen_merge": (i32, [vp, i32, vp, i32, i64, i64, vp, i32, vp, i64, vp, i32, vp, sz, vp, vp]),
         "zen_decode_dense_workspace": (sz, [i64, i64]),
         "zen_decode_dense": (i32, [vp, i32, vp, i32, i64, vp, i64, i32, vp, sz, vp, vp]),

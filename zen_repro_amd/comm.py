@@ -108,13 +108,15 @@ class LoadBalanceAllreduce:
         return idx, val
 
     def merge_sparse_flat(self, indices_tensors, values_tensors, dense_size, capacity=None, idx64=False,
-                          mode=_lib.MODE_FAST):
+                          mode=_lib.MODE_FAST, slot=0):
         """decode_sparse_tensors followed by encode_sparse_tensor (comm.py:125-127)
         without the dense intermediate and without host synchronisation.
         Returns (indices, fp32 sums, count int64[1], status int32[1]); the first
         `count` entries are valid and ascending.  In fast mode a status with
         STAT_RETRY means the outputs are unspecified and the call must be repeated
-        with mode=MODE_GENERAL (merge_sparse does that by itself)."""
+        with mode=MODE_GENERAL (merge_sparse does that by itself).  Calls that
+        may be in flight at the same time must use different `slot` numbers
+        (a slot owns its workspace)."""
         indices = self.stack_tensors(indices_tensors)
         values = self.stack_tensors(values_tensors)
         _lib.require_gpu(indices, "indices")
@@ -128,7 +130,7 @@ class LoadBalanceAllreduce:
         out_val = torch.empty(capacity, dtype=torch.float32, device=dev)
         count = torch.zeros(1, dtype=torch.int64, device=dev)
         status = _lib.status_word(dev)
-        ws = _lib.scratch.get(dev, "merge", L.zen_merge_workspace(r, dense_size))
+        ws = _lib.scratch.get(dev, f"merge/{slot}", L.zen_merge_workspace(r, dense_size))
         rc = L.zen_merge(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(values),
                          _lib.dtype_code(values), r, dense_size, _lib.ptr(out_idx), 1 if idx64 else 0,
                          _lib.ptr(out_val), capacity, _lib.ptr(count), mode, _lib.ptr(ws), ws.numel(),

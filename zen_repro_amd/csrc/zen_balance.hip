@@ -372,6 +372,12 @@ size_t zen_load_balance_workspace(int64_t n, int64_t m, int dtype, int64_t capac
   return general > slabs ? general : slabs;
 }
 
+int zen_load_balance_path(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions, int64_t k, int mode) {
+  if (mode != ZEN_MODE_FAST || partitions <= 0 || m <= 0 || m % partitions != 0) return 0;
+  if (zen::slab_balance_fits(n, m, partitions, dtype, capacity, k, nullptr)) return 2;
+  return m >= 4096 ? 1 : 0;
+}
+
 int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
                      const uint32_t *thr, int64_t k, uint32_t *thr_out, int32_t *out_idx, void *out_val,
                      int64_t capacity, int64_t *splits, int32_t *table, int mode, void *workspace,

@@ -478,6 +478,12 @@ size_t zen_merge_workspace(int64_t r, int64_t dense_n) {
   return zen::plan_merge(nullptr, r, dense_n).bytes;
 }
 
+int zen_merge_path(int64_t r, int64_t dense_n, int mode) {
+  if (mode != ZEN_MODE_FAST || r <= 0 || dense_n <= 0) return 0;
+  if (zen::slab_merge_fits(r, dense_n, nullptr)) return 2;
+  return zen::bucket_sort_fits(r, (uint32_t)dense_n) ? 1 : 0;
+}
+
 int zen_merge(const void *idx, int idx64_in, const void *val, int dtype, int64_t r, int64_t dense_n, void *out_idx,
               int idx64_out, float *out_val, int64_t capacity, int64_t *out_count, int mode, void *workspace,
               size_t workspace_bytes, int32_t *status, void *stream) {

@@ -3,7 +3,6 @@
 // (train.py:83), and the ordered single-pass compaction that turns a dense
 // tensor into ascending (index, value) lists (comm.py:47-50).
 #include <math.h>
-#include <stdlib.h>
 
 #include "zen_select.h"
 
@@ -162,7 +161,7 @@ __device__ inline void sample_pick_block(const uint32_t *hist, uint32_t rank, in
 template <typename S, bool ALIGNED>
 __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restrict__ in, int64_t n, int block_log2,
                                                               uint32_t *__restrict__ hist, uint32_t rank,
-                                                              uint32_t *floor_out, bool fused) {
+                                                              uint32_t *floor_out) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kShift = KeyOf<S>::kBits - 15;
   // one pad word per 32: the flush below reads 16 consecutive words per thread, which would otherwise put
@@ -238,13 +237,7 @@ __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restric
   if (threadIdx.x == 0) s_last = atomicAdd(&hist[kFineBins], 1u) == gridDim.x - 1;
   __syncthreads();
   if (!s_last) return;
-  if (fused) sample_pick_block(hist, rank, kShift, floor_out, smem);
-}
-
-__global__ __launch_bounds__(kSampleBlock) void k_sample_pick(const uint32_t *hist, uint32_t rank, int key_shift,
-                                                              uint32_t *floor_out) {
-  __shared__ uint32_t smem[kSampleBlock / 64 + 1];
-  sample_pick_block(hist, rank, key_shift, floor_out, smem);
+  sample_pick_block(hist, rank, kShift, floor_out, smem);
 }
 
 // Run by one whole block (BLOCK threads) over the complete candidate
@@ -648,7 +641,7 @@ int select_compact(const SelectArgs &a, hipStream_t stream) {
 // is flushed to the output list with one reservation and coalesced stores; the
 // candidate histogram is taken at flush time.
 
-constexpr int kScatStage = 4096;
+constexpr int kScatStage = 2048;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -866,6 +859,8 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   const int64_t tile = (int64_t)kSelBlock * kSelVecs * V * subs;
   const int64_t ntiles = ceil_div(a.n, tile);
   if (ntiles > 0x3fffffff) return fail(ZEN_EINVAL, "select_stage: too many tiles");
+  // three workgroups per compute unit (measured: two are 10 % slower, four no faster); their LDS, 60 KB per
+  // unit, leaves room for another stream's kernels next to this long one
   int64_t blocks = (int64_t)device_cus() * 3;
   if (blocks > ntiles) blocks = ntiles;
   const S *in = static_cast<const S *>(a.in);
@@ -949,20 +944,15 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
   int64_t blocks = ceil_div(nblocks * V, 32768);
   if (blocks < 128) blocks = 128;
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
-  const bool fused = getenv("ZSPLIT") == nullptr;
   {
     ProfScope prof(kProfTopkHist, stream);
     if (aligned)
       k_sample_hist<S, true><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist, rank,
-                                                                                        thr_lo, fused);
+                                                                                        thr_lo);
     else
       k_sample_hist<S, false><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist,
-                                                                                         rank, thr_lo, fused);
+                                                                                         rank, thr_lo);
     ZEN_LAUNCH_CHECK("k_sample_hist");
-    if (!fused) {
-      k_sample_pick<<<dim3(1), dim3(kSampleBlock), 0, stream>>>(hist, rank, KeyOf<S>::kBits - 15, thr_lo);
-      ZEN_LAUNCH_CHECK("k_sample_pick");
-    }
   }
   return ZEN_OK;
 }

@@ -64,16 +64,17 @@ class TensorPartition:
         return pos, val.view(torch.int32)
 
     # ------------------------------------------------------- fused path
-    def _table(self, device, m):
-        key = (torch.device(device), m)
+    def _table(self, device, m, slot=0):
+        key = (torch.device(device), m, slot)
         t = self._tables.get(key)
         if t is None:
-            self._tables.clear()  # one table per partitioner: sizes rarely change
+            # one table per partitioner and slot: sizes rarely change
+            self._tables = {k: v for k, v in self._tables.items() if k[:2] == key[:2]}
             t = torch.zeros(m, dtype=torch.int32, device=device)
             self._tables[key] = t
         return t
 
-    def load_balance_flat(self, tensor, thr=None, capacity=None, k=0, mode=_lib.MODE_FAST, thr_out=None):
+    def load_balance_flat(self, tensor, thr=None, capacity=None, k=0, mode=_lib.MODE_FAST, thr_out=None, slot=0):
         """Fused path without host synchronisation.  Returns (indices int32
         [capacity], values [capacity], splits int64[P] on device, status int32[1]
         on device); the first splits.sum() entries are valid, partition-major.
@@ -81,7 +82,10 @@ class TensorPartition:
         an int32[2] device tensor, receives the threshold key and the count);
         else `thr` is the device tensor written by topk_threshold; else the
         nonzeros.  A status with STAT_RETRY (fast mode only) means the call
-        must be repeated with mode=MODE_GENERAL; load_balance does that."""
+        must be repeated with mode=MODE_GENERAL; load_balance does that.
+        Calls that may be in flight at the same time (different streams, e.g.
+        one gradient bucket's encode next to the previous bucket's) must use
+        different `slot` numbers: a slot owns its workspace and its table."""
         _lib.require_gpu(tensor, "input")
         flat = tensor.reshape(-1)
         n = flat.numel()
@@ -96,8 +100,8 @@ class TensorPartition:
         splits = torch.zeros(self.partitions, dtype=torch.int64, device=dev)
         status = _lib.status_word(dev)
         nbytes = L.zen_load_balance_workspace(n, m, code, capacity, self.partitions)
-        ws = _lib.scratch.get(dev, "load_balance", nbytes)
-        table = self._table(dev, m)
+        ws = _lib.scratch.get(dev, f"load_balance/{slot}", nbytes)
+        table = self._table(dev, m, slot)
         rc = L.zen_load_balance(
             _lib.ptr(flat), code, n, m, self.partitions, self.rehash, _lib.ptr(thr), int(k), _lib.ptr(thr_out),
             _lib.ptr(out_idx), _lib.ptr(out_val), capacity, _lib.ptr(splits), _lib.ptr(table), mode,
