@@ -17,9 +17,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the dominant kernel on the full c3 workload, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by what the same counters read
-# for a plain 1 GiB copy (profiles/c3_select_compact_hbm_traffic.txt).  Other
+# for a plain 1 GiB copy (profiles/c3_select_stage_hbm_traffic.txt).  Other
 # workloads report null.
-MEASURED_TRAFFIC = {("c3", 1, "k_select_compact"): 1.519e9}
+MEASURED_TRAFFIC = {("c3", 1, "k_select_stage"): 1.513e9}
 
 
 def parse():
@@ -35,7 +35,7 @@ def parse():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run five device copies of 1 GiB and exit (scale for hardware byte counters)")
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
-    ap.add_argument("--depth", type=int, default=2,
+    ap.add_argument("--depth", type=int, default=1,
                     help="gradient buckets in flight: step i+1 is enqueued on its own streams next to step i "
                          "(1 = a step starts when the previous one has finished)")
     ap.add_argument("--no-kernel-timing", action="store_true",
@@ -176,6 +176,7 @@ def main():
     # dominant kernel: the one with the largest summed duration among the
     # kernels that stream the dense gradient; its algorithmic bytes per launch
     per_launch = {
+        "k_select_stage": n * esize + nnz * (4 + esize),
         "k_select_compact": n * esize + nnz * (4 + esize),
         "k_topk_hist": n * esize,
     }

@@ -72,6 +72,13 @@ enum ProfTag {
   kProfMergeReduce,
   kProfCompress,
   kProfInsertDense,
+  kProfSelectStage,
+  kProfFeed,
+  kProfSlabSort,
+  kProfSlabChains,
+  kProfSlabPlace,
+  kProfMergeFeed,
+  kProfMergeBucket,
   kProfCount
 };
 

@@ -355,7 +355,7 @@ int slab_merge_launch(const SlabGeom &geo, const I *idx, const S *val, int64_t r
   launch_fill<unsigned long long>(p.scan, 0ull, p.zero_bytes / sizeof(unsigned long long), s);
   ZEN_LAUNCH_CHECK("merge: clear prefix state");
   {
-    ProfScope prof(kProfMergePrep, s);
+    ProfScope prof(kProfMergeFeed, s);
     const MergeCountSrc<I> csrc{idx, (uint32_t)dense_n, status};
     const MergeWriteSrc<I, S> wsrc{idx, val, (uint32_t)dense_n};
     const int rc = feed_slabs(geo, csrc, wsrc, nullptr, r, p.hist, p.cursor, p.bucket_lo, p.slab_rec, status, s);
@@ -363,7 +363,7 @@ int slab_merge_launch(const SlabGeom &geo, const I *idx, const S *val, int64_t r
   }
   const ScanState st = scan_state(p.scan, (int64_t)geo.nbuckets);
   const int tie_bits = ceil_log2_u64((uint64_t)r);  // arrival numbers are < r
-  ProfScope prof(kProfMergeReduce, s);
+  ProfScope prof(kProfMergeBucket, s);
   if (idx64_out)
     k_merge_bucket<int64_t><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
         geo, p.cursor, p.bucket_lo, p.slab_rec, static_cast<int64_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);

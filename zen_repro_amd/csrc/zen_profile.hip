@@ -21,6 +21,8 @@ std::vector<Span> g_spans;
 const char *const kNames[kProfCount] = {
     "k_topk_hist", "k_select_compact", "k_insert_list", "k_final_key", "sort_pairs",
     "k_gather",    "k_merge_prep",     "k_merge_reduce", "k_compress", "k_insert_dense",
+    "k_select_stage", "k_feed_count+scan+write", "k_slab_sort", "k_slab_chains+classify", "k_slab_place",
+    "merge: k_feed_count+scan+write", "k_merge_bucket",
 };
 
 void drop_spans() {

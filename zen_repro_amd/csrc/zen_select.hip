@@ -865,7 +865,7 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   if (blocks > ntiles) blocks = ntiles;
   const S *in = static_cast<const S *>(a.in);
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
-  ProfScope prof(kProfSelectCompact, stream);
+  ProfScope prof(kProfSelectStage, stream);
   if (aligned)
     k_select_stage<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
         in, a.n, a.thr, a.list_count, a.list_idx, static_cast<S *>(a.list_val), (uint32_t)a.capacity, a.ticket,

@@ -130,8 +130,7 @@ struct EncodeWriteSrc {
 // ------------------------------------------------------------ sort a bucket
 
 template <typename S>
-__global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTables tb, const S *__restrict__ dense,
-                                                          int32_t *status) {
+__global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTables tb, int32_t *status) {
   __shared__ SlabSortShared sh;
   __shared__ S s_val[kSlabCap];
   __shared__ uint32_t s_lost, s_base;
@@ -655,25 +654,28 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
   const uint32_t *filter = a.k > 0 ? p.thr : nullptr;
   const S *dense = static_cast<const S *>(a.input);
   {
-    ProfScope prof(kProfInsertList, s);
+    ProfScope prof(kProfFeed, s);
     const S *list_val = static_cast<const S *>(p.list_val);
     const EncodeCountSrc<S> csrc{geo, p.list_idx, list_val, filter, p.list_key};
     const EncodeWriteSrc<S> wsrc{p.list_idx, list_val, p.list_key};
     const int rc = feed_slabs(geo, csrc, wsrc, p.list_count, p.list_cap, p.feed_hist, p.tb.cursor, p.tb.bucket_lo,
                               p.tb.slab_rec, a.status, s);
     if (rc != ZEN_OK) return rc;
-    k_slab_sort<S><<<dim3(B), dim3(kSlabBlock), 0, s>>>(geo, p.tb, dense, a.status);
+  }
+  {
+    ProfScope prof(kProfSlabSort, s);
+    k_slab_sort<S><<<dim3(B), dim3(kSlabBlock), 0, s>>>(geo, p.tb, a.status);
     ZEN_LAUNCH_CHECK("k_slab_sort");
   }
   {
-    ProfScope prof(kProfFinalKey, s);
+    ProfScope prof(kProfSlabChains, s);
     k_slab_chains<S><<<dim3(256), dim3(256), 0, s>>>(geo, a.g, p.tb, a.hash, a.hash_log2, a.status);
     ZEN_LAUNCH_CHECK("k_slab_chains");
     k_slab_classify<<<dim3(128), dim3(kSlabBlock), 0, s>>>(geo, a.g, p.tb, a.hash, a.hash_log2, a.spp, a.status);
     ZEN_LAUNCH_CHECK("k_slab_classify");
   }
   {
-    ProfScope prof(kProfGather, s);
+    ProfScope prof(kProfSlabPlace, s);
     k_slab_place<S><<<dim3(B), dim3(kSlabBlock), 0, s>>>(geo, p.tb, a.hash, a.partitions, a.spp, dense, a.out_idx,
                                                          static_cast<S *>(a.out_val), (uint32_t)a.capacity, a.splits,
                                                          a.status);
