@@ -35,6 +35,8 @@ def parse():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run five device copies of 1 GiB and exit (scale for hardware byte counters)")
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
+    ap.add_argument("--merge-follows", action="store_true",
+                    help="with --depth: a step's merge runs on its encode's stream, after it")
     ap.add_argument("--depth", type=int, default=1,
                     help="gradient buckets in flight: step i+1 is enqueued on its own streams next to step i "
                          "(1 = a step starts when the previous one has finished)")
@@ -123,7 +125,8 @@ def main():
     depth = 1 if args.one_stream else max(1, args.depth)
     main = torch.cuda.current_stream(dev)
     enc_streams = [main] + [torch.cuda.Stream(device=dev) for _ in range(depth - 1)]
-    mrg_streams = [None if args.one_stream else torch.cuda.Stream(device=dev) for _ in range(depth)]
+    mrg_streams = [None if (args.one_stream or args.merge_follows) else torch.cuda.Stream(device=dev)
+                   for _ in range(depth)]
 
     def step(i):
         slot = i % depth

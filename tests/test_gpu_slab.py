@@ -63,6 +63,32 @@ def test_slab_load_balance_bit_exact(zen, oracle, n, P, density, rehash, dtype):
     assert not tp._table(d.device, m).any()
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_slab_load_balance_odd_length_unaligned_and_empty(zen, oracle, dtype):
+    """A tensor whose length is no multiple of anything and whose first element is not 16-byte aligned (the
+    streaming kernel's element-wise loads and its ragged last tile), and a tensor of zeros."""
+    from zen_repro_amd import _lib
+
+    n, P = (1 << 23) + 1237, 16
+    g = make_grad(oracle, n, 0.03, dtype, seed=4242)
+    g[-1] = 0x3F80 if dtype == "bf16" else 1.0  # the very last element is selected
+    idx_o, val_o, splits_o, st_o = oracle.load_balance(g, P, 1, 3)
+    assert st_o == 0
+    capacity = len(idx_o) + 2048
+    assert lb_path(zen, n, P, dtype, capacity) == SLAB
+    buf = to_dev(np.concatenate([g[:3], g]))
+    d = buf[3:]
+    assert d.data_ptr() % 16 != 0
+    tp = zen.TensorPartition(P, 1, 3)
+    oi, ov, splits, status = tp.load_balance_flat(d, capacity=capacity)
+    total = int(splits_o.sum())
+    assert status.item() == 0 and np.array_equal(to_np(splits), splits_o)
+    assert np.array_equal(to_np(oi)[:total], idx_o) and np.array_equal(to_np(ov)[:total], val_o)
+    zeros = torch.zeros(n, dtype=d.dtype, device="cuda")
+    oi, ov, splits, status = tp.load_balance_flat(zeros, capacity=capacity)
+    assert status.item() == 0 and int(splits.sum()) == 0
+
+
 def test_slab_load_balance_declines_and_general_mode_takes_over(zen, oracle):
     """One rehash level at 15 % load sends every level-1 loser to the serial
     lists: far more than the slab path carries per partition.  It must say so

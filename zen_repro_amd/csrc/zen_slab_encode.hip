@@ -70,9 +70,20 @@ __global__ __launch_bounds__(kScanCols * kScanChunks) void k_feed_scan(SlabGeom 
   const uint32_t per = (batches + kScanChunks - 1) / kScanChunks;
   const uint32_t r0 = chunk * per < batches ? chunk * per : batches;
   const uint32_t r1 = r0 + per < batches ? r0 + per : batches;
+  // the loads of a thread do not depend on each other: eight at a time are in flight (a plain loop would
+  // wait for each before asking for the next)
   uint32_t sum = 0;
-  if (b < row_words)
-    for (uint32_t r = r0; r < r1; ++r) sum += hist[(size_t)r * row_words + b];
+  if (b < row_words) {
+    uint32_t r = r0;
+    for (; r + 8 <= r1; r += 8) {
+      uint32_t x[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) x[q] = hist[(size_t)(r + q) * row_words + b];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) sum += x[q];
+    }
+    for (; r < r1; ++r) sum += hist[(size_t)r * row_words + b];
+  }
   s_sum[chunk][col] = sum;
   __syncthreads();
   uint32_t running = 0, total = 0;
@@ -81,12 +92,24 @@ __global__ __launch_bounds__(kScanCols * kScanChunks) void k_feed_scan(SlabGeom 
     if ((uint32_t)c < chunk) running += x;
     total += x;
   }
-  if (b < row_words)
-    for (uint32_t r = r0; r < r1; ++r) {
+  if (b < row_words) {
+    uint32_t r = r0;
+    for (; r + 8 <= r1; r += 8) {
+      uint32_t x[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) x[q] = hist[(size_t)(r + q) * row_words + b];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        hist[(size_t)(r + q) * row_words + b] = running;
+        running += x[q];
+      }
+    }
+    for (; r < r1; ++r) {
       const uint32_t x = hist[(size_t)r * row_words + b];
       hist[(size_t)r * row_words + b] = running;
       running += x;
     }
+  }
   if (chunk == 0 && b < nbuckets) {
     cursor[b] = total;
     bucket_lo[b] = geo.first_key(b);  // a 64-bit division: once per bucket here, not once per thread later
