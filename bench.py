@@ -149,14 +149,25 @@ def main():
 
     run(args.warmup)
     torch.cuda.synchronize()
+    # An event between two kernels costs the device a few microseconds, about 40 of them per step with every
+    # stage timed.  So the stage breakdown comes from an untimed pass of its own, and in the timed region only
+    # the dominant kernel (the one the roofline figure is about) carries events.
+    streaming = ("k_select_stage", "k_select_compact", "k_topk_hist")  # kernels that read the dense gradient
+    stages, dom = {}, None
     if not args.no_kernel_timing:
         _lib.profile_enable(True)
+        run(args.steps)
+        torch.cuda.synchronize()
+        stages = _lib.profile_read()
+        cands = [(stages[name][0], name) for name in streaming if name in stages]
+        dom = max(cands)[1] if cands else None
+        _lib.profile_enable(dom is not None, only=dom)
     t0 = time.perf_counter()
     outs = run(args.steps)
     t_enq = time.perf_counter()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    kernels = {} if args.no_kernel_timing else _lib.profile_read()
+    kernels = _lib.profile_read() if dom else {}
     _lib.profile_enable(False)
 
     (o_idx, o_val, splits, st_enc), (m_idx, m_val, m_count, st_mrg) = outs[-1]
@@ -184,10 +195,8 @@ def main():
         "k_topk_hist": n * esize,
     }
     roofline = None
-    stage_ms = {name: round(total / args.steps, 4) for name, (total, _) in kernels.items()}
-    cands = [(kernels[name][0], name) for name in per_launch if name in kernels]
-    if cands:
-        _, dom = max(cands)
+    stage_ms = {name: round(total / args.steps, 4) for name, (total, _) in stages.items()}
+    if dom in kernels:
         total_ms, launches = kernels[dom]
         avg_ms = total_ms / launches
         achieved = per_launch[dom] / (avg_ms * 1e-3) / 1e9
@@ -217,6 +226,8 @@ def main():
         "path_frac_of_hbm_peak": round(b_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "host_enqueue_ms_per_step": round((t_enq - t0) * 1e3 / args.steps, 4),
         "stage_ms_per_step": stage_ms,
+        "stage_ms_note": "from an untimed pass with every stage's events on; the timed region times only the "
+                         "roofline kernel",
         "roofline": roofline,
         "cpu_baseline": None,
     }

@@ -238,9 +238,12 @@ int zen_bucket_sort_pairs(uint32_t *keys, uint32_t *vals, int64_t max_count,
  * (tensor_load_balance.py:25-38, comm.py:66-144).  zen_profile_enable(1)
  * clears earlier samples and starts recording; zen_profile_read synchronises
  * on the recorded events of one tag and returns their summed duration and the
- * number of launches.  Process-wide, serialised by a mutex.
+ * number of launches.  An event between two kernels costs a few microseconds
+ * on the device: zen_profile_only(tag) limits the recording to one tag (a
+ * negative tag lifts the limit).  Process-wide, serialised by a mutex.
  */
 int zen_profile_enable(int on);
+int zen_profile_only(int tag);
 int zen_profile_tags(void);
 const char *zen_profile_name(int tag);
 int zen_profile_read(int tag, double *total_ms, int64_t *launches);

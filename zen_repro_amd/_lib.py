@@ -62,6 +62,7 @@ def lib():
         "zen_bucket_sort_fits": (i32, [i64, ctypes.c_uint32]),
         "zen_bucket_sort_pairs": (i32, [vp, vp, i64, vp, ctypes.c_uint32, vp, sz, vp, vp]),
         "zen_profile_enable": (i32, [i32]),
+        "zen_profile_only": (i32, [i32]),
         "zen_profile_tags": (i32, []),
         "zen_profile_name": (ctypes.c_char_p, [i32]),
         "zen_profile_read": (i32, [i32, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]),
@@ -150,8 +151,15 @@ def describe_status(bits):
     return ", ".join(names) or "ok"
 
 
-def profile_enable(on=True):
-    check(lib().zen_profile_enable(1 if on else 0), "profile_enable")
+def profile_enable(on=True, only=None):
+    """Start (or stop) timing the tagged launches; `only` names the one kernel tag to time."""
+    L = lib()
+    tag = -1
+    if only is not None:
+        names = [L.zen_profile_name(t).decode() for t in range(L.zen_profile_tags())]
+        tag = names.index(only)
+    check(L.zen_profile_only(tag), "profile_only")
+    check(L.zen_profile_enable(1 if on else 0), "profile_enable")
 
 
 def profile_read():

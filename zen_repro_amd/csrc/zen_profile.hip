@@ -16,7 +16,21 @@ struct Span {
 
 std::mutex g_mu;
 bool g_on = false;
+int g_only = -1;  // >= 0: only launches with this tag are timed
 std::vector<Span> g_spans;
+std::vector<hipEvent_t> g_spare;  // created ahead of the timed launches: creating an event costs host time
+
+constexpr size_t kSpareEvents = 2048;
+
+hipEvent_t take_event() {
+  if (!g_spare.empty()) {
+    hipEvent_t e = g_spare.back();
+    g_spare.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  return hipEventCreate(&e) == hipSuccess ? e : nullptr;
+}
 
 const char *const kNames[kProfCount] = {
     "k_topk_hist", "k_select_compact", "k_insert_list", "k_final_key", "sort_pairs",
@@ -25,10 +39,10 @@ const char *const kNames[kProfCount] = {
     "merge: k_feed_count+scan+write", "k_merge_bucket",
 };
 
-void drop_spans() {
+void drop_spans() {  // the events go back to the spare list (a read has waited for them, or nobody will)
   for (Span &s : g_spans) {
-    (void)hipEventDestroy(s.start);
-    (void)hipEventDestroy(s.stop);
+    g_spare.push_back(s.start);
+    g_spare.push_back(s.stop);
   }
   g_spans.clear();
 }
@@ -37,9 +51,12 @@ void drop_spans() {
 
 ProfScope::ProfScope(int tag, hipStream_t stream) : tag_(tag), stream_(stream), start_(nullptr), stop_(nullptr) {
   std::lock_guard<std::mutex> lock(g_mu);
-  if (!g_on) return;
-  if (hipEventCreate(&start_) != hipSuccess || hipEventCreate(&stop_) != hipSuccess) {
-    start_ = stop_ = nullptr;
+  if (!g_on || (g_only >= 0 && tag != g_only)) return;
+  start_ = take_event();
+  stop_ = start_ ? take_event() : nullptr;
+  if (!stop_) {
+    if (start_) g_spare.push_back(start_);
+    start_ = nullptr;
     return;
   }
   (void)hipEventRecord(start_, stream_);
@@ -60,6 +77,18 @@ int zen_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(zen::g_mu);
   zen::drop_spans();
   zen::g_on = on != 0;
+  while (zen::g_on && zen::g_spare.size() < zen::kSpareEvents) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) break;
+    zen::g_spare.push_back(e);
+  }
+  return ZEN_OK;
+}
+
+int zen_profile_only(int tag) {
+  if (tag >= zen::kProfCount) return zen::fail(ZEN_EINVAL, "zen_profile_only: no such tag");
+  std::lock_guard<std::mutex> lock(zen::g_mu);
+  zen::g_only = tag < 0 ? -1 : tag;
   return ZEN_OK;
 }
 
