@@ -29,6 +29,7 @@ constexpr int kSlabSubsPer = kSlabSubs / kSlabBlock;
 constexpr int kSlabGroupLimit = 1024;                 // bounds the rank loop on piled-up keys
 constexpr int kSlabMaxBuckets = 2048;
 constexpr int kSlabTarget = 3584;                     // records a bucket is sized for (leaves 40 % to spare)
+constexpr int kSlabResident = 512;                    // per-bucket workgroups the chip holds at a time (256 CUs x 2)
 constexpr int kSlabMoveCap = 1024;                    // entries that may move into one bucket from elsewhere
 constexpr int kSlabSerialCap = 4096;                  // overflow entries per partition the fast path carries
 
@@ -88,6 +89,14 @@ inline bool slab_geometry(int64_t m, int partitions, int64_t expected, int targe
   int64_t bpp = ceil_div(expected, (int64_t)target * partitions);
   if (bpp < 1) bpp = 1;
   if (bpp * partitions > kSlabMaxBuckets) bpp = kSlabMaxBuckets / partitions;
+  // The per-bucket kernels run in rounds of kSlabResident workgroups, and a workgroup costs much the same whether
+  // its slab is half or three quarters full: a bucket count a little above a whole number of rounds wastes most
+  // of the last one.  Fewer, fuller buckets then do better, as long as a slab keeps a quarter to spare.
+  {
+    const int64_t rounds = ceil_div(bpp * partitions, (int64_t)kSlabResident);
+    const int64_t fewer = (rounds - 1) * kSlabResident / partitions;
+    if (fewer >= 1 && expected / (fewer * partitions) <= (int64_t)kSlabCap * 3 / 4) bpp = fewer;
+  }
   const int64_t nb = bpp * partitions;
   if (expected / nb > (int64_t)kSlabCap * 3 / 4) return false;  // too many records per bucket
   const int64_t npp = m / partitions;

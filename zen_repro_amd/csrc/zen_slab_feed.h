@@ -18,8 +18,8 @@ namespace zen {
 
 constexpr int kFeedItems = 8;
 constexpr int kFeedBatch = kSlabBlock * kFeedItems;  // list entries per workgroup
-constexpr int kScanChunks = 64;
-constexpr int kScanCols = 16;
+constexpr int kScanChunks = 32;
+constexpr int kScanCols = 8;  // 256 threads: a workgroup this small finds room on a CU other kernels are using
 constexpr uint32_t kNoSlot = 0xffffffffu;  // key of an entry that is dropped
 
 // Number of list entries: *list_count if given, never more than list_cap.
