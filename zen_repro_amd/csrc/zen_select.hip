@@ -711,16 +711,30 @@ __device__ inline void stage_flush(uint32_t count, const int32_t *st_idx, const 
   __syncthreads();
 }
 
+// How the sub-tiles (kSelBlock * kSelVecs vectors each) are handed out.  Every workgroup first takes
+// `fixed` tiles of kStageBig sub-tiles, tile i of workgroup b being number i * workgroups + b: no counter, and
+// neighbouring workgroups read neighbouring memory.  The rest of the tensor goes out in shorter tiles through a
+// ticket counter, so that workgroups that ran ahead take more and all finish within one short tile of each
+// other.  (A device-wide counter serves about 90 tickets per microsecond; 768 workgroups asking once per
+// kStageSmall sub-tiles stay below that.)
+constexpr int kStageBig = 16;
+constexpr int kStageSmall = 6;
+struct StageSched {
+  uint32_t fixed;        // counter-free tiles per workgroup
+  uint32_t fixed_subs;   // sub-tiles they cover together
+  uint32_t ticket_tiles; // tiles of kStageSmall sub-tiles after that
+};
+
 template <typename S, bool ALIGNED>
 __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
     const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, uint32_t *list_count,
-    int32_t *__restrict__ list_idx, S *__restrict__ list_val, uint32_t capacity, uint32_t *ticket, int ntiles,
-    int subs, uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *thr_copy, int32_t *status) {
+    int32_t *__restrict__ list_idx, S *__restrict__ list_val, uint32_t capacity, uint32_t *ticket, StageSched sch,
+    uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *thr_copy, int32_t *status) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kSub = kSelBlock * kSelVecs * V;
   constexpr int kWaves = kSelBlock / 64;
   __shared__ uint32_t s_wave[2][kWaves];
-  __shared__ int s_next[2];
+  __shared__ uint32_t s_next[2];
   __shared__ int32_t st_idx[kScatStage];
   __shared__ S st_val[kScatStage];
   __shared__ uint32_t s_base;
@@ -734,32 +748,48 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
   if (floor_key > KeyOf<S>::kMask) floor_key = KeyOf<S>::kMask + 1u;  // nothing qualifies
   const int wave = threadIdx.x >> 6;
 
-  // The first tile is the block's own number, later ones come from the ticket counter; the ticket for the
-  // tile after the current one is drawn while the current one is processed.  Two register sets take turns:
-  // while one sub-tile is examined the loads of the next one are in flight.
-  int tile = (int)blockIdx.x;
-  int turn = 0;        // tiles this block has started
+  // A tile is (first sub-tile, number of sub-tiles); length 0 means there is none.  The tile after the current
+  // one is always known before the current one ends: its ticket is drawn when the current tile starts and
+  // read behind the first barrier.  Three register sets take turns: while one sub-tile is examined the loads
+  // of the next two are in flight.
+  uint32_t cur_first = 0, cur_len = 0, nxt_first = 0, nxt_len = 0;
+  auto fixed_tile = [&](uint32_t i, uint32_t &first, uint32_t &len) {
+    first = (i * gridDim.x + blockIdx.x) * (uint32_t)kStageBig;
+    len = (uint32_t)kStageBig;
+  };
+  auto ticket_tile = [&](uint32_t j, uint32_t &first, uint32_t &len) {
+    first = sch.fixed_subs + j * (uint32_t)kStageSmall;
+    len = j < sch.ticket_tiles ? (uint32_t)kStageSmall : 0u;
+  };
+  uint32_t turn = 0;   // tiles this block has started
   uint32_t par = 0;    // sub-tiles this block has processed
   uint32_t count = 0;  // staged entries
-  int next_tile = ntiles;
+  bool ticket_pending = false;
   int64_t sub_base = 0;
-  int sub = 0;
-  uint4 qa[kSelVecs], qb[kSelVecs];
+  uint32_t sub = 0;
+  uint4 qa[kSelVecs], qb[kSelVecs], qc[kSelVecs];
 
-  // one sub-tile: cur holds its data, nxt receives the following sub-tile's
-  auto body = [&](uint4 (&cur)[kSelVecs], uint4 (&nxt)[kSelVecs]) {
+  // loads the sub-tile `ahead` places after the current one, if the block's sequence has one there
+  auto load_ahead = [&](uint32_t ahead, uint4 (&q)[kSelVecs]) {
+    const uint32_t p = sub + ahead;
+    if (p < cur_len)
+      stage_load<S, ALIGNED>(in, n, (int64_t)(cur_first + p) * kSub, q);
+    else if (p - cur_len < nxt_len)
+      stage_load<S, ALIGNED>(in, n, (int64_t)(nxt_first + p - cur_len) * kSub, q);
+  };
+
+  // one sub-tile: cur holds its data, far receives the data of the sub-tile two places on
+  auto body = [&](uint4 (&cur)[kSelVecs], uint4 (&far)[kSelVecs]) {
     uint32_t x = Flags<S>::build(cur, floor_key);
     const uint32_t cnt = (uint32_t)__popc(x);
     const uint32_t incl = wave_inclusive_scan_dpp(cnt);
     if ((threadIdx.x & 63) == 63) s_wave[par & 1][wave] = incl;
     __syncthreads();
-    // what comes next: the following sub-tile of this tile, or the first one of the next tile
-    if (sub + 1 < subs) {
-      stage_load<S, ALIGNED>(in, n, sub_base + kSub, nxt);
-    } else {
-      next_tile = s_next[turn & 1];
-      if (next_tile < ntiles) stage_load<S, ALIGNED>(in, n, (int64_t)next_tile * subs * kSub, nxt);
+    if (ticket_pending) {
+      ticket_tile(s_next[turn & 1], nxt_first, nxt_len);
+      ticket_pending = false;
     }
+    load_ahead(2, far);
     uint32_t before = incl - cnt, total = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
@@ -796,18 +826,39 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
     }
   };
 
-  if (tile < ntiles) stage_load<S, ALIGNED>(in, n, (int64_t)tile * subs * kSub, qa);
-  while (tile < ntiles) {
-    if (threadIdx.x == 0) s_next[turn & 1] = (int)gridDim.x + (int)atomicAdd(ticket, 1u);
-    const int64_t tile_base = (int64_t)tile * subs * kSub;
-    for (sub = 0; sub < subs; ++sub, ++par) {
-      sub_base = tile_base + (int64_t)sub * kSub;
-      if (par & 1)
+  if (sch.fixed > 0)
+    fixed_tile(0, cur_first, cur_len);
+  else
+    ticket_tile(blockIdx.x, cur_first, cur_len);
+  uint32_t rot = 0;  // par % 3
+  if (cur_len) {
+    stage_load<S, ALIGNED>(in, n, (int64_t)cur_first * kSub, qa);
+    sub = 0;
+    load_ahead(1, qb);  // tiles have at least two sub-tiles
+  }
+  while (cur_len) {
+    // the tile after this one
+    if (turn + 1 < sch.fixed) {
+      fixed_tile(turn + 1, nxt_first, nxt_len);
+    } else if (turn + 1 == sch.fixed) {
+      ticket_tile(blockIdx.x, nxt_first, nxt_len);
+    } else {
+      nxt_len = 0;
+      ticket_pending = true;
+      if (threadIdx.x == 0) s_next[turn & 1] = gridDim.x + atomicAdd(ticket, 1u);
+    }
+    for (sub = 0; sub < cur_len; ++sub, ++par) {
+      sub_base = (int64_t)(cur_first + sub) * kSub;
+      if (rot == 0)
+        body(qa, qc);
+      else if (rot == 1)
         body(qb, qa);
       else
-        body(qa, qb);
+        body(qc, qb);
+      rot = rot == 2 ? 0 : rot + 1;
     }
-    tile = next_tile;
+    cur_first = nxt_first;
+    cur_len = nxt_len;
     ++turn;
   }
   __syncthreads();
@@ -855,25 +906,30 @@ static int device_cus() {
 template <typename S>
 static int stage_launch(const StageArgs &a, hipStream_t stream) {
   constexpr int V = VecOf<S>::kN;
-  const int subs = select_subs(a.n, a.dtype);
-  const int64_t tile = (int64_t)kSelBlock * kSelVecs * V * subs;
-  const int64_t ntiles = ceil_div(a.n, tile);
-  if (ntiles > 0x3fffffff) return fail(ZEN_EINVAL, "select_stage: too many tiles");
+  const int64_t sub = (int64_t)kSelBlock * kSelVecs * V;
+  const int64_t subs = ceil_div(a.n > 0 ? a.n : 1, sub);
+  if (subs > 0x3fffffff) return fail(ZEN_EINVAL, "select_stage: tensor too large");
   // three workgroups per compute unit (measured: two are 10 % slower, four no faster); their LDS, 60 KB per
   // unit, leaves room for another stream's kernels next to this long one
   int64_t blocks = (int64_t)device_cus() * 3;
-  if (blocks > ntiles) blocks = ntiles;
+  const int64_t least = ceil_div(subs, kStageSmall);
+  if (blocks > least) blocks = least;
+  // about two thirds of the tensor in counter-free tiles, the rest through tickets
+  StageSched sch;
+  sch.fixed = (uint32_t)(subs * 2 / 3 / ((int64_t)kStageBig * blocks));
+  sch.fixed_subs = sch.fixed * (uint32_t)kStageBig * (uint32_t)blocks;
+  sch.ticket_tiles = (uint32_t)ceil_div(subs - (int64_t)sch.fixed_subs, kStageSmall);
   const S *in = static_cast<const S *>(a.in);
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
   ProfScope prof(kProfSelectStage, stream);
   if (aligned)
     k_select_stage<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
         in, a.n, a.thr, a.list_count, a.list_idx, static_cast<S *>(a.list_val), (uint32_t)a.capacity, a.ticket,
-        (int)ntiles, subs, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
+        sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
   else
     k_select_stage<S, false><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
         in, a.n, a.thr, a.list_count, a.list_idx, static_cast<S *>(a.list_val), (uint32_t)a.capacity, a.ticket,
-        (int)ntiles, subs, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
+        sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
   ZEN_LAUNCH_CHECK("k_select_stage");
   return ZEN_OK;
 }
