@@ -77,6 +77,50 @@ size_t zen_mapping_workspace(int64_t n, int partitions);
 int zen_mapping(int64_t n, int partitions, int64_t *out, int64_t *counts,
                 void *workspace, size_t workspace_bytes, int32_t *status, void *stream);
 
+/* ---------------------------------------------------------------- bitmap */
+
+/*
+ * Bitmap form of an index set, the wire format of the second exchange.
+ * mapping_p[mapping_n] is one partition's ascending index list (zen_mapping).
+ *
+ * zen_bitmap_encode replaces encode_bitmap (comm.py:59-85): bit j of the
+ * bitmap is set iff some idx[i] has lower-bound position j in mapping_p
+ * (torch.searchsorted, left side, comm.py:61-63; an index that is no member
+ * marks the next member, as in the reference).  Bits are numbered from the
+ * least significant bit of byte 0 (weights 2^0..2^7 per byte, comm.py:79-83).
+ * The bitmap is written as zen_bitmap_words(mapping_n) little-endian 32-bit
+ * words, i.e. (mapping_n + 7) / 8 meaningful bytes followed by zero padding up
+ * to a multiple of four; `bitmap_words` must be 4-byte aligned and that large.
+ * idx holds idx_n entries (int32, or int64 if idx64) in any order, of which
+ * only the first *idx_n_dev count if that device counter is given.  rank_at is
+ * optional: the rank dictionary zen_bitmap_ranks builds for this mapping and
+ * `numel` (zen_bitmap_rank_words(numel) words, 16-byte aligned: members below
+ * every multiple of 512 and one membership bit per index value; to be kept
+ * with the mapping, which the reference caches too, comm.py:132-134).  With it
+ * a lookup is two loads instead of a search through the list from an
+ * interpolated guess, and indices >= numel count as beyond the last member.
+ * For indices in [0, numel) the result is the same with and without.  A position past the end
+ * of the list (torch raises an IndexError there) sets ZEN_STAT_BAD_INDEX.
+ *
+ * zen_bitmap_decode replaces decode_bitmap (comm.py:87-99) for one rank's
+ * bitmap: out receives mapping_p[j] for every set bit j < mapping_n in
+ * ascending order, *out_count their number (ZEN_STAT_CAPACITY if it exceeds
+ * `capacity`; the excess is dropped).  Bits at positions >= mapping_n are
+ * ignored (comm.py:97); a bitmap of fewer than (mapping_n + 7) / 8 bytes is
+ * ZEN_EINVAL (the reference's mask would not fit the list).  No alignment
+ * requirement on `bitmap`.
+ */
+size_t zen_bitmap_words(int64_t mapping_n);
+size_t zen_bitmap_rank_words(int64_t numel);
+int zen_bitmap_ranks(const int64_t *mapping_p, int64_t mapping_n, int64_t numel, uint32_t *rank_at, void *stream);
+int zen_bitmap_encode(const int64_t *mapping_p, int64_t mapping_n, const void *idx, int idx64, int64_t idx_n,
+                      const int64_t *idx_n_dev, const uint32_t *rank_at, int64_t numel, uint32_t *bitmap_words,
+                      int32_t *status, void *stream);
+size_t zen_bitmap_decode_workspace(int64_t mapping_n);
+int zen_bitmap_decode(const int64_t *mapping_p, int64_t mapping_n, const uint8_t *bitmap, int64_t bitmap_bytes,
+                      int64_t *out, int64_t capacity, int64_t *out_count, void *workspace, size_t workspace_bytes,
+                      int32_t *status, void *stream);
+
 /* ---------------------------------------------------------------- insert */
 
 /*

@@ -3,6 +3,7 @@ amount of torch plumbing every wrapper shares: dtype codes, stream handles,
 cached workspaces and status words.  There is no fallback: if the library is
 missing or a call fails, an exception is raised."""
 import ctypes
+import threading
 import os
 
 import torch  # first: makes the process use torch's HIP runtime for libzen_hip too
@@ -43,6 +44,12 @@ def lib():
         "zen_hash_index": (i32, [vp, i64, i32, vp]),
         "zen_mapping_workspace": (sz, [i64, i32]),
         "zen_mapping": (i32, [i64, i32, vp, vp, vp, sz, vp, vp]),
+        "zen_bitmap_words": (sz, [i64]),
+        "zen_bitmap_rank_words": (sz, [i64]),
+        "zen_bitmap_ranks": (i32, [vp, i64, i64, vp, vp]),
+        "zen_bitmap_encode": (i32, [vp, i64, vp, i32, i64, vp, vp, i64, vp, vp, vp]),
+        "zen_bitmap_decode_workspace": (sz, [i64]),
+        "zen_bitmap_decode": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, sz, vp, vp]),
         "zen_sparse_balance": (i32, [vp, i32, i64, vp, i64, vp, i64, vp, i32, i32, vp, vp]),
         "zen_topk_threshold_workspace": (sz, []),
         "zen_topk_threshold": (i32, [vp, i32, i64, i64, vp, vp, sz, vp]),
@@ -109,15 +116,17 @@ def require_gpu(t, name):
 
 
 class Scratch:
-    """Per-device cache of raw byte buffers, grown on demand and reused.  A
-    buffer is tied to the stream order of its users, like any torch tensor."""
+    """Cache of raw byte buffers per device and host thread, grown on demand
+    and reused.  A buffer is tied to the stream order of its users, like any
+    torch tensor; two threads that enqueue calls side by side (their kernels
+    interleave even on one stream) never share one."""
 
     def __init__(self):
         self._bufs = {}
 
     def get(self, device, name, nbytes, zero=False):
         key = (torch.device(device).index if torch.device(device).index is not None
-               else torch.cuda.current_device(), name)
+               else torch.cuda.current_device(), threading.get_ident(), name)
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < nbytes:
             alloc = torch.zeros if zero else torch.empty

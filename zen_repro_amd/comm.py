@@ -61,6 +61,7 @@ class LoadBalanceAllreduce:
         self.tensor_partition = self.get_tensor_partition_obj(memory_scale, rehash)
         self.logger = logger
         self.mapping = {}
+        self._bitmap_ranks = {}  # numel -> (mapping list of this rank, its rank table)
 
     def get_tensor_partition_obj(self, memory_scale, rehash):
         return TensorPartition(partitions=self.partitions, memory_scale=memory_scale, rehash=rehash)
@@ -171,6 +172,119 @@ class LoadBalanceAllreduce:
             mapping.append(out[at:at + c])
             at += c
         return mapping
+
+    # ----------------------------------------------------------- bitmap
+
+    def encode_bitmap_flat(self, sparse_indices, numel, count=None):
+        """encode_bitmap without host synchronisation: (uint8 bitmap, status
+        int32[1]).  `count` (int64[1] on the device) limits the indices that
+        are looked at to the first `count`."""
+        mapping = self.mapping[numel][self.local_rank]
+        _lib.require_gpu(sparse_indices, "sparse_indices")
+        if sparse_indices.dtype not in (torch.int32, torch.int64):
+            raise RuntimeError("sparse_indices must be int32 or int64")
+        dev = sparse_indices.device
+        L = _lib.lib()
+        members = mapping.numel()
+        words = torch.empty(max(1, L.zen_bitmap_words(members)), dtype=torch.int32, device=dev)
+        status = _lib.status_word(dev)
+        # the rank table lives next to the mapping it belongs to (same cache, same lifetime)
+        cached = self._bitmap_ranks.get(numel)
+        if cached is None or cached[0] is not mapping:
+            rank_at = torch.empty(L.zen_bitmap_rank_words(numel), dtype=torch.int32, device=dev)
+            _lib.check(L.zen_bitmap_ranks(_lib.ptr(mapping), members, numel, _lib.ptr(rank_at),
+                                          _lib.stream_of(dev)), "encode_bitmap")
+            cached = self._bitmap_ranks[numel] = (mapping, rank_at)
+        rc = L.zen_bitmap_encode(_lib.ptr(mapping), members, _lib.ptr(sparse_indices),
+                                 int(sparse_indices.dtype == torch.int64), sparse_indices.numel(),
+                                 _lib.ptr(count) if count is not None else None, _lib.ptr(cached[1]), numel,
+                                 _lib.ptr(words), _lib.ptr(status), _lib.stream_of(dev))
+        _lib.check(rc, "encode_bitmap")
+        return words.view(torch.uint8)[:(members + 7) // 8], status
+
+    def encode_bitmap(self, sparse_indices, numel):
+        """One bit per member of this rank's mapping list, set where the member
+        is among sparse_indices; least significant bit first, padded to a whole
+        byte (comm.py:59-85).  self.mapping[numel] must exist (comm.py:135)."""
+        bitmap, status = self.encode_bitmap_flat(sparse_indices, numel)
+        bits = int(status.item())
+        if bits & _lib.STAT_BAD_INDEX:  # result[indices] = 1 with an index == len(result), comm.py:63
+            raise IndexError("encode_bitmap: an index lies beyond the last member of the mapping")
+        if bits:
+            raise RuntimeError("encode_bitmap: " + _lib.describe_status(bits))
+        return bitmap
+
+    def decode_bitmap(self, bitmap_indices, numel):
+        """For every rank i the members of mapping[numel][i] whose bit is set in
+        bitmap_indices[i], ascending int64 (comm.py:87-99)."""
+        mapping_tensor = self.mapping[numel]
+        L = _lib.lib()
+        outs, counts = [], []
+        status = None
+        for i, bitmap_tensor in enumerate(bitmap_indices):
+            mapping = mapping_tensor[i]
+            _lib.require_gpu(bitmap_tensor, "bitmap")
+            if bitmap_tensor.dtype != torch.uint8:
+                raise RuntimeError("bitmap must be uint8")
+            dev = bitmap_tensor.device
+            members = mapping.numel()
+            if bitmap_tensor.numel() * 8 < members:  # the mask would be shorter than the list it indexes, comm.py:97-98
+                raise IndexError("decode_bitmap: bitmap shorter than the mapping")
+            if status is None:
+                status = _lib.status_word(dev)
+            # a set bit costs eight bytes of output: room for every bit that can be set
+            capacity = min(members, bitmap_tensor.numel() * 8)
+            out = torch.empty(capacity, dtype=torch.int64, device=dev)
+            count = torch.zeros(1, dtype=torch.int64, device=dev)
+            ws = _lib.scratch.get(dev, "bitmap", L.zen_bitmap_decode_workspace(members))
+            rc = L.zen_bitmap_decode(_lib.ptr(mapping), members, _lib.ptr(bitmap_tensor), bitmap_tensor.numel(),
+                                     _lib.ptr(out), capacity, _lib.ptr(count), _lib.ptr(ws), ws.numel(),
+                                     _lib.ptr(status), _lib.stream_of(dev))
+            _lib.check(rc, "decode_bitmap")
+            outs.append(out)
+            counts.append(count)
+        if not outs:
+            return []
+        host = torch.cat(counts + [status.to(torch.int64)]).tolist()
+        if host[-1]:
+            raise RuntimeError("decode_bitmap: " + _lib.describe_status(host[-1]))
+        return [out[:c] for out, c in zip(outs, host)]
+
+    # ------------------------------------------------- the whole exchange
+
+    def zen_sparse_comm(self, tensor, method):
+        """The reference's driver of one sparse all-reduce (comm.py:101-150):
+        method 1 = all-gather of (indices, values); 2 = load balance, exchange of
+        the buckets, merge, all-gather of the merged indices; 3 = as 2 with the
+        indices travelling as bitmaps.  The exchanges themselves belong to
+        `self.ddp`, an object with the reference backend's allgather /
+        allgather_padding / alltoallv (DDPbackend.py:13-41, 71-81); this build
+        ships none, so the attribute has to be set by the caller."""
+        ddp = getattr(self, "ddp", None)
+        if ddp is None:
+            raise RuntimeError("zen_sparse_comm needs a communication backend in self.ddp")
+        numel = tensor.numel()
+        if method == 1:
+            sparse_indices, sparse_values = self.encode_sparse_tensor(tensor)
+            indices_tensors = ddp.allgather_padding(sparse_indices)
+            values_tensors = ddp.allgather_padding(sparse_values)
+            return self.decode_sparse_tensors(indices_tensors, values_tensors, numel)
+        indices, values, splits = self.tensor_partition.load_balance(tensor)
+        gather_splits = ddp.allgather(splits)
+        indices_tensors = ddp.alltoallv(indices, gather_splits)
+        values_tensors = ddp.alltoallv(values, gather_splits)
+        _dense_tensor = self.decode_sparse_tensors(indices_tensors, values_tensors, numel)
+        sparse_indices, sparse_values = self.encode_sparse_tensor(_dense_tensor)
+        if method == 2:
+            indices_tensors = ddp.allgather_padding(sparse_indices)
+        else:
+            if numel not in self.mapping:
+                self.mapping[numel] = self.calculate_mapping(numel)
+            bitmap_indices = self.encode_bitmap(sparse_indices, numel)
+            bitmap_indices_gather = ddp.allgather_padding(bitmap_indices)
+            indices_tensors = self.decode_bitmap(bitmap_indices_gather, numel)
+        values_tensors = ddp.allgather_padding(sparse_values)
+        return self.decode_sparse_tensors(indices_tensors, values_tensors, numel)
 
 
 def _as_one_buffer(tensors):
