@@ -34,6 +34,8 @@ def parse():
                     help="the CPU baseline runs on 1/div of the workload")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run five device copies of 1 GiB and exit (scale for hardware byte counters)")
+    ap.add_argument("--bitmap-codec", action="store_true",
+                    help="measure the bitmap index codec of the second exchange instead (prints its own line)")
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
     ap.add_argument("--merge-follows", action="store_true",
                     help="with --depth: a step's merge runs on its encode's stream, after it")
@@ -73,6 +75,60 @@ def cpu_baseline(cfg, grad_dev, div):
     }
 
 
+def bitmap_codec(args, dev):
+    """Rank 0's merged indices -> bitmap over its partition's member list -> indices again (comm.py:59-99):
+    one step = one encode_bitmap and one decode_bitmap of that bitmap, no host synchronisation in between.
+    Algorithmic bytes: the indices in (8 B each), the bitmap out and in again (members / 8 B each way), the
+    indices out (8 B each)."""
+    import torch
+
+    from zen_repro_amd import LoadBalanceAllreduce, LocalGroup, _lib, workloads
+
+    cfg, grad = workloads.make(args.config, device=dev, seed=0, shrink=args.shrink)
+    del grad
+    n, P = cfg.n, cfg.partitions
+    lba = LoadBalanceAllreduce(LocalGroup(P, 0), None, None)
+    lba.mapping[n] = lba.calculate_mapping(n)
+    members = lba.mapping[n][0]
+    _, _, flat_idx, flat_val = workloads.peer_payloads(cfg, max(1, (cfg.k or n // 100) // P), device=dev, seed=1)
+    m_idx, _ = lba.merge_sparse(flat_idx, flat_val, n)
+    L = _lib.lib()
+    out = torch.empty(m_idx.numel(), dtype=torch.int64, device=dev)
+    count = torch.zeros(1, dtype=torch.int64, device=dev)
+    ws = torch.empty(max(256, L.zen_bitmap_decode_workspace(members.numel())), dtype=torch.uint8, device=dev)
+    status = _lib.status_word(dev)
+
+    def step():
+        bitmap, st = lba.encode_bitmap_flat(m_idx, n)
+        _lib.check(L.zen_bitmap_decode(_lib.ptr(members), members.numel(), _lib.ptr(bitmap), bitmap.numel(),
+                                       _lib.ptr(out), out.numel(), _lib.ptr(count), _lib.ptr(ws), ws.numel(),
+                                       _lib.ptr(status), _lib.stream_of(dev)), "decode_bitmap")
+        return st
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    flags = [step() for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    bits = int(status.item())
+    for st in flags:
+        bits |= int(st.item())
+    if bits or int(count.item()) != m_idx.numel() or not torch.equal(out, m_idx):
+        print("bench.py: the bitmap round trip did not return the indices", file=sys.stderr)
+        sys.exit(1)
+    u, nbytes = m_idx.numel(), (members.numel() + 7) // 8
+    b_alg = 16 * u + 2 * nbytes
+    print(json.dumps({
+        "metric": "bitmap index codec, encode + decode of one rank's merged indices", "value": round(u / ms / 1e3, 2),
+        "unit": "M indices/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "dtype": "int64", "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: {cfg.note}", "elements": n, "partitions": P, "indices": u,
+                   "members": members.numel(), "bitmap_bytes": nbytes},
+        "algorithmic_bytes": b_alg, "algorithmic_GBps": round(b_alg / (ms * 1e-3) / 1e9, 2)}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -100,6 +156,10 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": {"bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4,
                                                "copies": 5}}))
+        return
+
+    if args.bitmap_codec:
+        bitmap_codec(args, dev)
         return
 
     cfg, grad = workloads.make(args.config, device=dev, seed=0, shrink=args.shrink)
