@@ -284,6 +284,17 @@ def test_compress_masked_copy(zen, oracle, dtype):
     assert np.array_equal(to_np(out), want2)
     small = d[:4096]
     assert zen.compress(1, small) is small  # train.py:77-78
+    # threshold over the samples of several ranks (train.py:56-73); the exchange is the caller's
+    others = [make_grad(oracle, n, 1.0, dtype, seed=6 + r) for r in range(3)]
+    everyone = np.concatenate([g[sample]] + [o[sample] for o in others])
+    gather = lambda mine: torch.cat([mine] + [to_dev(o)[torch.from_numpy(sample).cuda()] for o in others])  # noqa: E731
+    out = zen.compress_with_allgather(5, d, zen.LocalGroup(4), torch.from_numpy(sample).cuda(), gather)
+    want3, _ = oracle.mask_dense(g, oracle.kth_key(everyone, len(everyone) * 5 // 100))
+    assert np.array_equal(to_np(out), want3)
+    assert np.array_equal(to_np(zen.compress_with_allgather(5, d, zen.LocalGroup(1), torch.from_numpy(sample).cuda())),
+                          want2)
+    with pytest.raises(RuntimeError):
+        zen.compress_with_allgather(5, d, zen.LocalGroup(4))
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])

@@ -62,3 +62,32 @@ def compress(top_k, tensor, sample_index=None):
         raise RuntimeError("compress: top-k of the sample is empty")
     thr = topk_threshold(sample, k)
     return mask_below(flat, thr).view_as(tensor)
+
+
+def compress_with_allgather(top_k, tensor, pg_group, sample_index=None, all_gather=None):
+    """The reference's compress_with_allgather (train.py:56-73): as compress,
+    but the threshold is the (n_all*top_k//100)-th largest magnitude among
+    the 1 % samples of every rank of pg_group.  `all_gather(sample)` returns
+    the samples of all ranks as one tensor (the reference calls
+    dist.all_gather_into_tensor there); this build ships no exchange, so it
+    has to be passed in for groups of more than one rank."""
+    numel = tensor.numel()
+    if numel <= 4096:
+        return tensor
+    flat = tensor.reshape(-1)
+    if sample_index is None:
+        sample_index = torch.randint(0, numel, (math.ceil(0.01 * numel),), device=tensor.device)
+    sample = flat[sample_index]
+    if all_gather is not None:
+        samples = all_gather(sample)
+        if samples.numel() != pg_group.size() * sample.numel():
+            raise RuntimeError("compress_with_allgather: the gathered samples have the wrong size")
+    elif pg_group.size() == 1:
+        samples = sample
+    else:
+        raise RuntimeError("compress_with_allgather needs an all_gather callable for more than one rank")
+    k = samples.numel() * top_k // 100
+    if k < 1:
+        raise RuntimeError("compress_with_allgather: top-k of the samples is empty")
+    thr = topk_threshold(samples.contiguous(), k)
+    return mask_below(flat, thr).view_as(tensor)

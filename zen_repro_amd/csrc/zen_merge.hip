@@ -149,29 +149,38 @@ constexpr int kMergeTarget = 3072;   // records a bucket is sized for: duplicate
 constexpr int kMergeItems = 13;      // sorted records per thread while summing (odd: no LDS bank conflicts)
 static_assert(kSlabBlock * kMergeItems >= kSlabCap, "every sorted place needs an owner");
 
-template <typename I>
-struct MergeCountSrc {
-  const I *idx;
-  uint32_t dense_n;
-  int32_t *status;
-  __device__ inline uint32_t key(uint32_t e) const {
-    const I k = idx[e];
-    if (k >= 0 && (uint64_t)k < (uint64_t)dense_n) return (uint32_t)k;
-    atomicOr(status, ZEN_STAT_BAD_INDEX);  // skipped, like everything behind the good ones in the general path
-    return kNoSlot;
-  }
-};
+// An entry travels as (index, arrival number, value as fp32 bits).
 template <typename I, typename S>
-struct MergeWriteSrc {
+struct MergeSrc {
+  SlabGeom geo;
   const I *idx;
   const S *val;
   uint32_t dense_n;
-  __device__ inline void rec(uint32_t e, uint32_t *key, uint32_t *a, uint32_t *b) const {
-    const I k = idx[e];
-    *key = (k >= 0 && (uint64_t)k < (uint64_t)dense_n) ? (uint32_t)k : kNoSlot;
-    *a = e;
-    *b = __float_as_uint(KeyOf<S>::to_f32(val[e]));
+  int32_t *status;
+  // the value is fetched again by arrival number when the entry is written: a workgroup's 4096 arrival numbers
+  // are consecutive, so those loads hit the 8 KB it has just read
+  static constexpr int kStaged = 2;
+  __device__ inline uint32_t late(const uint32_t (&w)[3], int) const {
+    return __float_as_uint(KeyOf<S>::to_f32(val[w[1]]));
   }
+  __device__ inline bool load(uint32_t e, uint32_t (&w)[3], uint32_t *bucket) const {
+    const I k = idx[e];
+    if (k < 0 || (uint64_t)k >= (uint64_t)dense_n) {
+      atomicOr(status, ZEN_STAT_BAD_INDEX);  // skipped, like everything behind the good ones in the general path
+      return false;
+    }
+    w[0] = (uint32_t)k;
+    w[1] = e;
+    w[2] = 0;
+    *bucket = geo.bucket_of((uint32_t)k);
+    return true;
+  }
+};
+struct MergeSink {
+  SlabGeom geo;
+  uint4 *slab_rec;
+  __device__ inline uint32_t bucket(const uint32_t (&w)[3]) const { return geo.bucket_of(w[0]); }
+  __device__ inline void store(size_t at, const uint32_t (&w)[3]) const { slab_rec[at] = make_uint4(w[0], w[1], w[2], 0u); }
 };
 
 template <typename I>
@@ -190,8 +199,8 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
   const int nb = (int)geo.nbuckets;
   if (b >= nb) return;
   const size_t base = (size_t)b * kSlabCap;
-  uint32_t n_raw = cursor[b];
-  if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the scan flagged the overflow
+  uint32_t n_raw = cursor[b * kCursorPad];
+  if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the scatter flagged the overflow
   const uint32_t lo = bucket_lo[b];
   uint32_t off[kSlabItems], arr[kSlabItems], val[kSlabItems], rank[kSlabItems];
   uint32_t live = 0;
@@ -319,7 +328,8 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
 
 struct SlabMergePlan {
   unsigned long long *scan;  // prefix state over the buckets (zeroed before use)
-  uint32_t *cursor, *bucket_lo, *hist;
+  CoarseGeom cg;
+  FeedBuffers feed;
   uint4 *slab_rec;
   size_t zero_bytes;
   size_t bytes;
@@ -329,11 +339,14 @@ SlabMergePlan plan_slab_merge(void *workspace, const SlabGeom &geo, int64_t r) {
   Carver cv(workspace);
   SlabMergePlan p;
   const size_t B = geo.nbuckets;
+  // what must be zero when the first kernel starts sits together: one fill
   p.scan = cv.take<unsigned long long>(scan_words((int64_t)B));
+  p.feed.coarse_cursor = cv.take<uint32_t>(feed_coarse_cursor_words());
+  p.feed.cursor = cv.take<uint32_t>(B * kCursorPad);
   p.zero_bytes = cv.used;
-  p.cursor = cv.take<uint32_t>(B);
-  p.bucket_lo = cv.take<uint32_t>(B);
-  p.hist = cv.take<uint32_t>((size_t)feed_batches(r) * feed_row_words((uint32_t)B));
+  p.feed.bucket_lo = cv.take<uint32_t>(B);
+  p.cg = coarse_geometry(geo, r);
+  p.feed.coarse_words = cv.take<uint32_t>(feed_coarse_words(p.cg, 3));
   p.slab_rec = cv.take<uint4>(B * kSlabCap);
   p.bytes = cv.used;
   return p;
@@ -356,9 +369,9 @@ int slab_merge_launch(const SlabGeom &geo, const I *idx, const S *val, int64_t r
   ZEN_LAUNCH_CHECK("merge: clear prefix state");
   {
     ProfScope prof(kProfMergeFeed, s);
-    const MergeCountSrc<I> csrc{idx, (uint32_t)dense_n, status};
-    const MergeWriteSrc<I, S> wsrc{idx, val, (uint32_t)dense_n};
-    const int rc = feed_slabs(geo, csrc, wsrc, nullptr, r, p.hist, p.cursor, p.bucket_lo, p.slab_rec, status, s);
+    const MergeSrc<I, S> src{geo, idx, val, (uint32_t)dense_n, status};
+    const MergeSink sink{geo, p.slab_rec};
+    const int rc = feed_slabs<3>(geo, p.cg, src, sink, nullptr, r, p.feed, status, s);
     if (rc != ZEN_OK) return rc;
   }
   const ScanState st = scan_state(p.scan, (int64_t)geo.nbuckets);
@@ -366,10 +379,10 @@ int slab_merge_launch(const SlabGeom &geo, const I *idx, const S *val, int64_t r
   ProfScope prof(kProfMergeBucket, s);
   if (idx64_out)
     k_merge_bucket<int64_t><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
-        geo, p.cursor, p.bucket_lo, p.slab_rec, static_cast<int64_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
+        geo, p.feed.cursor, p.feed.bucket_lo, p.slab_rec, static_cast<int64_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
   else
     k_merge_bucket<int32_t><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
-        geo, p.cursor, p.bucket_lo, p.slab_rec, static_cast<int32_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
+        geo, p.feed.cursor, p.feed.bucket_lo, p.slab_rec, static_cast<int32_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
   ZEN_LAUNCH_CHECK("k_merge_bucket");
   return ZEN_OK;
 }

@@ -35,8 +35,8 @@ hipEvent_t take_event() {
 const char *const kNames[kProfCount] = {
     "k_topk_hist", "k_select_compact", "k_insert_list", "k_final_key", "sort_pairs",
     "k_gather",    "k_merge_prep",     "k_merge_reduce", "k_compress", "k_insert_dense",
-    "k_select_stage", "k_feed_count+scan+write", "k_slab_sort", "k_slab_chains+classify", "k_slab_place",
-    "merge: k_feed_count+scan+write", "k_merge_bucket",
+    "k_select_stage", "k_coarse_scatter+k_fine_scatter", "k_slab_sort", "k_slab_chains+classify", "k_slab_place",
+    "merge: k_coarse_scatter+k_fine_scatter", "k_merge_bucket",
 };
 
 void drop_spans() {  // the events go back to the spare list (a read has waited for them, or nobody will)

@@ -5,8 +5,10 @@
 // (functions_cuda_kernel.cu:97-167, tensor_load_balance.py:13-51).  Here the
 // select kernel leaves its candidates in one unordered list, and five short
 // kernels finish the job (a bucket is a range of level-1 hash slots, zen_slab.h):
-//   k_feed_*        the list, filtered by the exact threshold, goes to the bucket
-//                   slabs (count, scan, write);
+//   k_coarse_scatter, k_fine_scatter
+//                   the list, filtered by the exact threshold, goes to the bucket
+//                   slabs in two steps (64 groups of buckets first, then the buckets
+//                   of each group), so that every store belongs to a long run;
 //   k_slab_sort     one workgroup per bucket: applies the exact threshold, sorts
 //                   the bucket by (level-1 slot, index) inside LDS; in a run of
 //                   equal slots the first entry (smallest index) is the slot's
@@ -30,13 +32,13 @@ namespace zen {
 namespace {
 
 struct SlabTables {
-  uint32_t *cursor;     // [B] records in the bucket's slab
+  uint32_t *cursor;     // [B * kCursorPad] records in the bucket's slab, at [b * kCursorPad]
   uint32_t *bucket_lo;  // [B] smallest level-1 slot of the bucket
   uint32_t *bucket_n;   // [B] selected records, sorted, in the slab
   uint32_t *removed_n;  // [B] of which lost their level-1 slot
   uint32_t *movein_n;   // [B] entries whose final slot lies in the bucket but whose level-1 slot does not own it
   uint32_t *serial_n;   // [P] entries that found no slot
-  uint4 *slab_rec;      // [B * kSlabCap] records as they arrive: (level-1 slot, index, value, 0)
+  uint2 *slab_rec;      // [B * kSlabCap] records as they arrive: (index, value)
   int32_t *slab_idx;    // [B * kSlabCap] after the sort: index | kRemovedBit
   void *slab_val;       // [B * kSlabCap] after the sort: value
   uint32_t *slab_key;   // [B * kSlabCap] after the sort: level-1 slot, ascending inside a slab
@@ -53,101 +55,35 @@ __device__ inline uint32_t level1_slot(const Probe &g, uint32_t t) { return (pol
 
 // ------------------------------------------------- list -> bucket slabs
 
-}  // namespace
-
-__global__ __launch_bounds__(kScanCols * kScanChunks) void k_feed_scan(SlabGeom geo,
-                                                                       const uint32_t *__restrict__ list_count,
-                                                                       uint32_t list_cap, uint32_t nbuckets,
-                                                                       uint32_t row_words, uint32_t *__restrict__ hist,
-                                                                       uint32_t *__restrict__ cursor,
-                                                                       uint32_t *__restrict__ bucket_lo,
-                                                                       int32_t *status) {
-  __shared__ uint32_t s_sum[kScanChunks][kScanCols];
-  const uint32_t count = feed_count(list_count, list_cap);
-  const uint32_t batches = (count + kFeedBatch - 1) / kFeedBatch;
-  const uint32_t col = threadIdx.x % kScanCols, chunk = threadIdx.x / kScanCols;
-  const uint32_t b = blockIdx.x * kScanCols + col;
-  const uint32_t per = (batches + kScanChunks - 1) / kScanChunks;
-  const uint32_t r0 = chunk * per < batches ? chunk * per : batches;
-  const uint32_t r1 = r0 + per < batches ? r0 + per : batches;
-  // the loads of a thread do not depend on each other: eight at a time are in flight (a plain loop would
-  // wait for each before asking for the next)
-  uint32_t sum = 0;
-  if (b < row_words) {
-    uint32_t r = r0;
-    for (; r + 8 <= r1; r += 8) {
-      uint32_t x[8];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) x[q] = hist[(size_t)(r + q) * row_words + b];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) sum += x[q];
-    }
-    for (; r < r1; ++r) sum += hist[(size_t)r * row_words + b];
-  }
-  s_sum[chunk][col] = sum;
-  __syncthreads();
-  uint32_t running = 0, total = 0;
-  for (int c = 0; c < kScanChunks; ++c) {
-    const uint32_t x = s_sum[c][col];
-    if ((uint32_t)c < chunk) running += x;
-    total += x;
-  }
-  if (b < row_words) {
-    uint32_t r = r0;
-    for (; r + 8 <= r1; r += 8) {
-      uint32_t x[8];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) x[q] = hist[(size_t)(r + q) * row_words + b];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        hist[(size_t)(r + q) * row_words + b] = running;
-        running += x[q];
-      }
-    }
-    for (; r < r1; ++r) {
-      const uint32_t x = hist[(size_t)r * row_words + b];
-      hist[(size_t)r * row_words + b] = running;
-      running += x;
-    }
-  }
-  if (chunk == 0 && b < nbuckets) {
-    cursor[b] = total;
-    bucket_lo[b] = geo.first_key(b);  // a 64-bit division: once per bucket here, not once per thread later
-    if (total > (uint32_t)kSlabCap) atomicOr(status, ZEN_STAT_RETRY);
-  }
-}
-
-namespace {
-
-// The select kernel left its candidates in one list, in no particular order.  On the way to the slabs index 0
-// (never transmitted: 0 is the table's empty marker, tensor_load_balance.py:31) and whatever the exact
-// threshold excludes are dropped; every kept entry's level-1 slot is computed once, in the counting pass, and
-// kept in list_key for the writing pass.
+// The select kernel left its candidates in one list, in no particular order.  On the way to the slabs
+// (zen_slab_feed.h) index 0 (never transmitted: 0 is the table's empty marker, tensor_load_balance.py:31) and
+// whatever the exact threshold excludes are dropped.  An entry travels as (index, value); its level-1 slot is
+// hashed again wherever it is needed, which is cheaper than carrying it along.
 template <typename S>
-struct EncodeCountSrc {
+struct EncodeSrc {
   SlabGeom geo;
   const int32_t *list_idx;
   const S *list_val;
   const uint32_t *filter;  // optional exact threshold
-  uint32_t *list_key;
-  __device__ inline uint32_t key(uint32_t e) const {
+  static constexpr int kStaged = 2;
+  __device__ inline uint32_t late(const uint32_t (&)[2], int) const { return 0; }
+  __device__ inline bool load(uint32_t e, uint32_t (&w)[2], uint32_t *bucket) const {
     const uint32_t t = (uint32_t)list_idx[e];
-    uint32_t slot = kNoSlot;
-    if (t != 0 && (list_val[e] & KeyOf<S>::kMask) >= (filter ? filter[0] : 0u)) slot = geo.mod_m(poly(t) + kSeed1);
-    list_key[e] = slot;
-    return slot;
+    const S v = list_val[e];
+    if (t == 0 || (v & KeyOf<S>::kMask) < (filter ? filter[0] : 0u)) return false;
+    w[0] = t;
+    w[1] = (uint32_t)v;
+    *bucket = geo.bucket_of(geo.mod_m(poly(t) + kSeed1));
+    return true;
   }
 };
-template <typename S>
-struct EncodeWriteSrc {
-  const int32_t *list_idx;
-  const S *list_val;
-  const uint32_t *list_key;
-  __device__ inline void rec(uint32_t e, uint32_t *key, uint32_t *a, uint32_t *b) const {
-    *key = list_key[e];
-    *a = (uint32_t)list_idx[e];
-    *b = (uint32_t)list_val[e];
+struct EncodeSink {
+  SlabGeom geo;
+  uint2 *slab_rec;
+  __device__ inline uint32_t bucket(const uint32_t (&w)[2]) const {
+    return geo.bucket_of(geo.mod_m(poly(w[0]) + kSeed1));
   }
+  __device__ inline void store(size_t at, const uint32_t (&w)[2]) const { slab_rec[at] = make_uint2(w[0], w[1]); }
 };
 
 // ------------------------------------------------------------ sort a bucket
@@ -159,8 +95,8 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
   __shared__ uint32_t s_lost, s_base;
   const uint32_t b = blockIdx.x;
   const size_t base = (size_t)b * kSlabCap;
-  uint32_t n_raw = tb.cursor[b];
-  if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the scan flagged the overflow
+  uint32_t n_raw = tb.cursor[b * kCursorPad];
+  if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the scatter flagged the overflow
   const uint32_t lo = tb.bucket_lo[b];
   S *slab_val = static_cast<S *>(tb.slab_val);
   if (threadIdx.x == 0) s_lost = 0;
@@ -173,10 +109,10 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
     off[i] = idx[i] = pos[i] = 0;
     val[i] = 0;
     if (j < n_raw) {
-      const uint4 rec = tb.slab_rec[base + j];
-      off[i] = rec.x - lo;
-      idx[i] = rec.y;
-      val[i] = (S)rec.z;
+      const uint2 rec = tb.slab_rec[base + j];
+      off[i] = geo.mod_m(poly(rec.x) + kSeed1) - lo;  // the level-1 slot again: cheaper than carrying it along
+      idx[i] = rec.x;
+      val[i] = (S)rec.y;
       pos[i] = j;
       live |= 1u << i;
     }
@@ -620,9 +556,9 @@ struct SlabPlan {
   uint32_t *list_count;   // candidates the select kernel found
   int32_t *list_idx;      // [list_cap] the candidates, in no particular order
   void *list_val;
-  uint32_t *list_key;     // [list_cap] level-1 slot of every selected candidate
   uint32_t list_cap;
-  uint32_t *feed_hist;    // per-batch bucket counts, then run starts (zen_slab_feed.h)
+  CoarseGeom cg;
+  FeedBuffers feed;
   uint32_t *thr;          // [0..1] exact threshold + count, [2..3] sampled floor
   void *zero_begin;
   size_t zero_bytes;
@@ -639,7 +575,8 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.cand_hist = cv.take<uint32_t>((size_t)kCandHistWords);
   p.ticket = cv.take<uint32_t>(4);
   p.list_count = cv.take<uint32_t>(4);
-  p.tb.cursor = cv.take<uint32_t>(B);
+  p.tb.cursor = cv.take<uint32_t>(B * kCursorPad);
+  p.feed.coarse_cursor = cv.take<uint32_t>(feed_coarse_cursor_words());
   p.tb.movein_n = cv.take<uint32_t>(B);
   p.tb.serial_n = cv.take<uint32_t>((size_t)partitions);
   p.tb.ctr = cv.take<Counters>(1);
@@ -649,13 +586,15 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.list_cap = (uint32_t)list_cap;
   p.list_idx = cv.take<int32_t>((size_t)list_cap);
   p.list_val = cv.take<char>((size_t)list_cap * (dtype == ZEN_BF16 ? 2 : 4));
-  p.list_key = cv.take<uint32_t>((size_t)list_cap);
-  p.feed_hist = cv.take<uint32_t>((size_t)feed_batches(list_cap) * feed_row_words((uint32_t)B));
+  p.cg = coarse_geometry(geo, list_cap);
+  p.feed.coarse_words = cv.take<uint32_t>(feed_coarse_words(p.cg, 2));
   p.tb.bucket_lo = cv.take<uint32_t>(B);
+  p.feed.cursor = p.tb.cursor;
+  p.feed.bucket_lo = p.tb.bucket_lo;
   p.tb.out_start = cv.take<uint32_t>(B + 1);
   p.tb.bucket_n = cv.take<uint32_t>(B);
   p.tb.removed_n = cv.take<uint32_t>(B);
-  p.tb.slab_rec = cv.take<uint4>(B * kSlabCap);
+  p.tb.slab_rec = cv.take<uint2>(B * kSlabCap);
   p.tb.slab_idx = cv.take<int32_t>(B * kSlabCap);
   p.tb.slab_val = cv.take<char>(B * kSlabCap * (dtype == ZEN_BF16 ? 2 : 4));
   p.tb.slab_key = cv.take<uint32_t>(B * kSlabCap);
@@ -678,11 +617,9 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
   const S *dense = static_cast<const S *>(a.input);
   {
     ProfScope prof(kProfFeed, s);
-    const S *list_val = static_cast<const S *>(p.list_val);
-    const EncodeCountSrc<S> csrc{geo, p.list_idx, list_val, filter, p.list_key};
-    const EncodeWriteSrc<S> wsrc{p.list_idx, list_val, p.list_key};
-    const int rc = feed_slabs(geo, csrc, wsrc, p.list_count, p.list_cap, p.feed_hist, p.tb.cursor, p.tb.bucket_lo,
-                              p.tb.slab_rec, a.status, s);
+    const EncodeSrc<S> src{geo, p.list_idx, static_cast<const S *>(p.list_val), filter};
+    const EncodeSink sink{geo, p.tb.slab_rec};
+    const int rc = feed_slabs<2>(geo, p.cg, src, sink, p.list_count, p.list_cap, p.feed, a.status, s);
     if (rc != ZEN_OK) return rc;
   }
   {

@@ -1,15 +1,28 @@
 // Moving an unordered list of keyed entries into bucket slabs (zen_slab.h), shared by the encode and the
-// merge side.  Three kernels, no global atomic (a reservation per bucket and batch would be a million
-// device-wide atomics, and those on one cache line are carried out one after the other): every workgroup counts
-// its batch of the list per bucket (k_feed_count), a scan over the batches turns the counts of a bucket into
-// the places where each batch's run starts in the bucket's slab (k_feed_scan), and every workgroup orders its
-// batch by bucket in LDS and writes the runs as 16-byte records (k_feed_write).
+// merge side.
 //
-// What an entry is comes from two small functor types:
-//   CountSrc:  uint32_t key(uint32_t e)   key of list entry e, or kNoSlot if the entry is dropped (it may
-//                                         store the key for the write pass)
-//   WriteSrc:  void rec(uint32_t e, uint32_t *key, uint32_t *a, uint32_t *b)   the record of entry e: its key
-//                                         (kNoSlot: dropped) and two payload words
+// A direct scatter into a thousand slabs would write runs of three or four records, and memory serves such
+// stores one request at a time.  So the list goes to at most 64 coarse slabs first (a coarse slab = `per`
+// neighbouring buckets; k_coarse_scatter) and each coarse slab to its buckets afterwards (k_fine_scatter): a
+// workgroup orders its 4096 entries by destination in LDS, reserves one run per destination with one atomic
+// each and writes runs of dozens to hundreds of entries.  The order inside a slab is whatever the atomics make
+// it; the per-bucket sorts that follow do not depend on it.
+//
+// Atomics on one address are carried out one after the other (about 11 ns each), and a thousand workgroups
+// asking the same 64 cursors at once would wait 10 us for that alone: a coarse slab is therefore kept in
+// kCoarseSplit parts with a cursor each (workgroup i writes part i % kCoarseSplit), every coarse cursor has a
+// 128-byte line to itself, and the bucket cursors sit kCursorPad words apart.
+//
+// An entry travels as W 32-bit words.  What they are comes from two small functor types:
+//   Src:   bool load(uint32_t e, uint32_t (&w)[W], uint32_t *bucket)   words and bucket of list entry e;
+//                                                                      false: the entry is dropped
+//          kStaged, uint32_t late(const uint32_t (&w)[W], int q)       only the first kStaged words go through
+//                                                                      LDS in the first step; word q >= kStaged
+//                                                                      is asked for again when the entry is
+//                                                                      written (from the words before it), so
+//                                                                      that more workgroups fit a compute unit
+//   Sink:  uint32_t bucket(const uint32_t (&w)[W])                     the bucket again, from the words
+//          void store(size_t at, const uint32_t (&w)[W])               the record at slab place `at`
 #pragma once
 
 #include "zen_slab.h"
@@ -18,9 +31,44 @@ namespace zen {
 
 constexpr int kFeedItems = 8;
 constexpr int kFeedBatch = kSlabBlock * kFeedItems;  // list entries per workgroup
-constexpr int kScanChunks = 32;
-constexpr int kScanCols = 8;  // 256 threads: a workgroup this small finds room on a CU other kernels are using
-constexpr uint32_t kNoSlot = 0xffffffffu;  // key of an entry that is dropped
+constexpr int kCoarseMax = 64;
+constexpr int kCoarsePer = kSlabMaxBuckets / kCoarseMax;  // buckets per coarse slab, at most
+constexpr int kCoarsePad = 32;   // words between two coarse cursors
+constexpr int kCoarseSplit = 4;  // parts of a coarse slab
+constexpr int kCursorPad = 8;    // words between two bucket cursors
+
+struct CoarseGeom {
+  uint32_t groups;  // coarse slabs (<= kCoarseMax)
+  uint32_t per;     // buckets per coarse slab (<= kCoarsePer)
+  uint32_t cap;     // entries one part of a coarse slab holds
+  float inv_per;    // (1 / per)(1 - 2^-20), rounded down
+};
+
+// list_cap entries at most, spread over the buckets like hash values: a coarse slab receives its share give
+// or take a few hundred, and its parts equal shares of that.
+inline CoarseGeom coarse_geometry(const SlabGeom &geo, int64_t list_cap) {
+  CoarseGeom c;
+  c.per = (geo.nbuckets + kCoarseMax - 1) / kCoarseMax;
+  c.groups = (geo.nbuckets + c.per - 1) / c.per;
+  c.inv_per = slab_inverse_below(c.per);
+  const int64_t share = ceil_div(list_cap * c.per, (int64_t)geo.nbuckets * kCoarseSplit);
+  c.cap = (uint32_t)(share + share / 8 + 4096);
+  return c;
+}
+
+inline uint32_t feed_batches(int64_t entries) { return (uint32_t)ceil_div(entries > 0 ? entries : 1, kFeedBatch); }
+
+// Workspace of the two steps.
+struct FeedBuffers {
+  uint32_t *coarse_cursor;  // [feed_coarse_cursor_words()], zero before the first step
+  uint32_t *coarse_words;   // [W][groups * kCoarseSplit * cap]
+  uint32_t *cursor;         // [nbuckets * kCursorPad], zero before the second step; ends as the slab fill counts
+  uint32_t *bucket_lo;      // [nbuckets] smallest key of every bucket (written by the second step)
+};
+inline size_t feed_coarse_cursor_words() { return (size_t)kCoarseMax * kCoarseSplit * kCoarsePad; }
+inline size_t feed_coarse_words(const CoarseGeom &cg, int words) {
+  return (size_t)words * cg.groups * kCoarseSplit * cg.cap;
+}
 
 // Number of list entries: *list_count if given, never more than list_cap.
 __device__ inline uint32_t feed_count(const uint32_t *list_count, uint32_t list_cap) {
@@ -29,150 +77,161 @@ __device__ inline uint32_t feed_count(const uint32_t *list_count, uint32_t list_
   return c < list_cap ? c : list_cap;
 }
 
-inline uint32_t feed_row_words(uint32_t nbuckets) { return (nbuckets + 63u) / 64u * 64u; }
-inline uint32_t feed_batches(int64_t list_cap) { return (uint32_t)ceil_div(list_cap, kFeedBatch); }
-// hist needs feed_batches(list_cap) * feed_row_words(nbuckets) words
+// Orders the (up to kFeedBatch) live entries of a workgroup by destination d < NDST <= 64 and reserves, per
+// destination, a run behind `cursor_of(d)`.  On return s_pref[d] is where destination d starts in the ordered
+// batch (s_pref[NDST] = live entries) and s_gbase[d] where its run starts in the destination.
+template <int NDST, typename CursorOf>
+__device__ inline void feed_runs(const uint32_t (&dst)[kFeedItems], uint32_t (&rank)[kFeedItems], uint32_t *s_cnt,
+                                 uint32_t *s_pref, uint32_t *s_gbase, CursorOf cursor_of) {
+  static_assert(NDST <= 64, "one wave scans the destinations");
+  if (threadIdx.x < NDST) s_cnt[threadIdx.x] = 0;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kFeedItems; ++i) rank[i] = dst[i] != 0xffu ? atomicAdd(&s_cnt[dst[i]], 1u) : 0u;
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    const uint32_t n = threadIdx.x < NDST ? s_cnt[threadIdx.x] : 0u;
+    const uint32_t incl = wave_inclusive_scan(n);
+    if (threadIdx.x < NDST) {
+      s_pref[threadIdx.x] = incl - n;
+      s_gbase[threadIdx.x] = n ? atomicAdd(cursor_of(threadIdx.x), n) : 0u;
+    }
+    if (threadIdx.x == NDST - 1) s_pref[NDST] = incl;
+  }
+  __syncthreads();
+}
 
-template <typename CountSrc>
-__global__ __launch_bounds__(kSlabBlock) void k_feed_count(SlabGeom geo, CountSrc src,
-                                                           const uint32_t *__restrict__ list_count, uint32_t list_cap,
-                                                           uint32_t row_words, uint32_t *__restrict__ hist,
-                                                           int32_t *status) {
-  __shared__ uint32_t s_cnt[kSlabMaxBuckets];
+template <int W, typename Src>
+__global__ __launch_bounds__(kSlabBlock) void k_coarse_scatter(SlabGeom geo, CoarseGeom cg, Src src,
+                                                               const uint32_t *__restrict__ list_count,
+                                                               uint32_t list_cap, uint32_t *__restrict__ coarse_cursor,
+                                                               uint32_t *__restrict__ coarse_words, int32_t *status) {
+  constexpr int WS = Src::kStaged;
+  static_assert(WS >= 1 && WS <= W, "staged words");
+  __shared__ uint32_t s_cnt[kCoarseMax], s_pref[kCoarseMax + 1], s_gbase[kCoarseMax];
+  __shared__ uint32_t s_word[WS][kFeedBatch];
+  __shared__ uint8_t s_dst[kFeedBatch];
   if (list_count && *list_count > list_cap && blockIdx.x == 0 && threadIdx.x == 0)
     atomicOr(status, ZEN_STAT_RETRY);  // the list lost entries
   const uint32_t count = feed_count(list_count, list_cap);
   const uint32_t batch = blockIdx.x * (uint32_t)kFeedBatch;
   if (batch >= count) return;
-  for (uint32_t b = threadIdx.x; b < row_words; b += kSlabBlock) s_cnt[b] = 0;
-  __syncthreads();
-  uint32_t key[kFeedItems];
+  const uint32_t part = blockIdx.x % kCoarseSplit;
+  uint32_t w[kFeedItems][W], dst[kFeedItems], rank[kFeedItems];
 #pragma unroll
   for (int i = 0; i < kFeedItems; ++i) {
     const uint32_t e = batch + threadIdx.x + i * kSlabBlock;
-    key[i] = e < count ? src.key(e) : kNoSlot;
+    dst[i] = 0xffu;
+    uint32_t bucket = 0;
+    if (e < count && src.load(e, w[i], &bucket)) {
+      uint32_t rem;
+      dst[i] = SlabGeom::div_small(bucket, cg.per, cg.inv_per, &rem);
+    }
+  }
+  feed_runs<kCoarseMax>(dst, rank, s_cnt, s_pref, s_gbase,
+                        [&](uint32_t d) { return &coarse_cursor[(d * kCoarseSplit + part) * kCoarsePad]; });
+#pragma unroll
+  for (int i = 0; i < kFeedItems; ++i) {
+    if (dst[i] != 0xffu) {
+      const uint32_t p = s_pref[dst[i]] + rank[i];
+#pragma unroll
+      for (int q = 0; q < WS; ++q) s_word[q][p] = w[i][q];
+      s_dst[p] = (uint8_t)dst[i];
+    }
+  }
+  __syncthreads();
+  const uint32_t total = s_pref[kCoarseMax];
+  const size_t plane = (size_t)cg.groups * kCoarseSplit * cg.cap;  // words of one word plane
+  for (uint32_t p = threadIdx.x; p < total; p += kSlabBlock) {
+    const uint32_t d = s_dst[p];
+    const uint32_t at = s_gbase[d] + (p - s_pref[d]);
+    if (at < cg.cap) {
+      const size_t o = (size_t)(d * kCoarseSplit + part) * cg.cap + at;
+      uint32_t rec[W];
+#pragma unroll
+      for (int q = 0; q < WS; ++q) rec[q] = s_word[q][p];
+#pragma unroll
+      for (int q = WS; q < W; ++q) rec[q] = src.late(rec, q);
+#pragma unroll
+      for (int q = 0; q < W; ++q) coarse_words[q * plane + o] = rec[q];
+    } else {
+      atomicOr(status, ZEN_STAT_RETRY);  // a coarse slab is full: the general path answers
+    }
+  }
+}
+
+// Grid: (batches per part, parts of all coarse slabs).  Also writes bucket_lo for the coarse slab's buckets.
+template <int W, typename Sink>
+__global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, CoarseGeom cg, Sink sink,
+                                                             const uint32_t *__restrict__ coarse_cursor,
+                                                             const uint32_t *__restrict__ coarse_words,
+                                                             uint32_t *__restrict__ cursor,
+                                                             uint32_t *__restrict__ bucket_lo, int32_t *status) {
+  __shared__ uint32_t s_cnt[kCoarsePer], s_pref[kCoarsePer + 1], s_gbase[kCoarsePer];
+  __shared__ uint32_t s_word[W][kFeedBatch];
+  __shared__ uint8_t s_dst[kFeedBatch];
+  const uint32_t c = blockIdx.y / kCoarseSplit;
+  const uint32_t first_bucket = c * cg.per;
+  if (blockIdx.x == 0 && blockIdx.y % kCoarseSplit == 0 && threadIdx.x < cg.per &&
+      first_bucket + threadIdx.x < geo.nbuckets)
+    bucket_lo[first_bucket + threadIdx.x] = geo.first_key(first_bucket + threadIdx.x);  // a 64-bit division: once per bucket
+  uint32_t count = coarse_cursor[blockIdx.y * kCoarsePad];
+  if (count > cg.cap) count = cg.cap;  // the first step flagged the overflow
+  const uint32_t batch = blockIdx.x * (uint32_t)kFeedBatch;
+  if (batch >= count) return;
+  const size_t plane = (size_t)cg.groups * kCoarseSplit * cg.cap;
+  const uint32_t *from = coarse_words + (size_t)blockIdx.y * cg.cap;
+  uint32_t w[kFeedItems][W], dst[kFeedItems], rank[kFeedItems];
+#pragma unroll
+  for (int i = 0; i < kFeedItems; ++i) {
+    const uint32_t e = batch + threadIdx.x + i * kSlabBlock;
+    dst[i] = 0xffu;
+    if (e < count) {
+#pragma unroll
+      for (int q = 0; q < W; ++q) w[i][q] = from[q * plane + e];
+      dst[i] = 0;
+    }
   }
 #pragma unroll
   for (int i = 0; i < kFeedItems; ++i)
-    if (key[i] != kNoSlot) atomicAdd(&s_cnt[geo.bucket_of(key[i])], 1u);
-  __syncthreads();
-  uint32_t *row = hist + (size_t)blockIdx.x * row_words;
-  for (uint32_t b = threadIdx.x; b < row_words; b += kSlabBlock) row[b] = s_cnt[b];
-}
-
-// Workgroup = kScanCols buckets x kScanChunks ranges of batches.  hist[batch][bucket] becomes the number of the
-// bucket's entries in earlier batches; cursor[bucket] = the bucket's total; bucket_lo[bucket] = its first key.
-__global__ __launch_bounds__(kScanCols * kScanChunks) void k_feed_scan(SlabGeom geo,
-                                                                       const uint32_t *__restrict__ list_count,
-                                                                       uint32_t list_cap, uint32_t nbuckets,
-                                                                       uint32_t row_words, uint32_t *__restrict__ hist,
-                                                                       uint32_t *__restrict__ cursor,
-                                                                       uint32_t *__restrict__ bucket_lo,
-                                                                       int32_t *status);
-
-// Every kept entry of the batch goes to its bucket's slab as one 16-byte record (key, a, b, 0).  Scattered
-// stores cost one memory request each whatever their size (about 80 G requests/s on this part), so the batch
-// is first ordered by bucket in LDS: the records of a bucket then leave as one run, a few requests instead of
-// one per record.  A run's place in the slab comes from the scan.
-template <typename WriteSrc>
-__global__ __launch_bounds__(kSlabBlock) void k_feed_write(SlabGeom geo, WriteSrc src,
-                                                           const uint32_t *__restrict__ list_count, uint32_t list_cap,
-                                                           uint32_t row_words, const uint32_t *__restrict__ hist,
-                                                           uint4 *__restrict__ slab_rec) {
-  // entries of the batch per bucket; then (where the bucket's run starts in the ordered batch) << 13 | (where it
-  // starts in the slab).  One array, so that two workgroups fit into a compute unit's LDS.
-  __shared__ uint32_t s_cnt[kSlabMaxBuckets];
-  __shared__ uint4 s_rec[kFeedBatch];  // the ordered batch; .w = bucket << 13 | place in the slab
-  __shared__ uint32_t s_scan[kSlabBlock / 64 + 1];
-  static_assert(kSlabCap <= (1 << 13) && kFeedBatch < (1 << 13) && kSlabMaxBuckets <= (1 << 11), "packed fields");
-  const uint32_t count = feed_count(list_count, list_cap);
-  const uint32_t batch = blockIdx.x * (uint32_t)kFeedBatch;
-  if (batch >= count) return;
-  for (uint32_t b = threadIdx.x; b < (uint32_t)kSlabMaxBuckets; b += kSlabBlock) s_cnt[b] = 0;
-  // where the runs of this thread's buckets start in the slabs: asked for now, needed after the counting
-  constexpr int kPer = kSlabMaxBuckets / kSlabBlock;
-  uint32_t base[kPer];
-  {
-    const uint32_t *row = hist + (size_t)blockIdx.x * row_words;
-#pragma unroll
-    for (int e = 0; e < kPer; ++e) {
-      const uint32_t b = threadIdx.x * kPer + e;
-      base[e] = b < row_words ? row[b] : 0u;
-    }
-  }
-  __syncthreads();
-  uint32_t pa[kFeedItems], pb[kFeedItems], key[kFeedItems], bucket[kFeedItems], rank[kFeedItems];
+    if (dst[i] != 0xffu) dst[i] = sink.bucket(w[i]) - first_bucket;
+  feed_runs<kCoarsePer>(dst, rank, s_cnt, s_pref, s_gbase,
+                        [&](uint32_t d) { return &cursor[(first_bucket + d) * kCursorPad]; });
 #pragma unroll
   for (int i = 0; i < kFeedItems; ++i) {
-    const uint32_t e = batch + threadIdx.x + i * kSlabBlock;
-    pa[i] = pb[i] = 0;
-    key[i] = kNoSlot;
-    if (e < count) src.rec(e, &key[i], &pa[i], &pb[i]);
-  }
+    if (dst[i] != 0xffu) {
+      const uint32_t p = s_pref[dst[i]] + rank[i];
 #pragma unroll
-  for (int i = 0; i < kFeedItems; ++i) {
-    bucket[i] = rank[i] = 0;
-    if (key[i] != kNoSlot) {
-      bucket[i] = geo.bucket_of(key[i]);
-      rank[i] = atomicAdd(&s_cnt[bucket[i]], 1u);
+      for (int q = 0; q < W; ++q) s_word[q][p] = w[i][q];
+      s_dst[p] = (uint8_t)dst[i];
     }
   }
   __syncthreads();
-  uint32_t batch_live;
-  {
-    // thread owns kPer consecutive buckets: one exclusive prefix over the buckets gives every bucket's run a
-    // place in the ordered batch
-    uint32_t c[kPer];
-    uint32_t sum = 0;
+  const uint32_t total = s_pref[kCoarsePer];
+  for (uint32_t p = threadIdx.x; p < total; p += kSlabBlock) {
+    const uint32_t d = s_dst[p];
+    const uint32_t at = s_gbase[d] + (p - s_pref[d]);
+    if (at < (uint32_t)kSlabCap) {
+      uint32_t rec[W];
 #pragma unroll
-    for (int e = 0; e < kPer; ++e) {
-      c[e] = s_cnt[threadIdx.x * kPer + e];
-      sum += c[e];
+      for (int q = 0; q < W; ++q) rec[q] = s_word[q][p];
+      sink.store((size_t)(first_bucket + d) * kSlabCap + at, rec);
+    } else {
+      atomicOr(status, ZEN_STAT_RETRY);  // a slab is full: the general path answers
     }
-    uint32_t running = block_exclusive_scan<uint32_t, kSlabBlock>(sum, s_scan, &batch_live);
-#pragma unroll
-    for (int e = 0; e < kPer; ++e) {
-      // a run that starts past the slab's end (overflow, flagged by the scan) is clipped to the end
-      s_cnt[threadIdx.x * kPer + e] = (running << 13) | (base[e] < (uint32_t)kSlabCap ? base[e] : (uint32_t)kSlabCap);
-      running += c[e];
-    }
-  }
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < kFeedItems; ++i) {
-    if (key[i] != kNoSlot) {
-      const uint32_t sb = s_cnt[bucket[i]];
-      uint32_t pos = (sb & 8191u) + rank[i];
-      if (pos > 8191u) pos = 8191u;  // beyond the slab anyway: dropped below, must not spill into the bucket field
-      s_rec[(sb >> 13) + rank[i]] = make_uint4(key[i], pa[i], pb[i], (bucket[i] << 13) | pos);
-    }
-  }
-  __syncthreads();
-  // consecutive lanes write consecutive records of a run
-  for (uint32_t e = threadIdx.x; e < batch_live; e += kSlabBlock) {
-    uint4 rec = s_rec[e];
-    const uint32_t b = rec.w >> 13, pos = rec.w & 8191u;
-    rec.w = 0;
-    if (pos < (uint32_t)kSlabCap) slab_rec[(size_t)b * kSlabCap + pos] = rec;
   }
 }
 
-// Launches the three kernels.  hist: feed_batches(list_cap) * feed_row_words(nbuckets) words.
-template <typename CountSrc, typename WriteSrc>
-int feed_slabs(const SlabGeom &geo, const CountSrc &csrc, const WriteSrc &wsrc, const uint32_t *list_count,
-               int64_t list_cap, uint32_t *hist, uint32_t *cursor, uint32_t *bucket_lo, uint4 *slab_rec,
-               int32_t *status, hipStream_t s) {
-  const uint32_t row_words = feed_row_words(geo.nbuckets);
-  const unsigned batches = feed_batches(list_cap);
-  k_feed_count<CountSrc><<<dim3(batches), dim3(kSlabBlock), 0, s>>>(geo, csrc, list_count, (uint32_t)list_cap, row_words,
-                                                                    hist, status);
-  ZEN_LAUNCH_CHECK("k_feed_count");
-  k_feed_scan<<<dim3(row_words / kScanCols), dim3(kScanCols * kScanChunks), 0, s>>>(
-      geo, list_count, (uint32_t)list_cap, geo.nbuckets, row_words, hist, cursor, bucket_lo, status);
-  ZEN_LAUNCH_CHECK("k_feed_scan");
-  k_feed_write<WriteSrc><<<dim3(batches), dim3(kSlabBlock), 0, s>>>(geo, wsrc, list_count, (uint32_t)list_cap, row_words,
-                                                                    hist, slab_rec);
-  ZEN_LAUNCH_CHECK("k_feed_write");
+// Launches the two steps.  The cursors in `fb` must be zero.
+template <int W, typename Src, typename Sink>
+int feed_slabs(const SlabGeom &geo, const CoarseGeom &cg, const Src &src, const Sink &sink,
+               const uint32_t *list_count, int64_t list_cap, const FeedBuffers &fb, int32_t *status, hipStream_t s) {
+  k_coarse_scatter<W, Src><<<dim3(feed_batches(list_cap)), dim3(kSlabBlock), 0, s>>>(
+      geo, cg, src, list_count, (uint32_t)list_cap, fb.coarse_cursor, fb.coarse_words, status);
+  ZEN_LAUNCH_CHECK("k_coarse_scatter");
+  k_fine_scatter<W, Sink><<<dim3(feed_batches(cg.cap), cg.groups * kCoarseSplit), dim3(kSlabBlock), 0, s>>>(
+      geo, cg, sink, fb.coarse_cursor, fb.coarse_words, fb.cursor, fb.bucket_lo, status);
+  ZEN_LAUNCH_CHECK("k_fine_scatter");
   return ZEN_OK;
 }
 
