@@ -231,14 +231,17 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
     }
   }
   __syncthreads();
-  // Thread t owns the sorted places [t * kMergeItems, (t + 1) * kMergeItems).  It walks once from its first
+  // Thread t owns the sorted places [t * per, (t + 1) * per): as few per thread as cover the bucket, so that
+  // every thread has some (and an odd number, which keeps the lanes of a wave on different LDS banks).  It
+  // walks once from its first
   // place to the end of the last run that starts in its range, summing every run that starts there in arrival
   // order from +0 (like the dense tensor of comm.py:35), and leaves each sum in the value word of the run's
   // head.  (One walk: a loop per run would cost every lane of a wave the longest run of any lane, each time.)
   // A run's words are read by the thread of its head only, so the sums can be written in place.
-  const uint32_t first = threadIdx.x * kMergeItems;
+  const uint32_t per = ((n + kSlabBlock - 1) / kSlabBlock) | 1u;  // <= kMergeItems
+  const uint32_t first = threadIdx.x * per;
   if (first < n) {
-    const uint32_t end = first + kMergeItems < n ? first + kMergeItems : n;
+    const uint32_t end = first + per < n ? first + per : n;
     uint32_t cur = first > 0 ? sh.key[first - 1] : 0xffffffffu;  // index of the run the walk is in
     uint32_t head = 0xffffffffu;                                  // place of its head if it started in the range
     float acc = 0.0f;
@@ -268,7 +271,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
     const uint32_t p = first + q;
     k[q] = 0;
     sum[q] = 0.0f;
-    if (p < n) {
+    if ((uint32_t)q < per && p < n) {
       k[q] = sh.key[p];
       const bool is_head = p == 0 || k[q] != prev;
       prev = k[q];
