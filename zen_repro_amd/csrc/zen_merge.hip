@@ -149,7 +149,8 @@ constexpr int kMergeTarget = 3072;   // records a bucket is sized for: duplicate
 constexpr int kMergeItems = 13;      // sorted records per thread while summing (odd: no LDS bank conflicts)
 static_assert(kSlabBlock * kMergeItems >= kSlabCap, "every sorted place needs an owner");
 
-// An entry travels as (index, arrival number, value as fp32 bits).
+// An entry travels as (index, arrival number, value bits); in the bucket slabs the three sit in arrays of their
+// own (the value in its own type: ten bytes per bf16 entry).
 template <typename I, typename S>
 struct MergeSrc {
   SlabGeom geo;
@@ -160,9 +161,7 @@ struct MergeSrc {
   // the value is fetched again by arrival number when the entry is written: a workgroup's 4096 arrival numbers
   // are consecutive, so those loads hit the 8 KB it has just read
   static constexpr int kStaged = 2;
-  __device__ inline uint32_t late(const uint32_t (&w)[3], int) const {
-    return __float_as_uint(KeyOf<S>::to_f32(val[w[1]]));
-  }
+  __device__ inline uint32_t late(const uint32_t (&w)[3], int) const { return (uint32_t)val[w[1]]; }
   __device__ inline bool load(uint32_t e, uint32_t (&w)[3], uint32_t *bucket) const {
     const I k = idx[e];
     if (k < 0 || (uint64_t)k >= (uint64_t)dense_n) {
@@ -176,17 +175,25 @@ struct MergeSrc {
     return true;
   }
 };
+template <typename S>
 struct MergeSink {
   SlabGeom geo;
-  uint4 *slab_rec;
+  uint32_t *slab_idx, *slab_arr;
+  S *slab_val;
   __device__ inline uint32_t bucket(const uint32_t (&w)[3]) const { return geo.bucket_of(w[0]); }
-  __device__ inline void store(size_t at, const uint32_t (&w)[3]) const { slab_rec[at] = make_uint4(w[0], w[1], w[2], 0u); }
+  __device__ inline void store(size_t at, const uint32_t (&w)[3]) const {
+    slab_idx[at] = w[0];
+    slab_arr[at] = w[1];
+    slab_val[at] = (S)w[2];
+  }
 };
 
-template <typename I>
+template <typename I, typename S>
 __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const uint32_t *__restrict__ cursor,
                                                              const uint32_t *__restrict__ bucket_lo,
-                                                             const uint4 *__restrict__ slab_rec,
+                                                             const uint32_t *__restrict__ slab_idx,
+                                                             const uint32_t *__restrict__ slab_arr,
+                                                             const S *__restrict__ slab_val,
                                                              I *__restrict__ out_idx, float *__restrict__ out_val,
                                                              int64_t capacity, ScanState st, int tie_bits,
                                                              int64_t *out_count, int32_t *status) {
@@ -209,10 +216,9 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
     const uint32_t j = threadIdx.x + i * kSlabBlock;
     off[i] = arr[i] = val[i] = 0;
     if (j < n_raw) {
-      const uint4 rec = slab_rec[base + j];
-      off[i] = rec.x - lo;
-      arr[i] = rec.y;
-      val[i] = rec.z;
+      off[i] = slab_idx[base + j] - lo;
+      arr[i] = slab_arr[base + j];
+      val[i] = __float_as_uint(KeyOf<S>::to_f32(slab_val[base + j]));
       live |= 1u << i;
     }
   }
@@ -333,12 +339,13 @@ struct SlabMergePlan {
   unsigned long long *scan;  // prefix state over the buckets (zeroed before use)
   CoarseGeom cg;
   FeedBuffers feed;
-  uint4 *slab_rec;
+  uint32_t *slab_idx, *slab_arr;
+  void *slab_val;
   size_t zero_bytes;
   size_t bytes;
 };
 
-SlabMergePlan plan_slab_merge(void *workspace, const SlabGeom &geo, int64_t r) {
+SlabMergePlan plan_slab_merge(void *workspace, const SlabGeom &geo, int64_t r) {  // sized for 4-byte values
   Carver cv(workspace);
   SlabMergePlan p;
   const size_t B = geo.nbuckets;
@@ -350,7 +357,9 @@ SlabMergePlan plan_slab_merge(void *workspace, const SlabGeom &geo, int64_t r) {
   p.feed.bucket_lo = cv.take<uint32_t>(B);
   p.cg = coarse_geometry(geo, r);
   p.feed.coarse_words = cv.take<uint32_t>(feed_coarse_words(p.cg, 3));
-  p.slab_rec = cv.take<uint4>(B * kSlabCap);
+  p.slab_idx = cv.take<uint32_t>(B * kSlabCap);
+  p.slab_arr = cv.take<uint32_t>(B * kSlabCap);
+  p.slab_val = cv.take<uint32_t>(B * kSlabCap);
   p.bytes = cv.used;
   return p;
 }
@@ -373,7 +382,7 @@ int slab_merge_launch(const SlabGeom &geo, const I *idx, const S *val, int64_t r
   {
     ProfScope prof(kProfMergeFeed, s);
     const MergeSrc<I, S> src{geo, idx, val, (uint32_t)dense_n, status};
-    const MergeSink sink{geo, p.slab_rec};
+    const MergeSink<S> sink{geo, p.slab_idx, p.slab_arr, static_cast<S *>(p.slab_val)};
     const int rc = feed_slabs<3>(geo, p.cg, src, sink, nullptr, r, p.feed, status, s);
     if (rc != ZEN_OK) return rc;
   }
@@ -381,11 +390,13 @@ int slab_merge_launch(const SlabGeom &geo, const I *idx, const S *val, int64_t r
   const int tie_bits = ceil_log2_u64((uint64_t)r);  // arrival numbers are < r
   ProfScope prof(kProfMergeBucket, s);
   if (idx64_out)
-    k_merge_bucket<int64_t><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
-        geo, p.feed.cursor, p.feed.bucket_lo, p.slab_rec, static_cast<int64_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
+    k_merge_bucket<int64_t, S><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
+        geo, p.feed.cursor, p.feed.bucket_lo, p.slab_idx, p.slab_arr, static_cast<const S *>(p.slab_val),
+        static_cast<int64_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
   else
-    k_merge_bucket<int32_t><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
-        geo, p.feed.cursor, p.feed.bucket_lo, p.slab_rec, static_cast<int32_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
+    k_merge_bucket<int32_t, S><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
+        geo, p.feed.cursor, p.feed.bucket_lo, p.slab_idx, p.slab_arr, static_cast<const S *>(p.slab_val),
+        static_cast<int32_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
   ZEN_LAUNCH_CHECK("k_merge_bucket");
   return ZEN_OK;
 }
