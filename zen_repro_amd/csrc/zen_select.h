@@ -103,7 +103,7 @@ struct StageArgs {
   int32_t *list_idx = nullptr;
   void *list_val = nullptr;        // elements of the tensor's type
   int64_t capacity = 0;            // < 2^32
-  uint32_t *ticket = nullptr;
+  uint32_t *ticket = nullptr;      // select_stage_ticket_words() words
   uint32_t *cand_hist = nullptr;
   int64_t pick_k = 0;
   uint32_t *pick_thr = nullptr;
@@ -111,5 +111,6 @@ struct StageArgs {
   int32_t *status = nullptr;
 };
 int select_stage_list(const StageArgs &a, hipStream_t stream);
+size_t select_stage_ticket_words();
 
 }  // namespace zen

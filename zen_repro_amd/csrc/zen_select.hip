@@ -389,6 +389,7 @@ struct Flags<uint16_t> {
     const int a = bit & 15;
     return ((a >> 2) << 3) + ((a & 3) << 1) + (bit >> 4);
   }
+  static __device__ inline uint32_t vec_mask(int j) { return (0xfu << (4 * j)) * 0x00010001u; }  // flags of vector j
 };
 
 // fp32: element e sits at bit e.
@@ -408,6 +409,7 @@ struct Flags<uint32_t> {
   }
   static __device__ inline uint32_t below(int count) { return (uint32_t)((1ull << count) - 1ull); }
   static __device__ inline int offset_of(int bit) { return bit; }
+  static __device__ inline uint32_t vec_mask(int j) { return 0xfu << (4 * j); }  // flags of vector j
 };
 
 template <typename S, typename I, bool ALIGNED, bool STAGED>
@@ -664,6 +666,23 @@ __device__ inline void stage_load(const S *__restrict__ in, int64_t n, int64_t s
   }
 }
 
+// The same for a 16-byte aligned tensor, without a branch: vector numbers past the last complete vector are
+// pulled back onto it (their flags are cleared by the caller).  Loads that sit in branches make the compiler
+// wait for every load in flight wherever one of them is needed, and the point of the exercise is to have the
+// next two sub-tiles in flight while the current one is examined.
+template <typename S>
+__device__ inline void stage_load_fast(const S *__restrict__ in, uint32_t last_vec, uint32_t vec0,
+                                       uint4 (&q)[kSelVecs]) {
+  constexpr int V = VecOf<S>::kN;
+#pragma unroll
+  for (int j = 0; j < kSelVecs; ++j) {
+    uint32_t v = vec0 + (uint32_t)j * kSelBlock + threadIdx.x;
+    v = v < last_vec ? v : last_vec;
+    const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(in + (size_t)v * V));
+    q[j] = make_uint4(t.x, t.y, t.z, t.w);
+  }
+}
+
 // Word w (0..15) of the 64 bytes a thread holds, without indexing registers dynamically.
 __device__ inline uint32_t pick_word(const uint4 (&q)[kSelVecs], int w) {
   uint32_t r = 0;
@@ -714,11 +733,14 @@ __device__ inline void stage_flush(uint32_t count, const int32_t *st_idx, const 
 // How the sub-tiles (kSelBlock * kSelVecs vectors each) are handed out.  Every workgroup first takes
 // `fixed` tiles of kStageBig sub-tiles, tile i of workgroup b being number i * workgroups + b: no counter, and
 // the workgroups move through memory side by side (short tiles measured a little faster than long ones).  The rest of the tensor goes out in shorter tiles through a
-// ticket counter, so that workgroups that ran ahead take more and all finish within one short tile of each
-// other.  (A device-wide counter serves about 90 tickets per microsecond; 768 workgroups asking once per
-// kStageSmall sub-tiles stay below that.)
+// ticket counters, so that workgroups that ran ahead take more and all finish within one short tile of each
+// other.  A device-wide counter serves about 90 tickets per microsecond, and 768 workgroups asking one
+// counter every few microseconds would queue up for it: the workgroups form kStageGroups groups (by number
+// modulo kStageGroups) with a counter each, and ticket t of group g is short tile number g + t * kStageGroups.
 constexpr int kStageBig = 2;    // both tile lengths must be at least 2: the loads run two sub-tiles ahead
-constexpr int kStageSmall = 6;
+constexpr int kStageSmall = 2;
+constexpr int kStageGroups = 8;
+constexpr int kStageTicketPad = 32;  // words between two ticket counters: a 128-byte line each
 struct StageSched {
   uint32_t fixed;        // counter-free tiles per workgroup
   uint32_t fixed_subs;   // sub-tiles they cover together
@@ -748,9 +770,10 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
   if (floor_key > KeyOf<S>::kMask) floor_key = KeyOf<S>::kMask + 1u;  // nothing qualifies
   const int wave = threadIdx.x >> 6;
 
-  // A tile is (first sub-tile, number of sub-tiles); length 0 means there is none.  The tile after the current
-  // one is always known before the current one ends: its ticket is drawn when the current tile starts and
-  // handed to the other threads two sub-tiles before the end.  Three register sets take turns: while one sub-tile is examined the loads
+  // A tile is (first sub-tile, number of sub-tiles); length 0 means there is none.  The current tile and the
+  // one after it are always known (the loads run two sub-tiles ahead); the ticket of the tile after those is
+  // drawn when the current tile starts and handed to the other threads at its last sub-tile, so the counter
+  // has a whole tile's time to answer.  Three register sets take turns: while one sub-tile is examined the loads
   // of the next two are in flight.
   uint32_t cur_first = 0, cur_len = 0, nxt_first = 0, nxt_len = 0;
   auto fixed_tile = [&](uint32_t i, uint32_t &first, uint32_t &len) {
@@ -761,37 +784,71 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
     first = sch.fixed_subs + j * (uint32_t)kStageSmall;
     len = j < sch.ticket_tiles ? (uint32_t)kStageSmall : 0u;
   };
+  const uint32_t group = blockIdx.x % kStageGroups;
+  // workgroups of this group: its first tickets are theirs without asking (number blockIdx.x / kStageGroups)
+  const uint32_t group_size = (gridDim.x - group + kStageGroups - 1) / kStageGroups;
   uint32_t turn = 0;   // tiles this block has started
   uint32_t par = 0;    // sub-tiles this block has processed
   uint32_t count = 0;  // staged entries
   bool ticket_pending = false;
   uint32_t drawn = 0;  // thread 0: the ticket on its way
+  uint32_t far_first = 0, far_len = 0;  // the tile after the next one
+  // what the counter returns is kept as it is until it is handed over: any arithmetic on it here would make
+  // the wave wait for the answer, and for all its loads in flight with it
+  auto draw = [&]() { return atomicAdd(&ticket[group * kStageTicketPad], 1u); };
+  auto drawn_tile = [&](uint32_t raw) { return group + (group_size + raw) * kStageGroups; };
+  // tile number tn of this block if no ticket is needed for it: counter-free tiles first, then the block's
+  // own first short tile
+  auto known_tile = [&](uint32_t tn, uint32_t &first, uint32_t &len) {
+    if (tn < sch.fixed) {
+      fixed_tile(tn, first, len);
+      return true;
+    }
+    if (tn == sch.fixed) {
+      ticket_tile(blockIdx.x, first, len);  // = group + (blockIdx.x / kStageGroups) * kStageGroups
+      return true;
+    }
+    return false;
+  };
   int64_t sub_base = 0;
   uint32_t sub = 0;
   uint4 qa[kSelVecs], qb[kSelVecs], qc[kSelVecs];
 
-  // loads the sub-tile `ahead` places after the current one, if the block's sequence has one there
+  // complete vectors of the tensor (an aligned tensor's last n % V elements are looked at separately, below)
+  constexpr uint32_t kSubVecs = kSelBlock * kSelVecs;
+  const uint32_t full_vecs = (uint32_t)(n / V);
+  // loads the sub-tile `ahead` places after the current one in the block's sequence; if there is none, an
+  // aligned tensor still gets its loads (of the last vector: every wave always has the same number of loads
+  // in flight, which lets the compiler wait for exactly the ones it needs)
   auto load_ahead = [&](uint32_t ahead, uint4 (&q)[kSelVecs]) {
     const uint32_t p = sub + ahead;
-    if (p < cur_len)
-      stage_load<S, ALIGNED>(in, n, (int64_t)(cur_first + p) * kSub, q);
-    else if (p - cur_len < nxt_len)
-      stage_load<S, ALIGNED>(in, n, (int64_t)(nxt_first + p - cur_len) * kSub, q);
+    const bool here = p < cur_len, there = !here && p - cur_len < nxt_len;
+    const uint32_t unit = here ? cur_first + p : nxt_first + p - cur_len;
+    if (ALIGNED)
+      stage_load_fast<S>(in, full_vecs - 1u, here || there ? unit * kSubVecs : 0xffffffffu - kSubVecs, q);
+    else if (here || there)
+      stage_load<S, false>(in, n, (int64_t)unit * kSub, q);
   };
 
   // one sub-tile: cur holds its data, far receives the data of the sub-tile two places on
   auto body = [&](uint4 (&cur)[kSelVecs], uint4 (&far)[kSelVecs]) {
     uint32_t x = Flags<S>::build(cur, floor_key);
+    if (ALIGNED) {
+      const uint32_t vec0 = (cur_first + sub) * kSubVecs;
+      if (vec0 + kSubVecs > full_vecs) {  // the tensor ends inside this sub-tile (or before it)
+#pragma unroll
+        for (int j = 0; j < kSelVecs; ++j)
+          if (vec0 + (uint32_t)j * kSelBlock + threadIdx.x >= full_vecs) x &= ~Flags<S>::vec_mask(j);
+      }
+    }
     const uint32_t cnt = (uint32_t)__popc(x);
     const uint32_t incl = wave_inclusive_scan_dpp(cnt);
     if ((threadIdx.x & 63) == 63) s_wave[par & 1][wave] = incl;
-    // the ticket drawn when this tile started is first needed two sub-tiles before the tile ends; asking for
-    // it only now keeps the counter's round trip out of the way
-    const bool hand_over = ticket_pending && sub + 2 >= cur_len;
+    const bool hand_over = ticket_pending && sub + 1 == cur_len;
     if (hand_over && threadIdx.x == 0) s_next[turn & 1] = drawn;
     __syncthreads();
     if (hand_over) {
-      ticket_tile(s_next[turn & 1], nxt_first, nxt_len);
+      ticket_tile(drawn_tile(s_next[turn & 1]), far_first, far_len);
       ticket_pending = false;
     }
     load_ahead(2, far);
@@ -831,43 +888,71 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
     }
   };
 
-  if (sch.fixed > 0)
-    fixed_tile(0, cur_first, cur_len);
-  else
-    ticket_tile(blockIdx.x, cur_first, cur_len);
-  uint32_t rot = 0;  // par % 3
+  known_tile(0, cur_first, cur_len);
+  if (!known_tile(1, nxt_first, nxt_len)) {  // short inputs: the second tile already needs a ticket
+    if (threadIdx.x == 0) s_next[1] = draw();
+    __syncthreads();
+    ticket_tile(drawn_tile(s_next[1]), nxt_first, nxt_len);
+  }
   if (cur_len) {
-    stage_load<S, ALIGNED>(in, n, (int64_t)cur_first * kSub, qa);
     sub = 0;
+    if (ALIGNED)
+      stage_load_fast<S>(in, full_vecs - 1u, cur_first * kSubVecs, qa);
+    else
+      stage_load<S, false>(in, n, (int64_t)cur_first * kSub, qa);
     load_ahead(1, qb);  // tiles have at least two sub-tiles
   }
-  while (cur_len) {
-    // the tile after this one
-    if (turn + 1 < sch.fixed) {
-      fixed_tile(turn + 1, nxt_first, nxt_len);
-    } else if (turn + 1 == sch.fixed) {
-      ticket_tile(blockIdx.x, nxt_first, nxt_len);
-    } else {
-      nxt_len = 0;
+  // Starts a tile: the ticket of the tile after the next one is asked for.
+  auto open_tile = [&]() {
+    far_len = 0;
+    if (!known_tile(turn + 2, far_first, far_len)) {
       ticket_pending = true;
-      if (threadIdx.x == 0) drawn = gridDim.x + atomicAdd(ticket, 1u);
+      if (threadIdx.x == 0) drawn = draw();
     }
-    for (sub = 0; sub < cur_len; ++sub, ++par) {
-      sub_base = (int64_t)(cur_first + sub) * kSub;
-      if (rot == 0)
-        body(qa, qc);
-      else if (rot == 1)
-        body(qb, qa);
-      else
-        body(qc, qb);
-      rot = rot == 2 ? 0 : rot + 1;
+  };
+  // One sub-tile of the block's sequence, then on to the next place in it.  False when the sequence has ended.
+  auto step = [&](uint4 (&cur)[kSelVecs], uint4 (&far)[kSelVecs]) {
+    if (cur_len == 0) return false;
+    if (sub == 0) open_tile();
+    sub_base = (int64_t)(cur_first + sub) * kSub;
+    body(cur, far);
+    ++par;
+    if (++sub == cur_len) {
+      cur_first = nxt_first;
+      cur_len = nxt_len;
+      nxt_first = far_first;
+      nxt_len = far_len;
+      ++turn;
+      sub = 0;
     }
-    cur_first = nxt_first;
-    cur_len = nxt_len;
-    ++turn;
+    return true;
+  };
+  // The three register sets keep their roles in straight-line code (a set chosen by a run-time number would be
+  // copied from tile to tile, and the copy waits for every load in flight).
+  for (;;) {
+    if (!step(qa, qc)) break;
+    if (!step(qb, qa)) break;
+    if (!step(qc, qb)) break;
   }
   __syncthreads();
   if (count) stage_flush<S>(count, st_idx, st_val, &s_base, hist, floor_key, list_count, list_idx, list_val, capacity);
+  if (ALIGNED && blockIdx.x == 0 && threadIdx.x == 0) {
+    // the elements behind the last complete vector (fewer than V), one by one
+    for (int64_t e = (int64_t)full_vecs * V; e < n; ++e) {
+      const S v = in[e];
+      if ((v & KeyOf<S>::kMask) >= floor_key) {
+        const uint32_t at = atomicAdd(list_count, 1u);
+        if (at < capacity) {
+          list_idx[at] = (int32_t)e;
+          list_val[at] = v;
+        }
+        if (hist) {
+          const uint32_t bin = ((v & KeyOf<S>::kMask) - floor_key) >> (sizeof(S) == 2 ? 0 : 16);
+          atomicAdd(&s_hist[bin < (uint32_t)kCandBins - 1u ? bin : (uint32_t)kCandBins - 1u], 1u);
+        }
+      }
+    }
+  }
   if (hist) {
     __syncthreads();
     uint32_t *row = cand_hist + (size_t)(blockIdx.x % kCandRows) * kCandBins;
@@ -926,7 +1011,7 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   sch.fixed_subs = sch.fixed * (uint32_t)kStageBig * (uint32_t)blocks;
   sch.ticket_tiles = (uint32_t)ceil_div(subs - (int64_t)sch.fixed_subs, kStageSmall);
   const S *in = static_cast<const S *>(a.in);
-  const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+  const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0 && a.n >= V;
   ProfScope prof(kProfSelectStage, stream);
   if (aligned)
     k_select_stage<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
@@ -939,6 +1024,8 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   ZEN_LAUNCH_CHECK("k_select_stage");
   return ZEN_OK;
 }
+
+size_t select_stage_ticket_words() { return (size_t)kStageGroups * kStageTicketPad; }
 
 int select_stage_list(const StageArgs &a, hipStream_t stream) {
   if (a.dtype == ZEN_BF16) return stage_launch<uint16_t>(a, stream);

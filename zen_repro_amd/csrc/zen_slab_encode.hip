@@ -573,7 +573,7 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.zero_begin = cv.base + cv.used;
   p.sample_hist = cv.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
   p.cand_hist = cv.take<uint32_t>((size_t)kCandHistWords);
-  p.ticket = cv.take<uint32_t>(4);
+  p.ticket = cv.take<uint32_t>(select_stage_ticket_words());
   p.list_count = cv.take<uint32_t>(4);
   p.tb.cursor = cv.take<uint32_t>(B * kCursorPad);
   p.feed.coarse_cursor = cv.take<uint32_t>(feed_coarse_cursor_words());
