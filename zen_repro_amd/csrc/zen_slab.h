@@ -27,7 +27,7 @@ constexpr int kSlabCap = kSlabBlock * kSlabItems;     // records per slab (6144)
 constexpr int kSlabSubs = 4096;                       // narrow key ranges inside a bucket (about one record each)
 constexpr int kSlabSubsPer = kSlabSubs / kSlabBlock;
 constexpr int kSlabGroupLimit = 1024;                 // bounds the rank loop on piled-up keys
-constexpr int kSlabMaxBuckets = 2048;
+constexpr int kSlabMaxBuckets = 4096;
 constexpr int kSlabTarget = 3584;                     // records a bucket is sized for (leaves 40 % to spare)
 constexpr int kSlabResident = 512;                    // per-bucket workgroups the chip holds at a time (256 CUs x 2)
 constexpr int kSlabMoveCap = 1024;                    // entries that may move into one bucket from elsewhere
