@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
     }
   }
   uint32_t n = 0;
-  const bool ranked = slab_rank(sh, geo, tie_bits, off, arr, live, rank, &n);
+  const bool ranked = slab_rank<kSlabBlock>(sh, geo, tie_bits, off, arr, live, rank, &n);
   if (!ranked) {
     if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
     n = 0;  // the bucket contributes nothing; the prefix protocol still gets its (empty) tile

@@ -21,11 +21,11 @@ namespace zen {
 constexpr uint32_t kRemovedBit = 1u << 31;  // in a sorted index word: the entry lost its level-1 slot
 constexpr uint32_t kIndexMask = kRemovedBit - 1u;
 
-constexpr int kSlabBlock = 512;                       // threads of a per-bucket workgroup
+constexpr int kSlabBlock = 512;                       // threads of a per-bucket workgroup (the sort takes twice as many)
 constexpr int kSlabItems = 12;                        // records per thread
 constexpr int kSlabCap = kSlabBlock * kSlabItems;     // records per slab (6144)
 constexpr int kSlabSubs = 4096;                       // narrow key ranges inside a bucket (about one record each)
-constexpr int kSlabSubsPer = kSlabSubs / kSlabBlock;
+constexpr int kSlabMaxBlock = 1024;                   // largest workgroup that ranks a slab
 constexpr int kSlabGroupLimit = 1024;                 // bounds the rank loop on piled-up keys
 constexpr int kSlabMaxBuckets = 4096;
 constexpr int kSlabTarget = 3584;                     // records a bucket is sized for (leaves 40 % to spare)
@@ -116,11 +116,14 @@ inline bool slab_geometry(int64_t m, int partitions, int64_t expected, int targe
   return true;
 }
 
-// Where the counter of narrow range s lives in SlabSortShared::cnt: a thread owns kSlabSubsPer consecutive
-// ranges during the prefix step, and this keeps the lanes of a wave on different LDS banks while they walk
-// through their ranges.  Range kSlabSubs (the end marker) stays at index kSlabSubs.
+// Where the counter of narrow range s lives in SlabSortShared::cnt when BLOCK threads rank the slab: a thread
+// owns kSlabSubs / BLOCK consecutive ranges during the prefix step, and this keeps the lanes of a wave on
+// different LDS banks while they walk through their ranges.  Range kSlabSubs (the end marker) stays at index
+// kSlabSubs.
+template <int BLOCK>
 __device__ inline uint32_t sub_place(uint32_t s) {
-  return s < (uint32_t)kSlabSubs ? (s % kSlabSubsPer) * kSlabBlock + s / kSlabSubsPer : s;
+  constexpr uint32_t kPer = kSlabSubs / BLOCK;
+  return s < (uint32_t)kSlabSubs ? (s % kPer) * BLOCK + s / kPer : s;
 }
 
 // Shared memory of the in-LDS sort.
@@ -128,70 +131,75 @@ struct SlabSortShared {
   uint32_t key[kSlabCap];
   uint32_t tie[kSlabCap];
   uint32_t cnt[kSlabSubs + 1];
-  uint32_t scan[kSlabBlock / 64 + 1];
+  uint32_t scan[kSlabMaxBlock / 64 + 1];
   uint32_t bad;
 };
 
-// Ranks the live records of a workgroup by (key offset, tie); tie < 2^tie_bits, the pair unique, and
+// Ranks the live records of a workgroup of BLOCK threads (kSlabCap / BLOCK records each) by (key offset, tie);
+// tie < 2^tie_bits, the pair unique, and
 // geo.sub_shift + tie_bits <= 32.  off[i] < bucket width.  The records are first grouped by narrow key range
 // with one LDS atomic each; a record is then one word, (offset inside the range) << tie_bits | tie, and
 // inside its group every record counts the words smaller than its own.  Returns false (for every thread) if a
 // group is too large for that; else rank[i] for live records and *n_out = number of live records.  On return
 // sh.key / sh.tie may be overwritten at once (sh.tie is not touched at all).
+template <int BLOCK>
 __device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, int tie_bits,
-                                 const uint32_t (&off)[kSlabItems], const uint32_t (&tie)[kSlabItems], uint32_t live,
-                                 uint32_t (&rank)[kSlabItems], uint32_t *n_out) {
-  for (int d = threadIdx.x; d <= kSlabSubs; d += kSlabBlock) sh.cnt[d] = 0;
+                                 const uint32_t (&off)[kSlabCap / BLOCK], const uint32_t (&tie)[kSlabCap / BLOCK],
+                                 uint32_t live, uint32_t (&rank)[kSlabCap / BLOCK], uint32_t *n_out) {
+  static_assert(BLOCK <= kSlabMaxBlock && kSlabCap % BLOCK == 0 && kSlabSubs % BLOCK == 0, "workgroup size");
+  constexpr int kItems = kSlabCap / BLOCK;
+  constexpr int kSubsPer = kSlabSubs / BLOCK;
+  for (int d = threadIdx.x; d <= kSlabSubs; d += BLOCK) sh.cnt[d] = 0;
   if (threadIdx.x == 0) sh.bad = 0;
   __syncthreads();
   const uint32_t low_mask = (1u << geo.sub_shift) - 1u;
-  uint32_t sub[kSlabItems], at[kSlabItems];
+  uint32_t sub[kItems], at[kItems];
 #pragma unroll
-  for (int i = 0; i < kSlabItems; ++i) {
+  for (int i = 0; i < kItems; ++i) {
     sub[i] = at[i] = 0;
     if (live & (1u << i)) {
       sub[i] = off[i] >> geo.sub_shift;
-      at[i] = atomicAdd(&sh.cnt[sub_place(sub[i])], 1u);
+      at[i] = atomicAdd(&sh.cnt[sub_place<BLOCK>(sub[i])], 1u);
     }
   }
   __syncthreads();
   {
-    uint32_t c[kSlabSubsPer];
+    uint32_t c[kSubsPer];
     uint32_t sum = 0, big = 0;
 #pragma unroll
-    for (int e = 0; e < kSlabSubsPer; ++e) {
-      c[e] = sh.cnt[e * kSlabBlock + threadIdx.x];
+    for (int e = 0; e < kSubsPer; ++e) {
+      c[e] = sh.cnt[e * BLOCK + threadIdx.x];
       sum += c[e];
       big |= c[e] > (uint32_t)kSlabGroupLimit;
     }
     if (big) sh.bad = 1;
     uint32_t total;
-    uint32_t running = block_exclusive_scan<uint32_t, kSlabBlock>(sum, sh.scan, &total);
+    uint32_t running = block_exclusive_scan<uint32_t, BLOCK>(sum, sh.scan, &total);
 #pragma unroll
-    for (int e = 0; e < kSlabSubsPer; ++e) {
-      sh.cnt[e * kSlabBlock + threadIdx.x] = running;
+    for (int e = 0; e < kSubsPer; ++e) {
+      sh.cnt[e * BLOCK + threadIdx.x] = running;
       running += c[e];
     }
-    if (threadIdx.x == kSlabBlock - 1) sh.cnt[kSlabSubs] = running;
+    if (threadIdx.x == BLOCK - 1) sh.cnt[kSlabSubs] = running;
   }
   __syncthreads();
   if (sh.bad) return false;
-  uint32_t g0[kSlabItems], word[kSlabItems];
+  uint32_t g0[kItems], word[kItems];
 #pragma unroll
-  for (int i = 0; i < kSlabItems; ++i) {
+  for (int i = 0; i < kItems; ++i) {
     g0[i] = word[i] = 0;
     if (live & (1u << i)) {
-      g0[i] = sh.cnt[sub_place(sub[i])];
+      g0[i] = sh.cnt[sub_place<BLOCK>(sub[i])];
       word[i] = ((off[i] & low_mask) << tie_bits) | tie[i];
       sh.key[g0[i] + at[i]] = word[i];
     }
   }
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < kSlabItems; ++i) {
+  for (int i = 0; i < kItems; ++i) {
     rank[i] = 0;
     if (live & (1u << i)) {
-      const uint32_t g1 = sh.cnt[sub_place(sub[i] + 1)];
+      const uint32_t g1 = sh.cnt[sub_place<BLOCK>(sub[i] + 1)];
       uint32_t less = 0;
       for (uint32_t u = g0[i]; u < g1; ++u) less += sh.key[u] < word[i];
       rank[i] = g0[i] + less;

@@ -88,8 +88,14 @@ struct EncodeSink {
 
 // ------------------------------------------------------------ sort a bucket
 
+// Twice the threads of the other per-bucket kernels, half the records each: the phases of this kernel are
+// chains of LDS round trips, and eight waves per SIMD hide them better than four (38 -> 30 us); it needs
+// fewer than 64 registers, so two workgroups still share a compute unit.
+constexpr int kSortBlock = 1024;
+constexpr int kSortItems = kSlabCap / kSortBlock;
+
 template <typename S>
-__global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTables tb, int32_t *status) {
+__global__ __launch_bounds__(kSortBlock, 2) void k_slab_sort(SlabGeom geo, SlabTables tb, int32_t *status) {
   __shared__ SlabSortShared sh;
   __shared__ S s_val[kSlabCap];
   __shared__ uint32_t s_lost, s_base;
@@ -100,12 +106,12 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
   const uint32_t lo = tb.bucket_lo[b];
   S *slab_val = static_cast<S *>(tb.slab_val);
   if (threadIdx.x == 0) s_lost = 0;
-  uint32_t off[kSlabItems], idx[kSlabItems], pos[kSlabItems], rank[kSlabItems];
-  S val[kSlabItems];
+  uint32_t off[kSortItems], idx[kSortItems], pos[kSortItems], rank[kSortItems];
+  S val[kSortItems];
   uint32_t live = 0;
 #pragma unroll
-  for (int i = 0; i < kSlabItems; ++i) {
-    const uint32_t j = threadIdx.x + i * kSlabBlock;
+  for (int i = 0; i < kSortItems; ++i) {
+    const uint32_t j = threadIdx.x + i * kSortBlock;
     off[i] = idx[i] = pos[i] = 0;
     val[i] = 0;
     if (j < n_raw) {
@@ -121,7 +127,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
   // while it is ranked); the runs of equal slots, few and short, are put right afterwards
   static_assert(kSlabCap <= (1 << 13), "slab places in 13 bits");
   uint32_t n = 0;
-  if (!slab_rank(sh, geo, 13, off, pos, live, rank, &n)) {
+  if (!slab_rank<kSortBlock>(sh, geo, 13, off, pos, live, rank, &n)) {
     if (threadIdx.x == 0) {
       atomicOr(status, ZEN_STAT_RETRY);
       tb.bucket_n[b] = 0;
@@ -130,7 +136,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
     return;
   }
 #pragma unroll
-  for (int i = 0; i < kSlabItems; ++i) {
+  for (int i = 0; i < kSortItems; ++i) {
     if (live & (1u << i)) {
       sh.key[rank[i]] = off[i];
       sh.tie[rank[i]] = idx[i];
@@ -139,7 +145,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
   }
   __syncthreads();
   // a run of equal slots gets its smallest index in front (the thread at the run's first place does it)
-  for (uint32_t p = threadIdx.x; p + 1 < n; p += kSlabBlock) {
+  for (uint32_t p = threadIdx.x; p + 1 < n; p += kSortBlock) {
     const uint32_t k = sh.key[p];
     if (sh.key[p + 1] == k && (p == 0 || sh.key[p - 1] != k)) {
       uint32_t best = p;
@@ -159,7 +165,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
   // In a run of equal slots the first entry has the smallest index: the slot's level-1 owner.  The others
   // lost level 1.  Their places in the sorted slab are collected in sh.cnt (a bucket has at most kSlabSubs
   // of them, else the call is declined).
-  for (uint32_t p = threadIdx.x; p < n; p += kSlabBlock) {
+  for (uint32_t p = threadIdx.x; p < n; p += kSortBlock) {
     const uint32_t k = sh.key[p];
     const bool lost = p > 0 && sh.key[p - 1] == k;
     tb.slab_key[base + p] = k + lo;
@@ -182,7 +188,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_sort(SlabGeom geo, SlabTabl
     s_base = lost_n ? atomicAdd(&tb.ctr->losers, lost_n) : 0u;
   }
   __syncthreads();
-  for (uint32_t i = threadIdx.x; i < lost_n; i += kSlabBlock) {
+  for (uint32_t i = threadIdx.x; i < lost_n; i += kSortBlock) {
     const uint32_t at = s_base + i;
     const uint32_t p = sh.cnt[i];
     if (at < tb.log_cap) {
@@ -624,7 +630,7 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
   }
   {
     ProfScope prof(kProfSlabSort, s);
-    k_slab_sort<S><<<dim3(B), dim3(kSlabBlock), 0, s>>>(geo, p.tb, a.status);
+    k_slab_sort<S><<<dim3(B), dim3(kSortBlock), 0, s>>>(geo, p.tb, a.status);
     ZEN_LAUNCH_CHECK("k_slab_sort");
   }
   {
