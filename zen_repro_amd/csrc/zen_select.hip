@@ -390,6 +390,13 @@ struct Flags<uint16_t> {
     return ((a >> 2) << 3) + ((a & 3) << 1) + (bit >> 4);
   }
   static __device__ inline uint32_t vec_mask(int j) { return (0xfu << (4 * j)) * 0x00010001u; }  // flags of vector j
+  // where the element of flag `bit` sits relative to the thread's first element of the sub-tile, when vector j
+  // of thread t starts at element (j * kSelBlock + t) * 8: bit = 4j + w + 16h is element 2w + h of vector j
+  static __device__ inline uint32_t elem_step(uint32_t bit) {
+    const uint32_t a = bit & 15u;
+    return (a >> 2) * (uint32_t)(kSelBlock * 8) + ((a & 3u) << 1) + (bit >> 4);
+  }
+  static __device__ inline uint16_t pick(const uint4 (&q)[kSelVecs], uint32_t bit);
 };
 
 // fp32: element e sits at bit e.
@@ -410,6 +417,10 @@ struct Flags<uint32_t> {
   static __device__ inline uint32_t below(int count) { return (uint32_t)((1ull << count) - 1ull); }
   static __device__ inline int offset_of(int bit) { return bit; }
   static __device__ inline uint32_t vec_mask(int j) { return 0xfu << (4 * j); }  // flags of vector j
+  static __device__ inline uint32_t elem_step(uint32_t bit) {  // bit = 4j + w is element w of vector j
+    return (bit >> 2) * (uint32_t)(kSelBlock * 4) + (bit & 3u);
+  }
+  static __device__ inline uint32_t pick(const uint4 (&q)[kSelVecs], uint32_t bit);
 };
 
 template <typename S, typename I, bool ALIGNED, bool STAGED>
@@ -695,6 +706,15 @@ __device__ inline uint32_t pick_word(const uint4 (&q)[kSelVecs], int w) {
   }
   return r;
 }
+// The element a flag bit stands for, straight from the flag's number (word 4j + w, half h for bf16).
+__device__ inline uint16_t Flags<uint16_t>::pick(const uint4 (&q)[kSelVecs], uint32_t bit) {
+  const uint32_t w = pick_word(q, (int)(bit & 15u));
+  return (uint16_t)((bit >> 4) ? (w >> 16) : (w & 0xffffu));
+}
+__device__ inline uint32_t Flags<uint32_t>::pick(const uint4 (&q)[kSelVecs], uint32_t bit) {
+  return pick_word(q, (int)bit);
+}
+
 template <typename S>
 __device__ inline S pick_elem(const uint4 (&q)[kSelVecs], int off);
 template <>
@@ -860,21 +880,23 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
       total += t;
     }
     const uint32_t all = x;
+    const uint32_t first_elem = (uint32_t)sub_base + threadIdx.x * (uint32_t)V;  // indices are below 2^31
     uint32_t done = 0;
     for (;;) {
       const uint32_t room = (uint32_t)kScatStage - count;
       const uint32_t hi = done + room;
       uint32_t y = x;
       while (y) {
-        const int bit = __ffs((int)y) - 1;
+        const uint32_t bit = (uint32_t)__ffs((int)y) - 1u;
         y &= y - 1;
-        const int off = Flags<S>::offset_of(bit);
-        const uint32_t pos = before + (uint32_t)__popc(all & Flags<S>::below(off));
+        // the thread's candidates take their places in the order of their flag bits (the list has no order
+        // to keep, and a place counted off the flag word costs two instructions)
+        const uint32_t pos = before + (uint32_t)__popc(all & ((1u << bit) - 1u));
         if (pos < hi) {
           x &= ~(1u << bit);
           const uint32_t at = count + pos - done;
-          st_idx[at] = (int32_t)(sub_base + ((int64_t)(off / V) * kSelBlock + threadIdx.x) * V + (off % V));
-          st_val[at] = pick_elem<S>(cur, off);
+          st_idx[at] = (int32_t)(first_elem + Flags<S>::elem_step(bit));
+          st_val[at] = Flags<S>::pick(cur, bit);
         }
       }
       const uint32_t take = total - done < room ? total - done : room;
