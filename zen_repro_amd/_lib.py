@@ -119,23 +119,32 @@ class Scratch:
     """Cache of raw byte buffers per device and host thread, grown on demand
     and reused.  A buffer is tied to the stream order of its users, like any
     torch tensor; two threads that enqueue calls side by side (their kernels
-    interleave even on one stream) never share one."""
+    interleave even on one stream) never share one, and a thread's buffers go
+    when the thread does."""
 
     def __init__(self):
-        self._bufs = {}
+        self._local = threading.local()
+
+    def _bufs(self):
+        bufs = getattr(self._local, "bufs", None)
+        if bufs is None:
+            bufs = self._local.bufs = {}
+        return bufs
 
     def get(self, device, name, nbytes, zero=False):
         key = (torch.device(device).index if torch.device(device).index is not None
-               else torch.cuda.current_device(), threading.get_ident(), name)
-        buf = self._bufs.get(key)
+               else torch.cuda.current_device(), name)
+        bufs = self._bufs()
+        buf = bufs.get(key)
         if buf is None or buf.numel() < nbytes:
             alloc = torch.zeros if zero else torch.empty
             buf = alloc(max(int(nbytes), 256), dtype=torch.uint8, device=device)
-            self._bufs[key] = buf
+            bufs[key] = buf
         return buf
 
     def drop(self):
-        self._bufs.clear()
+        """Forget the calling thread's buffers."""
+        self._bufs().clear()
 
 
 scratch = Scratch()
