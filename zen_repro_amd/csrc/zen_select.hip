@@ -13,7 +13,8 @@ namespace {
 
 constexpr int kHistBins = 2048;
 constexpr int kHistBlock = 256;
-constexpr int kSampleLog2 = 8;  // the sample is one 16-byte vector in 256
+constexpr int kSampleLog2Min = 6, kSampleLog2Max = 10;  // the sample is one 16-byte vector in 64 ... 1024
+constexpr int64_t kSampleHits = 7000;  // sample elements wanted at or above the threshold
 
 struct TopkState {
   uint32_t prefix;    // key bits fixed so far (right aligned)
@@ -1100,7 +1101,12 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
   constexpr int V = VecOf<S>::kN;
   uint32_t *hist = static_cast<uint32_t *>(workspace);
   const int64_t nvec = ceil_div(n, V);
-  const int64_t nblocks = ceil_div(nvec, 1ll << kSampleLog2);
+  // Every sampled vector lies on a page of its own, and the kernel spends its time waiting for their address
+  // translations: the sample is as thin as leaves about kSampleHits of its elements above the threshold
+  // (their count then scatters by 1.2 %, and the six deviations allowed for below cost 7 % more candidates).
+  int sample_log2 = kSampleLog2Max;
+  while (sample_log2 > kSampleLog2Min && (k >> sample_log2) < kSampleHits) --sample_log2;
+  const int64_t nblocks = ceil_div(nvec, 1ll << sample_log2);
   // rank to look for in the sample: the expected one plus six standard
   // deviations of a binomial count, so that the full tensor almost surely holds
   // at least k elements at or above the bin found (callers verify and retry)
@@ -1118,10 +1124,10 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
   {
     ProfScope prof(kProfTopkHist, stream);
     if (aligned)
-      k_sample_hist<S, true><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist, rank,
+      k_sample_hist<S, true><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, sample_log2, hist, rank,
                                                                                         thr_lo);
     else
-      k_sample_hist<S, false><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, kSampleLog2, hist,
+      k_sample_hist<S, false><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, sample_log2, hist,
                                                                                          rank, thr_lo);
     ZEN_LAUNCH_CHECK("k_sample_hist");
   }
