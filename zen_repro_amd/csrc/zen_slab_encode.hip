@@ -39,9 +39,9 @@ struct SlabTables {
   uint32_t *movein_n;   // [B] entries whose final slot lies in the bucket but whose level-1 slot does not own it
   uint32_t *serial_n;   // [P] entries that found no slot
   uint2 *slab_rec;      // [B * kSlabCap] records as they arrive: (index, value)
-  int32_t *slab_idx;    // [B * kSlabCap] after the sort: index | kRemovedBit
+  int32_t *slab_idx;    // [B * kSlabCap] after the sort: index | kRemovedBit, by ascending level-1 slot (the slot
+                        // itself is not kept: hashing the index again is cheaper than a trip to memory)
   void *slab_val;       // [B * kSlabCap] after the sort: value
-  uint32_t *slab_key;   // [B * kSlabCap] after the sort: level-1 slot, ascending inside a slab
   uint32_t *mv_key, *mv_idx, *mv_val;  // [B * kSlabMoveCap]
   uint32_t *ser_idx;    // [P * kSlabSerialCap]
   uint32_t *log_t, *log_v, *log_cell;  // [log_cap]
@@ -168,7 +168,6 @@ __global__ __launch_bounds__(kSortBlock, 2) void k_slab_sort(SlabGeom geo, SlabT
   for (uint32_t p = threadIdx.x; p < n; p += kSortBlock) {
     const uint32_t k = sh.key[p];
     const bool lost = p > 0 && sh.key[p - 1] == k;
-    tb.slab_key[base + p] = k + lo;
     tb.slab_idx[base + p] = (int32_t)(sh.tie[p] | (lost ? kRemovedBit : 0u));
     slab_val[base + p] = s_val[p];  // every thread has read its records: in place is safe
     if (lost) {
@@ -202,17 +201,27 @@ __global__ __launch_bounds__(kSortBlock, 2) void k_slab_sort(SlabGeom geo, SlabT
 
 // ------------------------------------------------------ levels 2 and 3
 
-// Smallest index whose level-1 slot is `slot` (kNone if nobody's), and where it sits.
+// Smallest index whose level-1 slot is `slot` (kNone if nobody's), and where it sits: bisection over the
+// bucket's sorted indices by their level-1 slots.
 __device__ inline uint32_t slab_head(const SlabGeom &geo, const SlabTables &tb, uint32_t slot, size_t *pos_out,
                                      uint32_t *bucket_out) {
   const uint32_t b = geo.bucket_of(slot);
-  const uint32_t *keys = tb.slab_key + (size_t)b * kSlabCap;
+  const int32_t *idx = tb.slab_idx + (size_t)b * kSlabCap;
   const uint32_t n = tb.bucket_n[b];
-  const uint32_t p = lower_bound_u32(keys, n, slot);
-  if (p >= n || keys[p] != slot) return kNone;
-  *pos_out = (size_t)b * kSlabCap + p;
+  uint32_t lo = 0, hi = n;
+  while (lo < hi) {
+    const uint32_t mid = lo + ((hi - lo) >> 1);
+    if (geo.mod_m(poly((uint32_t)idx[mid] & kIndexMask) + kSeed1) < slot)
+      lo = mid + 1;
+    else
+      hi = mid;
+  }
+  if (lo >= n) return kNone;
+  const uint32_t t = (uint32_t)idx[lo] & kIndexMask;
+  if (geo.mod_m(poly(t) + kSeed1) != slot) return kNone;
+  *pos_out = (size_t)b * kSlabCap + lo;
   *bucket_out = b;
-  return (uint32_t)tb.slab_idx[*pos_out] & kIndexMask;
+  return t;
 }
 
 template <typename S>
@@ -435,8 +444,8 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
     idx[i] = kRemovedBit;
     val[i] = 0;
     if (p < n) {
-      s_key[p] = tb.slab_key[base + p];
       idx[i] = (uint32_t)tb.slab_idx[base + p];
+      s_key[p] = geo.mod_m(poly(idx[i] & kIndexMask) + kSeed1);
       val[i] = slab_val[base + p];
     }
   }
@@ -603,7 +612,6 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.tb.slab_rec = cv.take<uint2>(B * kSlabCap);
   p.tb.slab_idx = cv.take<int32_t>(B * kSlabCap);
   p.tb.slab_val = cv.take<char>(B * kSlabCap * (dtype == ZEN_BF16 ? 2 : 4));
-  p.tb.slab_key = cv.take<uint32_t>(B * kSlabCap);
   p.tb.mv_key = cv.take<uint32_t>(B * kSlabMoveCap);
   p.tb.mv_idx = cv.take<uint32_t>(B * kSlabMoveCap);
   p.tb.mv_val = cv.take<uint32_t>(B * kSlabMoveCap);
