@@ -160,6 +160,7 @@ struct MergeSrc {
   int32_t *status;
   // the value is fetched again by arrival number when the entry is written: a workgroup's 4096 arrival numbers
   // are consecutive, so those loads hit the 8 KB it has just read
+  using Last = S;
   static constexpr int kStaged = 2;
   __device__ inline uint32_t late(const uint32_t (&w)[3], int) const { return (uint32_t)val[w[1]]; }
   __device__ inline bool load(uint32_t e, uint32_t (&w)[3], uint32_t *bucket) const {

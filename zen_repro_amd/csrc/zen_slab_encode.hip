@@ -38,7 +38,8 @@ struct SlabTables {
   uint32_t *removed_n;  // [B] of which lost their level-1 slot
   uint32_t *movein_n;   // [B] entries whose final slot lies in the bucket but whose level-1 slot does not own it
   uint32_t *serial_n;   // [P] entries that found no slot
-  uint2 *slab_rec;      // [B * kSlabCap] records as they arrive: (index, value)
+  uint32_t *raw_idx;    // [B * kSlabCap] entries as they arrive: index ...
+  void *raw_val;        // ... and value
   int32_t *slab_idx;    // [B * kSlabCap] after the sort: index | kRemovedBit, by ascending level-1 slot (the slot
                         // itself is not kept: hashing the index again is cheaper than a trip to memory)
   void *slab_val;       // [B * kSlabCap] after the sort: value
@@ -65,6 +66,7 @@ struct EncodeSrc {
   const int32_t *list_idx;
   const S *list_val;
   const uint32_t *filter;  // optional exact threshold
+  using Last = S;
   static constexpr int kStaged = 2;
   __device__ inline uint32_t late(const uint32_t (&)[2], int) const { return 0; }
   __device__ inline bool load(uint32_t e, uint32_t (&w)[2], uint32_t *bucket) const {
@@ -77,13 +79,18 @@ struct EncodeSrc {
     return true;
   }
 };
+template <typename S>
 struct EncodeSink {
   SlabGeom geo;
-  uint2 *slab_rec;
+  uint32_t *raw_idx;
+  S *raw_val;
   __device__ inline uint32_t bucket(const uint32_t (&w)[2]) const {
     return geo.bucket_of(geo.mod_m(poly(w[0]) + kSeed1));
   }
-  __device__ inline void store(size_t at, const uint32_t (&w)[2]) const { slab_rec[at] = make_uint2(w[0], w[1]); }
+  __device__ inline void store(size_t at, const uint32_t (&w)[2]) const {
+    raw_idx[at] = w[0];
+    raw_val[at] = (S)w[1];
+  }
 };
 
 // ------------------------------------------------------------ sort a bucket
@@ -115,10 +122,9 @@ __global__ __launch_bounds__(kSortBlock, 2) void k_slab_sort(SlabGeom geo, SlabT
     off[i] = idx[i] = pos[i] = 0;
     val[i] = 0;
     if (j < n_raw) {
-      const uint2 rec = tb.slab_rec[base + j];
-      off[i] = geo.mod_m(poly(rec.x) + kSeed1) - lo;  // the level-1 slot again: cheaper than carrying it along
-      idx[i] = rec.x;
-      val[i] = (S)rec.y;
+      idx[i] = tb.raw_idx[base + j];
+      val[i] = static_cast<const S *>(tb.raw_val)[base + j];
+      off[i] = geo.mod_m(poly(idx[i]) + kSeed1) - lo;  // the level-1 slot again: cheaper than carrying it along
       pos[i] = j;
       live |= 1u << i;
     }
@@ -609,7 +615,8 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.tb.out_start = cv.take<uint32_t>(B + 1);
   p.tb.bucket_n = cv.take<uint32_t>(B);
   p.tb.removed_n = cv.take<uint32_t>(B);
-  p.tb.slab_rec = cv.take<uint2>(B * kSlabCap);
+  p.tb.raw_idx = cv.take<uint32_t>(B * kSlabCap);
+  p.tb.raw_val = cv.take<char>(B * kSlabCap * (dtype == ZEN_BF16 ? 2 : 4));
   p.tb.slab_idx = cv.take<int32_t>(B * kSlabCap);
   p.tb.slab_val = cv.take<char>(B * kSlabCap * (dtype == ZEN_BF16 ? 2 : 4));
   p.tb.mv_key = cv.take<uint32_t>(B * kSlabMoveCap);
@@ -632,7 +639,7 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
   {
     ProfScope prof(kProfFeed, s);
     const EncodeSrc<S> src{geo, p.list_idx, static_cast<const S *>(p.list_val), filter};
-    const EncodeSink sink{geo, p.tb.slab_rec};
+    const EncodeSink<S> sink{geo, p.tb.raw_idx, static_cast<S *>(p.tb.raw_val)};
     const int rc = feed_slabs<2>(geo, p.cg, src, sink, p.list_count, p.list_cap, p.feed, a.status, s);
     if (rc != ZEN_OK) return rc;
   }

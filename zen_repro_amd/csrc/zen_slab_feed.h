@@ -13,7 +13,8 @@
 // kCoarseSplit parts with a cursor each (workgroup i writes part i % kCoarseSplit), every coarse cursor has a
 // 128-byte line to itself, and the bucket cursors sit kCursorPad words apart.
 //
-// An entry travels as W 32-bit words.  What they are comes from two small functor types:
+// An entry travels as W 32-bit words, the last of which is kept in memory as the narrower type Src::Last (a
+// bf16 value takes two bytes on its way, not four).  What they are comes from two small functor types:
 //   Src:   bool load(uint32_t e, uint32_t (&w)[W], uint32_t *bucket)   words and bucket of list entry e;
 //                                                                      false: the entry is dropped
 //          kStaged, uint32_t late(const uint32_t (&w)[W], int q)       only the first kStaged words go through
@@ -61,7 +62,7 @@ inline uint32_t feed_batches(int64_t entries) { return (uint32_t)ceil_div(entrie
 // Workspace of the two steps.
 struct FeedBuffers {
   uint32_t *coarse_cursor;  // [feed_coarse_cursor_words()], zero before the first step
-  uint32_t *coarse_words;   // [W][groups * kCoarseSplit * cap]
+  uint32_t *coarse_words;   // [W][groups * kCoarseSplit * cap]; the last plane holds Src::Last, not words
   uint32_t *cursor;         // [nbuckets * kCursorPad], zero before the second step; ends as the slab fill counts
   uint32_t *bucket_lo;      // [nbuckets] smallest key of every bucket (written by the second step)
 };
@@ -153,7 +154,8 @@ __global__ __launch_bounds__(kSlabBlock) void k_coarse_scatter(SlabGeom geo, Coa
 #pragma unroll
       for (int q = WS; q < W; ++q) rec[q] = src.late(rec, q);
 #pragma unroll
-      for (int q = 0; q < W; ++q) coarse_words[q * plane + o] = rec[q];
+      for (int q = 0; q < W - 1; ++q) coarse_words[q * plane + o] = rec[q];
+      reinterpret_cast<typename Src::Last *>(coarse_words + (size_t)(W - 1) * plane)[o] = (typename Src::Last)rec[W - 1];
     } else {
       atomicOr(status, ZEN_STAT_RETRY);  // a coarse slab is full: the general path answers
     }
@@ -161,7 +163,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_coarse_scatter(SlabGeom geo, Coa
 }
 
 // Grid: (batches per part, parts of all coarse slabs).  Also writes bucket_lo for the coarse slab's buckets.
-template <int W, typename Sink>
+template <int W, typename Last, typename Sink>
 __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, CoarseGeom cg, Sink sink,
                                                              const uint32_t *__restrict__ coarse_cursor,
                                                              const uint32_t *__restrict__ coarse_words,
@@ -181,6 +183,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, Coars
   if (batch >= count) return;
   const size_t plane = (size_t)cg.groups * kCoarseSplit * cg.cap;
   const uint32_t *from = coarse_words + (size_t)blockIdx.y * cg.cap;
+  const Last *from_last = reinterpret_cast<const Last *>(coarse_words + (size_t)(W - 1) * plane) + (size_t)blockIdx.y * cg.cap;
   uint32_t w[kFeedItems][W], dst[kFeedItems], rank[kFeedItems];
 #pragma unroll
   for (int i = 0; i < kFeedItems; ++i) {
@@ -188,7 +191,8 @@ __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, Coars
     dst[i] = 0xffu;
     if (e < count) {
 #pragma unroll
-      for (int q = 0; q < W; ++q) w[i][q] = from[q * plane + e];
+      for (int q = 0; q < W - 1; ++q) w[i][q] = from[q * plane + e];
+      w[i][W - 1] = (uint32_t)from_last[e];
       dst[i] = 0;
     }
   }
@@ -229,7 +233,7 @@ int feed_slabs(const SlabGeom &geo, const CoarseGeom &cg, const Src &src, const 
   k_coarse_scatter<W, Src><<<dim3(feed_batches(list_cap)), dim3(kSlabBlock), 0, s>>>(
       geo, cg, src, list_count, (uint32_t)list_cap, fb.coarse_cursor, fb.coarse_words, status);
   ZEN_LAUNCH_CHECK("k_coarse_scatter");
-  k_fine_scatter<W, Sink><<<dim3(feed_batches(cg.cap), cg.groups * kCoarseSplit), dim3(kSlabBlock), 0, s>>>(
+  k_fine_scatter<W, typename Src::Last, Sink><<<dim3(feed_batches(cg.cap), cg.groups * kCoarseSplit), dim3(kSlabBlock), 0, s>>>(
       geo, cg, sink, fb.coarse_cursor, fb.coarse_words, fb.cursor, fb.bucket_lo, status);
   ZEN_LAUNCH_CHECK("k_fine_scatter");
   return ZEN_OK;
