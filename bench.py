@@ -42,6 +42,8 @@ def parse():
     ap.add_argument("--depth", type=int, default=1,
                     help="gradient buckets in flight: step i+1 is enqueued on its own streams next to step i "
                          "(1 = a step starts when the previous one has finished)")
+    ap.add_argument("--time-every", type=int, default=4,
+                    help="in the timed region every n-th launch of the roofline kernel carries HIP events")
     ap.add_argument("--no-kernel-timing", action="store_true",
                     help="leave the HIP-event kernel timers off during the timed region")
     return ap.parse_args()
@@ -211,7 +213,8 @@ def main():
     torch.cuda.synchronize()
     # An event between two kernels costs the device a few microseconds, about 40 of them per step with every
     # stage timed.  So the stage breakdown comes from an untimed pass of its own, and in the timed region only
-    # the dominant kernel (the one the roofline figure is about) carries events.
+    # the dominant kernel (the one the roofline figure is about) carries events, on every --time-every-th of
+    # its launches (the pair of events around one launch holds the stream up for 10 us or so).
     streaming = ("k_select_stage", "k_select_compact", "k_topk_hist")  # kernels that read the dense gradient
     stages, dom = {}, None
     if not args.no_kernel_timing:
@@ -221,7 +224,7 @@ def main():
         stages = _lib.profile_read()
         cands = [(stages[name][0], name) for name in streaming if name in stages]
         dom = max(cands)[1] if cands else None
-        _lib.profile_enable(dom is not None, only=dom)
+        _lib.profile_enable(dom is not None, only=dom, every=max(1, args.time_every))
     t0 = time.perf_counter()
     outs = run(args.steps)
     t_enq = time.perf_counter()
@@ -263,7 +266,8 @@ def main():
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                     "traffic": MEASURED_TRAFFIC.get((cfg.name, args.shrink, dom)),
-                    "avg_launch_ms": round(avg_ms, 4), "launches_per_step": launches // args.steps,
+                    "avg_launch_ms": round(avg_ms, 4), "launches_per_step": stages[dom][1] // args.steps,
+                    "timed_launches": launches,
                     "algorithmic_bytes_per_launch": per_launch[dom]}
 
     line = {

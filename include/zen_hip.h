@@ -284,10 +284,13 @@ int zen_bucket_sort_pairs(uint32_t *keys, uint32_t *vals, int64_t max_count,
  * on the recorded events of one tag and returns their summed duration and the
  * number of launches.  An event between two kernels costs a few microseconds
  * on the device: zen_profile_only(tag) limits the recording to one tag (a
- * negative tag lifts the limit).  Process-wide, serialised by a mutex.
+ * negative tag lifts the limit), and zen_profile_every(n) to every n-th
+ * launch of a tag, counted from zen_profile_enable (n = 1: all of them).
+ * Process-wide, serialised by a mutex.
  */
 int zen_profile_enable(int on);
 int zen_profile_only(int tag);
+int zen_profile_every(int n);
 int zen_profile_tags(void);
 const char *zen_profile_name(int tag);
 int zen_profile_read(int tag, double *total_ms, int64_t *launches);

@@ -84,6 +84,13 @@ def test_slab_load_balance_odd_length_unaligned_and_empty(zen, oracle, dtype):
     total = int(splits_o.sum())
     assert status.item() == 0 and np.array_equal(to_np(splits), splits_o)
     assert np.array_equal(to_np(oi)[:total], idx_o) and np.array_equal(to_np(ov)[:total], val_o)
+    # the same tensor 16-byte aligned: whole vectors stream, the few elements behind the last one (the
+    # selected last element among them) go through a stage of their own
+    a = to_dev(g)
+    assert a.data_ptr() % 16 == 0 and n % 8 != 0
+    oi, ov, splits, status = tp.load_balance_flat(a, capacity=capacity)
+    assert status.item() == 0 and np.array_equal(to_np(splits), splits_o)
+    assert np.array_equal(to_np(oi)[:total], idx_o) and np.array_equal(to_np(ov)[:total], val_o)
     zeros = torch.zeros(n, dtype=d.dtype, device="cuda")
     oi, ov, splits, status = tp.load_balance_flat(zeros, capacity=capacity)
     assert status.item() == 0 and int(splits.sum()) == 0

@@ -70,6 +70,7 @@ def lib():
         "zen_bucket_sort_pairs": (i32, [vp, vp, i64, vp, ctypes.c_uint32, vp, sz, vp, vp]),
         "zen_profile_enable": (i32, [i32]),
         "zen_profile_only": (i32, [i32]),
+        "zen_profile_every": (i32, [i32]),
         "zen_profile_tags": (i32, []),
         "zen_profile_name": (ctypes.c_char_p, [i32]),
         "zen_profile_read": (i32, [i32, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]),
@@ -150,8 +151,44 @@ class Scratch:
 scratch = Scratch()
 
 
+class ZeroPool:
+    """Small zeroed device buffers (status words, counters, split sizes).  A
+    fill kernel for four bytes costs the device as much as one for a megabyte,
+    and a call on the hot path needs two or three such buffers: they are cut
+    from a block that one fill zeroed.  Every piece is handed out once (its
+    holder may write to it).  A block belongs to the host thread and the stream
+    that were current when it was made, so a piece is only ever used in the
+    stream order of its block's fill."""
+
+    BLOCK = 1 << 16
+    ALIGN = 16
+
+    def __init__(self):
+        self._local = threading.local()
+
+    def take(self, device, count, dtype):
+        dev = torch.device(device)
+        index = dev.index if dev.index is not None else torch.cuda.current_device()
+        nbytes = count * torch.empty((), dtype=dtype).element_size()
+        if nbytes > self.BLOCK // 4:
+            return torch.zeros(count, dtype=dtype, device=dev)
+        blocks = getattr(self._local, "blocks", None)
+        if blocks is None:
+            blocks = self._local.blocks = {}
+        key = (index, torch.cuda.current_stream(dev).cuda_stream)
+        entry = blocks.get(key)
+        if entry is None or entry[1] + nbytes > self.BLOCK:
+            entry = blocks[key] = [torch.zeros(self.BLOCK, dtype=torch.uint8, device=dev), 0]
+        at = entry[1]
+        entry[1] = (at + nbytes + self.ALIGN - 1) // self.ALIGN * self.ALIGN
+        return entry[0][at:at + nbytes].view(dtype)
+
+
+zeros = ZeroPool()
+
+
 def status_word(device):
-    return torch.zeros(1, dtype=torch.int32, device=device)
+    return zeros.take(device, 1, torch.int32)
 
 
 def describe_status(bits):
@@ -169,14 +206,16 @@ def describe_status(bits):
     return ", ".join(names) or "ok"
 
 
-def profile_enable(on=True, only=None):
-    """Start (or stop) timing the tagged launches; `only` names the one kernel tag to time."""
+def profile_enable(on=True, only=None, every=1):
+    """Start (or stop) timing the tagged launches; `only` names the one kernel
+    tag to time, `every` = n times every n-th launch of a tag."""
     L = lib()
     tag = -1
     if only is not None:
         names = [L.zen_profile_name(t).decode() for t in range(L.zen_profile_tags())]
         tag = names.index(only)
     check(L.zen_profile_only(tag), "profile_only")
+    check(L.zen_profile_every(int(every)), "profile_every")
     check(L.zen_profile_enable(1 if on else 0), "profile_enable")
 
 

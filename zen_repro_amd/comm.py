@@ -129,7 +129,7 @@ class LoadBalanceAllreduce:
             capacity = r
         out_idx = torch.empty(capacity, dtype=torch.int64 if idx64 else torch.int32, device=dev)
         out_val = torch.empty(capacity, dtype=torch.float32, device=dev)
-        count = torch.zeros(1, dtype=torch.int64, device=dev)
+        count = _lib.zeros.take(dev, 1, torch.int64)
         status = _lib.status_word(dev)
         ws = _lib.scratch.get(dev, f"merge/{slot}", L.zen_merge_workspace(r, dense_size))
         rc = L.zen_merge(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(values),

@@ -181,6 +181,7 @@ struct MergeSink {
   SlabGeom geo;
   uint32_t *slab_idx, *slab_arr;
   S *slab_val;
+  __device__ inline bool keep(const uint32_t (&)[3]) const { return true; }
   __device__ inline uint32_t bucket(const uint32_t (&w)[3]) const { return geo.bucket_of(w[0]); }
   __device__ inline void store(size_t at, const uint32_t (&w)[3]) const {
     slab_idx[at] = w[0];
@@ -198,7 +199,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
                                                              I *__restrict__ out_idx, float *__restrict__ out_val,
                                                              int64_t capacity, ScanState st, int tie_bits,
                                                              int64_t *out_count, int32_t *status) {
-  __shared__ SlabSortShared sh;
+  __shared__ SlabSortSharedT<true> sh;  // the values take the counters' place once the ranks are known
   __shared__ uint64_t s_scan64[kSlabBlock / 64 + 1];
   __shared__ int s_tile;
   if (threadIdx.x == 0) s_tile = (int)atomicAdd(st.ticket, 1u);

@@ -17,6 +17,8 @@ struct Span {
 std::mutex g_mu;
 bool g_on = false;
 int g_only = -1;  // >= 0: only launches with this tag are timed
+int g_every = 1;  // of which every g_every-th one
+int64_t g_seen[kProfCount];  // launches per tag since recording began
 std::vector<Span> g_spans;
 std::vector<hipEvent_t> g_spare;  // created ahead of the timed launches: creating an event costs host time
 
@@ -52,6 +54,7 @@ void drop_spans() {  // the events go back to the spare list (a read has waited 
 ProfScope::ProfScope(int tag, hipStream_t stream) : tag_(tag), stream_(stream), start_(nullptr), stop_(nullptr) {
   std::lock_guard<std::mutex> lock(g_mu);
   if (!g_on || (g_only >= 0 && tag != g_only)) return;
+  if (g_seen[tag]++ % g_every != 0) return;
   start_ = take_event();
   stop_ = start_ ? take_event() : nullptr;
   if (!stop_) {
@@ -77,6 +80,7 @@ int zen_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(zen::g_mu);
   zen::drop_spans();
   zen::g_on = on != 0;
+  for (int64_t &c : zen::g_seen) c = 0;
   while (zen::g_on && zen::g_spare.size() < zen::kSpareEvents) {
     hipEvent_t e = nullptr;
     if (hipEventCreate(&e) != hipSuccess) break;
@@ -89,6 +93,13 @@ int zen_profile_only(int tag) {
   if (tag >= zen::kProfCount) return zen::fail(ZEN_EINVAL, "zen_profile_only: no such tag");
   std::lock_guard<std::mutex> lock(zen::g_mu);
   zen::g_only = tag < 0 ? -1 : tag;
+  return ZEN_OK;
+}
+
+int zen_profile_every(int n) {
+  if (n < 1) return zen::fail(ZEN_EINVAL, "zen_profile_every: n must be at least 1");
+  std::lock_guard<std::mutex> lock(zen::g_mu);
+  zen::g_every = n;
   return ZEN_OK;
 }
 

@@ -4,6 +4,7 @@
 
 #include "zen_common.h"
 #include "zen_slab.h"
+#include "zen_slab_feed.h"
 
 namespace zen {
 
@@ -84,33 +85,34 @@ int topk_exact(const void *in, int dtype, int64_t n, const uint32_t *n_dev, int6
 int topk_sampled_floor(const void *in, int dtype, int64_t n, int64_t k, uint32_t *thr_lo, void *scratch,
                        hipStream_t stream, bool scratch_is_zero = false);
 size_t sampled_floor_zero_bytes();  // leading part of the scratch that must be zero (scratch_is_zero: the caller did it)
-constexpr int kCandBins = 2048;
+constexpr int kCandBins = 512;   // four octaves of 15-bit magnitudes above the floor; the rest shares the last bin
 constexpr int kCandRows = 8;   // partial candidate histograms (blocks spread over them)
 constexpr int kCandHistWords = kCandRows * kCandBins + 1;
 
-// One pass over a dense tensor that appends every element with key >= max(thr[0], 1) (thr == nullptr: the
-// nonzero ones), as (index, value), to a list, in no particular order, by persistent workgroups.
-// *list_count, *ticket and cand_hist must be zero on entry; *list_count ends as the number found, which may
-// exceed `capacity` (the excess is dropped; callers compare).  With cand_hist / pick_k / pick_thr the exact
-// k-th largest key is read off the candidates' histogram as in SelectArgs (and copied to thr_copy if that
-// is not null).
+// One pass over a dense tensor, by persistent workgroups, that hands every element with key >= max(thr[0], 1)
+// (thr == nullptr: the nonzero ones) except element 0 to the coarse slabs of zen_slab_feed.h, as (index,
+// value) and keyed by the level-1 hash slot of its index: whenever a workgroup has gathered a couple of
+// thousand candidates it orders them by coarse slab in LDS and appends one run per slab.  coarse_cursor,
+// *ticket and cand_hist must be zero on entry; a coarse slab that overflows raises ZEN_STAT_RETRY.  With
+// cand_hist / pick_k / pick_thr the exact k-th largest key is read off the candidates' histogram (element 0
+// included) as in SelectArgs (and copied to thr_copy if that is not null).
 struct StageArgs {
   const void *in = nullptr;
   int dtype = ZEN_F32;
   int64_t n = 0;
   const uint32_t *thr = nullptr;
-  uint32_t *list_count = nullptr;
-  int32_t *list_idx = nullptr;
-  void *list_val = nullptr;        // elements of the tensor's type
-  int64_t capacity = 0;            // < 2^32
-  uint32_t *ticket = nullptr;      // select_stage_ticket_words() words
+  SlabGeom geo;                     // buckets of the level-1 hash slots
+  CoarseGeom cg;
+  uint32_t *coarse_cursor = nullptr;
+  uint32_t *coarse_words = nullptr;  // plane 0: indices; plane 1: values in the tensor's type
+  uint32_t *ticket = nullptr;       // select_stage_ticket_words() words
   uint32_t *cand_hist = nullptr;
   int64_t pick_k = 0;
   uint32_t *pick_thr = nullptr;
   uint32_t *thr_copy = nullptr;
   int32_t *status = nullptr;
 };
-int select_stage_list(const StageArgs &a, hipStream_t stream);
+int select_stage_slabs(const StageArgs &a, hipStream_t stream);
 size_t select_stage_ticket_words();
 
 }  // namespace zen

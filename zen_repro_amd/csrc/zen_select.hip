@@ -248,8 +248,10 @@ __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restric
 // key).  Too few candidates, or the k-th lies in the clipped last bin:
 // ZEN_STAT_RETRY.
 // Place of a candidate bin inside its row of the global histogram: neighbours 256 bytes apart (see fine_place).
-__device__ inline uint32_t cand_place(uint32_t bin) { return ((bin & 31u) << 6) | (bin >> 5); }
-__device__ inline uint32_t cand_bin_at(uint32_t place) { return ((place & 63u) << 5) | (place >> 6); }
+constexpr uint32_t kCandCols = kCandBins / 32;
+static_assert(kCandBins % 32 == 0, "bins are laid out in 32 groups");
+__device__ inline uint32_t cand_place(uint32_t bin) { return (bin & 31u) * kCandCols + (bin >> 5); }
+__device__ inline uint32_t cand_bin_at(uint32_t place) { return ((place % kCandCols) << 5) | (place / kCandCols); }
 
 template <int BLOCK>
 __device__ inline void cand_pick_block(const uint32_t *hist, uint32_t base, uint32_t k, int shift,
@@ -652,8 +654,9 @@ int select_compact(const SelectArgs &a, hipStream_t stream) {
 // (the next sub-tile is already in flight while the current one is examined),
 // needs one barrier per sub-tile (the wave totals are double buffered), and
 // stages candidates in LDS until kScatStage of them are there.  A full stage
-// is flushed to the output list with one reservation and coalesced stores; the
-// candidate histogram is taken at flush time.
+// is flushed to the coarse slabs (zen_slab_feed.h): ordered by coarse slab
+// inside LDS, one reservation per slab, consecutive lanes writing consecutive
+// places of a run; the candidate histogram is taken at flush time.
 
 constexpr int kScatStage = 2048;
 
@@ -728,24 +731,88 @@ __device__ inline uint32_t pick_elem<uint32_t>(const uint4 (&q)[kSelVecs], int o
   return pick_word(q, off);
 }
 
-// Called by the whole block after a barrier made the staged entries visible:
-// one reservation in the output list, consecutive lanes write consecutive entries.
+// Where the candidates go.
+struct StageSlabs {
+  SlabGeom geo;
+  CoarseGeom cg;
+  uint32_t *cursor;  // coarse cursors
+  uint32_t *words;   // word planes of the coarse slabs
+};
+
+struct StageFlushShared {
+  uint32_t cnt[kCoarseMax], pref[kCoarseMax + 1], gbase[kCoarseMax];
+  uint8_t dst[kScatStage];
+};
+
+// Called by the whole block after a barrier made the staged entries visible.  What k_coarse_scatter does for
+// a list, done for the staged candidates: every entry finds its coarse slab (from the level-1 hash slot of
+// its index), the stage is put in slab order in place, every slab's run is reserved with one atomic and
+// consecutive lanes write consecutive places.  Element 0 is not handed on (index 0 is never transmitted:
+// 0 is the table's empty marker, tensor_load_balance.py:31), but counts in the histogram.
 template <typename S>
-__device__ inline void stage_flush(uint32_t count, const int32_t *st_idx, const S *st_val, uint32_t *s_base,
-                                   uint32_t *s_hist, uint32_t floor_key, uint32_t *list_count,
-                                   int32_t *__restrict__ list_idx, S *__restrict__ list_val, uint32_t capacity) {
-  if (threadIdx.x == 0) *s_base = atomicAdd(list_count, count);
+__device__ inline void stage_flush(uint32_t count, int32_t *st_idx, S *st_val, StageFlushShared &fl,
+                                   uint32_t *s_hist, uint32_t floor_key, const StageSlabs &out, int32_t *status) {
+  constexpr int kPer = kScatStage / kSelBlock;
+  static_assert(kScatStage % kSelBlock == 0 && kCoarseMax <= 64, "flush layout");
+  if (threadIdx.x < kCoarseMax) fl.cnt[threadIdx.x] = 0;
   __syncthreads();
-  const uint32_t base = *s_base;
-  for (uint32_t e = threadIdx.x; e < count; e += kSelBlock) {
-    const S v = st_val[e];
-    if (base + e < capacity) {
-      list_idx[base + e] = st_idx[e];
-      list_val[base + e] = v;
+  const uint32_t part = blockIdx.x % kCoarseSplit;
+  uint32_t t[kPer], d[kPer], r[kPer];
+  S v[kPer];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const uint32_t e = threadIdx.x + i * kSelBlock;
+    d[i] = 0xffu;
+    t[i] = r[i] = 0;
+    v[i] = 0;
+    if (e < count) {
+      t[i] = (uint32_t)st_idx[e];
+      v[i] = st_val[e];
+      if (s_hist) {
+        const uint32_t bin = ((v[i] & KeyOf<S>::kMask) - floor_key) >> (sizeof(S) == 2 ? 0 : 16);
+        atomicAdd(&s_hist[bin < (uint32_t)kCandBins - 1u ? bin : (uint32_t)kCandBins - 1u], 1u);
+      }
+      if (t[i] != 0) {
+        uint32_t rem;
+        const uint32_t bucket = out.geo.bucket_of(out.geo.mod_m(poly(t[i]) + kSeed1));
+        d[i] = SlabGeom::div_small(bucket, out.cg.per, out.cg.inv_per, &rem);
+        r[i] = atomicAdd(&fl.cnt[d[i]], 1u);
+      }
     }
-    if (s_hist) {
-      const uint32_t bin = ((v & KeyOf<S>::kMask) - floor_key) >> (sizeof(S) == 2 ? 0 : 16);
-      atomicAdd(&s_hist[bin < (uint32_t)kCandBins - 1u ? bin : (uint32_t)kCandBins - 1u], 1u);
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    const uint32_t c = threadIdx.x < kCoarseMax ? fl.cnt[threadIdx.x] : 0u;
+    const uint32_t incl = wave_inclusive_scan(c);
+    if (threadIdx.x < kCoarseMax) {
+      fl.pref[threadIdx.x] = incl - c;
+      fl.gbase[threadIdx.x] = c ? atomicAdd(&out.cursor[(threadIdx.x * kCoarseSplit + part) * kCoarsePad], c) : 0u;
+    }
+    if (threadIdx.x == kCoarseMax - 1) fl.pref[kCoarseMax] = incl;
+  }
+  __syncthreads();  // every thread holds its entries in registers: the stage is reordered in place
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    if (d[i] != 0xffu) {
+      const uint32_t p = fl.pref[d[i]] + r[i];
+      st_idx[p] = (int32_t)t[i];
+      st_val[p] = v[i];
+      fl.dst[p] = (uint8_t)d[i];
+    }
+  }
+  __syncthreads();
+  const uint32_t total = fl.pref[kCoarseMax];
+  const size_t plane = (size_t)out.cg.groups * kCoarseSplit * out.cg.cap;
+  S *val_plane = reinterpret_cast<S *>(out.words + plane);
+  for (uint32_t p = threadIdx.x; p < total; p += kSelBlock) {
+    const uint32_t g = fl.dst[p];
+    const uint32_t at = fl.gbase[g] + (p - fl.pref[g]);
+    if (at < out.cg.cap) {
+      const size_t o = (size_t)(g * kCoarseSplit + part) * out.cg.cap + at;
+      out.words[o] = (uint32_t)st_idx[p];
+      val_plane[o] = st_val[p];
+    } else {
+      atomicOr(status, ZEN_STAT_RETRY);  // a coarse slab is full: the general path answers
     }
   }
   __syncthreads();
@@ -770,9 +837,8 @@ struct StageSched {
 
 template <typename S, bool ALIGNED>
 __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
-    const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, uint32_t *list_count,
-    int32_t *__restrict__ list_idx, S *__restrict__ list_val, uint32_t capacity, uint32_t *ticket, StageSched sch,
-    uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *thr_copy, int32_t *status) {
+    const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, StageSlabs out, uint32_t *ticket,
+    StageSched sch, uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *thr_copy, int32_t *status) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kSub = kSelBlock * kSelVecs * V;
   constexpr int kWaves = kSelBlock / 64;
@@ -780,7 +846,8 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
   __shared__ uint32_t s_next[2];
   __shared__ int32_t st_idx[kScatStage];
   __shared__ S st_val[kScatStage];
-  __shared__ uint32_t s_base;
+  __shared__ StageFlushShared s_flush;
+  __shared__ uint32_t s_tail;
   __shared__ uint32_t s_pick[kSelBlock / 64 + 1];
   __shared__ uint32_t s_hist[kCandBins];
   uint32_t *hist = cand_hist ? s_hist : nullptr;
@@ -905,7 +972,7 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
       done += take;
       if (count < (uint32_t)kScatStage) break;
       __syncthreads();
-      stage_flush<S>(count, st_idx, st_val, &s_base, hist, floor_key, list_count, list_idx, list_val, capacity);
+      stage_flush<S>(count, st_idx, st_val, s_flush, hist, floor_key, out, status);
       count = 0;
       if (done == total) break;
     }
@@ -958,23 +1025,24 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
     if (!step(qc, qb)) break;
   }
   __syncthreads();
-  if (count) stage_flush<S>(count, st_idx, st_val, &s_base, hist, floor_key, list_count, list_idx, list_val, capacity);
-  if (ALIGNED && blockIdx.x == 0 && threadIdx.x == 0) {
-    // the elements behind the last complete vector (fewer than V), one by one
-    for (int64_t e = (int64_t)full_vecs * V; e < n; ++e) {
-      const S v = in[e];
-      if ((v & KeyOf<S>::kMask) >= floor_key) {
-        const uint32_t at = atomicAdd(list_count, 1u);
-        if (at < capacity) {
-          list_idx[at] = (int32_t)e;
-          list_val[at] = v;
-        }
-        if (hist) {
-          const uint32_t bin = ((v & KeyOf<S>::kMask) - floor_key) >> (sizeof(S) == 2 ? 0 : 16);
-          atomicAdd(&s_hist[bin < (uint32_t)kCandBins - 1u ? bin : (uint32_t)kCandBins - 1u], 1u);
+  if (count) stage_flush<S>(count, st_idx, st_val, s_flush, hist, floor_key, out, status);
+  if (ALIGNED && blockIdx.x == 0 && (int64_t)full_vecs * V < n) {
+    // the elements behind the last complete vector (fewer than V): a small stage of their own
+    if (threadIdx.x == 0) {
+      uint32_t c = 0;
+      for (int64_t e = (int64_t)full_vecs * V; e < n; ++e) {
+        const S v = in[e];
+        if ((v & KeyOf<S>::kMask) >= floor_key) {
+          st_idx[c] = (int32_t)e;
+          st_val[c] = v;
+          ++c;
         }
       }
+      s_tail = c;
     }
+    __syncthreads();
+    const uint32_t c = s_tail;
+    if (c) stage_flush<S>(c, st_idx, st_val, s_flush, hist, floor_key, out, status);
   }
   if (hist) {
     __syncthreads();
@@ -1035,22 +1103,21 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   sch.ticket_tiles = (uint32_t)ceil_div(subs - (int64_t)sch.fixed_subs, kStageSmall);
   const S *in = static_cast<const S *>(a.in);
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0 && a.n >= V;
+  const StageSlabs out{a.geo, a.cg, a.coarse_cursor, a.coarse_words};
   ProfScope prof(kProfSelectStage, stream);
   if (aligned)
     k_select_stage<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
-        in, a.n, a.thr, a.list_count, a.list_idx, static_cast<S *>(a.list_val), (uint32_t)a.capacity, a.ticket,
-        sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
+        in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
   else
     k_select_stage<S, false><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
-        in, a.n, a.thr, a.list_count, a.list_idx, static_cast<S *>(a.list_val), (uint32_t)a.capacity, a.ticket,
-        sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
+        in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
   ZEN_LAUNCH_CHECK("k_select_stage");
   return ZEN_OK;
 }
 
 size_t select_stage_ticket_words() { return (size_t)kStageGroups * kStageTicketPad; }
 
-int select_stage_list(const StageArgs &a, hipStream_t stream) {
+int select_stage_slabs(const StageArgs &a, hipStream_t stream) {
   if (a.dtype == ZEN_BF16) return stage_launch<uint16_t>(a, stream);
   return stage_launch<uint32_t>(a, stream);
 }

@@ -126,14 +126,31 @@ __device__ inline uint32_t sub_place(uint32_t s) {
   return s < (uint32_t)kSlabSubs ? (s % kPer) * BLOCK + s / kPer : s;
 }
 
-// Shared memory of the in-LDS sort.
-struct SlabSortShared {
+// Shared memory of the in-LDS sort.  slab_rank does not touch `tie`, and a caller that fills it only after
+// slab_rank has returned and has no use for `cnt` from then on lets the two share their memory (OVERLAY):
+// LDS decides how many workgroups share a compute unit.
+template <bool OVERLAY>
+struct SlabSortSharedT;
+template <>
+struct SlabSortSharedT<false> {
   uint32_t key[kSlabCap];
   uint32_t tie[kSlabCap];
   uint32_t cnt[kSlabSubs + 1];
   uint32_t scan[kSlabMaxBlock / 64 + 1];
   uint32_t bad;
 };
+template <>
+struct SlabSortSharedT<true> {
+  uint32_t key[kSlabCap];
+  union {
+    uint32_t tie[kSlabCap];
+    uint32_t cnt[kSlabSubs + 1];
+  };
+  uint32_t scan[kSlabMaxBlock / 64 + 1];
+  uint32_t bad;
+};
+static_assert(kSlabSubs + 1 <= kSlabCap, "the counters fit under the ties");
+using SlabSortShared = SlabSortSharedT<false>;
 
 // Ranks the live records of a workgroup of BLOCK threads (kSlabCap / BLOCK records each) by (key offset, tie);
 // tie < 2^tie_bits, the pair unique, and
@@ -142,8 +159,8 @@ struct SlabSortShared {
 // inside its group every record counts the words smaller than its own.  Returns false (for every thread) if a
 // group is too large for that; else rank[i] for live records and *n_out = number of live records.  On return
 // sh.key / sh.tie may be overwritten at once (sh.tie is not touched at all).
-template <int BLOCK>
-__device__ inline bool slab_rank(SlabSortShared &sh, const SlabGeom &geo, int tie_bits,
+template <int BLOCK, typename Shared>
+__device__ inline bool slab_rank(Shared &sh, const SlabGeom &geo, int tie_bits,
                                  const uint32_t (&off)[kSlabCap / BLOCK], const uint32_t (&tie)[kSlabCap / BLOCK],
                                  uint32_t live, uint32_t (&rank)[kSlabCap / BLOCK], uint32_t *n_out) {
   static_assert(BLOCK <= kSlabMaxBlock && kSlabCap % BLOCK == 0 && kSlabSubs % BLOCK == 0, "workgroup size");

@@ -3,13 +3,12 @@
 // The reference inserts every selected index into an int32 table as large as
 // the gradient and then scans that table partition by partition
 // (functions_cuda_kernel.cu:97-167, tensor_load_balance.py:13-51).  Here the
-// select kernel leaves its candidates in one unordered list, and five short
-// kernels finish the job (a bucket is a range of level-1 hash slots, zen_slab.h):
-//   k_coarse_scatter, k_fine_scatter
-//                   the list, filtered by the exact threshold, goes to the bucket
-//                   slabs in two steps (64 groups of buckets first, then the buckets
-//                   of each group), so that every store belongs to a long run;
-//   k_slab_sort     one workgroup per bucket: applies the exact threshold, sorts
+// select kernel leaves its candidates in 64 coarse slabs (a coarse slab = the
+// level-1 hash slots of a group of buckets; a bucket is a range of level-1
+// slots, zen_slab.h), and five short kernels finish the job:
+//   k_fine_scatter  the coarse slabs, filtered by the exact threshold, go to the
+//                   bucket slabs, so that every store belongs to a long run;
+//   k_slab_sort     one workgroup per bucket: sorts
 //                   the bucket by (level-1 slot, index) inside LDS; in a run of
 //                   equal slots the first entry (smallest index) is the slot's
 //                   level-1 owner, the others lost level 1 and are logged;
@@ -54,36 +53,21 @@ struct SlabTables {
 
 __device__ inline uint32_t level1_slot(const Probe &g, uint32_t t) { return (poly(t) + kSeed1) % g.m; }
 
-// ------------------------------------------------- list -> bucket slabs
+// ---------------------------------------------- coarse slabs -> bucket slabs
 
-// The select kernel left its candidates in one list, in no particular order.  On the way to the slabs
-// (zen_slab_feed.h) index 0 (never transmitted: 0 is the table's empty marker, tensor_load_balance.py:31) and
-// whatever the exact threshold excludes are dropped.  An entry travels as (index, value); its level-1 slot is
-// hashed again wherever it is needed, which is cheaper than carrying it along.
-template <typename S>
-struct EncodeSrc {
-  SlabGeom geo;
-  const int32_t *list_idx;
-  const S *list_val;
-  const uint32_t *filter;  // optional exact threshold
-  using Last = S;
-  static constexpr int kStaged = 2;
-  __device__ inline uint32_t late(const uint32_t (&)[2], int) const { return 0; }
-  __device__ inline bool load(uint32_t e, uint32_t (&w)[2], uint32_t *bucket) const {
-    const uint32_t t = (uint32_t)list_idx[e];
-    const S v = list_val[e];
-    if (t == 0 || (v & KeyOf<S>::kMask) < (filter ? filter[0] : 0u)) return false;
-    w[0] = t;
-    w[1] = (uint32_t)v;
-    *bucket = geo.bucket_of(geo.mod_m(poly(t) + kSeed1));
-    return true;
-  }
-};
+// The select kernel leaves its candidates in the coarse slabs (zen_slab_feed.h), as (index, value): index 0 is
+// dropped there already, what the exact threshold excludes is dropped on the way to the buckets (the threshold
+// is known only when the select kernel has ended).  An entry's level-1 slot is hashed again wherever it is
+// needed, which is cheaper than carrying it along.
 template <typename S>
 struct EncodeSink {
   SlabGeom geo;
   uint32_t *raw_idx;
   S *raw_val;
+  const uint32_t *filter;  // optional exact threshold
+  __device__ inline bool keep(const uint32_t (&w)[2]) const {
+    return (w[1] & KeyOf<S>::kMask) >= (filter ? filter[0] : 0u);
+  }
   __device__ inline uint32_t bucket(const uint32_t (&w)[2]) const {
     return geo.bucket_of(geo.mod_m(poly(w[0]) + kSeed1));
   }
@@ -574,10 +558,6 @@ struct SlabPlan {
   uint32_t *sample_hist;  // sampled floor histogram (+ finished-block count)
   uint32_t *cand_hist;
   uint32_t *ticket;
-  uint32_t *list_count;   // candidates the select kernel found
-  int32_t *list_idx;      // [list_cap] the candidates, in no particular order
-  void *list_val;
-  uint32_t list_cap;
   CoarseGeom cg;
   FeedBuffers feed;
   uint32_t *thr;          // [0..1] exact threshold + count, [2..3] sampled floor
@@ -595,7 +575,6 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.sample_hist = cv.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
   p.cand_hist = cv.take<uint32_t>((size_t)kCandHistWords);
   p.ticket = cv.take<uint32_t>(select_stage_ticket_words());
-  p.list_count = cv.take<uint32_t>(4);
   p.tb.cursor = cv.take<uint32_t>(B * kCursorPad);
   p.feed.coarse_cursor = cv.take<uint32_t>(feed_coarse_cursor_words());
   p.tb.movein_n = cv.take<uint32_t>(B);
@@ -604,9 +583,6 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.tb.done = cv.take<uint32_t>(1);
   p.zero_bytes = (size_t)(cv.base + cv.used - static_cast<char *>(p.zero_begin));
   p.thr = cv.take<uint32_t>(4);
-  p.list_cap = (uint32_t)list_cap;
-  p.list_idx = cv.take<int32_t>((size_t)list_cap);
-  p.list_val = cv.take<char>((size_t)list_cap * (dtype == ZEN_BF16 ? 2 : 4));
   p.cg = coarse_geometry(geo, list_cap);
   p.feed.coarse_words = cv.take<uint32_t>(feed_coarse_words(p.cg, 2));
   p.tb.bucket_lo = cv.take<uint32_t>(B);
@@ -638,9 +614,8 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
   const S *dense = static_cast<const S *>(a.input);
   {
     ProfScope prof(kProfFeed, s);
-    const EncodeSrc<S> src{geo, p.list_idx, static_cast<const S *>(p.list_val), filter};
-    const EncodeSink<S> sink{geo, p.tb.raw_idx, static_cast<S *>(p.tb.raw_val)};
-    const int rc = feed_slabs<2>(geo, p.cg, src, sink, p.list_count, p.list_cap, p.feed, a.status, s);
+    const EncodeSink<S> sink{geo, p.tb.raw_idx, static_cast<S *>(p.tb.raw_val), filter};
+    const int rc = feed_fine<2, S>(geo, p.cg, sink, p.feed, a.status, s);
     if (rc != ZEN_OK) return rc;
   }
   {
@@ -695,10 +670,10 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
   sc.dtype = a.dtype;
   sc.n = a.n;
   sc.thr = a.thr;
-  sc.list_count = p.list_count;
-  sc.list_idx = p.list_idx;
-  sc.list_val = p.list_val;
-  sc.capacity = p.list_cap;
+  sc.geo = geo;
+  sc.cg = p.cg;
+  sc.coarse_cursor = p.feed.coarse_cursor;
+  sc.coarse_words = p.feed.coarse_words;
   sc.ticket = p.ticket;
   sc.status = a.status;
   int rc;
@@ -712,7 +687,7 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
     sc.pick_thr = p.thr;
     sc.thr_copy = a.thr_out;
   }
-  if ((rc = select_stage_list(sc, s)) != ZEN_OK) return rc;
+  if ((rc = select_stage_slabs(sc, s)) != ZEN_OK) return rc;
   if (a.dtype == ZEN_BF16) return slab_launch<uint16_t>(a, geo, p, s);
   return slab_launch<uint32_t>(a, geo, p, s);
 }

@@ -3,7 +3,8 @@
 //
 // A direct scatter into a thousand slabs would write runs of three or four records, and memory serves such
 // stores one request at a time.  So the list goes to at most 64 coarse slabs first (a coarse slab = `per`
-// neighbouring buckets; k_coarse_scatter) and each coarse slab to its buckets afterwards (k_fine_scatter): a
+// neighbouring buckets; k_coarse_scatter, or the producer of the entries itself in the same manner: the select
+// kernel of the encode side does) and each coarse slab to its buckets afterwards (k_fine_scatter): a
 // workgroup orders its 4096 entries by destination in LDS, reserves one run per destination with one atomic
 // each and writes runs of dozens to hundreds of entries.  The order inside a slab is whatever the atomics make
 // it; the per-bucket sorts that follow do not depend on it.
@@ -22,7 +23,8 @@
 //                                                                      is asked for again when the entry is
 //                                                                      written (from the words before it), so
 //                                                                      that more workgroups fit a compute unit
-//   Sink:  uint32_t bucket(const uint32_t (&w)[W])                     the bucket again, from the words
+//   Sink:  bool keep(const uint32_t (&w)[W])                           false: the entry is dropped after all
+//          uint32_t bucket(const uint32_t (&w)[W])                     the bucket again, from the words
 //          void store(size_t at, const uint32_t (&w)[W])               the record at slab place `at`
 #pragma once
 
@@ -170,7 +172,8 @@ __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, Coars
                                                              uint32_t *__restrict__ cursor,
                                                              uint32_t *__restrict__ bucket_lo, int32_t *status) {
   __shared__ uint32_t s_cnt[kCoarsePer], s_pref[kCoarsePer + 1], s_gbase[kCoarsePer];
-  __shared__ uint32_t s_word[W][kFeedBatch];
+  __shared__ uint32_t s_word[W - 1][kFeedBatch];
+  __shared__ Last s_last[kFeedBatch];  // the last word in its own type here too: LDS decides how many workgroups share a compute unit
   __shared__ uint8_t s_dst[kFeedBatch];
   const uint32_t c = blockIdx.y / kCoarseSplit;
   const uint32_t first_bucket = c * cg.per;
@@ -198,7 +201,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, Coars
   }
 #pragma unroll
   for (int i = 0; i < kFeedItems; ++i)
-    if (dst[i] != 0xffu) dst[i] = sink.bucket(w[i]) - first_bucket;
+    if (dst[i] != 0xffu) dst[i] = sink.keep(w[i]) ? sink.bucket(w[i]) - first_bucket : 0xffu;
   feed_runs<kCoarsePer>(dst, rank, s_cnt, s_pref, s_gbase,
                         [&](uint32_t d) { return &cursor[(first_bucket + d) * kCursorPad]; });
 #pragma unroll
@@ -206,7 +209,8 @@ __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, Coars
     if (dst[i] != 0xffu) {
       const uint32_t p = s_pref[dst[i]] + rank[i];
 #pragma unroll
-      for (int q = 0; q < W; ++q) s_word[q][p] = w[i][q];
+      for (int q = 0; q < W - 1; ++q) s_word[q][p] = w[i][q];
+      s_last[p] = (Last)w[i][W - 1];
       s_dst[p] = (uint8_t)dst[i];
     }
   }
@@ -218,7 +222,8 @@ __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, Coars
     if (at < (uint32_t)kSlabCap) {
       uint32_t rec[W];
 #pragma unroll
-      for (int q = 0; q < W; ++q) rec[q] = s_word[q][p];
+      for (int q = 0; q < W - 1; ++q) rec[q] = s_word[q][p];
+      rec[W - 1] = (uint32_t)s_last[p];
       sink.store((size_t)(first_bucket + d) * kSlabCap + at, rec);
     } else {
       atomicOr(status, ZEN_STAT_RETRY);  // a slab is full: the general path answers
@@ -226,17 +231,24 @@ __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, Coars
   }
 }
 
-// Launches the two steps.  The cursors in `fb` must be zero.
+// Launches the second step alone (for a producer that fills the coarse slabs itself), and the two steps.  The
+// cursors in `fb` must be zero before the coarse slabs are filled.
+template <int W, typename Last, typename Sink>
+int feed_fine(const SlabGeom &geo, const CoarseGeom &cg, const Sink &sink, const FeedBuffers &fb, int32_t *status,
+              hipStream_t s) {
+  k_fine_scatter<W, Last, Sink><<<dim3(feed_batches(cg.cap), cg.groups * kCoarseSplit), dim3(kSlabBlock), 0, s>>>(
+      geo, cg, sink, fb.coarse_cursor, fb.coarse_words, fb.cursor, fb.bucket_lo, status);
+  ZEN_LAUNCH_CHECK("k_fine_scatter");
+  return ZEN_OK;
+}
+
 template <int W, typename Src, typename Sink>
 int feed_slabs(const SlabGeom &geo, const CoarseGeom &cg, const Src &src, const Sink &sink,
                const uint32_t *list_count, int64_t list_cap, const FeedBuffers &fb, int32_t *status, hipStream_t s) {
   k_coarse_scatter<W, Src><<<dim3(feed_batches(list_cap)), dim3(kSlabBlock), 0, s>>>(
       geo, cg, src, list_count, (uint32_t)list_cap, fb.coarse_cursor, fb.coarse_words, status);
   ZEN_LAUNCH_CHECK("k_coarse_scatter");
-  k_fine_scatter<W, typename Src::Last, Sink><<<dim3(feed_batches(cg.cap), cg.groups * kCoarseSplit), dim3(kSlabBlock), 0, s>>>(
-      geo, cg, sink, fb.coarse_cursor, fb.coarse_words, fb.cursor, fb.bucket_lo, status);
-  ZEN_LAUNCH_CHECK("k_fine_scatter");
-  return ZEN_OK;
+  return feed_fine<W, typename Src::Last, Sink>(geo, cg, sink, fb, status, s);
 }
 
 }  // namespace zen

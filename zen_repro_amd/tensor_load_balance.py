@@ -97,7 +97,7 @@ class TensorPartition:
         L = _lib.lib()
         out_idx = torch.empty(capacity, dtype=torch.int32, device=dev)
         out_val = torch.empty(capacity, dtype=flat.dtype, device=dev)
-        splits = torch.zeros(self.partitions, dtype=torch.int64, device=dev)
+        splits = _lib.zeros.take(dev, self.partitions, torch.int64)
         status = _lib.status_word(dev)
         nbytes = L.zen_load_balance_workspace(n, m, code, capacity, self.partitions)
         ws = _lib.scratch.get(dev, f"load_balance/{slot}", nbytes)
