@@ -1168,9 +1168,9 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
   constexpr int V = VecOf<S>::kN;
   uint32_t *hist = static_cast<uint32_t *>(workspace);
   const int64_t nvec = ceil_div(n, V);
-  // Every sampled vector lies on a page of its own, and the kernel spends its time waiting for their address
-  // translations: the sample is as thin as leaves about kSampleHits of its elements above the threshold
-  // (their count then scatters by 1.2 %, and the six deviations allowed for below cost 7 % more candidates).
+  // The sample is as thin as leaves about kSampleHits of its elements above the threshold (their count then
+  // scatters by 1.2 %, and the six deviations allowed for below cost 7 % more candidates): a thicker one
+  // lengthens the kernel's load and histogram phases and buys nothing.
   int sample_log2 = kSampleLog2Max;
   while (sample_log2 > kSampleLog2Min && (k >> sample_log2) < kSampleHits) --sample_log2;
   const int64_t nblocks = ceil_div(nvec, 1ll << sample_log2);
