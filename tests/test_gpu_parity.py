@@ -576,3 +576,59 @@ def test_stack_tensors_views_are_not_copied(zen):
     assert lba.stack_tensors(parts).data_ptr() == buf.data_ptr()
     other = [buf[0:10], buf[20:30]]
     assert lba.stack_tensors(other).tolist() == list(range(10)) + list(range(20, 30))
+
+
+def test_zero_pool_pieces_are_zero_apart_and_per_stream(zen):
+    """Status words, counts and split sizes are cut from pooled zeroed blocks: every piece is zero, aligned,
+    handed out once, and belongs to the stream that was current when its block was made."""
+    from zen_repro_amd import _lib
+
+    pool = _lib.ZeroPool()
+    a = pool.take("cuda", 1, torch.int32)
+    b = pool.take("cuda", 16, torch.int64)
+    c = pool.take("cuda", 3, torch.int32)
+    for t, n, dt in ((a, 1, torch.int32), (b, 16, torch.int64), (c, 3, torch.int32)):
+        assert t.dtype == dt and t.numel() == n and t.data_ptr() % 16 == 0 and int(t.abs().sum()) == 0
+    spans = sorted((t.data_ptr(), t.data_ptr() + t.numel() * t.element_size()) for t in (a, b, c))
+    assert all(spans[i][1] <= spans[i + 1][0] for i in range(2))
+    a.fill_(7)  # a holder may write: the neighbours stay zero
+    assert int(b.abs().sum()) == 0 and int(c.abs().sum()) == 0
+    base = a.data_ptr()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        d = pool.take("cuda", 1, torch.int32)
+        assert int(d.item()) == 0
+    assert not (base <= d.data_ptr() < base + pool.BLOCK)  # another stream, another block
+    # a block that is used up is replaced, not reused
+    seen = set()
+    for _ in range(2 * pool.BLOCK // 16 + 3):
+        t = pool.take("cuda", 1, torch.int32)
+        assert t.data_ptr() not in seen
+        seen.add(t.data_ptr())
+    assert int(t.item()) == 0
+    big = pool.take("cuda", pool.BLOCK, torch.uint8)  # too large for a block: a tensor of its own
+    assert big.numel() == pool.BLOCK and int(big.sum()) == 0
+
+
+def test_profile_every_nth_launch(zen, oracle):
+    """zen_profile_every(n): of a tag's launches since recording began, the first and every n-th after it
+    carry events."""
+    from zen_repro_amd import _lib
+
+    vals = to_dev(make_grad(oracle, 1 << 16, 0.05, "f32", seed=5))
+    try:
+        _lib.profile_enable(True, only="k_compress", every=3)
+        for _ in range(7):
+            zen.compress(10, vals)
+        torch.cuda.synchronize()
+        got = _lib.profile_read()
+        assert set(got) == {"k_compress"} and got["k_compress"][1] == 3 and got["k_compress"][0] > 0
+        _lib.profile_enable(True, every=1)
+        for _ in range(2):
+            zen.compress(10, vals)
+        assert _lib.profile_read()["k_compress"][1] == 2
+        with pytest.raises(ValueError):
+            _lib.profile_enable(True, every=0)
+    finally:
+        _lib.profile_enable(False)
+        _lib.check(_lib.lib().zen_profile_every(1), "profile_every")
