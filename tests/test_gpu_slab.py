@@ -134,6 +134,41 @@ def test_slab_load_balance_too_many_candidates_declines(zen, oracle):
     assert status.item() & (_lib.STAT_RETRY | _lib.STAT_CAPACITY)
 
 
+def test_slab_load_balance_fused_topk_fp32(zen, oracle):
+    """fp32 top-k inside the call on the slab path: the candidates' histogram resolves 15 key bits, the last
+    16 come from a second histogram over the candidates of the threshold's bin.  The k-th value is shared
+    by many elements (ties are kept), element 0 lies in the threshold's bin above the threshold (it counts
+    towards k and is never transmitted), and the very last element holds the largest value."""
+    n, P = (1 << 24) + 24, 16
+    rng = np.random.default_rng(77)
+    x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    k = n // 100
+    key0 = int(oracle.kth_key(x, k))
+    tie = np.array([key0], dtype=np.uint32).view(np.float32)[0]
+    x[rng.integers(1, n - 1, 300)] = -tie                                    # 300 more elements at the k-th magnitude
+    x[0] = np.array([key0 + 5], dtype=np.uint32).view(np.float32)[0]         # same bin of 65536 keys, above it
+    x[-1] = 1.0
+    key = int(oracle.kth_key(x, k))
+    assert key >> 16 == key0 >> 16
+    masked, kept = oracle.mask_dense(x, key)
+    assert kept > k and masked[0] != 0
+    idx_o, val_o, splits_o, st_o = oracle.load_balance(masked, P, 1, 3)
+    assert st_o == 0 and 0 not in idx_o
+    capacity = int(1.25 * k) + 4096
+    assert lb_path(zen, n, P, "f32", capacity, k=k) == SLAB
+    tp = zen.TensorPartition(P, 1, 3)
+    d = to_dev(x)
+    thr_out = torch.zeros(2, dtype=torch.int32, device="cuda")
+    for rep in range(2):  # the second call finds its counters cleared again
+        oi, ov, splits, status = tp.load_balance_flat(d, capacity=capacity, k=k, thr_out=thr_out)
+        assert status.item() == 0
+        assert to_np(thr_out).tolist() == [key, kept]
+        assert np.array_equal(to_np(splits), splits_o)
+        total = int(splits_o.sum())
+        assert np.array_equal(to_np(oi)[:total], idx_o)
+        assert np.array_equal(to_np(ov)[:total], val_o)
+
+
 def test_slab_load_balance_threshold_given(zen, oracle):
     """Selection by a threshold the caller computed (topk_threshold) instead of k."""
     from zen_repro_amd import _lib

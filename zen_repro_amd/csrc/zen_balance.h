@@ -130,7 +130,7 @@ struct SlabBalanceArgs {
   int partitions;
   int64_t spp;                // serial slots per partition
   const uint32_t *thr;        // optional threshold key (device); with k == 0 and no thr: the nonzeros
-  int64_t k;                  // > 0: the k largest magnitudes, ties kept (bf16 only)
+  int64_t k;                  // > 0: the k largest magnitudes, ties kept
   uint32_t *thr_out;          // optional, k > 0: receives (threshold key, number selected)
   int32_t *out_idx;
   void *out_val;

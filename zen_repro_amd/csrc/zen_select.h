@@ -94,8 +94,9 @@ constexpr int kCandHistWords = kCandRows * kCandBins + 1;
 // value) and keyed by the level-1 hash slot of its index: whenever a workgroup has gathered a couple of
 // thousand candidates it orders them by coarse slab in LDS and appends one run per slab.  coarse_cursor,
 // *ticket and cand_hist must be zero on entry; a coarse slab that overflows raises ZEN_STAT_RETRY.  With
-// cand_hist / pick_k / pick_thr the exact k-th largest key is read off the candidates' histogram (element 0
-// included) as in SelectArgs (and copied to thr_copy if that is not null).
+// cand_hist / pick_k / pick_thr the k-th largest key is read off the candidates' histogram (element 0
+// included) as in SelectArgs (and copied to thr_copy if that is not null): exactly for bf16, for fp32 the
+// lowest key of its bin of 65536 keys.
 struct StageArgs {
   const void *in = nullptr;
   int dtype = ZEN_F32;
@@ -109,6 +110,7 @@ struct StageArgs {
   uint32_t *cand_hist = nullptr;
   int64_t pick_k = 0;
   uint32_t *pick_thr = nullptr;
+  uint32_t *pick_above = nullptr;   // optional: number of candidates in the histogram bins above the k-th's
   uint32_t *thr_copy = nullptr;
   int32_t *status = nullptr;
 };

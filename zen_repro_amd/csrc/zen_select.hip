@@ -255,7 +255,8 @@ __device__ inline uint32_t cand_bin_at(uint32_t place) { return ((place % kCandC
 
 template <int BLOCK>
 __device__ inline void cand_pick_block(const uint32_t *hist, uint32_t base, uint32_t k, int shift,
-                                       uint32_t *thr_out, int32_t *status, uint32_t *smem, uint32_t *s_sum) {
+                                       uint32_t *thr_out, int32_t *status, uint32_t *smem, uint32_t *s_sum,
+                                       uint32_t *above_out = nullptr) {
   constexpr int kPer = kCandBins / BLOCK;
   // the rows are summed into s_sum (kCandBins words of LDS) with consecutive lanes on consecutive words
   __syncthreads();
@@ -288,6 +289,7 @@ __device__ inline void cand_pick_block(const uint32_t *hist, uint32_t base, uint
         const uint32_t bin = kCandBins - 1 - (threadIdx.x * kPer + j);
         thr_out[0] = base + (bin << shift);
         thr_out[1] = above + c[j];
+        if (above_out) *above_out = above;  // candidates in the bins above the k-th's
         if (bin == kCandBins - 1) atomicOr(status, ZEN_STAT_RETRY);
       }
       above += c[j];
@@ -838,7 +840,8 @@ struct StageSched {
 template <typename S, bool ALIGNED>
 __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
     const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, StageSlabs out, uint32_t *ticket,
-    StageSched sch, uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *thr_copy, int32_t *status) {
+    StageSched sch, uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *pick_above,
+    uint32_t *thr_copy, int32_t *status) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kSub = kSelBlock * kSelVecs * V;
   constexpr int kWaves = kSelBlock / 64;
@@ -957,7 +960,7 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
       while (y) {
         const uint32_t bit = (uint32_t)__ffs((int)y) - 1u;
         y &= y - 1;
-        // the thread's candidates take their places in the order of their flag bits (the list has no order
+        // the thread's candidates take their places in the order of their flag bits (the stage has no order
         // to keep, and a place counted off the flag word costs two instructions)
         const uint32_t pos = before + (uint32_t)__popc(all & ((1u << bit) - 1u));
         if (pos < hi) {
@@ -1062,7 +1065,7 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
       __syncthreads();
       if (s_last) {
         cand_pick_block<kSelBlock>(cand_hist, floor_key, pick_k, KeyOf<S>::kBits == 15 ? 0 : 16, pick_thr, status,
-                                   s_pick, s_hist);
+                                   s_pick, s_hist, pick_above);
         __syncthreads();
         if (thr_copy && threadIdx.x < 2)
           thr_copy[threadIdx.x] = __hip_atomic_load(&pick_thr[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1107,10 +1110,12 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   ProfScope prof(kProfSelectStage, stream);
   if (aligned)
     k_select_stage<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
-        in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
+        in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.pick_above, a.thr_copy,
+        a.status);
   else
     k_select_stage<S, false><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
-        in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.thr_copy, a.status);
+        in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.pick_above, a.thr_copy,
+        a.status);
   ZEN_LAUNCH_CHECK("k_select_stage");
   return ZEN_OK;
 }

@@ -77,6 +77,74 @@ struct EncodeSink {
   }
 };
 
+// --------------------------------------------- fp32: the threshold's last 16 bits
+
+constexpr int kRefineBins = 65536;
+constexpr int kRefineBlock = 512;
+
+// The candidates' histogram resolves the 15 leading bits of an fp32 key: after the select kernel thr[0] is
+// the lowest key of the bin the k-th largest lies in, thr[1] the number of candidates at or above it and
+// *above the number in the bins above.  This kernel histograms the low 16 key bits of the candidates of that
+// bin (they sit in the coarse slabs; element 0, which is never handed on, is looked at in the tensor), and the
+// workgroup that finishes last replaces thr[0..1] by the exact key and the number of elements at or above it.
+// Grid: (batches per part, parts of all coarse slabs), like k_fine_scatter.  hist: kRefineBins + 1 zeroed words.
+__global__ __launch_bounds__(kRefineBlock) void k_refine_threshold(CoarseGeom cg,
+                                                                   const uint32_t *__restrict__ coarse_cursor,
+                                                                   const uint32_t *__restrict__ coarse_words,
+                                                                   const uint32_t *__restrict__ dense,
+                                                                   uint32_t *thr, const uint32_t *above, uint32_t k,
+                                                                   uint32_t *hist, uint32_t *thr_copy, int32_t *status) {
+  __shared__ uint32_t s_scan[kRefineBlock / 64 + 1];
+  __shared__ bool s_last;
+  const uint32_t base = thr[0];
+  uint32_t count = coarse_cursor[blockIdx.y * kCoarsePad];
+  if (count > cg.cap) count = cg.cap;
+  const size_t plane = (size_t)cg.groups * kCoarseSplit * cg.cap;
+  const uint32_t *vals = coarse_words + plane + (size_t)blockIdx.y * cg.cap;
+  const uint32_t first = blockIdx.x * (uint32_t)kFeedBatch;
+  const uint32_t last = first + (uint32_t)kFeedBatch < count ? first + (uint32_t)kFeedBatch : count;
+  for (uint32_t e = first + threadIdx.x; e < last; e += kRefineBlock) {
+    const uint32_t d = (vals[e] & KeyOf<uint32_t>::kMask) - base;
+    if (d < (uint32_t)kRefineBins) atomicAdd(&hist[d], 1u);
+  }
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+    const uint32_t key0 = dense[0] & KeyOf<uint32_t>::kMask;  // counted by the select kernel if it was a candidate
+    if (key0 - base < (uint32_t)kRefineBins) atomicAdd(&hist[key0 - base], 1u);  // base is at or above the floor
+  }
+  wait_global_acks();
+  __syncthreads();
+  if (threadIdx.x == 0) s_last = atomicAdd(&hist[kRefineBins], 1u) == gridDim.x * gridDim.y - 1u;
+  __syncthreads();
+  if (!s_last) return;
+  // from the top down: thread t owns the kPer bins below kRefineBins - t * kPer
+  constexpr int kPer = kRefineBins / kRefineBlock;
+  const uint32_t hi = (uint32_t)kRefineBins - threadIdx.x * (uint32_t)kPer;
+  uint32_t mine = 0;
+  for (int j = 1; j <= kPer; ++j) mine += load_fresh(&hist[hi - (uint32_t)j]);
+  uint32_t total;
+  uint32_t before = block_exclusive_scan<uint32_t, kRefineBlock>(mine, s_scan, &total);
+  const uint32_t over = above[0];
+  const uint32_t need = k > over ? k - over : 1u;  // rank inside the bin, from the top
+  if (total < need) {
+    if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);  // the two histograms disagree: let the general mode answer
+    return;
+  }
+  if (before < need && need <= before + mine) {
+    for (int j = 1; j <= kPer; ++j) {
+      const uint32_t c = load_fresh(&hist[hi - (uint32_t)j]);
+      if (before < need && need <= before + c) {
+        thr[0] = base + hi - (uint32_t)j;
+        thr[1] = over + before + c;
+        if (thr_copy) {
+          thr_copy[0] = base + hi - (uint32_t)j;
+          thr_copy[1] = over + before + c;
+        }
+      }
+      before += c;
+    }
+  }
+}
+
 // ------------------------------------------------------------ sort a bucket
 
 // Twice the threads of the other per-bucket kernels, half the records each: the phases of this kernel are
@@ -560,9 +628,12 @@ struct SlabPlan {
   uint32_t *ticket;
   CoarseGeom cg;
   FeedBuffers feed;
-  uint32_t *thr;          // [0..1] exact threshold + count, [2..3] sampled floor
+  uint32_t *thr;          // [0..1] exact threshold + count, [2..3] sampled floor, [4] candidates above the k-th's bin
+  uint32_t *refine_hist;  // fp32: histogram of the threshold's last 16 bits (+ finished-workgroup count), last in
+                          // the zero region and cleared only for a top-k call
   void *zero_begin;
   size_t zero_bytes;
+  size_t zero_bytes_topk;
   size_t bytes;
 };
 
@@ -582,7 +653,9 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.tb.ctr = cv.take<Counters>(1);
   p.tb.done = cv.take<uint32_t>(1);
   p.zero_bytes = (size_t)(cv.base + cv.used - static_cast<char *>(p.zero_begin));
-  p.thr = cv.take<uint32_t>(4);
+  p.refine_hist = cv.take<uint32_t>(dtype == ZEN_BF16 ? 1 : (size_t)kRefineBins + 1);
+  p.zero_bytes_topk = (size_t)(cv.base + cv.used - static_cast<char *>(p.zero_begin));
+  p.thr = cv.take<uint32_t>(8);
   p.cg = coarse_geometry(geo, list_cap);
   p.feed.coarse_words = cv.take<uint32_t>(feed_coarse_words(p.cg, 2));
   p.tb.bucket_lo = cv.take<uint32_t>(B);
@@ -644,7 +717,7 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
 
 bool slab_balance_fits(int64_t n, int64_t m, int partitions, int dtype, int64_t capacity, int64_t k, SlabGeom *geo) {
   (void)n;
-  if (k > 0 && dtype != ZEN_BF16) return false;  // the candidate histogram resolves bf16 keys only
+  (void)k;
   if (capacity > 0x1fffffffll) return false;
   SlabGeom g;
   if (!slab_geometry(m, partitions, capacity, kSlabTarget, &g)) return false;
@@ -663,7 +736,9 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
   if (!slab_balance_fits(a.n, a.g.m, a.partitions, a.dtype, a.capacity, a.k, &geo))
     return fail(ZEN_EINVAL, "slab_load_balance: sizes do not suit the slab layout");
   const SlabPlan p = plan_slab(a.workspace, geo, a.partitions, a.dtype, list_capacity(a.capacity));
-  launch_fill<uint32_t>(static_cast<uint32_t *>(p.zero_begin), 0u, p.zero_bytes / sizeof(uint32_t), s);
+  const bool refine = a.k > 0 && a.dtype == ZEN_F32;
+  launch_fill<uint32_t>(static_cast<uint32_t *>(p.zero_begin), 0u,
+                        (refine ? p.zero_bytes_topk : p.zero_bytes) / sizeof(uint32_t), s);
   ZEN_LAUNCH_CHECK("slab: clear counters");
   StageArgs sc;
   sc.in = a.input;
@@ -685,9 +760,16 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
     sc.cand_hist = p.cand_hist;
     sc.pick_k = a.k;
     sc.pick_thr = p.thr;
-    sc.thr_copy = a.thr_out;
+    sc.pick_above = p.thr + 4;
+    sc.thr_copy = refine ? nullptr : a.thr_out;  // fp32: the threshold is not final yet
   }
   if ((rc = select_stage_slabs(sc, s)) != ZEN_OK) return rc;
+  if (refine) {
+    k_refine_threshold<<<dim3(feed_batches(p.cg.cap), p.cg.groups * kCoarseSplit), dim3(kRefineBlock), 0, s>>>(
+        p.cg, p.feed.coarse_cursor, p.feed.coarse_words, static_cast<const uint32_t *>(a.input), p.thr,
+        p.thr + 4, (uint32_t)a.k, p.refine_hist, a.thr_out, a.status);
+    ZEN_LAUNCH_CHECK("k_refine_threshold");
+  }
   if (a.dtype == ZEN_BF16) return slab_launch<uint16_t>(a, geo, p, s);
   return slab_launch<uint32_t>(a, geo, p, s);
 }
