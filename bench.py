@@ -19,7 +19,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by what the same counters read
 # for a plain 1 GiB copy (profiles/c3_select_stage_hbm_traffic.txt).  Other
 # workloads report null.
-MEASURED_TRAFFIC = {("c3", 1, "k_select_stage"): 1.522e9}
+MEASURED_TRAFFIC = {("c3", 1, "k_select_stage"): 1.519e9}
 
 
 def parse():
