@@ -42,6 +42,8 @@ struct SlabTables {
   int32_t *slab_idx;    // [B * kSlabCap] after the sort: index | kRemovedBit, by ascending level-1 slot (the slot
                         // itself is not kept: hashing the index again is cheaper than a trip to memory)
   void *slab_val;       // [B * kSlabCap] after the sort: value
+  uint16_t *sub_index;  // [B * kSlabIndexLen] sorted place of the first record of every kSlabIndexStep-th narrow
+                        // key range of the bucket (the last entry: the number of records)
   uint32_t *mv_key, *mv_idx, *mv_val;  // [B * kSlabMoveCap]
   uint32_t *ser_idx;    // [P * kSlabSerialCap]
   uint32_t *log_t, *log_v, *log_cell;  // [log_cap]
@@ -50,6 +52,14 @@ struct SlabTables {
   Counters *ctr;
   uint32_t log_cap;
 };
+
+// Every kSlabIndexStep-th narrow key range of a bucket (zen_slab.h; about one record per range) has its first
+// sorted place written down by the sort kernel: whoever asks who owns a level-1 slot reads two of these places
+// and the three or four records between them instead of bisecting the whole bucket (thirteen loads, one
+// after the other).
+constexpr int kSlabIndexStep = 4;
+constexpr int kSlabIndexLen = kSlabSubs / kSlabIndexStep + 1;
+static_assert(kSlabSubs % kSlabIndexStep == 0 && kSlabCap < 65536, "index layout");
 
 __device__ inline uint32_t level1_slot(const Probe &g, uint32_t t) { return (poly(t) + kSeed1) % g.m; }
 
@@ -193,6 +203,10 @@ __global__ __launch_bounds__(kSortBlock, 2) void k_slab_sort(SlabGeom geo, SlabT
     }
     return;
   }
+  // the counters hold where every narrow range starts in the sorted bucket: every kSlabIndexStep-th goes to
+  // the index (before the counters' memory is used for the list of losers below)
+  for (int j = threadIdx.x; j < kSlabIndexLen; j += kSortBlock)
+    tb.sub_index[(size_t)b * kSlabIndexLen + j] = (uint16_t)sh.cnt[sub_place<kSortBlock>((uint32_t)j * kSlabIndexStep)];
 #pragma unroll
   for (int i = 0; i < kSortItems; ++i) {
     if (live & (1u << i)) {
@@ -259,27 +273,36 @@ __global__ __launch_bounds__(kSortBlock, 2) void k_slab_sort(SlabGeom geo, SlabT
 
 // ------------------------------------------------------ levels 2 and 3
 
-// Smallest index whose level-1 slot is `slot` (kNone if nobody's), and where it sits: bisection over the
-// bucket's sorted indices by their level-1 slots.
+// Smallest index whose level-1 slot is `slot` (kNone if nobody's), and where it sits.  The bucket's index
+// narrows the search to the records of kSlabIndexStep narrow ranges (three or four); they are fetched four at
+// a time and looked at in sorted order: by ascending slot, and in a run of equal slots the smallest index
+// comes first.
 __device__ inline uint32_t slab_head(const SlabGeom &geo, const SlabTables &tb, uint32_t slot, size_t *pos_out,
                                      uint32_t *bucket_out) {
   const uint32_t b = geo.bucket_of(slot);
   const int32_t *idx = tb.slab_idx + (size_t)b * kSlabCap;
   const uint32_t n = tb.bucket_n[b];
-  uint32_t lo = 0, hi = n;
-  while (lo < hi) {
-    const uint32_t mid = lo + ((hi - lo) >> 1);
-    if (geo.mod_m(poly((uint32_t)idx[mid] & kIndexMask) + kSeed1) < slot)
-      lo = mid + 1;
-    else
-      hi = mid;
+  const uint32_t j = ((slot - tb.bucket_lo[b]) >> geo.sub_shift) / (uint32_t)kSlabIndexStep;
+  const uint16_t *index = tb.sub_index + (size_t)b * kSlabIndexLen;
+  uint32_t p = index[j], end = index[j + 1];
+  if (end > n) end = n;  // a bucket the sort declined has no index (and no records)
+  for (; p < end; p += 4) {
+    uint32_t t[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) t[q] = (uint32_t)idx[p + q < end ? p + q : p] & kIndexMask;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (p + q >= end) return kNone;
+      const uint32_t s1 = geo.mod_m(poly(t[q]) + kSeed1);
+      if (s1 > slot) return kNone;
+      if (s1 == slot) {
+        *pos_out = (size_t)b * kSlabCap + p + q;
+        *bucket_out = b;
+        return t[q];
+      }
+    }
   }
-  if (lo >= n) return kNone;
-  const uint32_t t = (uint32_t)idx[lo] & kIndexMask;
-  if (geo.mod_m(poly(t) + kSeed1) != slot) return kNone;
-  *pos_out = (size_t)b * kSlabCap + lo;
-  *bucket_out = b;
-  return t;
+  return kNone;
 }
 
 template <typename S>
@@ -668,6 +691,7 @@ SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dty
   p.tb.raw_val = cv.take<char>(B * kSlabCap * (dtype == ZEN_BF16 ? 2 : 4));
   p.tb.slab_idx = cv.take<int32_t>(B * kSlabCap);
   p.tb.slab_val = cv.take<char>(B * kSlabCap * (dtype == ZEN_BF16 ? 2 : 4));
+  p.tb.sub_index = cv.take<uint16_t>(B * kSlabIndexLen);
   p.tb.mv_key = cv.take<uint32_t>(B * kSlabMoveCap);
   p.tb.mv_idx = cv.take<uint32_t>(B * kSlabMoveCap);
   p.tb.mv_val = cv.take<uint32_t>(B * kSlabMoveCap);
