@@ -30,7 +30,7 @@ def parse():
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--shrink", type=int, default=1, help="divide the workload size (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-div", type=int, default=2,
+    ap.add_argument("--cpu-sample-div", type=int, default=1,
                     help="the CPU baseline runs on 1/div of the workload")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run five device copies of 1 GiB and exit (scale for hardware byte counters)")
@@ -64,9 +64,10 @@ def cpu_baseline(cfg, grad_dev, div):
     nnz_est = sub.k if sub.k else int(torch.count_nonzero(g))
     per_peer = max(1, nnz_est // cfg.partitions)
     idx_l, val_l, _, _ = workloads.peer_payloads(sub, per_peer, device="cpu", seed=1)
-    times, _ = torch_path.timed_pass(g, sub.k, cfg.partitions, idx_l, val_l)
+    times, (c_idx, c_val, c_splits, _, _, _) = torch_path.timed_pass(g, sub.k, cfg.partitions, idx_l, val_l)
     total = sum(times.values())
-    return {
+    parity = parity_gate(sub, grad_dev[:n_s], idx_l, val_l, c_idx, c_val, c_splits)
+    return parity, {
         "value": n_s * g.element_size() / total / 1e9,
         "unit": "GB/s",
         "cores": torch.get_num_threads(),
@@ -75,6 +76,35 @@ def cpu_baseline(cfg, grad_dev, div):
                   f"select {times['select']:.2f}s partition {times['partition']:.2f}s merge {times['merge']:.2f}s; "
                   f"torch ops use {torch.get_num_threads()} threads, the sequential insert 1",
     }
+
+
+def parity_gate(sub, grad_dev, idx_l, val_l, c_idx, c_val, c_splits):
+    """The HIP path on the sample the CPU baseline has just worked through, checked against that pass's
+    results (untimed): split sizes, the buckets' indices in their order and their values bit for bit; the
+    merged indices and fp32 sums bit for bit against a sequential fp32 scatter_add_ on the CPU (the baseline
+    itself accumulates in the values' own type, as the reference does)."""
+    import torch
+
+    from zen_repro_amd import LoadBalanceAllreduce, LocalGroup, TensorPartition
+
+    dev, P = grad_dev.device, sub.partitions
+    n_s = grad_dev.numel()
+    capacity = int(sub.k * 1.25) + 4096 if sub.k else int(sum(t.numel() for t in c_idx)) + 16
+    g_idx, g_val, g_splits = TensorPartition(P, 1, 3).load_balance(grad_dev, capacity=capacity, k=sub.k)
+    bits = torch.int16 if grad_dev.dtype == torch.bfloat16 else torch.int32
+    encode_ok = (torch.equal(g_splits.cpu(), c_splits.to(torch.int64))
+                 and torch.equal(torch.cat(g_idx).cpu(), torch.cat(c_idx).to(torch.int32))
+                 and torch.equal(torch.cat(g_val).cpu().view(bits), torch.cat(c_val).view(bits)))
+    lba = LoadBalanceAllreduce(LocalGroup(P), None, None)
+    m_idx, m_val = lba.merge_sparse([t.to(dev) for t in idx_l], [t.to(dev) for t in val_l], n_s)
+    dense = torch.zeros(n_s, dtype=torch.float32)
+    dense.scatter_add_(0, torch.cat(idx_l).to(torch.int64), torch.cat(val_l).to(torch.float32))
+    want_idx = torch.nonzero(dense, as_tuple=True)[0]
+    merge_ok = (torch.equal(m_idx.cpu(), want_idx)
+                and torch.equal(m_val.cpu().view(torch.int32), dense[want_idx].view(torch.int32)))
+    return {"ok": bool(encode_ok and merge_ok), "encode_bit_exact": bool(encode_ok), "merge_bit_exact": bool(merge_ok),
+            "checked": f"the CPU baseline's sample: {int(g_splits.sum())} selected entries in {P} buckets, "
+                       f"{int(m_idx.numel())} merged entries"}
 
 
 def bitmap_codec(args, dev):
@@ -296,8 +326,11 @@ def main():
         "cpu_baseline": None,
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(cfg, grad, args.cpu_sample_div)
+        line["parity_vs_cpu_baseline"], line["cpu_baseline"] = cpu_baseline(cfg, grad, args.cpu_sample_div)
     print(json.dumps(line))
+    if line.get("parity_vs_cpu_baseline") and not line["parity_vs_cpu_baseline"]["ok"]:
+        print("bench.py: the HIP path and the CPU baseline disagree on the sample", file=sys.stderr)
+        sys.exit(1)
 
 
 if __name__ == "__main__":
