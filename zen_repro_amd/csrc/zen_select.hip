@@ -822,8 +822,8 @@ __device__ inline void stage_flush(uint32_t count, int32_t *st_idx, S *st_val, S
 
 // How the sub-tiles (kSelBlock * kSelVecs vectors each) are handed out.  Every workgroup first takes
 // `fixed` tiles of kStageBig sub-tiles, tile i of workgroup b being number i * workgroups + b: no counter, and
-// the workgroups move through memory side by side (short tiles measured a little faster than long ones).  The rest of the tensor goes out in shorter tiles through a
-// ticket counters, so that workgroups that ran ahead take more and all finish within one short tile of each
+// the workgroups move through memory side by side (short tiles measured a little faster than long ones).
+// The rest of the tensor goes out in short tiles through ticket counters, so that workgroups that ran ahead take more and all finish within one short tile of each
 // other.  A device-wide counter serves about 90 tickets per microsecond, and 768 workgroups asking one
 // counter every few microseconds would queue up for it: the workgroups form kStageGroups groups (by number
 // modulo kStageGroups) with a counter each, and ticket t of group g is short tile number g + t * kStageGroups.
