@@ -3,7 +3,9 @@
 
 One step = exact top-k selection fused with the hash partition and slot-order
 compaction of the rank's own gradient + merge of the P peer payloads addressed
-to rank 0, all inputs resident in HBM.  Prints one JSON line (see README / DESIGN).
+to rank 0, all inputs resident in HBM.  Prints one JSON line: the step's dense-gradient
+throughput, the roofline figures of the kernel that streams the gradient, the stage
+times, the CPU baseline on the same workload and whether the HIP path reproduced it.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--shrink S]
 """
