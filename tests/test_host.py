@@ -46,9 +46,9 @@ def test_workspace_queries_are_host_only(L):
 
 def test_path_selection_is_host_only(L):
     """Which implementation a call takes depends on sizes alone."""
-    # c3: 743 M bf16 elements, top 0.5 %, 16 partitions -> bucket slabs; fp32 top-k is not on that path
+    # c3: 743 M bf16 elements, top 0.5 %, 16 partitions -> bucket slabs; the same as fp32 too
     assert L.zen_load_balance_path(743440384, 743440384, 1, 4650000, 16, 3717201, 0) == 2
-    assert L.zen_load_balance_path(743440384, 743440384, 0, 4650000, 16, 3717201, 0) == 1
+    assert L.zen_load_balance_path(743440384, 743440384, 0, 4650000, 16, 3717201, 0) == 2
     assert L.zen_load_balance_path(743440384, 743440384, 0, 4650000, 16, 0, 0) == 2
     assert L.zen_load_balance_path(743440384, 743440384, 1, 4650000, 16, 3717201, 1) == 0   # general mode
     assert L.zen_load_balance_path(1 << 20, 1 << 20, 1, 1 << 14, 4, 0, 0) == 1             # small table
