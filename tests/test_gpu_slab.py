@@ -249,6 +249,8 @@ def payloads(oracle, rng, n, peers, per_peer, overlap, dtype):
 @pytest.mark.parametrize("n,peers,per_peer,overlap", [
     (1 << 24, 16, 20000, 0.3),
     (50000000, 64, 4000, 0.5),   # every shared index arrives 64 times
+    (1 << 24, 16, 20000, 0.9),   # nine records in ten share their index with fifteen others: more than a
+                                 # workgroup sets aside for ranking in a second round
     ((1 << 23) + 12345, 4, 30000, 0.0),
 ])
 def test_slab_merge_bit_exact(zen, oracle, n, peers, per_peer, overlap, dtype, idx64):

@@ -131,8 +131,12 @@ __device__ inline uint32_t sub_place(uint32_t s) {
 // LDS decides how many workgroups share a compute unit.
 template <bool OVERLAY>
 struct SlabSortSharedT;
+constexpr int kSlabQueueCap = kSlabCap - kSlabSubs - 1;  // large-group records a workgroup sets aside
+constexpr int kSlabInline = 4;                            // groups up to this size are ranked by their own threads
+constexpr int kSlabQueueMin = 256;                        // records in larger groups below which nothing is set aside
 template <>
 struct SlabSortSharedT<false> {
+  static constexpr bool kQueue = false;
   uint32_t key[kSlabCap];
   uint32_t tie[kSlabCap];
   uint32_t cnt[kSlabSubs + 1];
@@ -141,14 +145,20 @@ struct SlabSortSharedT<false> {
 };
 template <>
 struct SlabSortSharedT<true> {
+  static constexpr bool kQueue = true;
   uint32_t key[kSlabCap];
   union {
     uint32_t tie[kSlabCap];
-    uint32_t cnt[kSlabSubs + 1];
+    struct {
+      uint32_t cnt[kSlabSubs + 1];
+      uint32_t queue[kSlabQueueCap];  // the rest of the ties' memory: records of large groups (see slab_rank)
+    };
   };
   uint32_t scan[kSlabMaxBlock / 64 + 1];
   uint32_t bad;
+  uint32_t queued;
 };
+
 static_assert(kSlabSubs + 1 <= kSlabCap, "the counters fit under the ties");
 using SlabSortShared = SlabSortSharedT<false>;
 
@@ -156,7 +166,12 @@ using SlabSortShared = SlabSortSharedT<false>;
 // tie < 2^tie_bits, the pair unique, and
 // geo.sub_shift + tie_bits <= 32.  off[i] < bucket width.  The records are first grouped by narrow key range
 // with one LDS atomic each; a record is then one word, (offset inside the range) << tie_bits | tie, and
-// inside its group every record counts the words smaller than its own.  Returns false (for every thread) if a
+// inside its group every record counts the words smaller than its own.  Where many records share a key (a
+// merge of payloads that overlap) every wave has, for each of its threads' records in turn, a few lanes that
+// walk through a group of dozens while the others wait, and the LDS instructions of all those half-empty
+// rounds are what the workgroup then spends its time on: with a Shared that has a queue, records of groups
+// larger than kSlabInline are set aside instead and handed out again afterwards, one per lane, so that the
+// lanes of a wave walk through large groups together.  Returns false (for every thread) if a
 // group is too large for that; else rank[i] for live records and *n_out = number of live records.  On return
 // sh.key / sh.tie may be overwritten at once (sh.tie is not touched at all).
 template <int BLOCK, typename Shared>
@@ -167,10 +182,14 @@ __device__ inline bool slab_rank(Shared &sh, const SlabGeom &geo, int tie_bits,
   constexpr int kItems = kSlabCap / BLOCK;
   constexpr int kSubsPer = kSlabSubs / BLOCK;
   for (int d = threadIdx.x; d <= kSlabSubs; d += BLOCK) sh.cnt[d] = 0;
-  if (threadIdx.x == 0) sh.bad = 0;
+  if (threadIdx.x == 0) {
+    sh.bad = 0;
+    if constexpr (Shared::kQueue) sh.queued = 0;
+  }
   __syncthreads();
   const uint32_t low_mask = (1u << geo.sub_shift) - 1u;
   uint32_t sub[kItems], at[kItems];
+  uint32_t in_large = 0;  // records in groups larger than kSlabInline
 #pragma unroll
   for (int i = 0; i < kItems; ++i) {
     sub[i] = at[i] = 0;
@@ -182,16 +201,18 @@ __device__ inline bool slab_rank(Shared &sh, const SlabGeom &geo, int tie_bits,
   __syncthreads();
   {
     uint32_t c[kSubsPer];
-    uint32_t sum = 0, big = 0;
+    uint32_t sum = 0, big = 0;  // sum: records in the low half, records of groups larger than kSlabInline in the high half
+    static_assert(kSlabCap < 65536, "two counts in one word");
 #pragma unroll
     for (int e = 0; e < kSubsPer; ++e) {
       c[e] = sh.cnt[e * BLOCK + threadIdx.x];
-      sum += c[e];
+      sum += c[e] + (c[e] > (uint32_t)kSlabInline ? c[e] << 16 : 0u);
       big |= c[e] > (uint32_t)kSlabGroupLimit;
     }
     if (big) sh.bad = 1;
     uint32_t total;
-    uint32_t running = block_exclusive_scan<uint32_t, BLOCK>(sum, sh.scan, &total);
+    uint32_t running = block_exclusive_scan<uint32_t, BLOCK>(sum, sh.scan, &total) & 0xffffu;
+    in_large = total >> 16;
 #pragma unroll
     for (int e = 0; e < kSubsPer; ++e) {
       sh.cnt[e * BLOCK + threadIdx.x] = running;
@@ -212,15 +233,67 @@ __device__ inline bool slab_rank(Shared &sh, const SlabGeom &geo, int tie_bits,
     }
   }
   __syncthreads();
+  constexpr uint32_t kSetAside = 0x80000000u;
+  uint32_t g1[kItems];
 #pragma unroll
   for (int i = 0; i < kItems; ++i) {
     rank[i] = 0;
-    if (live & (1u << i)) {
-      const uint32_t g1 = sh.cnt[sub_place<BLOCK>(sub[i] + 1)];
+    g1[i] = (live & (1u << i)) ? sh.cnt[sub_place<BLOCK>(sub[i] + 1)] : g0[i];
+  }
+  // a few large groups are not worth the two extra barriers
+  const bool set_aside = Shared::kQueue && in_large >= (uint32_t)kSlabQueueMin;
+  if constexpr (Shared::kQueue) {
+    // records of large groups are set aside: one LDS atomic per wave and round, not per lane (they would all
+    // meet on the one counter)
+    if (set_aside) {
+#pragma unroll
+      for (int i = 0; i < kItems; ++i) {
+        if (g1[i] - g0[i] > (uint32_t)kSlabInline) {
+          const uint64_t peers = __ballot(1);
+          const uint32_t before = (uint32_t)__popcll(peers & ((1ull << (threadIdx.x & 63u)) - 1ull));
+          uint32_t q = 0;
+          if (before == 0) q = atomicAdd(&sh.queued, (uint32_t)__popcll(peers));
+          q = (uint32_t)__shfl((int)q, (int)__ffsll((long long)peers) - 1) + before;
+          if (q < (uint32_t)kSlabQueueCap) {
+            sh.queue[q] = sub[i] | (at[i] << 12);  // sub < 2^12, at < group size <= kSlabGroupLimit
+            rank[i] = kSetAside | q;
+            g1[i] = g0[i];  // nothing left to do for it below
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kItems; ++i) {
+    if (g1[i] > g0[i]) {
       uint32_t less = 0;
-      for (uint32_t u = g0[i]; u < g1; ++u) less += sh.key[u] < word[i];
+      for (uint32_t u = g0[i]; u < g1[i]; ++u) less += sh.key[u] < word[i];
       rank[i] = g0[i] + less;
     }
+  }
+  if constexpr (Shared::kQueue) {
+    static_assert(kSlabSubs <= (1 << 12) && kSlabGroupLimit <= (1 << 19), "a queue entry is one word");
+    if (!set_aside) {
+      *n_out = sh.cnt[kSlabSubs];
+      __syncthreads();
+      return true;
+    }
+    __syncthreads();
+    const uint32_t queued = sh.queued < (uint32_t)kSlabQueueCap ? sh.queued : (uint32_t)kSlabQueueCap;
+    // the thread that takes a queue entry also overwrites it with the rank
+#pragma unroll 1
+    for (uint32_t q = threadIdx.x; q < queued; q += BLOCK) {
+      const uint32_t e = sh.queue[q];
+      const uint32_t b0 = sh.cnt[sub_place<BLOCK>(e & 4095u)], b1 = sh.cnt[sub_place<BLOCK>((e & 4095u) + 1)];
+      const uint32_t w = sh.key[b0 + (e >> 12)];
+      uint32_t less = 0;
+      for (uint32_t u = b0; u < b1; ++u) less += sh.key[u] < w;
+      sh.queue[q] = b0 + less;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kItems; ++i)
+      if (rank[i] & kSetAside) rank[i] = sh.queue[rank[i] & ~kSetAside];
   }
   *n_out = sh.cnt[kSlabSubs];
   __syncthreads();
