@@ -248,6 +248,21 @@ int zen_decode_dense(const void *idx, int idx64_in, const void *val, int dtype,
                      void *workspace, size_t workspace_bytes,
                      int32_t *status, void *stream);
 
+/*
+ * The same for payloads that arrive as `nlists` strictly ascending index lists back to back (list l is
+ * idx[list_start[l] .. list_start[l + 1]), list_start a HOST array of nlists + 1 offsets, at most 64 lists):
+ * the second exchange of the sparse all-reduce, where every rank receives all ranks' merged shards
+ * (comm.py:142-145), and method 1, where it receives all ranks' own selections (comm.py:113-117).  No sort
+ * and no cleared dense tensor: one workgroup per tile of the dense tensor gathers its stretch of every list
+ * and writes the tile once.  Same result as zen_decode_dense, bit for bit (lists may share indices).  A list
+ * that is not strictly ascending or an index outside [0, dense_n) raises ZEN_STAT_RETRY: the dense tensor
+ * is then unspecified and the caller repeats with zen_decode_dense.
+ */
+size_t zen_decode_dense_sorted_workspace(int64_t dense_n, int nlists);
+int zen_decode_dense_sorted(const void *idx, int idx64_in, const void *val, int dtype,
+                            const int64_t *list_start, int nlists, void *dense, int64_t dense_n,
+                            void *workspace, size_t workspace_bytes, int32_t *status, void *stream);
+
 /* --------------------------------------------------------------- utility */
 
 /*

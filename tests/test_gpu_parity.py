@@ -569,6 +569,113 @@ def test_decode_sparse_tensors_dense(zen, oracle, dtype):
         assert (np.abs(oracle.bf16_bits_to_f32(got) - native) <= 2e-2 * scale + 1e-30).all()
 
 
+def ascending_lists(oracle, rng, n, nlists, per_list, shared, dtype, idx_dtype):
+    """nlists strictly ascending index lists over [0, n); a fraction `shared` of every list comes from one pool
+    (lists meet on those indices), the rest lies in the list's own residue class (disjoint)."""
+    pool = rng.choice(n // nlists, max(1, int(per_list * shared) * 2), replace=False) * nlists
+    idx, val = [], []
+    for l in range(nlists):
+        common = rng.choice(pool, int(per_list * shared), replace=False) if shared > 0 else np.empty(0, np.int64)
+        own = rng.choice(n // nlists, per_list - len(common), replace=False) * nlists + (l if l else 0)
+        i = np.unique(np.concatenate([common, own])).astype(idx_dtype)
+        v = (rng.standard_normal(len(i)) * 1e-3).astype(np.float32)
+        v[::97] = -0.0  # +0 + -0 = +0: the dense element stays a plain zero
+        idx.append(i)
+        val.append(oracle.f32_to_bf16_bits(v) if dtype == "bf16" else v)
+    return idx, val
+
+
+@pytest.mark.parametrize("idx_dtype", [np.int64, np.int32])
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("n,nlists,per_list,shared", [
+    ((1 << 22) + 4099, 16, 20000, 0.0),   # the second exchange: disjoint shards; size not a multiple of the tile
+    (1 << 22, 16, 20000, 0.4),            # method 1: every rank's own selection, lists meet on many indices
+    (1 << 20, 1, 5000, 0.0),
+    (3000, 5, 40, 0.5),                   # less than one tile
+    (1 << 21, 64, 3000, 0.1),
+])
+def test_decode_ascending_lists_without_a_sort(zen, oracle, n, nlists, per_list, shared, dtype, idx_dtype):
+    """zen_decode_dense_sorted through decode_sparse_tensors(ascending=True): bit-identical to the oracle's
+    sequential fp32 scatter_add (and therefore to zen_decode_dense), straight through the C-ABI too."""
+    from zen_repro_amd import _lib
+
+    rng = np.random.default_rng(n % 977 + nlists)
+    idx, val = ascending_lists(oracle, rng, n, nlists, per_list, shared, dtype, idx_dtype)
+    ci, cv = np.concatenate(idx), np.concatenate(val)
+    f32 = oracle.decode(ci.astype(np.int64), cv, n, "f32acc")
+    want = oracle.f32_to_bf16_bits(f32) if dtype == "bf16" else f32
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(max(nlists, 2)), None, None)
+    d_idx, d_val = [to_dev(i) for i in idx], [to_dev(v) for v in val]
+    got = lba.decode_sparse_tensors(d_idx, d_val, n, ascending=True)
+    assert np.array_equal(to_np(got).view(want.dtype), want)
+    assert np.array_equal(to_np(lba.decode_sparse_tensors(d_idx, d_val, n)).view(want.dtype), want)
+    # the entry point itself: it must have taken the lists as they are (status 0), into a buffer full of ones
+    L = _lib.lib()
+    flat_i, flat_v = to_dev(ci), to_dev(cv)
+    dense = torch.full((n,), 1.0, dtype=flat_v.dtype, device="cuda")
+    starts = (ctypes.c_int64 * (nlists + 1))(0, *np.cumsum([len(i) for i in idx]).tolist())
+    ws = torch.empty(L.zen_decode_dense_sorted_workspace(n, nlists), dtype=torch.uint8, device="cuda")
+    status = _lib.status_word("cuda")
+    rc = L.zen_decode_dense_sorted(_lib.ptr(flat_i), int(idx_dtype == np.int64), _lib.ptr(flat_v), _lib.dtype_code(flat_v),
+                                   starts, nlists, _lib.ptr(dense), n, _lib.ptr(ws), ws.numel(), _lib.ptr(status),
+                                   _lib.stream_of("cuda"))
+    assert rc == 0 and status.item() == 0
+    assert np.array_equal(to_np(dense).view(want.dtype), want)
+
+
+def test_decode_ascending_declines_what_is_not_ascending(zen, oracle):
+    """A list with a descent, a repeated index inside one list or an index outside the dense tensor raise
+    ZEN_STAT_RETRY; decode_sparse_tensors then answers through the general entry point (or raises, for the
+    bad index, as the reference's scatter_add_ does)."""
+    from zen_repro_amd import _lib
+
+    n = 1 << 20
+    rng = np.random.default_rng(3)
+    idx, val = ascending_lists(oracle, rng, n, 4, 3000, 0.2, "f32", np.int64)
+    L = _lib.lib()
+
+    def status_of(lists):
+        flat_i, flat_v = to_dev(np.concatenate(lists)), to_dev(np.concatenate(val))
+        dense = torch.empty(n, dtype=torch.float32, device="cuda")
+        starts = (ctypes.c_int64 * 5)(0, *np.cumsum([len(i) for i in lists]).tolist())
+        ws = torch.empty(L.zen_decode_dense_sorted_workspace(n, 4), dtype=torch.uint8, device="cuda")
+        status = _lib.status_word("cuda")
+        rc = L.zen_decode_dense_sorted(_lib.ptr(flat_i), 1, _lib.ptr(flat_v), _lib.F32, starts, 4, _lib.ptr(dense), n,
+                                       _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of("cuda"))
+        assert rc == 0
+        return int(status.item())
+
+    assert status_of(idx) == 0
+    swapped = [i.copy() for i in idx]
+    swapped[2][[100, 101]] = swapped[2][[101, 100]]          # one descent
+    assert status_of(swapped) == _lib.STAT_RETRY
+    twice = [i.copy() for i in idx]
+    twice[1][500] = twice[1][499]                             # the same index twice in one list
+    assert status_of(twice) == _lib.STAT_RETRY
+    beyond = [i.copy() for i in idx]
+    beyond[3][-1] = n + 5                                     # ascending, but outside the tensor
+    assert status_of(beyond) == _lib.STAT_RETRY
+    below = [i.copy() for i in idx]
+    below[0][0] = -3
+    assert status_of(below) == _lib.STAT_RETRY
+    # through the wrapper the result is right all the same
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(4), None, None)
+    for lists in (swapped, twice):
+        got = lba.decode_sparse_tensors([to_dev(i) for i in lists], [to_dev(v) for v in val], n, ascending=True)
+        assert np.array_equal(to_np(got), oracle.decode(np.concatenate(lists), np.concatenate(val), n, "f32acc"))
+    with pytest.raises(RuntimeError):
+        lba.decode_sparse_tensors([to_dev(i) for i in beyond], [to_dev(v) for v in val], n, ascending=True)
+    # bad arguments are the host's business
+    ws = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    status = _lib.status_word("cuda")
+    bad = (ctypes.c_int64 * 3)(0, 10, 5)
+    assert L.zen_decode_dense_sorted(_lib.ptr(ws), 1, _lib.ptr(ws), _lib.F32, bad, 2, _lib.ptr(ws), 100, _lib.ptr(ws),
+                                     ws.numel(), _lib.ptr(status), None) == _lib.EINVAL
+    ok = (ctypes.c_int64 * 2)(0, 10)
+    assert L.zen_decode_dense_sorted(_lib.ptr(ws), 1, _lib.ptr(ws), _lib.F32, ok, 1, _lib.ptr(ws), 1 << 30,
+                                     _lib.ptr(ws), ws.numel(), _lib.ptr(status), None) == _lib.EWORKSPACE
+
+
 def test_stack_tensors_views_are_not_copied(zen):
     buf = torch.arange(100, device="cuda", dtype=torch.int32)
     parts = [buf[0:10], buf[10:45], buf[45:100]]

@@ -2,6 +2,9 @@
 (LoadBalanceAllreduce).  The collectives around it are not part of this
 package: one GPU computes its own share, the full P-way partition of its
 gradient and the merge of P incoming payloads."""
+import ctypes
+import itertools
+
 import torch
 
 from . import _lib
@@ -75,10 +78,16 @@ class LoadBalanceAllreduce:
         return tensors.reshape(shape)
 
     # ------------------------------------------------------------ merge
-    def decode_sparse_tensors(self, indices_tensors, values_tensors, alltoall_dense_size):
+    def decode_sparse_tensors(self, indices_tensors, values_tensors, alltoall_dense_size, ascending=False):
         """Dense tensor of `alltoall_dense_size` elements in the value dtype with
         every payload scatter-added into it (comm.py:32-44).  Sums are taken in
-        fp32 in payload order and rounded once."""
+        fp32 in payload order and rounded once.  `ascending` says that every
+        tensor of the list is a strictly ascending index list (what the second
+        exchange and method 1 deliver, comm.py:113-117, 142-145): the dense
+        tensor is then built tile by tile without a sort; a list that is not
+        ascending after all only costs the time of the attempt."""
+        lists = indices_tensors if isinstance(indices_tensors, (list, tuple)) else [indices_tensors]
+        sizes = [int(t.numel()) for t in lists]
         indices = self.stack_tensors(indices_tensors)
         values = self.stack_tensors(values_tensors)
         assert indices.dtype in (torch.int32, torch.int64)
@@ -88,6 +97,18 @@ class LoadBalanceAllreduce:
         L = _lib.lib()
         r = indices.numel()
         dense = torch.empty(alltoall_dense_size, dtype=values.dtype, device=dev)
+        if ascending and 1 <= len(sizes) <= 64 and sum(sizes) == r == values.numel():
+            starts = (ctypes.c_int64 * (len(sizes) + 1))(0, *itertools.accumulate(sizes))
+            ws = _lib.scratch.get(dev, "decode_sorted",
+                                  L.zen_decode_dense_sorted_workspace(alltoall_dense_size, len(sizes)))
+            status = _lib.status_word(dev)
+            rc = L.zen_decode_dense_sorted(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(values),
+                                           _lib.dtype_code(values), starts, len(sizes), _lib.ptr(dense),
+                                           alltoall_dense_size, _lib.ptr(ws), ws.numel(), _lib.ptr(status),
+                                           _lib.stream_of(dev))
+            _lib.check(rc, "decode_sparse_tensors")
+            if not int(status.item()):  # the reference's scatter_add_ raises on a bad index, also a sync
+                return dense
         ws = _lib.scratch.get(dev, "decode", L.zen_decode_dense_workspace(r, alltoall_dense_size))
         for mode in (_lib.MODE_FAST, _lib.MODE_GENERAL):
             status = _lib.status_word(dev)
@@ -268,7 +289,7 @@ class LoadBalanceAllreduce:
             sparse_indices, sparse_values = self.encode_sparse_tensor(tensor)
             indices_tensors = ddp.allgather_padding(sparse_indices)
             values_tensors = ddp.allgather_padding(sparse_values)
-            return self.decode_sparse_tensors(indices_tensors, values_tensors, numel)
+            return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
         indices, values, splits = self.tensor_partition.load_balance(tensor)
         gather_splits = ddp.allgather(splits)
         indices_tensors = ddp.alltoallv(indices, gather_splits)
@@ -284,7 +305,7 @@ class LoadBalanceAllreduce:
             bitmap_indices_gather = ddp.allgather_padding(bitmap_indices)
             indices_tensors = self.decode_bitmap(bitmap_indices_gather, numel)
         values_tensors = ddp.allgather_padding(sparse_values)
-        return self.decode_sparse_tensors(indices_tensors, values_tensors, numel)
+        return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
 
 
 def _as_one_buffer(tensors):
