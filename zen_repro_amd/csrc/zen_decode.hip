@@ -7,7 +7,7 @@
 // dense result needs no sort: the dense tensor is cut into tiles of kDecTile
 // elements, a first kernel finds where every tile starts in every list, and one
 // workgroup per tile gathers its entries (a contiguous stretch of every list)
-// into fp32 accumulators in LDS and writes the tile out with full-width
+// into a copy of the tile in LDS and writes the tile out with full-width
 // stores.  The dense tensor is written exactly once and never cleared first.
 //
 // Sums are taken in fp32 from +0 in payload order and rounded once, like
@@ -20,7 +20,7 @@
 namespace zen {
 namespace {
 
-constexpr int kDecTile = 4096;   // dense elements per workgroup (16 KB of fp32 accumulators)
+constexpr int kDecTile = 8192;   // dense elements per workgroup (its LDS copy: 16 KB for bf16, 32 KB for fp32)
 constexpr int kDecBlock = 256;
 constexpr int kDecMaxLists = 64;
 
@@ -59,43 +59,30 @@ __global__ __launch_bounds__(256) void k_decode_starts(const I *__restrict__ idx
   starts[g] = lo;
 }
 
+// The value a dense element gets from one entry: +0 + v in fp32, rounded to the tensor's type (-0 becomes +0,
+// like in a scatter_add_ into zeros).
+__device__ inline uint16_t single_value(uint16_t v) { return f32_to_bf16_rne(0.0f + KeyOf<uint16_t>::to_f32(v)); }
+__device__ inline uint32_t single_value(uint32_t v) { return __float_as_uint(0.0f + __uint_as_float(v)); }
+__device__ inline uint16_t rounded(float f, uint16_t) { return f32_to_bf16_rne(f); }
+__device__ inline uint32_t rounded(float f, uint32_t) { return __float_as_uint(f); }
+
+// n elements (a multiple of 16 bytes' worth, from a 16-byte aligned LDS array) to dense[first ..), as wide as
+// the tensor's end and alignment allow.
 template <typename S>
-__device__ inline void store_tile(const float *acc, S *__restrict__ dense, int64_t first, int64_t dense_n);
-
-template <>
-__device__ inline void store_tile<uint16_t>(const float *acc, uint16_t *__restrict__ dense, int64_t first,
-                                            int64_t dense_n) {
-  for (int j = threadIdx.x * 8; j < kDecTile; j += kDecBlock * 8) {
-    uint16_t out[8];
-#pragma unroll
-    for (int q = 0; q < 8; ++q) out[q] = f32_to_bf16_rne(acc[j + q]);
-    if (first + j + 8 <= dense_n && ((reinterpret_cast<uintptr_t>(dense) & 15u) == 0)) {
-      uint4 v;
-      __builtin_memcpy(&v, out, 16);
-      *reinterpret_cast<uint4 *>(dense + first + j) = v;
+__device__ inline void store_run(const S *src, int n, S *__restrict__ dense, int64_t first, int64_t dense_n) {
+  constexpr int V = 16 / sizeof(S);
+  const bool wide = (reinterpret_cast<uintptr_t>(dense + first) & 15u) == 0;
+  for (int j = threadIdx.x * V; j < n; j += kDecBlock * V) {
+    if (wide && first + j + V <= dense_n) {
+      *reinterpret_cast<uint4 *>(dense + first + j) = *reinterpret_cast<const uint4 *>(src + j);
     } else {
-      for (int q = 0; q < 8; ++q)
-        if (first + j + q < dense_n) dense[first + j + q] = out[q];
+      for (int q = 0; q < V; ++q)
+        if (first + j + q < dense_n) dense[first + j + q] = src[j + q];
     }
   }
 }
 
-template <>
-__device__ inline void store_tile<uint32_t>(const float *acc, uint32_t *__restrict__ dense, int64_t first,
-                                            int64_t dense_n) {
-  for (int j = threadIdx.x * 4; j < kDecTile; j += kDecBlock * 4) {
-    if (first + j + 4 <= dense_n && ((reinterpret_cast<uintptr_t>(dense) & 15u) == 0)) {
-      const uint4 v = make_uint4(__float_as_uint(acc[j]), __float_as_uint(acc[j + 1]), __float_as_uint(acc[j + 2]),
-                                 __float_as_uint(acc[j + 3]));
-      *reinterpret_cast<uint4 *>(dense + first + j) = v;
-    } else {
-      for (int q = 0; q < 4; ++q)
-        if (first + j + q < dense_n) dense[first + j + q] = __float_as_uint(acc[j + q]);
-    }
-  }
-}
-
-constexpr int kDecStage = 1024;  // entries of a tile kept in LDS for the case that lists meet
+constexpr int kDecStage = 2048;  // entries of a tile kept in LDS for the case that lists meet
 
 // One workgroup per tile.  Anything that contradicts "every list strictly ascending, every index inside
 // [0, dense_n)" raises ZEN_STAT_RETRY (the caller repeats with zen_decode_dense, which takes any input).
@@ -106,24 +93,26 @@ __global__ __launch_bounds__(kDecBlock) void k_decode_tiles(const I *__restrict_
                                                             DecLists lists, int64_t ntiles,
                                                             const uint32_t *__restrict__ starts, S *__restrict__ dense,
                                                             int64_t dense_n, int32_t *status) {
-  __shared__ float acc[kDecTile];
+  // The tile in the tensor's own type; where lists meet the same memory holds fp32 sums for a part of the tile
+  // at a time (LDS decides how many tiles a compute unit has in flight, and the kernel lives on that).
+  __shared__ __attribute__((aligned(16))) S tile[kDecTile];
   __shared__ uint32_t occ[kDecTile / 32];
   __shared__ int64_t s_base[kDecMaxLists];      // where the list's stretch starts in idx / val
   __shared__ uint32_t s_first[kDecMaxLists];    // entry number inside the list of the stretch's first entry
   __shared__ uint32_t s_pref[kDecMaxLists + 1];  // entries of the lists before, in this tile
   __shared__ uint16_t st_off[kDecStage];
-  __shared__ float st_val[kDecStage];
+  __shared__ S st_val[kDecStage];
   __shared__ uint32_t s_meet, s_wrong;
   static_assert(kDecMaxLists == 64 && kDecTile <= 65536, "one wave scans the lists; offsets are 16 bits");
   const int64_t t = blockIdx.x;
   const int64_t first = t * (int64_t)kDecTile;
   const int64_t per_list = ntiles + 1;
-  uint32_t a = 0, b = 0;  // asked for first: the answer is on its way while the accumulators are cleared
+  uint32_t a = 0, b = 0;  // asked for first: the answer is on its way while the tile is cleared
   if ((int)threadIdx.x < lists.n) {
     a = starts[threadIdx.x * per_list + t];
     b = starts[threadIdx.x * per_list + t + 1];
   }
-  for (int j = threadIdx.x; j < kDecTile; j += kDecBlock) acc[j] = 0.0f;
+  for (int j = threadIdx.x; j < kDecTile; j += kDecBlock) tile[j] = 0;
   for (int j = threadIdx.x; j < kDecTile / 32; j += kDecBlock) occ[j] = 0;
   if (threadIdx.x == 0) s_meet = s_wrong = 0;
   if (threadIdx.x < 64) {
@@ -162,10 +151,10 @@ __global__ __launch_bounds__(kDecBlock) void k_decode_tiles(const I *__restrict_
       wrong = true;
       continue;
     }
-    const float v = KeyOf<S>::to_f32(val[at]);
+    const S v = val[at];
     const uint32_t bit = 1u << (off & 31u);
     if (atomicOr(&occ[off >> 5], bit) & bit) meet = true;
-    acc[off] = 0.0f + v;
+    tile[off] = single_value(v);
     if (f < (uint32_t)kDecStage) {
       st_off[f] = (uint16_t)off;
       st_val[f] = v;
@@ -178,25 +167,53 @@ __global__ __launch_bounds__(kDecBlock) void k_decode_tiles(const I *__restrict_
     if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
     return;  // the caller repeats the whole call: what this tile holds does not matter
   }
-  if (s_meet) {
-    // two lists share an index here: the lists one after the other (inside a list every index occurs once),
-    // from the staged copy, or from memory again if the tile holds more entries than the stage
-    for (int j = threadIdx.x; j < kDecTile; j += kDecBlock) acc[j] = 0.0f;
+  if (!s_meet) {
+    store_run<S>(tile, kDecTile, dense, first, dense_n);
+    return;
+  }
+  // Two lists share an index here: fp32 sums, the lists one after the other (inside a list every index occurs
+  // once), from the staged copy, or from memory again if the tile holds more entries than the stage.  The
+  // tile's memory holds the sums of kPart elements at a time; each part is rounded in place and written out.
+  constexpr int kPart = kDecTile * (int)sizeof(S) / (int)sizeof(float);
+  float *acc = reinterpret_cast<float *>(tile);
+  for (int part = 0; part < kDecTile; part += kPart) {
+    for (int j = threadIdx.x; j < kPart; j += kDecBlock) acc[j] = 0.0f;
     __syncthreads();
     for (int l = 0; l < lists.n; ++l) {
       const uint32_t f0 = s_pref[l], f1 = s_pref[l + 1];
       for (uint32_t f = f0 + threadIdx.x; f < f1; f += kDecBlock) {
+        uint32_t off;
+        S v;
         if (f < (uint32_t)kDecStage) {
-          acc[st_off[f]] += st_val[f];
+          off = st_off[f];
+          v = st_val[f];
         } else {
           const int64_t at = s_base[l] + (f - f0);
-          acc[(uint32_t)((int64_t)idx[at] - first)] += KeyOf<S>::to_f32(val[at]);
+          off = (uint32_t)((int64_t)idx[at] - first);
+          v = val[at];
         }
+        if (off - (uint32_t)part < (uint32_t)kPart) acc[off - (uint32_t)part] += KeyOf<S>::to_f32(v);
       }
       __syncthreads();
     }
+    // rounded where it stands: a thread reads the sums of its own 16 bytes of output before it writes them
+    // (the narrower type's array overlays the first part of the sums' memory, ahead of what is still unread
+    // only for other threads' elements, hence the barrier between reading and writing)
+    constexpr int V = 16 / (int)sizeof(S);
+    S out[kPart / kDecBlock];
+#pragma unroll
+    for (int i = 0; i < kPart / kDecBlock / V; ++i)
+#pragma unroll
+      for (int q = 0; q < V; ++q) out[i * V + q] = rounded(acc[(threadIdx.x + i * kDecBlock) * V + q], S(0));
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kPart / kDecBlock / V; ++i)
+#pragma unroll
+      for (int q = 0; q < V; ++q) tile[(threadIdx.x + i * kDecBlock) * V + q] = out[i * V + q];
+    __syncthreads();
+    store_run<S>(tile, kPart, dense, first + part, dense_n);
+    __syncthreads();
   }
-  store_tile<S>(acc, dense, first, dense_n);
 }
 
 template <typename I, typename S>
