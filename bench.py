@@ -38,6 +38,8 @@ def parse():
                     help="run five device copies of 1 GiB and exit (scale for hardware byte counters)")
     ap.add_argument("--bitmap-codec", action="store_true",
                     help="measure the bitmap index codec of the second exchange instead (prints its own line)")
+    ap.add_argument("--phase2-decode", action="store_true",
+                    help="measure the decode of the second exchange instead (prints its own line)")
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
     ap.add_argument("--merge-follows", action="store_true",
                     help="with --depth: a step's merge runs on its encode's stream, after it")
@@ -163,6 +165,64 @@ def bitmap_codec(args, dev):
         "algorithmic_bytes": b_alg, "algorithmic_GBps": round(b_alg / (ms * 1e-3) / 1e9, 2)}))
 
 
+def phase2_decode(args, dev):
+    """The second exchange's decode (comm.py:142-145): P ascending, pairwise disjoint shards of merged entries
+    (rank p's shard holds indices of hash partition p, as many as rank 0 merges in the main benchmark) into
+    the dense gradient.  One step = one decode_sparse_tensors(ascending=True) of the concatenated shards;
+    the result is checked against a plain assignment (the shards are disjoint)."""
+    import torch
+
+    from zen_repro_amd import LoadBalanceAllreduce, LocalGroup, workloads
+
+    cfg, grad = workloads.make(args.config, device=dev, seed=0, shrink=args.shrink)
+    dtype = grad.dtype
+    del grad
+    n, P = cfg.n, cfg.partitions
+    lba = LoadBalanceAllreduce(LocalGroup(P, 0), None, None)
+    part = torch.empty(n, dtype=torch.int32, device=dev)
+    from zen_repro_amd.functions import hash_index
+    hash_index(part, P)
+    per = max(1, int((cfg.k or n // 100) * 0.766))  # what a rank keeps after merging P payloads that overlap by a quarter
+    gen = torch.Generator(device=dev).manual_seed(2)
+    idx, val = [], []
+    for p in range(P):
+        members = torch.nonzero(part == p, as_tuple=True)[0]
+        pick = torch.randperm(members.numel(), device=dev, generator=gen)[:per].sort().values
+        idx.append(members[pick].contiguous())
+        val.append((torch.randn(per, device=dev, generator=gen) * 1e-3).to(dtype))
+        del members, pick
+    del part
+    flat_i, flat_v = torch.cat(idx), torch.cat(val)
+    sizes = [t.numel() for t in idx]
+    views = list(torch.split(flat_i, sizes)), list(torch.split(flat_v, sizes))  # what an all-gather into one buffer leaves
+
+    def step():
+        return lba.decode_sparse_tensors(views[0], views[1], n, ascending=True)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        dense = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    want = torch.zeros(n, dtype=dtype, device=dev)
+    want[flat_i] = flat_v
+    bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
+    if not torch.equal(dense.view(bits), want.view(bits)):
+        print("bench.py: the decoded dense tensor is not the shards' assignment", file=sys.stderr)
+        sys.exit(1)
+    r, s_ = flat_i.numel(), flat_v.element_size()
+    b_alg = r * (8 + s_) + n * s_
+    print(json.dumps({
+        "metric": "phase-2 decode: all ranks' merged shards into the dense gradient", "value": round(b_alg / (ms * 1e-3) / 1e9, 2),
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "dtype": "bf16" if dtype == torch.bfloat16 else "f32", "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: {cfg.note}", "elements": n, "shards": P, "entries": r},
+        "algorithmic_bytes": b_alg}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -194,6 +254,9 @@ def main():
 
     if args.bitmap_codec:
         bitmap_codec(args, dev)
+        return
+    if args.phase2_decode:
+        phase2_decode(args, dev)
         return
 
     cfg, grad = workloads.make(args.config, device=dev, seed=0, shrink=args.shrink)
