@@ -294,8 +294,13 @@ class LoadBalanceAllreduce:
         gather_splits = ddp.allgather(splits)
         indices_tensors = ddp.alltoallv(indices, gather_splits)
         values_tensors = ddp.alltoallv(values, gather_splits)
-        _dense_tensor = self.decode_sparse_tensors(indices_tensors, values_tensors, numel)
-        sparse_indices, sparse_values = self.encode_sparse_tensor(_dense_tensor)
+        # decode_sparse_tensors + encode_sparse_tensor (comm.py:125-127) without the dense tensor in between:
+        # fp32 sums in payload order, rounded once to the tensor's type, what rounds to zero dropped
+        sparse_indices, sums = self.merge_sparse(indices_tensors, values_tensors, numel)
+        sparse_values = sums.to(tensor.dtype)
+        nonzero = sparse_values != 0
+        if not bool(nonzero.all()):
+            sparse_indices, sparse_values = sparse_indices[nonzero], sparse_values[nonzero]
         if method == 2:
             indices_tensors = ddp.allgather_padding(sparse_indices)
         else:
