@@ -156,6 +156,23 @@ int zen_topk_threshold(const void *input, int dtype, int64_t n, int64_t k,
                        void *stream);
 
 /*
+ * zen_topk_threshold without a workspace argument and without any allocation.
+ * No counterpart in the reference: it is for callers that cannot allocate or
+ * carry a workspace (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  The radix select's counters and histogram
+ * (8448 bytes) live in a static device array inside the library, one copy per
+ * GPU, held until the process ends.  Same arguments otherwise, same result.
+ * n > ZEN_TOPK_STATIC_MAX_N is ZEN_EINVAL.  All calls on one GPU share that
+ * array: calls that overlap on one GPU (two streams, two host threads) race;
+ * calls in stream order do not, each clears the array before it counts.  The
+ * first call on a device looks the array's address up
+ * (hipGetSymbolAddress); make it outside graph capture.
+ */
+#define ZEN_TOPK_STATIC_MAX_N 0x7fffffffll
+int zen_topk_threshold_static(const void *input, int dtype, int64_t n, int64_t k,
+                              uint32_t *thr, void *stream);
+
+/*
  * out[i] = key(input[i]) >= thr[0] ? input[i] : 0.  Replaces
  * torch.where(tensor_abs >= threshold, tensor, 0) (train.py:83).
  */

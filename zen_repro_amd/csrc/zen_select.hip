@@ -4,6 +4,8 @@
 // tensor into ascending (index, value) lists (comm.py:47-50).
 #include <math.h>
 
+#include <mutex>
+
 #include "zen_select.h"
 
 namespace zen {
@@ -1249,9 +1251,56 @@ size_t sampled_floor_zero_bytes() { return (kFineBins + 2) * sizeof(uint32_t); }
 
 }  // namespace zen
 
+// The radix select's counters and histogram for callers that cannot bring a workspace along: one array per
+// GPU, part of the loaded code object, which that GPU holds until the process ends.  Host code never passes
+// the array's name to a kernel (on the host it is a stand-in, not a device address): it asks for the address
+// once per device and keeps it.
+namespace {
+
+constexpr size_t kTopkStaticBytes = 256 /* TopkState */ + zen::kHistBins * sizeof(uint32_t);
+static_assert(sizeof(zen::TopkState) <= 256, "TopkState outgrew its slot");
+static __device__ __align__(256) unsigned char g_topk_static[kTopkStaticBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_topk_static_mu;
+void *g_topk_static_at[kMaxDevices];  // device address of g_topk_static, per device; null = not asked yet
+
+// Address of the current device's copy of g_topk_static.
+int topk_static_scratch(void **out) {
+  int dev = -1;
+  ZEN_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return zen::fail(ZEN_EINVAL, "zen_topk_threshold_static: device number out of range");
+  std::lock_guard<std::mutex> lock(g_topk_static_mu);
+  if (!g_topk_static_at[dev]) {
+    void *p = nullptr;
+    ZEN_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(g_topk_static)));
+    if (!p) return zen::fail(ZEN_EHIP, "zen_topk_threshold_static: no address for the static scratch array");
+    g_topk_static_at[dev] = p;
+  }
+  *out = g_topk_static_at[dev];
+  return ZEN_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 size_t zen_topk_threshold_workspace(void) { return zen::topk_scratch_bytes(); }
+
+int zen_topk_threshold_static(const void *input, int dtype, int64_t n, int64_t k, uint32_t *thr, void *stream) {
+  using namespace zen;
+  if (!input || !thr) return fail(ZEN_EINVAL, "zen_topk_threshold_static: null pointer");
+  if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_topk_threshold_static: bad dtype");
+  if (n <= 0 || n > ZEN_TOPK_STATIC_MAX_N)
+    return fail(ZEN_EINVAL, "zen_topk_threshold_static: n exceeds ZEN_TOPK_STATIC_MAX_N (2^31 - 1 elements)");
+  if (k < 1 || k > n) return fail(ZEN_EINVAL, "zen_topk_threshold_static: need 1 <= k <= n");
+  void *scratch_at = nullptr;
+  const int rc = topk_static_scratch(&scratch_at);
+  if (rc != ZEN_OK) return rc;
+  // k_topk_init clears the counters and the histogram at the head of every call, so what the previous call
+  // left in the array does not matter.
+  return topk_exact(input, dtype, n, nullptr, k, thr, scratch_at, nullptr, 0, static_cast<hipStream_t>(stream));
+}
 
 int zen_topk_threshold(const void *input, int dtype, int64_t n, int64_t k, uint32_t *thr, void *workspace,
                        size_t workspace_bytes, void *stream) {
