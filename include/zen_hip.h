@@ -50,6 +50,11 @@ extern "C" {
 /* `mode` argument of the sort-based entry points */
 #define ZEN_MODE_FAST 0    /* bucket sort in LDS; flags ZEN_STAT_RETRY on pathological key distributions */
 #define ZEN_MODE_GENERAL 1 /* one radix pass per 8 key bits; any input */
+/* OR-ed into the `mode` of zen_merge: the caller vouches that the first zen_merge_zero_bytes() bytes of the
+   workspace are zero.  The call then skips the kernel that clears them, and leaves them zero again when it
+   returns ZEN_OK and raises neither ZEN_STAT_RETRY nor ZEN_STAT_INTERNAL (after those the caller clears
+   them).  A workspace allocated zeroed and used for zen_merge only therefore needs no clearing at all. */
+#define ZEN_MODE_ZEROED 0x100
 
 int zen_abi_version(void);
 
@@ -211,9 +216,10 @@ int zen_select(const void *input, int dtype, int64_t n, const uint32_t *thr,
  * tensor_load_balance.py:15-16; the serial capacity is n / partitions / 10
  * per partition (tensor_load_balance.py:18).
  * `table` is int32[m] scratch that must be all zero on entry and is all zero
- * again on return (so one allocation serves every call); after a call that
- * raised ZEN_STAT_RETRY or ZEN_STAT_INTERNAL its contents are undefined and the
- * caller clears it.  ZEN_MODE_GENERAL keeps the owner of every probed slot in
+ * again on return (so one allocation serves every call, and no call spends a
+ * kernel on clearing counters: those live in the table too); after a call that
+ * raised ZEN_STAT_RETRY or ZEN_STAT_INTERNAL, or returned an error code, its
+ * contents are undefined and the caller clears it.  ZEN_MODE_GENERAL keeps the owner of every probed slot in
  * it, like the reference; ZEN_MODE_FAST sorts the selected entries by their
  * level-1 slot instead and only borrows a corner of the table as a hash map
  * for the few entries that collide (ZEN_STAT_RETRY if there are too many).
@@ -243,9 +249,11 @@ int zen_load_balance_path(int64_t n, int64_t m, int dtype, int64_t capacity, int
  * encode_sparse_tensor of the first exchange (comm.py:32-50, 125-127) without
  * the dense intermediate.  idx is int32 (idx64_in == 0) or int64.  out_idx is
  * int64 when idx64_out != 0.  out_val is fp32.  *out_count is int64.
- * `mode` is ZEN_MODE_FAST or ZEN_MODE_GENERAL; both give identical results.
+ * `mode` is ZEN_MODE_FAST or ZEN_MODE_GENERAL (both give identical results),
+ * optionally with ZEN_MODE_ZEROED.
  */
 size_t zen_merge_workspace(int64_t r, int64_t dense_n);
+size_t zen_merge_zero_bytes(void); /* see ZEN_MODE_ZEROED; the same for every r and dense_n */
 /* 0 = radix sort (general mode), 1 = one bucket pass + per-range sorts, 2 = bucket slabs; see zen_load_balance_path */
 int zen_merge_path(int64_t r, int64_t dense_n, int mode);
 int zen_merge(const void *idx, int idx64_in, const void *val, int dtype,

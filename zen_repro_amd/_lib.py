@@ -12,9 +12,11 @@ F32, BF16 = 0, 1
 OK, EINVAL, EHIP, EWORKSPACE = 0, -1, -2, -3
 STAT_SERIAL_OVERFLOW, STAT_CAPACITY, STAT_INTERNAL, STAT_BAD_INDEX, STAT_RETRY = 1, 2, 4, 8, 16
 MODE_FAST, MODE_GENERAL = 0, 1
+MODE_ZEROED = 0x100  # zen_merge: the head of the workspace is zero (and stays so)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libzen_hip.so")
+# ZEN_HIP_LIB names another build of the library (a debug build, a build with other compile-time settings)
+LIB_PATH = os.environ.get("ZEN_HIP_LIB") or os.path.join(_HERE, "csrc", "libzen_hip.so")
 
 _lib = None
 
@@ -62,6 +64,7 @@ def lib():
         "zen_load_balance_path": (i32, [i64, i64, i32, i64, i32, i64, i32]),
         "zen_merge_workspace": (sz, [i64, i64]),
         "zen_merge_path": (i32, [i64, i64, i32]),
+        "zen_merge_zero_bytes": (sz, []),
         "zen_merge": (i32, [vp, i32, vp, i32, i64, i64, vp, i32, vp, i64, vp, i32, vp, sz, vp, vp]),
         "zen_decode_dense_workspace": (sz, [i64, i64]),
         "zen_decode_dense": (i32, [vp, i32, vp, i32, i64, vp, i64, i32, vp, sz, vp, vp]),

@@ -152,13 +152,24 @@ class LoadBalanceAllreduce:
         out_val = torch.empty(capacity, dtype=torch.float32, device=dev)
         count = _lib.zeros.take(dev, 1, torch.int64)
         status = _lib.status_word(dev)
-        ws = _lib.scratch.get(dev, f"merge/{slot}", L.zen_merge_workspace(r, dense_size))
+        # The workspace is allocated zeroed and serves zen_merge only, which leaves its head (the counters
+        # that must start at zero) zero again: no call spends a kernel on clearing it.
+        ws = _lib.scratch.get(dev, f"merge/{slot}", L.zen_merge_workspace(r, dense_size), zero=True)
         rc = L.zen_merge(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(values),
                          _lib.dtype_code(values), r, dense_size, _lib.ptr(out_idx), 1 if idx64 else 0,
-                         _lib.ptr(out_val), capacity, _lib.ptr(count), mode, _lib.ptr(ws), ws.numel(),
-                         _lib.ptr(status), _lib.stream_of(dev))
+                         _lib.ptr(out_val), capacity, _lib.ptr(count), mode | _lib.MODE_ZEROED, _lib.ptr(ws),
+                         ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
+        if rc != _lib.OK:
+            ws[:L.zen_merge_zero_bytes()].zero_()
         _lib.check(rc, "merge_sparse")
         return out_idx, out_val, count, status
+
+    def reset_merge_workspace(self, device, slot=0):
+        """After a merge_sparse_flat whose status carried STAT_RETRY or
+        STAT_INTERNAL: clears the head of the slot's workspace again."""
+        L = _lib.lib()
+        ws = _lib.scratch.get(device, f"merge/{slot}", 256, zero=True)
+        ws[:min(ws.numel(), L.zen_merge_zero_bytes())].zero_()
 
     def merge_sparse(self, indices_tensors, values_tensors, dense_size):
         """Synchronising form of merge_sparse_flat: (int64 indices, fp32 sums)."""
@@ -166,6 +177,8 @@ class LoadBalanceAllreduce:
             idx, val, count, status = self.merge_sparse_flat(indices_tensors, values_tensors, dense_size,
                                                              idx64=True, mode=mode)
             host = torch.cat([count, status.to(torch.int64)]).tolist()
+            if host[1] & (_lib.STAT_RETRY | _lib.STAT_INTERNAL):
+                self.reset_merge_workspace(idx.device)
             if not host[1] & _lib.STAT_RETRY:
                 break
         if host[1]:

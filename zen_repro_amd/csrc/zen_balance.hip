@@ -418,8 +418,9 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
     sa.capacity = capacity;
     sa.splits = splits;
     sa.hash = reinterpret_cast<unsigned long long *>(table);
+    // the map takes the head of the table; the megabyte behind it is left to the path's counters
     uint32_t log2 = 0;
-    while (log2 < 24 && (2ull << log2) <= (uint64_t)m / 2) ++log2;
+    while (log2 < 24 && (16ull << log2) + (1ull << 20) <= (uint64_t)m * sizeof(int32_t)) ++log2;
     sa.hash_log2 = log2;
     sa.workspace = workspace;
     sa.status = status;

@@ -222,7 +222,8 @@ constexpr uint64_t kDescPrefix = 2ull << 62;
 constexpr uint64_t kDescValue = (1ull << 62) - 1;
 constexpr uint32_t kSpinLimit = 1u << 22;  // bounded wait: flag ZEN_STAT_INTERNAL instead of hanging
 
-inline size_t scan_words(int64_t ntiles) { return (size_t)ntiles + 2; }
+constexpr size_t scan_words_c(int64_t ntiles) { return (size_t)ntiles + 2; }
+inline size_t scan_words(int64_t ntiles) { return scan_words_c(ntiles); }
 
 struct ScanState {
   unsigned long long *desc;

@@ -146,8 +146,13 @@ __global__ __launch_bounds__(256) void k_scatter_dense<uint16_t>(const int32_t *
 // leave off (every bucket publishes how much it keeps and adds up what the earlier ones published).
 
 constexpr int kMergeTarget = 3072;   // records a bucket is sized for: duplicates make the buckets less even
-constexpr int kMergeItems = 13;      // sorted records per thread while summing (odd: no LDS bank conflicts)
-static_assert(kSlabBlock * kMergeItems >= kSlabCap, "every sorted place needs an owner");
+// Twice the threads of the scatter kernels, half the records each: the kernel's phases are chains of LDS round
+// trips, which eight waves per SIMD hide better than four, and a thread's records then fit 64 registers, so
+// that two workgroups share a compute unit.
+constexpr int kMergeBlock = 1024;
+constexpr int kMergeRecs = kSlabCap / kMergeBlock;  // slab records per thread
+constexpr int kMergeItems = 7;       // sorted records per thread while summing (odd: no LDS bank conflicts)
+static_assert(kMergeBlock * kMergeItems >= kSlabCap, "every sorted place needs an owner");
 
 // An entry travels as (index, arrival number, value bits); in the bucket slabs the three sit in arrays of their
 // own (the value in its own type: ten bytes per bf16 entry).
@@ -191,7 +196,8 @@ struct MergeSink {
 };
 
 template <typename I, typename S>
-__global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const uint32_t *__restrict__ cursor,
+__global__ __launch_bounds__(kMergeBlock, 8) void k_merge_bucket(SlabGeom geo, uint32_t *__restrict__ cursor,
+                                                             uint32_t *__restrict__ coarse_cursor,
                                                              const uint32_t *__restrict__ bucket_lo,
                                                              const uint32_t *__restrict__ slab_idx,
                                                              const uint32_t *__restrict__ slab_arr,
@@ -200,7 +206,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
                                                              int64_t capacity, ScanState st, int tie_bits,
                                                              int64_t *out_count, int32_t *status) {
   __shared__ SlabSortSharedT<true> sh;  // the values take the counters' place once the ranks are known
-  __shared__ uint64_t s_scan64[kSlabBlock / 64 + 1];
+  __shared__ uint64_t s_scan64[kMergeBlock / 64 + 1];
   __shared__ int s_tile;
   if (threadIdx.x == 0) s_tile = (int)atomicAdd(st.ticket, 1u);
   __syncthreads();
@@ -211,27 +217,33 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
   uint32_t n_raw = cursor[b * kCursorPad];
   if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the scatter flagged the overflow
   const uint32_t lo = bucket_lo[b];
-  uint32_t off[kSlabItems], arr[kSlabItems], val[kSlabItems], rank[kSlabItems];
+  // The counters of the scatter kernels go back to zero (this workgroup was the only reader of its slab's
+  // count; the coarse cursors a slice per workgroup), and the last workgroup to finish clears the prefix
+  // state: the memory that must be zero when a call starts is zero again when it ends.
+  if (threadIdx.x == 0) cursor[b * kCursorPad] = 0;
+  for (uint32_t i = (uint32_t)b * kMergeBlock + threadIdx.x; i < kCoarseCursorWords; i += (uint32_t)nb * kMergeBlock)
+    coarse_cursor[i] = 0;
+  uint32_t off[kMergeRecs], arr[kMergeRecs], val[kMergeRecs], rank[kMergeRecs];
   uint32_t live = 0;
+  // the loads sit in no branch (places past the end are pulled back onto the slab's first record), so that
+  // they are all in flight together
 #pragma unroll
-  for (int i = 0; i < kSlabItems; ++i) {
-    const uint32_t j = threadIdx.x + i * kSlabBlock;
-    off[i] = arr[i] = val[i] = 0;
-    if (j < n_raw) {
-      off[i] = slab_idx[base + j] - lo;
-      arr[i] = slab_arr[base + j];
-      val[i] = __float_as_uint(KeyOf<S>::to_f32(slab_val[base + j]));
-      live |= 1u << i;
-    }
+  for (int i = 0; i < kMergeRecs; ++i) {
+    const uint32_t j = threadIdx.x + i * kMergeBlock;
+    const size_t from = base + (j < n_raw ? j : 0u);
+    off[i] = slab_idx[from] - lo;
+    arr[i] = slab_arr[from];
+    val[i] = __float_as_uint(KeyOf<S>::to_f32(slab_val[from]));
+    if (j < n_raw) live |= 1u << i;
   }
   uint32_t n = 0;
-  const bool ranked = slab_rank<kSlabBlock>(sh, geo, tie_bits, off, arr, live, rank, &n);
+  const bool ranked = slab_rank<kMergeBlock>(sh, geo, tie_bits, off, arr, live, rank, &n);
   if (!ranked) {
     if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
     n = 0;  // the bucket contributes nothing; the prefix protocol still gets its (empty) tile
   } else {
 #pragma unroll
-    for (int i = 0; i < kSlabItems; ++i) {
+    for (int i = 0; i < kMergeRecs; ++i) {
       if (live & (1u << i)) {
         sh.key[rank[i]] = off[i];
         sh.tie[rank[i]] = val[i];  // the arrival numbers have done their work: their place takes the values
@@ -239,85 +251,85 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
     }
   }
   __syncthreads();
-  // Thread t owns the sorted places [t * per, (t + 1) * per): as few per thread as cover the bucket, so that
-  // every thread has some (and an odd number, which keeps the lanes of a wave on different LDS banks).  It
-  // walks once from its first
-  // place to the end of the last run that starts in its range, summing every run that starts there in arrival
-  // order from +0 (like the dense tensor of comm.py:35), and leaves each sum in the value word of the run's
-  // head.  (One walk: a loop per run would cost every lane of a wave the longest run of any lane, each time.)
-  // A run's words are read by the thread of its head only, so the sums can be written in place.
-  const uint32_t per = ((n + kSlabBlock - 1) / kSlabBlock) | 1u;  // <= kMergeItems
+  // Thread t owns the sorted places [t * per, (t + 1) * per): as few per thread as cover the bucket (and an odd
+  // number, which keeps the lanes of a wave on different LDS banks).  It fetches them all at once and walks
+  // through them in registers.  A run of equal indices is summed in arrival order from +0 (like the dense
+  // tensor of comm.py:35) and belongs to the thread that holds its last record; where that run began before
+  // the thread's first place (rare: runs are short next to `per`, long ones come from payloads that overlap),
+  // the part in front is summed first, from the run's head on.
+  const uint32_t per = ((n + kMergeBlock - 1) / kMergeBlock) | 1u;  // <= kMergeItems
   const uint32_t first = threadIdx.x * per;
-  if (first < n) {
-    const uint32_t end = first + per < n ? first + per : n;
-    uint32_t cur = first > 0 ? sh.key[first - 1] : 0xffffffffu;  // index of the run the walk is in
-    uint32_t head = 0xffffffffu;                                  // place of its head if it started in the range
-    float acc = 0.0f;
-    for (uint32_t u = first; u < n; ++u) {
-      const uint32_t ku = sh.key[u];
-      if (ku != cur) {
-        if (head != 0xffffffffu) sh.tie[head] = __float_as_uint(acc);
-        if (u >= end) {
-          head = 0xffffffffu;
-          break;
-        }
-        cur = ku;
-        head = u;
-        acc = 0.0f;
-      }
-      if (head != 0xffffffffu) acc += __uint_as_float(sh.tie[u]);
-    }
-    if (head != 0xffffffffu) sh.tie[head] = __float_as_uint(acc);  // the bucket's last run
-  }
-  __syncthreads();
   uint32_t k[kMergeItems];
   float sum[kMergeItems];
   uint32_t keep = 0;
-  uint32_t prev = first > 0 && first <= n ? sh.key[first - 1] : 0xffffffffu;
+  {
+    constexpr uint32_t kNoKey = 0xffffffffu;  // offsets are below the bucket width
+    float v[kMergeItems];
 #pragma unroll
-  for (int q = 0; q < kMergeItems; ++q) {
-    const uint32_t p = first + q;
-    k[q] = 0;
-    sum[q] = 0.0f;
-    if ((uint32_t)q < per && p < n) {
-      k[q] = sh.key[p];
-      const bool is_head = p == 0 || k[q] != prev;
-      prev = k[q];
-      sum[q] = __uint_as_float(sh.tie[p]);
-      if (is_head && sum[q] != 0.0f) keep |= 1u << q;  // torch.nonzero keeps NaN, drops +-0
+    for (int q = 0; q < kMergeItems; ++q) {
+      const uint32_t p = first + q;
+      const bool have = (uint32_t)q < per && p < n;
+      const uint32_t from = have ? p : 0u;
+      k[q] = sh.key[from];
+      v[q] = __uint_as_float(sh.tie[from]);
+      if (!have) k[q] = kNoKey;
+    }
+    const uint32_t before_k = first > 0 && first < n ? sh.key[first - 1] : kNoKey;
+    const uint32_t after_k = first + per < n ? sh.key[first + per] : kNoKey;
+    float acc = 0.0f;
+    if (first < n && before_k == k[0]) {
+      // the run began before this thread's places: find its head, sum up to the place in front of `first`
+      uint32_t head = first - 1;
+      while (head > 0) {
+        const uint32_t a0 = sh.key[head - 1];
+        const uint32_t a1 = sh.key[head >= 2 ? head - 2 : 0u];
+        const uint32_t a2 = sh.key[head >= 3 ? head - 3 : 0u];
+        const uint32_t a3 = sh.key[head >= 4 ? head - 4 : 0u];
+        if (a0 != before_k) break;
+        if (head < 2 || a1 != before_k) { head -= 1; break; }
+        if (head < 3 || a2 != before_k) { head -= 2; break; }
+        if (head < 4 || a3 != before_k) { head -= 3; break; }
+        head -= 4;
+      }
+      for (uint32_t u = head; u < first; u += 4) {
+        const float f0 = __uint_as_float(sh.tie[u]);
+        const float f1 = __uint_as_float(sh.tie[u + 1 < first ? u + 1 : u]);
+        const float f2 = __uint_as_float(sh.tie[u + 2 < first ? u + 2 : u]);
+        const float f3 = __uint_as_float(sh.tie[u + 3 < first ? u + 3 : u]);
+        acc += f0;
+        if (u + 1 < first) acc += f1;
+        if (u + 2 < first) acc += f2;
+        if (u + 3 < first) acc += f3;
+      }
+    }
+    uint32_t prev = before_k;
+#pragma unroll
+    for (int q = 0; q < kMergeItems; ++q) {
+      const uint32_t next = q + 1 < kMergeItems ? ((uint32_t)(q + 1) < per ? k[q + 1] : after_k) : after_k;
+      if (k[q] != kNoKey) {
+        if (k[q] != prev) acc = 0.0f;
+        acc += v[q];
+        prev = k[q];
+        sum[q] = acc;
+        if (k[q] != next && acc != 0.0f) keep |= 1u << q;  // torch.nonzero keeps NaN, drops +-0
+      } else {
+        sum[q] = 0.0f;
+      }
     }
   }
   uint32_t total;
-  const uint32_t before = block_exclusive_scan<uint32_t, kSlabBlock>((uint32_t)__popc(keep), sh.scan, &total);
-  // where this bucket's output starts: the sum of what all earlier buckets keep.  Every thread waits for a
-  // few of them (bounded), nobody waits for a chain of prefixes.
+  const uint32_t before = block_exclusive_scan<uint32_t, kMergeBlock>((uint32_t)__popc(keep), sh.scan, &total);
+  // where this bucket's output starts: the sum of what all earlier buckets keep.  Every thread asks for a
+  // few of them (bounded wait), nobody waits for a chain of prefixes; while the answers are on their way the
+  // kept entries are gathered in LDS (everybody is past reading the sorted bucket: the scan synchronised).
   if (threadIdx.x == 0) desc_store(&st.desc[b], kDescAggregate | total);
-  uint64_t mine = 0;
-  bool gave_up = false;
-  for (int p = (int)threadIdx.x; p < b; p += kSlabBlock) {
-    uint64_t d = desc_load(&st.desc[p]);
-    uint32_t spins = 0;
-    while ((d >> 62) == 0) {
-      if (++spins > kSpinLimit) {
-        gave_up = true;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(2);
-      d = desc_load(&st.desc[p]);
-    }
-    mine += d & kDescValue;
+  constexpr int kAsk = kSlabMaxBuckets / kMergeBlock;
+  uint64_t d[kAsk];
+#pragma unroll
+  for (int e = 0; e < kAsk; ++e) {
+    const int p = (int)threadIdx.x + e * kMergeBlock;
+    d[e] = p < b ? desc_load(&st.desc[p]) : kDescAggregate;
   }
-  if (gave_up) atomicOr(status, ZEN_STAT_INTERNAL);
-  uint64_t all_before;
-  block_exclusive_scan<uint64_t, kSlabBlock>(mine, s_scan64, &all_before);
-  const uint64_t tile_start = all_before;
-  if (b == nb - 1 && threadIdx.x == 0) {
-    const uint64_t all = tile_start + total;
-    *out_count = (int64_t)all;
-    if (all > (uint64_t)capacity) atomicOr(status, ZEN_STAT_CAPACITY);
-  }
-  // gather what is kept in LDS (everybody is past reading the sorted bucket: the scans synchronised), then
-  // write it with consecutive lanes
   uint32_t li = before;
 #pragma unroll
   for (int q = 0; q < kMergeItems; ++q) {
@@ -327,15 +339,59 @@ __global__ __launch_bounds__(kSlabBlock) void k_merge_bucket(SlabGeom geo, const
       ++li;
     }
   }
-  __syncthreads();
-  for (uint32_t i = threadIdx.x; i < total; i += kSlabBlock) {
+  uint64_t mine = 0;
+  bool gave_up = false;
+#pragma unroll
+  for (int e = 0; e < kAsk; ++e) {
+    const int p = (int)threadIdx.x + e * kMergeBlock;
+    uint32_t spins = 0;
+    while ((d[e] >> 62) == 0) {
+      if (++spins > kSpinLimit) {
+        gave_up = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+      d[e] = desc_load(&st.desc[p]);
+    }
+    mine += d[e] & kDescValue;
+  }
+  if (gave_up) atomicOr(status, ZEN_STAT_INTERNAL);
+  uint64_t all_before;
+  block_exclusive_scan<uint64_t, kMergeBlock>(mine, s_scan64, &all_before);  // its barriers also publish the gathered entries
+  const uint64_t tile_start = all_before;
+  if (b == nb - 1 && threadIdx.x == 0) {
+    const uint64_t all = tile_start + total;
+    *out_count = (int64_t)all;
+    if (all > (uint64_t)capacity) atomicOr(status, ZEN_STAT_CAPACITY);
+  }
+  for (uint32_t i = threadIdx.x; i < total; i += kMergeBlock) {
     const uint64_t pos = tile_start + i;
     if (pos < (uint64_t)capacity) {
       out_idx[pos] = (I)sh.key[i];
       out_val[pos] = __uint_as_float(sh.tie[i]);
     }
   }
+  // every workgroup has read the descriptors it needs before it gets here
+  uint32_t *finished = reinterpret_cast<uint32_t *>(st.desc + nb + 1);
+  __syncthreads();
+  if (threadIdx.x == 0) s_tile = atomicAdd(finished, 1u) == (uint32_t)nb - 1u;
+  __syncthreads();
+  if (s_tile) {
+    for (int i = threadIdx.x; i < nb; i += kMergeBlock) st.desc[i] = 0ull;
+    if (threadIdx.x == 0) {
+      *st.ticket = 0;
+      *finished = 0;
+    }
+  }
 }
+
+// Memory that must be zero when a merge starts: the prefix state over the buckets and the scatter kernels'
+// counters, for the largest geometry.  It sits at the head of the workspace whatever path a call takes, and a
+// call on bucket slabs leaves it zero again, so that a caller who vouches for it (ZEN_MODE_ZEROED) saves the
+// kernel that would clear it.
+constexpr size_t kMergeZeroBytes =
+    ((scan_words_c(kSlabMaxBuckets) * sizeof(unsigned long long) + 255) / 256 * 256) +
+    (size_t)kCoarseCursorWords * sizeof(uint32_t) + (size_t)kSlabMaxBuckets * kCursorPad * sizeof(uint32_t);
 
 struct SlabMergePlan {
   unsigned long long *scan;  // prefix state over the buckets (zeroed before use)
@@ -351,11 +407,11 @@ SlabMergePlan plan_slab_merge(void *workspace, const SlabGeom &geo, int64_t r) {
   Carver cv(workspace);
   SlabMergePlan p;
   const size_t B = geo.nbuckets;
-  // what must be zero when the first kernel starts sits together: one fill
   p.scan = cv.take<unsigned long long>(scan_words((int64_t)B));
   p.feed.coarse_cursor = cv.take<uint32_t>(feed_coarse_cursor_words());
   p.feed.cursor = cv.take<uint32_t>(B * kCursorPad);
   p.zero_bytes = cv.used;
+  cv.used = kMergeZeroBytes;  // whatever the geometry, the rest starts behind the largest zero region
   p.feed.bucket_lo = cv.take<uint32_t>(B);
   p.cg = coarse_geometry(geo, r);
   p.feed.coarse_words = cv.take<uint32_t>(feed_coarse_words(p.cg, 3));
@@ -377,10 +433,12 @@ bool slab_merge_fits(int64_t r, int64_t dense_n, SlabGeom *geo) {
 template <typename I, typename S>
 int slab_merge_launch(const SlabGeom &geo, const I *idx, const S *val, int64_t r, int64_t dense_n, void *out_idx,
                       int idx64_out, float *out_val, int64_t capacity, int64_t *out_count, void *workspace,
-                      int32_t *status, hipStream_t s) {
+                      bool zeroed, int32_t *status, hipStream_t s) {
   const SlabMergePlan p = plan_slab_merge(workspace, geo, r);
-  launch_fill<unsigned long long>(p.scan, 0ull, p.zero_bytes / sizeof(unsigned long long), s);
-  ZEN_LAUNCH_CHECK("merge: clear prefix state");
+  if (!zeroed) {
+    launch_fill<unsigned long long>(p.scan, 0ull, p.zero_bytes / sizeof(unsigned long long), s);
+    ZEN_LAUNCH_CHECK("merge: clear prefix state");
+  }
   {
     ProfScope prof(kProfMergeFeed, s);
     const MergeSrc<I, S> src{geo, idx, val, (uint32_t)dense_n, status};
@@ -392,13 +450,15 @@ int slab_merge_launch(const SlabGeom &geo, const I *idx, const S *val, int64_t r
   const int tie_bits = ceil_log2_u64((uint64_t)r);  // arrival numbers are < r
   ProfScope prof(kProfMergeBucket, s);
   if (idx64_out)
-    k_merge_bucket<int64_t, S><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
-        geo, p.feed.cursor, p.feed.bucket_lo, p.slab_idx, p.slab_arr, static_cast<const S *>(p.slab_val),
-        static_cast<int64_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
+    k_merge_bucket<int64_t, S><<<dim3(geo.nbuckets), dim3(kMergeBlock), 0, s>>>(
+        geo, p.feed.cursor, p.feed.coarse_cursor, p.feed.bucket_lo, p.slab_idx, p.slab_arr,
+        static_cast<const S *>(p.slab_val), static_cast<int64_t *>(out_idx), out_val, capacity, st, tie_bits, out_count,
+        status);
   else
-    k_merge_bucket<int32_t, S><<<dim3(geo.nbuckets), dim3(kSlabBlock), 0, s>>>(
-        geo, p.feed.cursor, p.feed.bucket_lo, p.slab_idx, p.slab_arr, static_cast<const S *>(p.slab_val),
-        static_cast<int32_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
+    k_merge_bucket<int32_t, S><<<dim3(geo.nbuckets), dim3(kMergeBlock), 0, s>>>(
+        geo, p.feed.cursor, p.feed.coarse_cursor, p.feed.bucket_lo, p.slab_idx, p.slab_arr,
+        static_cast<const S *>(p.slab_val), static_cast<int32_t *>(out_idx), out_val, capacity, st, tie_bits, out_count,
+        status);
   ZEN_LAUNCH_CHECK("k_merge_bucket");
   return ZEN_OK;
 }
@@ -413,6 +473,7 @@ struct MergePlan {
 
 MergePlan plan_merge(void *workspace, int64_t r, int64_t dense_n) {
   Carver cv(workspace);
+  cv.used = kMergeZeroBytes;  // the head of the workspace belongs to the bucket-slab path's counters
   MergePlan p;
   const size_t cap = (size_t)(r > 0 ? r : 1);
   p.keys = cv.take<uint32_t>(cap);
@@ -435,13 +496,15 @@ template <typename S>
 int merge_launch(const void *idx, int idx64_in, const S *val, int64_t r, int64_t dense_n, void *out_idx,
                  int idx64_out, float *out_val, int64_t capacity, int64_t *out_count, int mode, void *workspace,
                  int32_t *status, hipStream_t s) {
+  const bool zeroed = (mode & ZEN_MODE_ZEROED) != 0;
+  mode &= ~ZEN_MODE_ZEROED;
   SlabGeom geo;
   if (mode == ZEN_MODE_FAST && slab_merge_fits(r, dense_n, &geo)) {
     if (idx64_in)
       return slab_merge_launch(geo, static_cast<const int64_t *>(idx), val, r, dense_n, out_idx, idx64_out, out_val,
-                               capacity, out_count, workspace, status, s);
+                               capacity, out_count, workspace, zeroed, status, s);
     return slab_merge_launch(geo, static_cast<const int32_t *>(idx), val, r, dense_n, out_idx, idx64_out, out_val,
-                             capacity, out_count, workspace, status, s);
+                             capacity, out_count, workspace, zeroed, status, s);
   }
   MergePlan p = plan_merge(workspace, r, dense_n);
   const unsigned blocks = (unsigned)ceil_div(r, 256);
@@ -488,7 +551,10 @@ int merge_launch(const void *idx, int idx64_in, const S *val, int64_t r, int64_t
 
 int merge_check(const void *idx, const void *val, int dtype, int64_t r, int64_t dense_n, int mode, const char **why) {
   if (dtype != ZEN_F32 && dtype != ZEN_BF16) { *why = "bad dtype"; return ZEN_EINVAL; }
-  if (mode != ZEN_MODE_FAST && mode != ZEN_MODE_GENERAL) { *why = "bad mode"; return ZEN_EINVAL; }
+  if ((mode & ~ZEN_MODE_ZEROED) != ZEN_MODE_FAST && (mode & ~ZEN_MODE_ZEROED) != ZEN_MODE_GENERAL) {
+    *why = "bad mode";
+    return ZEN_EINVAL;
+  }
   if (r < 0 || r > 0x7ffffffell || dense_n <= 0 || dense_n > 0x7fffffffll) {
     *why = "need 0 <= r < 2^31 - 1 and 0 < dense_n < 2^31";
     return ZEN_EINVAL;
@@ -507,7 +573,10 @@ size_t zen_merge_workspace(int64_t r, int64_t dense_n) {
   return zen::plan_merge(nullptr, r, dense_n).bytes;
 }
 
+size_t zen_merge_zero_bytes(void) { return zen::kMergeZeroBytes; }
+
 int zen_merge_path(int64_t r, int64_t dense_n, int mode) {
+  mode &= ~ZEN_MODE_ZEROED;
   if (mode != ZEN_MODE_FAST || r <= 0 || dense_n <= 0) return 0;
   if (zen::slab_merge_fits(r, dense_n, nullptr)) return 2;
   return zen::bucket_sort_fits(r, (uint32_t)dense_n) ? 1 : 0;
@@ -566,11 +635,11 @@ int zen_decode_dense(const void *idx, int idx64_in, const void *val, int dtype, 
   void *inner = cv.take<char>(zen_merge_workspace(r, dense_n));
   int rc;
   if (dtype == ZEN_BF16)
-    rc = merge_launch(idx, idx64_in, static_cast<const uint16_t *>(val), r, dense_n, m_idx, 0, m_val, r, m_count, mode,
-                      inner, status, s);
+    rc = merge_launch(idx, idx64_in, static_cast<const uint16_t *>(val), r, dense_n, m_idx, 0, m_val, r, m_count,
+                      mode & ~ZEN_MODE_ZEROED, inner, status, s);
   else
-    rc = merge_launch(idx, idx64_in, static_cast<const uint32_t *>(val), r, dense_n, m_idx, 0, m_val, r, m_count, mode,
-                      inner, status, s);
+    rc = merge_launch(idx, idx64_in, static_cast<const uint32_t *>(val), r, dense_n, m_idx, 0, m_val, r, m_count,
+                      mode & ~ZEN_MODE_ZEROED, inner, status, s);
   if (rc != ZEN_OK) return rc;
   const unsigned blocks = (unsigned)ceil_div(r, 256);
   if (dtype == ZEN_BF16)

@@ -241,6 +241,9 @@ __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restric
   __syncthreads();
   if (!s_last) return;
   sample_pick_block(hist, rank, kShift, floor_out, smem);
+  // the histogram is left as it was found, all zero: a caller that keeps it between calls need not clear it
+  __syncthreads();
+  for (int i = threadIdx.x; i < kFineBins + 2; i += kSampleBlock) hist[i] = 0;
 }
 
 // Run by one whole block (BLOCK threads) over the complete candidate
@@ -1071,6 +1074,8 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
         __syncthreads();
         if (thr_copy && threadIdx.x < 2)
           thr_copy[threadIdx.x] = __hip_atomic_load(&pick_thr[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // the histogram and its count of finished workgroups are left all zero, as they were found
+        for (int i = threadIdx.x; i < kCandHistWords; i += kSelBlock) cand_hist[i] = 0;
       }
     }
   }

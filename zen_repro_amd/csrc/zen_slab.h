@@ -156,40 +156,55 @@ struct SlabSortSharedT<true> {
   };
   uint32_t scan[kSlabMaxBlock / 64 + 1];
   uint32_t bad;
-  uint32_t queued;
 };
 
 static_assert(kSlabSubs + 1 <= kSlabCap, "the counters fit under the ties");
 using SlabSortShared = SlabSortSharedT<false>;
 
+// Number of words in sh.key[b0, b1) that are smaller than w.  The words are fetched four at a time (places past
+// the end are pulled back onto the last word and not counted): a loop that fetches one word per turn waits
+// for LDS once per word, and that wait is what such a loop spends its time on.
+template <typename Shared>
+__device__ inline uint32_t slab_count_less(const Shared &sh, uint32_t b0, uint32_t b1, uint32_t w) {
+  uint32_t less = 0;
+  const uint32_t last = b1 - 1u;
+  for (uint32_t u = b0; u < b1; u += 4) {
+    const uint32_t a0 = sh.key[u];
+    const uint32_t a1 = sh.key[u + 1 < last ? u + 1 : last];
+    const uint32_t a2 = sh.key[u + 2 < last ? u + 2 : last];
+    const uint32_t a3 = sh.key[u + 3 < last ? u + 3 : last];
+    less += (a0 < w) + (u + 1 < b1 && a1 < w) + (u + 2 < b1 && a2 < w) + (u + 3 < b1 && a3 < w);
+  }
+  return less;
+}
+
 // Ranks the live records of a workgroup of BLOCK threads (kSlabCap / BLOCK records each) by (key offset, tie);
 // tie < 2^tie_bits, the pair unique, and
 // geo.sub_shift + tie_bits <= 32.  off[i] < bucket width.  The records are first grouped by narrow key range
 // with one LDS atomic each; a record is then one word, (offset inside the range) << tie_bits | tie, and
-// inside its group every record counts the words smaller than its own.  Where many records share a key (a
-// merge of payloads that overlap) every wave has, for each of its threads' records in turn, a few lanes that
-// walk through a group of dozens while the others wait, and the LDS instructions of all those half-empty
-// rounds are what the workgroup then spends its time on: with a Shared that has a queue, records of groups
-// larger than kSlabInline are set aside instead and handed out again afterwards, one per lane, so that the
-// lanes of a wave walk through large groups together.  Returns false (for every thread) if a
+// inside its group every record counts the words smaller than its own: the first kSlabInline words of every
+// record's group are fetched in one go (all of them in flight together), which settles groups up to that size.
+// Where many records share a key (a merge of payloads that overlap) a few lanes of every wave would then walk
+// through groups of dozens while the others wait: with a Shared that has a queue, records of groups larger
+// than kSlabInline are set aside instead (their places in the queue follow from the same prefix sums as the
+// groups' places: the counters carry both, 16 bits each) and handed out again afterwards, one per lane, so
+// that the lanes of a wave walk through large groups together.  Returns false (for every thread) if a
 // group is too large for that; else rank[i] for live records and *n_out = number of live records.  On return
-// sh.key / sh.tie may be overwritten at once (sh.tie is not touched at all).
+// sh.key / sh.tie may be overwritten at once (sh.tie is not touched at all), and the low 16 bits of
+// sh.cnt[sub_place(s)] hold the sorted place of the first record of narrow range s.
 template <int BLOCK, typename Shared>
 __device__ inline bool slab_rank(Shared &sh, const SlabGeom &geo, int tie_bits,
                                  const uint32_t (&off)[kSlabCap / BLOCK], const uint32_t (&tie)[kSlabCap / BLOCK],
                                  uint32_t live, uint32_t (&rank)[kSlabCap / BLOCK], uint32_t *n_out) {
   static_assert(BLOCK <= kSlabMaxBlock && kSlabCap % BLOCK == 0 && kSlabSubs % BLOCK == 0, "workgroup size");
+  static_assert(kSlabCap < 65536, "two prefixes in one word");
   constexpr int kItems = kSlabCap / BLOCK;
   constexpr int kSubsPer = kSlabSubs / BLOCK;
   for (int d = threadIdx.x; d <= kSlabSubs; d += BLOCK) sh.cnt[d] = 0;
-  if (threadIdx.x == 0) {
-    sh.bad = 0;
-    if constexpr (Shared::kQueue) sh.queued = 0;
-  }
+  if (threadIdx.x == 0) sh.bad = 0;
   __syncthreads();
   const uint32_t low_mask = (1u << geo.sub_shift) - 1u;
   uint32_t sub[kItems], at[kItems];
-  uint32_t in_large = 0;  // records in groups larger than kSlabInline
 #pragma unroll
   for (int i = 0; i < kItems; ++i) {
     sub[i] = at[i] = 0;
@@ -202,7 +217,6 @@ __device__ inline bool slab_rank(Shared &sh, const SlabGeom &geo, int tie_bits,
   {
     uint32_t c[kSubsPer];
     uint32_t sum = 0, big = 0;  // sum: records in the low half, records of groups larger than kSlabInline in the high half
-    static_assert(kSlabCap < 65536, "two counts in one word");
 #pragma unroll
     for (int e = 0; e < kSubsPer; ++e) {
       c[e] = sh.cnt[e * BLOCK + threadIdx.x];
@@ -211,91 +225,91 @@ __device__ inline bool slab_rank(Shared &sh, const SlabGeom &geo, int tie_bits,
     }
     if (big) sh.bad = 1;
     uint32_t total;
-    uint32_t running = block_exclusive_scan<uint32_t, BLOCK>(sum, sh.scan, &total) & 0xffffu;
-    in_large = total >> 16;
+    uint32_t running = block_exclusive_scan<uint32_t, BLOCK>(sum, sh.scan, &total);
 #pragma unroll
     for (int e = 0; e < kSubsPer; ++e) {
       sh.cnt[e * BLOCK + threadIdx.x] = running;
-      running += c[e];
+      running += c[e] + (c[e] > (uint32_t)kSlabInline ? c[e] << 16 : 0u);
     }
-    if (threadIdx.x == BLOCK - 1) sh.cnt[kSlabSubs] = running;
+    if (threadIdx.x == BLOCK - 1) sh.cnt[kSlabSubs] = running;  // = total
   }
   __syncthreads();
   if (sh.bad) return false;
-  uint32_t g0[kItems], word[kItems];
+  const uint32_t totals = sh.cnt[kSlabSubs];
+  // a few large groups are not worth the extra barrier
+  const bool set_aside = Shared::kQueue && (totals >> 16) >= (uint32_t)kSlabQueueMin;
+  constexpr uint32_t kSetAside = 0x80000000u;
+  uint32_t g0[kItems], g1[kItems], word[kItems];
 #pragma unroll
   for (int i = 0; i < kItems; ++i) {
-    g0[i] = word[i] = 0;
+    g0[i] = g1[i] = word[i] = rank[i] = 0;
     if (live & (1u << i)) {
-      g0[i] = sh.cnt[sub_place<BLOCK>(sub[i])];
+      const uint32_t here = sh.cnt[sub_place<BLOCK>(sub[i])];
+      g0[i] = here & 0xffffu;
+      g1[i] = sh.cnt[sub_place<BLOCK>(sub[i] + 1)] & 0xffffu;
       word[i] = ((off[i] & low_mask) << tie_bits) | tie[i];
       sh.key[g0[i] + at[i]] = word[i];
-    }
-  }
-  __syncthreads();
-  constexpr uint32_t kSetAside = 0x80000000u;
-  uint32_t g1[kItems];
-#pragma unroll
-  for (int i = 0; i < kItems; ++i) {
-    rank[i] = 0;
-    g1[i] = (live & (1u << i)) ? sh.cnt[sub_place<BLOCK>(sub[i] + 1)] : g0[i];
-  }
-  // a few large groups are not worth the two extra barriers
-  const bool set_aside = Shared::kQueue && in_large >= (uint32_t)kSlabQueueMin;
-  if constexpr (Shared::kQueue) {
-    // records of large groups are set aside: one LDS atomic per wave and round, not per lane (they would all
-    // meet on the one counter)
-    if (set_aside) {
-#pragma unroll
-      for (int i = 0; i < kItems; ++i) {
-        if (g1[i] - g0[i] > (uint32_t)kSlabInline) {
-          const uint64_t peers = __ballot(1);
-          const uint32_t before = (uint32_t)__popcll(peers & ((1ull << (threadIdx.x & 63u)) - 1ull));
-          uint32_t q = 0;
-          if (before == 0) q = atomicAdd(&sh.queued, (uint32_t)__popcll(peers));
-          q = (uint32_t)__shfl((int)q, (int)__ffsll((long long)peers) - 1) + before;
-          if (q < (uint32_t)kSlabQueueCap) {
-            sh.queue[q] = sub[i] | (at[i] << 12);  // sub < 2^12, at < group size <= kSlabGroupLimit
-            rank[i] = kSetAside | q;
-            g1[i] = g0[i];  // nothing left to do for it below
-          }
+      if constexpr (Shared::kQueue) {
+        static_assert(kSlabSubs <= (1 << 12) && kSlabGroupLimit <= (1 << 19), "a queue entry is one word");
+        const uint32_t q = (here >> 16) + at[i];
+        if (set_aside && g1[i] - g0[i] > (uint32_t)kSlabInline && q < (uint32_t)kSlabQueueCap) {
+          sh.queue[q] = sub[i] | (at[i] << 12);  // sub < 2^12, at < group size <= kSlabGroupLimit
+          rank[i] = kSetAside | q;
+          g1[i] = g0[i];  // nothing left to do for it below
         }
       }
     }
   }
+  __syncthreads();
+  // the first kRankAhead words of every record's group, those of kBatch records fetched before any is looked
+  // at (most groups are no larger); the rest of a group one word per turn, or four where it is large
+#ifndef ZEN_RANK_AHEAD
+#define ZEN_RANK_AHEAD 2
+#endif
+  constexpr int kRankAhead = ZEN_RANK_AHEAD;
+  constexpr int kBatch = kItems % 3 == 0 ? 3 : kItems;
 #pragma unroll
-  for (int i = 0; i < kItems; ++i) {
-    if (g1[i] > g0[i]) {
-      uint32_t less = 0;
-      for (uint32_t u = g0[i]; u < g1[i]; ++u) less += sh.key[u] < word[i];
-      rank[i] = g0[i] + less;
+  for (int h = 0; h < kItems; h += kBatch) {
+    uint32_t a[kBatch][kRankAhead];
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      const uint32_t last = g1[h + i] > g0[h + i] ? g1[h + i] - 1u : g0[h + i];
+#pragma unroll
+      for (int j = 0; j < kRankAhead; ++j) a[i][j] = sh.key[g0[h + i] + j < last ? g0[h + i] + j : last];
+    }
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      if (g1[h + i] > g0[h + i]) {
+        uint32_t less = 0;
+#pragma unroll
+        for (int j = 0; j < kRankAhead; ++j) less += g0[h + i] + j < g1[h + i] && a[i][j] < word[h + i];
+        const uint32_t size = g1[h + i] - g0[h + i];
+        if (size > (uint32_t)kSlabInline)
+          less += slab_count_less(sh, g0[h + i] + kRankAhead, g1[h + i], word[h + i]);
+        else
+          for (uint32_t u = g0[h + i] + kRankAhead; u < g1[h + i]; ++u) less += sh.key[u] < word[h + i];
+        rank[h + i] = g0[h + i] + less;
+      }
     }
   }
   if constexpr (Shared::kQueue) {
-    static_assert(kSlabSubs <= (1 << 12) && kSlabGroupLimit <= (1 << 19), "a queue entry is one word");
-    if (!set_aside) {
-      *n_out = sh.cnt[kSlabSubs];
-      __syncthreads();
-      return true;
-    }
-    __syncthreads();
-    const uint32_t queued = sh.queued < (uint32_t)kSlabQueueCap ? sh.queued : (uint32_t)kSlabQueueCap;
-    // the thread that takes a queue entry also overwrites it with the rank
+    if (set_aside) {
+      const uint32_t queued = (totals >> 16) < (uint32_t)kSlabQueueCap ? (totals >> 16) : (uint32_t)kSlabQueueCap;
+      // the thread that takes a queue entry also overwrites it with the rank
 #pragma unroll 1
-    for (uint32_t q = threadIdx.x; q < queued; q += BLOCK) {
-      const uint32_t e = sh.queue[q];
-      const uint32_t b0 = sh.cnt[sub_place<BLOCK>(e & 4095u)], b1 = sh.cnt[sub_place<BLOCK>((e & 4095u) + 1)];
-      const uint32_t w = sh.key[b0 + (e >> 12)];
-      uint32_t less = 0;
-      for (uint32_t u = b0; u < b1; ++u) less += sh.key[u] < w;
-      sh.queue[q] = b0 + less;
-    }
-    __syncthreads();
+      for (uint32_t q = threadIdx.x; q < queued; q += BLOCK) {
+        const uint32_t e = sh.queue[q];
+        const uint32_t b0 = sh.cnt[sub_place<BLOCK>(e & 4095u)] & 0xffffu;
+        const uint32_t b1 = sh.cnt[sub_place<BLOCK>((e & 4095u) + 1)] & 0xffffu;
+        sh.queue[q] = b0 + slab_count_less(sh, b0, b1, sh.key[b0 + (e >> 12)]);
+      }
+      __syncthreads();
 #pragma unroll
-    for (int i = 0; i < kItems; ++i)
-      if (rank[i] & kSetAside) rank[i] = sh.queue[rank[i] & ~kSetAside];
+      for (int i = 0; i < kItems; ++i)
+        if (rank[i] & kSetAside) rank[i] = sh.queue[rank[i] & ~kSetAside];
+    }
   }
-  *n_out = sh.cnt[kSlabSubs];
+  *n_out = totals & 0xffffu;
   __syncthreads();
   return true;
 }

@@ -48,10 +48,17 @@ struct SlabTables {
   uint32_t *ser_idx;    // [P * kSlabSerialCap]
   uint32_t *log_t, *log_v, *log_cell;  // [log_cap]
   uint32_t *out_start;  // [B + 1] where every bucket starts in the output
-  uint32_t *done;       // [1] workgroups of k_slab_classify that have finished
+  uint32_t *done;       // [2] workgroups of k_slab_classify / of k_slab_place that have finished
   Counters *ctr;
+  uint32_t *coarse_cursor;  // the feed's coarse cursors and, for an fp32 top-k, the refinement histogram (else
+  uint32_t *refine_hist;    // null): k_slab_sort puts them back to zero
+  int partitions;
   uint32_t log_cap;
 };
+
+// The counters and histograms that must be zero when a call starts live in memory that is zero between calls
+// (the part of the caller's table the hash map does not use), and every one of them is put back to zero by the
+// last kernel that needs it: no kernel spends its time clearing them up front.
 
 // Every kSlabIndexStep-th narrow key range of a bucket (zen_slab.h; about one record per range) has its first
 // sorted place written down by the sort kernel: whoever asks who owns a level-1 slot reads two of these places
@@ -164,7 +171,7 @@ constexpr int kSortBlock = 1024;
 constexpr int kSortItems = kSlabCap / kSortBlock;
 
 template <typename S>
-__global__ __launch_bounds__(kSortBlock, 2) void k_slab_sort(SlabGeom geo, SlabTables tb, int32_t *status) {
+__global__ __launch_bounds__(kSortBlock, 8) void k_slab_sort(SlabGeom geo, SlabTables tb, int32_t *status) {
   __shared__ SlabSortShared sh;
   __shared__ S s_val[kSlabCap];
   __shared__ uint32_t s_lost, s_base;
@@ -174,18 +181,29 @@ __global__ __launch_bounds__(kSortBlock, 2) void k_slab_sort(SlabGeom geo, SlabT
   if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the scatter flagged the overflow
   const uint32_t lo = tb.bucket_lo[b];
   S *slab_val = static_cast<S *>(tb.slab_val);
-  if (threadIdx.x == 0) s_lost = 0;
+  if (threadIdx.x == 0) {
+    s_lost = 0;
+    tb.cursor[b * kCursorPad] = 0;  // this workgroup was its only reader
+  }
+  // the kernels before this one were the last to need these: back to zero, a slice per workgroup
+  for (uint32_t i = b * kSortBlock + threadIdx.x; i < kCoarseCursorWords; i += gridDim.x * kSortBlock)
+    tb.coarse_cursor[i] = 0;
+  if (tb.refine_hist)
+    for (uint32_t i = b * kSortBlock + threadIdx.x; i <= (uint32_t)kRefineBins; i += gridDim.x * kSortBlock)
+      tb.refine_hist[i] = 0;
   uint32_t off[kSortItems], idx[kSortItems], pos[kSortItems], rank[kSortItems];
   S val[kSortItems];
   uint32_t live = 0;
 #pragma unroll
   for (int i = 0; i < kSortItems; ++i) {
     const uint32_t j = threadIdx.x + i * kSortBlock;
-    off[i] = idx[i] = pos[i] = 0;
-    val[i] = 0;
+    // no branch around the loads (places past the end are pulled back onto the slab's first record): they are
+    // all in flight together
+    const size_t from = base + (j < n_raw ? j : 0u);
+    idx[i] = tb.raw_idx[from];
+    val[i] = static_cast<const S *>(tb.raw_val)[from];
+    off[i] = pos[i] = 0;
     if (j < n_raw) {
-      idx[i] = tb.raw_idx[base + j];
-      val[i] = static_cast<const S *>(tb.raw_val)[base + j];
       off[i] = geo.mod_m(poly(idx[i]) + kSeed1) - lo;  // the level-1 slot again: cheaper than carrying it along
       pos[i] = j;
       live |= 1u << i;
@@ -515,6 +533,21 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
   const uint32_t n = tb.bucket_n[b];
   uint32_t mv_n = tb.movein_n[b];
   if (mv_n > (uint32_t)kSlabMoveCap) mv_n = kSlabMoveCap;
+  // Called by every thread of the workgroup on its way out: the counters every workgroup of this kernel reads
+  // go back to zero once the last workgroup has read them (its own count of moved-in entries right away).
+  auto finish = [&]() {
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      tb.movein_n[b] = 0;
+      s_nrm = atomicAdd(&tb.done[1], 1u) == B - 1u;
+    }
+    __syncthreads();
+    if (s_nrm) {
+      for (int i = threadIdx.x; i < tb.partitions; i += kSlabBlock) tb.serial_n[i] = 0;
+      if (threadIdx.x < sizeof(Counters) / sizeof(uint32_t)) reinterpret_cast<uint32_t *>(tb.ctr)[threadIdx.x] = 0;
+      if (threadIdx.x < 2) tb.done[threadIdx.x] = 0;
+    }
+  };
   // the thread's entries (sorted places threadIdx.x + i * kSlabBlock) stay in registers; the slots go to LDS
   // for the searches, the places of removed entries are collected
   uint32_t idx[kSlabItems];
@@ -544,6 +577,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
   uint32_t rm_n = s_nrm;
   if (rm_n > (uint32_t)kPlaceRemoved) {  // more collisions than this path carries
     if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
+    finish();
     return;
   }
   if (rm_n > 1) sort_small(s_rm, rm_n);
@@ -642,6 +676,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
     if (hi > capacity) atomicOr(status, ZEN_STAT_CAPACITY);
   }
   (void)partitions;
+  finish();
 }
 
 struct SlabPlan {
@@ -652,38 +687,39 @@ struct SlabPlan {
   CoarseGeom cg;
   FeedBuffers feed;
   uint32_t *thr;          // [0..1] exact threshold + count, [2..3] sampled floor, [4] candidates above the k-th's bin
-  uint32_t *refine_hist;  // fp32: histogram of the threshold's last 16 bits (+ finished-workgroup count), last in
-                          // the zero region and cleared only for a top-k call
-  void *zero_begin;
-  size_t zero_bytes;
-  size_t zero_bytes_topk;
-  size_t bytes;
+  uint32_t *refine_hist;  // fp32: histogram of the threshold's last 16 bits (+ finished-workgroup count)
+  size_t state_bytes;     // of the zero-between-calls memory
+  size_t bytes;           // of the workspace
 };
 
-SlabPlan plan_slab(void *workspace, const SlabGeom &geo, int partitions, int dtype, int64_t list_cap) {
-  Carver cv(workspace);
+// `state` is memory that is zero between calls (see above); everything else comes out of the workspace.
+SlabPlan plan_slab(void *workspace, void *state, const SlabGeom &geo, int partitions, int dtype, int64_t list_cap) {
   SlabPlan p;
   const size_t B = geo.nbuckets;
-  // everything that must be zero when the first kernel starts sits together: one fill
-  p.zero_begin = cv.base + cv.used;
-  p.sample_hist = cv.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
-  p.cand_hist = cv.take<uint32_t>((size_t)kCandHistWords);
-  p.ticket = cv.take<uint32_t>(select_stage_ticket_words());
-  p.tb.cursor = cv.take<uint32_t>(B * kCursorPad);
-  p.feed.coarse_cursor = cv.take<uint32_t>(feed_coarse_cursor_words());
-  p.tb.movein_n = cv.take<uint32_t>(B);
-  p.tb.serial_n = cv.take<uint32_t>((size_t)partitions);
-  p.tb.ctr = cv.take<Counters>(1);
-  p.tb.done = cv.take<uint32_t>(1);
-  p.zero_bytes = (size_t)(cv.base + cv.used - static_cast<char *>(p.zero_begin));
-  p.refine_hist = cv.take<uint32_t>(dtype == ZEN_BF16 ? 1 : (size_t)kRefineBins + 1);
-  p.zero_bytes_topk = (size_t)(cv.base + cv.used - static_cast<char *>(p.zero_begin));
+  {
+    Carver cv(state);
+    p.sample_hist = cv.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
+    p.cand_hist = cv.take<uint32_t>((size_t)kCandHistWords);
+    p.ticket = cv.take<uint32_t>(select_stage_ticket_words());
+    p.tb.cursor = cv.take<uint32_t>(B * kCursorPad);
+    p.feed.coarse_cursor = cv.take<uint32_t>(feed_coarse_cursor_words());
+    p.tb.movein_n = cv.take<uint32_t>(B);
+    p.tb.serial_n = cv.take<uint32_t>((size_t)partitions);
+    p.tb.ctr = cv.take<Counters>(1);
+    p.tb.done = cv.take<uint32_t>(2);
+    p.refine_hist = cv.take<uint32_t>(dtype == ZEN_BF16 ? 1 : (size_t)kRefineBins + 1);
+    p.state_bytes = cv.used;
+  }
+  Carver cv(workspace);
   p.thr = cv.take<uint32_t>(8);
   p.cg = coarse_geometry(geo, list_cap);
   p.feed.coarse_words = cv.take<uint32_t>(feed_coarse_words(p.cg, 2));
   p.tb.bucket_lo = cv.take<uint32_t>(B);
   p.feed.cursor = p.tb.cursor;
   p.feed.bucket_lo = p.tb.bucket_lo;
+  p.tb.coarse_cursor = p.feed.coarse_cursor;
+  p.tb.refine_hist = nullptr;
+  p.tb.partitions = partitions;
   p.tb.out_start = cv.take<uint32_t>(B + 1);
   p.tb.bucket_n = cv.take<uint32_t>(B);
   p.tb.removed_n = cv.take<uint32_t>(B);
@@ -712,7 +748,7 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
   {
     ProfScope prof(kProfFeed, s);
     const EncodeSink<S> sink{geo, p.tb.raw_idx, static_cast<S *>(p.tb.raw_val), filter};
-    const int rc = feed_fine<2, S>(geo, p.cg, sink, p.feed, a.status, s);
+    const int rc = feed_fine<2, S>(geo, p.cg, sink, p.feed, a.status, s, p.ticket, (uint32_t)select_stage_ticket_words());
     if (rc != ZEN_OK) return rc;
   }
   {
@@ -739,31 +775,38 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
 
 }  // namespace
 
+size_t slab_balance_bytes(int64_t m, int partitions, int dtype, int64_t capacity) {
+  SlabGeom geo;
+  if (!slab_geometry(m, partitions, capacity, kSlabTarget, &geo)) return 0;
+  return plan_slab(nullptr, nullptr, geo, partitions, dtype, list_capacity(capacity)).bytes;
+}
+
+// The hash map takes the first 8 << hash_log2 bytes of the caller's table (at most half of it: zen_load_balance
+// sizes the map so); the counters sit behind it.
+static size_t slab_state_offset(uint32_t hash_log2) { return align_up((size_t)8 << hash_log2, 256); }
+
 bool slab_balance_fits(int64_t n, int64_t m, int partitions, int dtype, int64_t capacity, int64_t k, SlabGeom *geo) {
   (void)n;
   (void)k;
   if (capacity > 0x1fffffffll) return false;
   SlabGeom g;
   if (!slab_geometry(m, partitions, capacity, kSlabTarget, &g)) return false;
+  // slab_geometry wants m >= 2^22: a table of 16 MB or more, of which the map takes at most half and the
+  // counters less than 1 MB
   if (geo) *geo = g;
   return true;
-}
-
-size_t slab_balance_bytes(int64_t m, int partitions, int dtype, int64_t capacity) {
-  SlabGeom geo;
-  if (!slab_geometry(m, partitions, capacity, kSlabTarget, &geo)) return 0;
-  return plan_slab(nullptr, geo, partitions, dtype, list_capacity(capacity)).bytes;
 }
 
 int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
   SlabGeom geo;
   if (!slab_balance_fits(a.n, a.g.m, a.partitions, a.dtype, a.capacity, a.k, &geo))
     return fail(ZEN_EINVAL, "slab_load_balance: sizes do not suit the slab layout");
-  const SlabPlan p = plan_slab(a.workspace, geo, a.partitions, a.dtype, list_capacity(a.capacity));
+  char *state = reinterpret_cast<char *>(a.hash) + slab_state_offset(a.hash_log2);
+  SlabPlan p = plan_slab(a.workspace, state, geo, a.partitions, a.dtype, list_capacity(a.capacity));
+  if (slab_state_offset(a.hash_log2) + p.state_bytes > (size_t)a.g.m * sizeof(int32_t))
+    return fail(ZEN_EINVAL, "slab_load_balance: table too small for the counters");
   const bool refine = a.k > 0 && a.dtype == ZEN_F32;
-  launch_fill<uint32_t>(static_cast<uint32_t *>(p.zero_begin), 0u,
-                        (refine ? p.zero_bytes_topk : p.zero_bytes) / sizeof(uint32_t), s);
-  ZEN_LAUNCH_CHECK("slab: clear counters");
+  if (refine) p.tb.refine_hist = p.refine_hist;
   StageArgs sc;
   sc.in = a.input;
   sc.dtype = a.dtype;

@@ -66,12 +66,15 @@ inline uint32_t feed_batches(int64_t entries) { return (uint32_t)ceil_div(entrie
 
 // Workspace of the two steps.
 struct FeedBuffers {
-  uint32_t *coarse_cursor;  // [feed_coarse_cursor_words()], zero before the first step
+  uint32_t *coarse_cursor;  // [feed_coarse_cursor_words()], zero before the first step (the consumer of the
+                            // bucket slabs puts it back to zero)
   uint32_t *coarse_words;   // [W][groups * kCoarseSplit * cap]; the last plane holds Src::Last, not words
   uint32_t *cursor;         // [nbuckets * kCursorPad], zero before the second step; ends as the slab fill counts
+                            // (the consumer of a slab puts its count back to zero)
   uint32_t *bucket_lo;      // [nbuckets] smallest key of every bucket (written by the second step)
 };
-inline size_t feed_coarse_cursor_words() { return (size_t)kCoarseMax * kCoarseSplit * kCoarsePad; }
+constexpr uint32_t kCoarseCursorWords = kCoarseMax * kCoarseSplit * kCoarsePad;
+inline size_t feed_coarse_cursor_words() { return kCoarseCursorWords; }
 inline size_t feed_coarse_words(const CoarseGeom &cg, int words) {
   return (size_t)words * cg.groups * kCoarseSplit * cg.cap;
 }
@@ -173,8 +176,12 @@ __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, Coars
                                                              const uint32_t *__restrict__ coarse_cursor,
                                                              const uint32_t *__restrict__ coarse_words,
                                                              uint32_t *__restrict__ cursor,
-                                                             uint32_t *__restrict__ bucket_lo, int32_t *status) {
+                                                             uint32_t *__restrict__ bucket_lo, uint32_t *clear,
+                                                             uint32_t clear_words, int32_t *status) {
   __shared__ uint32_t s_cnt[kCoarsePer], s_pref[kCoarsePer + 1], s_gbase[kCoarsePer];
+  // counters of the kernel that filled the coarse slabs, which the caller wants back at zero
+  if (blockIdx.x == 0 && blockIdx.y == 0)
+    for (uint32_t i = threadIdx.x; i < clear_words; i += kSlabBlock) clear[i] = 0;
   __shared__ uint32_t s_word[W - 1][kFeedBatch];
   __shared__ Last s_last[kFeedBatch];  // the last word in its own type here too: LDS decides how many workgroups share a compute unit
   __shared__ uint8_t s_dst[kFeedBatch];
@@ -238,9 +245,9 @@ __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, Coars
 // cursors in `fb` must be zero before the coarse slabs are filled.
 template <int W, typename Last, typename Sink>
 int feed_fine(const SlabGeom &geo, const CoarseGeom &cg, const Sink &sink, const FeedBuffers &fb, int32_t *status,
-              hipStream_t s) {
+              hipStream_t s, uint32_t *clear = nullptr, uint32_t clear_words = 0) {
   k_fine_scatter<W, Last, Sink><<<dim3(feed_batches(cg.cap), cg.groups * kCoarseSplit), dim3(kSlabBlock), 0, s>>>(
-      geo, cg, sink, fb.coarse_cursor, fb.coarse_words, fb.cursor, fb.bucket_lo, status);
+      geo, cg, sink, fb.coarse_cursor, fb.coarse_words, fb.cursor, fb.bucket_lo, clear, clear_words, status);
   ZEN_LAUNCH_CHECK("k_fine_scatter");
   return ZEN_OK;
 }

@@ -118,10 +118,12 @@ class TensorPartition:
             out_idx, out_val, splits, status = self.load_balance_flat(tensor, thr, capacity, k, mode)
             host = torch.cat([splits, status.to(torch.int64)]).tolist()
             bits = host[-1]
+            if bits & (_lib.STAT_RETRY | _lib.STAT_INTERNAL):
+                # a declined or aborted call may leave entries and counters behind in the table
+                m, _ = self.table_sizes(tensor.numel())
+                self._table(tensor.device, m).zero_()
             if not bits & _lib.STAT_RETRY:
                 break
-            m, _ = self.table_sizes(tensor.numel())
-            self._table(tensor.device, m).zero_()  # a declined call may leave entries behind
         if bits:
             raise RuntimeError("load_balance: " + _lib.describe_status(bits))
         indices, values, at = [], [], 0
