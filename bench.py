@@ -335,7 +335,8 @@ def main():
     for enc, mrg in outs:  # every step of the timed region must have gone through cleanly and agree
         flags |= int(enc[3]) | int(mrg[3])
         if int(enc[2].sum()) != nnz or int(mrg[2]) != merged:
-            print("bench.py: steps disagree on their result sizes", file=sys.stderr)
+            print(f"bench.py: steps disagree on their result sizes (selected {int(enc[2].sum())} vs {nnz}, "
+                  f"merged {int(mrg[2])} vs {merged}, status {int(enc[3])} / {int(mrg[3])})", file=sys.stderr)
             sys.exit(1)
     if flags:
         print("bench.py: device status " + _lib.describe_status(flags), file=sys.stderr)

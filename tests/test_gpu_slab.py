@@ -300,3 +300,56 @@ def test_slab_merge_bad_indices_cancellation_and_pile_up(zen, oracle):
     gi2, gv2 = lba.merge_sparse(to_dev(idx2), to_dev(val2), n)
     wi2, wv2 = oracle.merge_sparse(idx2, val2, n)
     assert np.array_equal(to_np(gi2), wi2) and np.array_equal(to_np(gv2).view(np.uint32), wv2.view(np.uint32))
+
+
+# ------------------------------------------------ counters are left at zero
+
+def test_table_and_merge_workspace_are_zero_again_after_every_call(zen, oracle):
+    """The slab paths clear no counters up front: they rely on the table (encode) and the head of the merge
+    workspace being zero, and put them back to zero themselves.  Calls of different sizes and selections in a
+    row, on one table and one workspace, must each give the oracle's answer and leave both all zero."""
+    from zen_repro_amd import _lib
+
+    L = _lib.lib()
+    P = 8
+    n = 1 << 23
+    tp = zen.TensorPartition(P, 1, 3)
+    rng = np.random.default_rng(5)
+    g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    cases = [("f32", 0.004, 0), ("bf16", 0.01, 0), ("f32", 1.0, n // 200), ("bf16", 1.0, n // 100), ("f32", 0.002, 0)]
+    for dtype, density, k in cases:
+        x = np.where(rng.random(n) < density, g, 0).astype(np.float32)
+        x_np = oracle.f32_to_bf16_bits(x) if dtype == "bf16" else x
+        grad = to_dev(x_np)
+        if k:
+            key = oracle.kth_key(x_np, k)
+            masked, kept = oracle.mask_dense(x_np, key)
+            cap = kept + 1024
+        else:
+            masked, cap = x_np, int(np.count_nonzero(x)) + 1024
+        m, _ = tp.table_sizes(n)
+        assert L.zen_load_balance_path(n, m, _lib.dtype_code(grad), cap, P, k, _lib.MODE_FAST) == 2
+        idx, val, splits, st = tp.load_balance_flat(grad, None, cap, k=k)
+        idx_o, val_o, splits_o, st_o = oracle.load_balance(masked, P, 1, 3)
+        assert int(st.item()) == 0 and st_o == 0
+        total = int(splits.sum())
+        assert np.array_equal(splits.cpu().numpy(), splits_o)
+        assert np.array_equal(idx[:total].cpu().numpy(), idx_o)
+        assert np.array_equal(to_np(val[:total]), val_o)
+        assert int(tp._table(grad.device, m).count_nonzero()) == 0, (dtype, density, k)
+
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P), None, None)
+    dense_n = 1 << 26
+    for r in (400_000, 3_000_000, 70_000):
+        idx = rng.integers(1, dense_n, r).astype(np.int32)
+        idx[rng.integers(0, r, r // 3)] = idx[rng.integers(0, r, r // 3)]  # duplicates
+        val = (rng.standard_normal(r) * 1e-3).astype(np.float32)
+        assert L.zen_merge_path(r, dense_n, _lib.MODE_FAST) == 2
+        m_idx, m_val, count, st = lba.merge_sparse_flat(to_dev(idx), to_dev(val), dense_n)
+        assert int(st.item()) == 0
+        mi_o, mv_o = oracle.merge_sparse(idx, val, dense_n)
+        c = int(count.item())
+        assert np.array_equal(m_idx[:c].cpu().numpy(), mi_o)
+        assert np.array_equal(m_val[:c].cpu().numpy().view(np.uint32), mv_o.view(np.uint32))
+        ws = _lib.scratch.get(m_idx.device, "merge/0", 256, zero=True)
+        assert int(ws[:L.zen_merge_zero_bytes()].count_nonzero()) == 0, r

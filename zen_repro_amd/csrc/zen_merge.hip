@@ -220,7 +220,6 @@ __global__ __launch_bounds__(kMergeBlock, 8) void k_merge_bucket(SlabGeom geo, u
   // The counters of the scatter kernels go back to zero (this workgroup was the only reader of its slab's
   // count; the coarse cursors a slice per workgroup), and the last workgroup to finish clears the prefix
   // state: the memory that must be zero when a call starts is zero again when it ends.
-  if (threadIdx.x == 0) cursor[b * kCursorPad] = 0;
   for (uint32_t i = (uint32_t)b * kMergeBlock + threadIdx.x; i < kCoarseCursorWords; i += (uint32_t)nb * kMergeBlock)
     coarse_cursor[i] = 0;
   uint32_t off[kMergeRecs], arr[kMergeRecs], val[kMergeRecs], rank[kMergeRecs];
@@ -238,6 +237,7 @@ __global__ __launch_bounds__(kMergeBlock, 8) void k_merge_bucket(SlabGeom geo, u
   }
   uint32_t n = 0;
   const bool ranked = slab_rank<kMergeBlock>(sh, geo, tie_bits, off, arr, live, rank, &n);
+  if (threadIdx.x == 0) cursor[b * kCursorPad] = 0;  // every thread has read it: slab_rank synchronised
   if (!ranked) {
     if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
     n = 0;  // the bucket contributes nothing; the prefix protocol still gets its (empty) tile

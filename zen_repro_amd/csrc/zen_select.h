@@ -112,6 +112,8 @@ struct StageArgs {
   uint32_t *pick_thr = nullptr;
   uint32_t *pick_above = nullptr;   // optional: number of candidates in the histogram bins above the k-th's
   uint32_t *thr_copy = nullptr;
+  uint32_t *clear = nullptr;        // optional: clear_words words the kernel sets to zero (memory of an earlier
+  uint32_t clear_words = 0;         // kernel that nobody needs any more)
   int32_t *status = nullptr;
 };
 int select_stage_slabs(const StageArgs &a, hipStream_t stream);

@@ -241,9 +241,6 @@ __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restric
   __syncthreads();
   if (!s_last) return;
   sample_pick_block(hist, rank, kShift, floor_out, smem);
-  // the histogram is left as it was found, all zero: a caller that keeps it between calls need not clear it
-  __syncthreads();
-  for (int i = threadIdx.x; i < kFineBins + 2; i += kSampleBlock) hist[i] = 0;
 }
 
 // Run by one whole block (BLOCK threads) over the complete candidate
@@ -846,10 +843,13 @@ template <typename S, bool ALIGNED>
 __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
     const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, StageSlabs out, uint32_t *ticket,
     StageSched sch, uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *pick_above,
-    uint32_t *thr_copy, int32_t *status) {
+    uint32_t *thr_copy, uint32_t *clear, uint32_t clear_words, int32_t *status) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kSub = kSelBlock * kSelVecs * V;
   constexpr int kWaves = kSelBlock / 64;
+  // what the kernel before this one needed at zero and nobody needs any more (the sample's histogram): back
+  // to zero, a slice per workgroup
+  for (uint32_t i = blockIdx.x * kSelBlock + threadIdx.x; i < clear_words; i += gridDim.x * kSelBlock) clear[i] = 0;
   __shared__ uint32_t s_wave[2][kWaves];
   __shared__ uint32_t s_next[2];
   __shared__ int32_t st_idx[kScatStage];
@@ -1074,8 +1074,6 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
         __syncthreads();
         if (thr_copy && threadIdx.x < 2)
           thr_copy[threadIdx.x] = __hip_atomic_load(&pick_thr[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // the histogram and its count of finished workgroups are left all zero, as they were found
-        for (int i = threadIdx.x; i < kCandHistWords; i += kSelBlock) cand_hist[i] = 0;
       }
     }
   }
@@ -1118,11 +1116,11 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   if (aligned)
     k_select_stage<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
         in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.pick_above, a.thr_copy,
-        a.status);
+        a.clear, a.clear_words, a.status);
   else
     k_select_stage<S, false><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
         in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.pick_above, a.thr_copy,
-        a.status);
+        a.clear, a.clear_words, a.status);
   ZEN_LAUNCH_CHECK("k_select_stage");
   return ZEN_OK;
 }

@@ -48,7 +48,10 @@ struct SlabTables {
   uint32_t *ser_idx;    // [P * kSlabSerialCap]
   uint32_t *log_t, *log_v, *log_cell;  // [log_cap]
   uint32_t *out_start;  // [B + 1] where every bucket starts in the output
-  uint32_t *done;       // [2] workgroups of k_slab_classify / of k_slab_place that have finished
+  uint32_t *done;       // [1] workgroups of k_slab_classify that have finished
+  uint32_t *final_n;    // [B + P + 2] what k_slab_place needs of the counters above, copied by the last workgroup of
+                        // k_slab_classify before it puts them back to zero: moved-in entries per bucket, serial
+                        // entries per partition, logged losers, displaced owners
   Counters *ctr;
   uint32_t *coarse_cursor;  // the feed's coarse cursors and, for an fp32 top-k, the refinement histogram (else
   uint32_t *refine_hist;    // null): k_slab_sort puts them back to zero
@@ -181,10 +184,7 @@ __global__ __launch_bounds__(kSortBlock, 8) void k_slab_sort(SlabGeom geo, SlabT
   if (n_raw > (uint32_t)kSlabCap) n_raw = kSlabCap;  // the scatter flagged the overflow
   const uint32_t lo = tb.bucket_lo[b];
   S *slab_val = static_cast<S *>(tb.slab_val);
-  if (threadIdx.x == 0) {
-    s_lost = 0;
-    tb.cursor[b * kCursorPad] = 0;  // this workgroup was its only reader
-  }
+  if (threadIdx.x == 0) s_lost = 0;
   // the kernels before this one were the last to need these: back to zero, a slice per workgroup
   for (uint32_t i = b * kSortBlock + threadIdx.x; i < kCoarseCursorWords; i += gridDim.x * kSortBlock)
     tb.coarse_cursor[i] = 0;
@@ -215,12 +215,15 @@ __global__ __launch_bounds__(kSortBlock, 8) void k_slab_sort(SlabGeom geo, SlabT
   uint32_t n = 0;
   if (!slab_rank<kSortBlock>(sh, geo, 13, off, pos, live, rank, &n)) {
     if (threadIdx.x == 0) {
+      tb.cursor[b * kCursorPad] = 0;
       atomicOr(status, ZEN_STAT_RETRY);
       tb.bucket_n[b] = 0;
       tb.removed_n[b] = 0;
     }
     return;
   }
+  // every thread has read the slab's fill count (slab_rank synchronised); this workgroup was its only reader
+  if (threadIdx.x == 0) tb.cursor[b * kCursorPad] = 0;
   // the counters hold where every narrow range starts in the sorted bucket: every kSlabIndexStep-th goes to
   // the index (before the counters' memory is used for the list of losers below)
   for (int j = threadIdx.x; j < kSlabIndexLen; j += kSortBlock)
@@ -384,7 +387,9 @@ __global__ __launch_bounds__(256) void k_slab_chains(SlabGeom geo, Probe g, Slab
 }
 
 // Where every bucket starts in the output: survivors + moved-in entries, the partition's serial entries
-// behind its last bucket.  Run by one workgroup of kSlabBlock threads once all counts are final.
+// behind its last bucket.  Run by one workgroup of kSlabBlock threads once all counts are final: it is the last
+// to need the counters the chains and the classification raised with atomics, hands what k_slab_place still
+// wants of them on in final_n and puts them back to zero.
 __device__ inline void slab_output_starts(const SlabGeom &geo, const SlabTables &tb, uint32_t *s_scan) {
   constexpr int kPer = kSlabMaxBuckets / kSlabBlock;
   const uint32_t B = geo.nbuckets;
@@ -395,13 +400,16 @@ __device__ inline void slab_output_starts(const SlabGeom &geo, const SlabTables 
     const uint32_t x = threadIdx.x * kPer + e;
     c[e] = 0;
     if (x < B) {
-      uint32_t mv = load_fresh(&tb.movein_n[x]);
-      if (mv > (uint32_t)kSlabMoveCap) mv = kSlabMoveCap;
+      const uint32_t mv_raw = load_fresh(&tb.movein_n[x]);
+      const uint32_t mv = mv_raw > (uint32_t)kSlabMoveCap ? (uint32_t)kSlabMoveCap : mv_raw;
+      tb.final_n[x] = mv_raw;
+      tb.movein_n[x] = 0;
       c[e] = tb.bucket_n[x] - load_fresh(&tb.removed_n[x]) + mv;
       if (x % geo.bpp == geo.bpp - 1) {
-        uint32_t sn = load_fresh(&tb.serial_n[x / geo.bpp]);
-        if (sn > (uint32_t)kSlabSerialCap) sn = kSlabSerialCap;
-        c[e] += sn;
+        const uint32_t sn_raw = load_fresh(&tb.serial_n[x / geo.bpp]);
+        tb.final_n[B + x / geo.bpp] = sn_raw;
+        tb.serial_n[x / geo.bpp] = 0;
+        c[e] += sn_raw > (uint32_t)kSlabSerialCap ? (uint32_t)kSlabSerialCap : sn_raw;
       }
     }
     sum += c[e];
@@ -415,6 +423,13 @@ __device__ inline void slab_output_starts(const SlabGeom &geo, const SlabTables 
     running += c[e];
   }
   if (B == (uint32_t)kSlabMaxBuckets && threadIdx.x == kSlabBlock - 1) tb.out_start[B] = running;
+  if (threadIdx.x == 0) {
+    const uint32_t P = (uint32_t)tb.partitions;
+    tb.final_n[B + P] = load_fresh(&tb.ctr->losers);
+    tb.final_n[B + P + 1] = load_fresh(&tb.ctr->displaced);
+    tb.ctr->logged = tb.ctr->losers = tb.ctr->claims = tb.ctr->displaced = 0;
+    *tb.done = 0;
+  }
 }
 
 // Final place of every logged entry: the level-2/3 slot it holds in the map, or its partition's serial list.
@@ -519,10 +534,11 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
 
   // every occupied map cell ends with the index that finally holds its slot, and that index recorded the
   // cell: clearing by cell number leaves the borrowed memory zero again
+  const uint32_t *serial_n = tb.final_n + B;
   {
-    uint32_t losers = tb.ctr->losers;
+    uint32_t losers = tb.final_n[B + tb.partitions];
     if (losers > tb.log_cap) losers = tb.log_cap;
-    uint32_t total = losers + tb.ctr->displaced;
+    uint32_t total = losers + tb.final_n[B + tb.partitions + 1];
     if (total > tb.log_cap) total = tb.log_cap;
     for (uint32_t i = b * kSlabBlock + threadIdx.x; i < total; i += B * kSlabBlock) {
       const uint32_t cell = tb.log_cell[i];
@@ -531,23 +547,8 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
   }
 
   const uint32_t n = tb.bucket_n[b];
-  uint32_t mv_n = tb.movein_n[b];
+  uint32_t mv_n = tb.final_n[b];
   if (mv_n > (uint32_t)kSlabMoveCap) mv_n = kSlabMoveCap;
-  // Called by every thread of the workgroup on its way out: the counters every workgroup of this kernel reads
-  // go back to zero once the last workgroup has read them (its own count of moved-in entries right away).
-  auto finish = [&]() {
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      tb.movein_n[b] = 0;
-      s_nrm = atomicAdd(&tb.done[1], 1u) == B - 1u;
-    }
-    __syncthreads();
-    if (s_nrm) {
-      for (int i = threadIdx.x; i < tb.partitions; i += kSlabBlock) tb.serial_n[i] = 0;
-      if (threadIdx.x < sizeof(Counters) / sizeof(uint32_t)) reinterpret_cast<uint32_t *>(tb.ctr)[threadIdx.x] = 0;
-      if (threadIdx.x < 2) tb.done[threadIdx.x] = 0;
-    }
-  };
   // the thread's entries (sorted places threadIdx.x + i * kSlabBlock) stay in registers; the slots go to LDS
   // for the searches, the places of removed entries are collected
   uint32_t idx[kSlabItems];
@@ -577,7 +578,6 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
   uint32_t rm_n = s_nrm;
   if (rm_n > (uint32_t)kPlaceRemoved) {  // more collisions than this path carries
     if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);
-    finish();
     return;
   }
   if (rm_n > 1) sort_small(s_rm, rm_n);
@@ -650,7 +650,7 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
   const bool last_of_part = b % geo.bpp == geo.bpp - 1;
   uint32_t serial = 0;
   if (last_of_part) {
-    serial = tb.serial_n[part];
+    serial = serial_n[part];
     if (serial > (uint32_t)kSlabSerialCap) serial = kSlabSerialCap;
   }
   const uint32_t own_n = out_n - serial;  // survivors + moved-in
@@ -672,11 +672,10 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
   if (b % geo.bpp == 0 && threadIdx.x == 0) {
     const uint32_t lo = tb.out_start[b], hi = tb.out_start[b + geo.bpp];
     splits[part] = (int64_t)(hi - lo);
-    if ((int64_t)tb.serial_n[part] > spp) atomicOr(status, ZEN_STAT_SERIAL_OVERFLOW);
+    if ((int64_t)serial_n[part] > spp) atomicOr(status, ZEN_STAT_SERIAL_OVERFLOW);
     if (hi > capacity) atomicOr(status, ZEN_STAT_CAPACITY);
   }
   (void)partitions;
-  finish();
 }
 
 struct SlabPlan {
@@ -706,7 +705,7 @@ SlabPlan plan_slab(void *workspace, void *state, const SlabGeom &geo, int partit
     p.tb.movein_n = cv.take<uint32_t>(B);
     p.tb.serial_n = cv.take<uint32_t>((size_t)partitions);
     p.tb.ctr = cv.take<Counters>(1);
-    p.tb.done = cv.take<uint32_t>(2);
+    p.tb.done = cv.take<uint32_t>(1);
     p.refine_hist = cv.take<uint32_t>(dtype == ZEN_BF16 ? 1 : (size_t)kRefineBins + 1);
     p.state_bytes = cv.used;
   }
@@ -721,6 +720,7 @@ SlabPlan plan_slab(void *workspace, void *state, const SlabGeom &geo, int partit
   p.tb.refine_hist = nullptr;
   p.tb.partitions = partitions;
   p.tb.out_start = cv.take<uint32_t>(B + 1);
+  p.tb.final_n = cv.take<uint32_t>(B + (size_t)partitions + 2);
   p.tb.bucket_n = cv.take<uint32_t>(B);
   p.tb.removed_n = cv.take<uint32_t>(B);
   p.tb.raw_idx = cv.take<uint32_t>(B * kSlabCap);
@@ -748,7 +748,9 @@ int slab_launch(const SlabBalanceArgs &a, const SlabGeom &geo, const SlabPlan &p
   {
     ProfScope prof(kProfFeed, s);
     const EncodeSink<S> sink{geo, p.tb.raw_idx, static_cast<S *>(p.tb.raw_val), filter};
-    const int rc = feed_fine<2, S>(geo, p.cg, sink, p.feed, a.status, s, p.ticket, (uint32_t)select_stage_ticket_words());
+    // the select kernel's candidate histogram and ticket counters lie side by side: back to zero here
+    const int rc = feed_fine<2, S>(geo, p.cg, sink, p.feed, a.status, s, p.cand_hist,
+                                   (uint32_t)(reinterpret_cast<char *>(p.tb.cursor) - reinterpret_cast<char *>(p.cand_hist)) / 4u);
     if (rc != ZEN_OK) return rc;
   }
   {
@@ -829,6 +831,8 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
     sc.pick_thr = p.thr;
     sc.pick_above = p.thr + 4;
     sc.thr_copy = refine ? nullptr : a.thr_out;  // fp32: the threshold is not final yet
+    sc.clear = p.sample_hist;  // the sample kernel is through with its histogram
+    sc.clear_words = (uint32_t)(sampled_floor_zero_bytes() / sizeof(uint32_t));
   }
   if ((rc = select_stage_slabs(sc, s)) != ZEN_OK) return rc;
   if (refine) {

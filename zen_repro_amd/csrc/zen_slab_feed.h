@@ -179,9 +179,10 @@ __global__ __launch_bounds__(kSlabBlock) void k_fine_scatter(SlabGeom geo, Coars
                                                              uint32_t *__restrict__ bucket_lo, uint32_t *clear,
                                                              uint32_t clear_words, int32_t *status) {
   __shared__ uint32_t s_cnt[kCoarsePer], s_pref[kCoarsePer + 1], s_gbase[kCoarsePer];
-  // counters of the kernel that filled the coarse slabs, which the caller wants back at zero
-  if (blockIdx.x == 0 && blockIdx.y == 0)
-    for (uint32_t i = threadIdx.x; i < clear_words; i += kSlabBlock) clear[i] = 0;
+  // counters of the kernel that filled the coarse slabs, which the caller wants back at zero: a slice per workgroup
+  for (uint32_t i = (blockIdx.y * gridDim.x + blockIdx.x) * kSlabBlock + threadIdx.x; i < clear_words;
+       i += gridDim.x * gridDim.y * kSlabBlock)
+    clear[i] = 0;
   __shared__ uint32_t s_word[W - 1][kFeedBatch];
   __shared__ Last s_last[kFeedBatch];  // the last word in its own type here too: LDS decides how many workgroups share a compute unit
   __shared__ uint8_t s_dst[kFeedBatch];
