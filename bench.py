@@ -19,15 +19,15 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the dominant kernel on the full c3 workload, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by what the same counters read
-# for a plain 1 GiB copy (profiles/c3_select_stage_hbm_traffic.txt).  Other
+# for a plain 1 GiB copy, and the summary that holds the figures.  Other
 # workloads report null.
-MEASURED_TRAFFIC = {("c3", 1, "k_select_stage"): 1.519e9}
+MEASURED_TRAFFIC = {("c3", 1, "k_select_stage"): (1.519e9, "profiles/c3_select_stage_hbm_traffic.txt")}
 
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=40)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--shrink", type=int, default=1, help="divide the workload size (debugging)")
@@ -46,69 +46,142 @@ def parse():
     ap.add_argument("--depth", type=int, default=1,
                     help="gradient buckets in flight: step i+1 is enqueued on its own streams next to step i "
                          "(1 = a step starts when the previous one has finished)")
-    ap.add_argument("--time-every", type=int, default=4,
+    ap.add_argument("--rotate", type=int, default=16,
+                    help="at most this many copies of the inputs, used in turn (as many as make 512 MB)")
+    ap.add_argument("--imbalance", action="store_true", help="report the per-bucket load imbalance (always for c4)")
+    ap.add_argument("--time-every", type=int, default=2,
                     help="in the timed region every n-th launch of the roofline kernel carries HIP events")
     ap.add_argument("--no-kernel-timing", action="store_true",
                     help="leave the HIP-event kernel timers off during the timed region")
     return ap.parse_args()
 
 
-def cpu_baseline(cfg, grad_dev, div):
-    """The reference's torch-op sequence (insert: sequential C oracle) on this
-    box's host cores, on the first 1/div of the gradient."""
+def cpu_pass(buckets, grads, payloads, threads):
+    """The reference's torch-op sequence (insert: sequential C oracle) over every gradient bucket on this
+    box's host cores: (seconds per stage summed over the buckets, per-bucket results)."""
     import torch
 
     from oracle import torch_path
-    from zen_repro_amd import workloads
 
-    n_s = cfg.n // div // (16 * cfg.partitions) * (16 * cfg.partitions)
-    sub = workloads.Config(cfg.name, n_s, cfg.dtype, cfg.partitions, cfg.peers, cfg.overlap,
-                           k=int(cfg.k * n_s / cfg.n) if cfg.k else 0)
-    g = grad_dev[:n_s].cpu()
-    nnz_est = sub.k if sub.k else int(torch.count_nonzero(g))
-    per_peer = max(1, nnz_est // cfg.partitions)
-    idx_l, val_l, _, _ = workloads.peer_payloads(sub, per_peer, device="cpu", seed=1)
-    times, (c_idx, c_val, c_splits, _, _, _) = torch_path.timed_pass(g, sub.k, cfg.partitions, idx_l, val_l)
-    total = sum(times.values())
-    parity = parity_gate(sub, grad_dev[:n_s], idx_l, val_l, c_idx, c_val, c_splits)
-    return parity, {
-        "value": n_s * g.element_size() / total / 1e9,
-        "unit": "GB/s",
-        "cores": torch.get_num_threads(),
-        "kind": "port",
-        "sample": f"first {n_s} of {cfg.n} elements (1/{div}), k={sub.k}, {cfg.peers} peer payloads of {per_peer}; "
-                  f"select {times['select']:.2f}s partition {times['partition']:.2f}s merge {times['merge']:.2f}s; "
-                  f"torch ops use {torch.get_num_threads()} threads, the sequential insert 1",
-    }
+    torch.set_num_threads(threads)
+    total = {"select": 0.0, "partition": 0.0, "merge": 0.0}
+    results = []
+    for b, g, (idx_l, val_l) in zip(buckets, grads, payloads):
+        times, res = torch_path.timed_pass(g, b.k, b.partitions, idx_l, val_l)
+        for key, sec in times.items():
+            total[key] += sec
+        results.append(res)
+    return total, results
 
 
-def parity_gate(sub, grad_dev, idx_l, val_l, c_idx, c_val, c_splits):
-    """The HIP path on the sample the CPU baseline has just worked through, checked against that pass's
-    results (untimed): split sizes, the buckets' indices in their order and their values bit for bit; the
-    merged indices and fp32 sums bit for bit against a sequential fp32 scatter_add_ on the CPU (the baseline
-    itself accumulates in the values' own type, as the reference does)."""
+def cpu_baseline(buckets, grads_dev, payloads_dev, outs, div):
+    """CPU baseline on the whole workload (div == 1: the very tensors and payloads of the timed steps, and the
+    last timed step's outputs are what is checked against it) or on the first 1/div of every bucket (then the
+    HIP path repeats that sample, untimed, for the check).  A second pass on one host thread runs on a quarter
+    of that, to keep the run short."""
     import torch
 
+    from zen_repro_amd import workloads
+
+    all_threads = torch.get_num_threads()
+    if div == 1:
+        subs = buckets
+        grads = [g.cpu() for g in grads_dev]
+        payloads = [([t.cpu() for t in idx_l], [t.cpu() for t in val_l]) for idx_l, val_l in payloads_dev]
+        hip = outs
+    else:
+        subs, grads, payloads = [], [], []
+        for b, g in zip(buckets, grads_dev):
+            n_s = b.n // div // (16 * b.partitions) * (16 * b.partitions)
+            sub = workloads.Config(b.name, n_s, b.dtype, b.partitions, b.peers, b.overlap, k=int(b.k * n_s / b.n) if b.k else 0)
+            gs = g[:n_s].cpu()
+            nnz_est = sub.k if sub.k else int(torch.count_nonzero(gs))
+            idx_l, val_l, _, _ = workloads.peer_payloads(sub, max(1, nnz_est // b.partitions), device=g.device, seed=1)
+            subs.append(sub)
+            grads.append(gs)
+            payloads.append(([t.cpu() for t in idx_l], [t.cpu() for t in val_l]))
+        hip = hip_pass(subs, [g[:s.n] for g, s in zip(grads_dev, subs)],
+                       [([t.to(grads_dev[0].device) for t in i], [t.to(grads_dev[0].device) for t in v]) for i, v in payloads])
+    times, results = cpu_pass(subs, grads, payloads, all_threads)
+    parity = parity_gate(subs, payloads, results, hip, "the last timed step's outputs" if div == 1 else
+                         f"an untimed repeat on the first 1/{div} of every bucket")
+    nbytes = sum(s.n * g.element_size() for s, g in zip(subs, grads))
+    base = {
+        "value": nbytes / sum(times.values()) / 1e9,
+        "unit": "GB/s",
+        "cores": all_threads,
+        "kind": "port",
+        "sample": f"{'the whole workload' if div == 1 else f'the first 1/{div} of every bucket'}: "
+                  f"{sum(s.n for s in subs)} elements in {len(subs)} bucket(s); "
+                  f"select {times['select']:.2f}s partition {times['partition']:.2f}s merge {times['merge']:.2f}s; "
+                  f"torch ops use {all_threads} threads, the sequential insert 1",
+    }
+    # one host thread, on the first quarter of that sample
+    q_subs, q_grads, q_pay = [], [], []
+    for s_, g in zip(subs, grads):
+        n_q = s_.n // 4 // (16 * s_.partitions) * (16 * s_.partitions)
+        if n_q < 16 * s_.partitions:
+            continue
+        q = workloads.Config(s_.name, n_q, s_.dtype, s_.partitions, s_.peers, s_.overlap, k=int(s_.k * n_q / s_.n) if s_.k else 0)
+        gq = g[:n_q]
+        nnz_est = q.k if q.k else int(torch.count_nonzero(gq))
+        idx_l, val_l, _, _ = workloads.peer_payloads(q, max(1, nnz_est // q.partitions), device="cpu", seed=1)
+        q_subs.append(q)
+        q_grads.append(gq)
+        q_pay.append((idx_l, val_l))
+    if q_subs:
+        t1, _ = cpu_pass(q_subs, q_grads, q_pay, 1)
+        base["value_1thread"] = sum(q.n * g.element_size() for q, g in zip(q_subs, q_grads)) / sum(t1.values()) / 1e9
+        base["sample_1thread"] = f"the first quarter of that sample ({sum(q.n for q in q_subs)} elements), one host thread"
+    torch.set_num_threads(all_threads)
+    return parity, base
+
+
+def hip_pass(buckets, grads, payloads):
+    """One untimed pass of the HIP path: per bucket ((idx, val, splits, status), (m_idx, m_val, m_count, status))."""
     from zen_repro_amd import LoadBalanceAllreduce, LocalGroup, TensorPartition
 
-    dev, P = grad_dev.device, sub.partitions
-    n_s = grad_dev.numel()
-    capacity = int(sub.k * 1.25) + 4096 if sub.k else int(sum(t.numel() for t in c_idx)) + 16
-    g_idx, g_val, g_splits = TensorPartition(P, 1, 3).load_balance(grad_dev, capacity=capacity, k=sub.k)
-    bits = torch.int16 if grad_dev.dtype == torch.bfloat16 else torch.int32
-    encode_ok = (torch.equal(g_splits.cpu(), c_splits.to(torch.int64))
-                 and torch.equal(torch.cat(g_idx).cpu(), torch.cat(c_idx).to(torch.int32))
-                 and torch.equal(torch.cat(g_val).cpu().view(bits), torch.cat(c_val).view(bits)))
-    lba = LoadBalanceAllreduce(LocalGroup(P), None, None)
-    m_idx, m_val = lba.merge_sparse([t.to(dev) for t in idx_l], [t.to(dev) for t in val_l], n_s)
-    dense = torch.zeros(n_s, dtype=torch.float32)
-    dense.scatter_add_(0, torch.cat(idx_l).to(torch.int64), torch.cat(val_l).to(torch.float32))
-    want_idx = torch.nonzero(dense, as_tuple=True)[0]
-    merge_ok = (torch.equal(m_idx.cpu(), want_idx)
-                and torch.equal(m_val.cpu().view(torch.int32), dense[want_idx].view(torch.int32)))
+    outs = []
+    for b, g, (idx_l, val_l) in zip(buckets, grads, payloads):
+        import torch
+
+        capacity = int(b.k * 1.25) + 4096 if b.k else int(torch.count_nonzero(g)) + 16
+        enc = TensorPartition(b.partitions, 1, 3).load_balance_flat(g, None, capacity, k=b.k)
+        lba = LoadBalanceAllreduce(LocalGroup(b.partitions), None, None)
+        flat_i, flat_v = torch.cat(idx_l), torch.cat(val_l)
+        mrg = lba.merge_sparse_flat(flat_i, flat_v, b.n, capacity=flat_i.numel())
+        outs.append((enc, mrg))
+    return outs
+
+
+def parity_gate(buckets, payloads, cpu_results, hip_outs, what):
+    """The HIP path's outputs against the CPU pass on the same inputs: split sizes, the buckets' indices in
+    their order and their values bit for bit; the merged indices and fp32 sums bit for bit against a sequential
+    fp32 scatter_add_ on the CPU (the baseline itself accumulates in the values' own type, as the reference
+    does)."""
+    import torch
+
+    encode_ok = merge_ok = True
+    selected = merged = 0
+    for b, (idx_l, val_l), (c_idx, c_val, c_splits, _, _, _), (enc, mrg) in zip(buckets, payloads, cpu_results, hip_outs):
+        g_idx, g_val, g_splits, _ = enc
+        count = int(g_splits.sum())
+        bits = torch.int16 if g_val.dtype == torch.bfloat16 else torch.int32
+        encode_ok = (encode_ok and torch.equal(g_splits.cpu(), c_splits.to(torch.int64))
+                     and torch.equal(g_idx[:count].cpu(), torch.cat(c_idx).to(torch.int32))
+                     and torch.equal(g_val[:count].cpu().view(bits), torch.cat(c_val).view(bits)))
+        m_idx, m_val, m_count, _ = mrg
+        u = int(m_count)
+        dense = torch.zeros(b.n, dtype=torch.float32)
+        dense.scatter_add_(0, torch.cat(idx_l).to(torch.int64), torch.cat(val_l).to(torch.float32))
+        want_idx = torch.nonzero(dense, as_tuple=True)[0]
+        merge_ok = (merge_ok and u == want_idx.numel() and torch.equal(m_idx[:u].cpu().to(torch.int64), want_idx)
+                    and torch.equal(m_val[:u].cpu().view(torch.int32), dense[want_idx].view(torch.int32)))
+        selected += count
+        merged += u
+        del dense
     return {"ok": bool(encode_ok and merge_ok), "encode_bit_exact": bool(encode_ok), "merge_bit_exact": bool(merge_ok),
-            "checked": f"the CPU baseline's sample: {int(g_splits.sum())} selected entries in {P} buckets, "
-                       f"{int(m_idx.numel())} merged entries"}
+            "checked": f"{what}: {selected} selected entries, {merged} merged entries"}
 
 
 def bitmap_codec(args, dev):
@@ -260,19 +333,32 @@ def main():
         return
 
     cfg, grad = workloads.make(args.config, device=dev, seed=0, shrink=args.shrink)
-    n, esize, P = cfg.n, grad.element_size(), cfg.partitions
+    esize, P = grad.element_size(), cfg.partitions
+    buckets = workloads.buckets(cfg)  # the gradient buckets the tensor is handed over in (c2: two; else one)
     tp = TensorPartition(P, 1, 3)
     lba = LoadBalanceAllreduce(LocalGroup(P), None, None)
 
-    if cfg.k:
-        nnz_guess = cfg.k
-        capacity = int(cfg.k * 1.25) + 4096  # room for ties at the threshold
-    else:
-        nnz_guess = int(torch.count_nonzero(grad))
-        capacity = nnz_guess + 16
-    per_peer = max(1, nnz_guess // P)
-    idx_l, val_l, flat_idx, flat_val = workloads.peer_payloads(cfg, per_peer, device=dev, seed=1)
-    received = flat_idx.numel()
+    # Per bucket: its stretch of the gradient, the capacity of its selection and the payloads the P peers send
+    # to rank 0, generated on the device (the CPU baseline gets copies of these very tensors).
+    grads, caps, payloads, flats = [], [], [], []
+    for b in buckets:
+        g = grad[b.offset:b.offset + b.n]
+        nnz_guess = b.k if b.k else int(torch.count_nonzero(g))
+        caps.append(int(b.k * 1.25) + 4096 if b.k else nnz_guess + 16)  # room for ties at the threshold
+        idx_l, val_l, flat_idx, flat_val = workloads.peer_payloads(b, max(1, nnz_guess // P), device=dev, seed=1)
+        grads.append(g)
+        payloads.append((idx_l, val_l))
+        flats.append((flat_idx, flat_val))
+    received = sum(fi.numel() for fi, _ in flats)
+    total_bytes = sum(b.n for b in buckets) * esize
+
+    # Inputs rotate between copies at different addresses so that nothing of a step's input is still in the
+    # 256 MB last-level cache when the next step reads it (the copies hold the same values: one check serves).
+    def copies_of(nbytes):
+        return max(1, min(args.rotate, -(-(512 << 20) // max(1, nbytes))))
+    grad_sets = [[g] + [g.clone() for _ in range(copies_of(total_bytes) - 1)] for g in grads]
+    pay_bytes = sum(fi.numel() * (4 + esize) for fi, _ in flats)
+    flat_sets = [[(fi, fv)] + [(fi.clone(), fv.clone()) for _ in range(copies_of(pay_bytes) - 1)] for fi, fv in flats]
 
     # The merge of the received payloads does not depend on this rank's own encode, so it runs on a second
     # stream.  A training step hands over one gradient bucket after the other (train.py:167-185 is called
@@ -288,30 +374,55 @@ def main():
     def step(i):
         slot = i % depth
         es, ms_ = enc_streams[slot], mrg_streams[slot]
+        enc, mrg = [], []
         with torch.cuda.stream(es):
-            enc = tp.load_balance_flat(grad, None, capacity, k=cfg.k, slot=slot)
+            for j, b in enumerate(buckets):
+                g = grad_sets[j][i % len(grad_sets[j])]
+                enc.append(tp.load_balance_flat(g, None, caps[j], k=b.k, slot=slot))
         with torch.cuda.stream(ms_ if ms_ is not None else es):
-            mrg = lba.merge_sparse_flat(flat_idx, flat_val, n, capacity=received, slot=slot)
-        return enc, mrg
+            for j, b in enumerate(buckets):
+                fi, fv = flat_sets[j][i % len(flat_sets[j])]
+                mrg.append(lba.merge_sparse_flat(fi, fv, b.n, capacity=fi.numel(), slot=slot))
+        return list(zip(enc, mrg))
+
+    side = enc_streams[1:] + [m for m in mrg_streams if m is not None]
 
     def run(count):
         outs = []
-        for s_ in enc_streams[1:] + [m for m in mrg_streams if m is not None]:
+        for s_ in side:
             s_.wait_stream(main)  # the inputs were produced on the main stream
         for i in range(count):
             outs.append(step(i))
-        for s_ in enc_streams[1:] + [m for m in mrg_streams if m is not None]:
+        for s_ in side:
             main.wait_stream(s_)
         return outs
 
     run(args.warmup)
     torch.cuda.synchronize()
+
+    # what a read-only pass over the gradient reaches on this box (plain non-temporal streaming loads)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    ceiling = None
+    if total_bytes >= 1 << 26:
+        L = _lib.lib()
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(11)]
+        for r in range(10):
+            evs[r].record()
+            for gs in grad_sets:
+                g = gs[r % len(gs)]
+                _lib.check(L.zen_stream_read(_lib.ptr(g), g.numel() * esize, _lib.ptr(sink), _lib.stream_of(dev)), "stream_read")
+        evs[10].record()
+        torch.cuda.synchronize()
+        per = sorted(evs[r].elapsed_time(evs[r + 1]) for r in range(10))
+        ceiling = total_bytes / (per[len(per) // 2] * 1e-3) / 1e9
+
     # An event between two kernels costs the device a few microseconds, about 40 of them per step with every
     # stage timed.  So the stage breakdown comes from an untimed pass of its own, and in the timed region only
     # the dominant kernel (the one the roofline figure is about) carries events, on every --time-every-th of
     # its launches (the pair of events around one launch holds the stream up for 10 us or so).
     streaming = ("k_select_stage", "k_select_compact", "k_topk_hist")  # kernels that read the dense gradient
     stages, dom = {}, None
+    every = 1 if len(buckets) > 1 else max(1, args.time_every)  # several buckets: every launch, or one bucket's only
     if not args.no_kernel_timing:
         _lib.profile_enable(True)
         run(args.steps)
@@ -319,7 +430,7 @@ def main():
         stages = _lib.profile_read()
         cands = [(stages[name][0], name) for name in streaming if name in stages]
         dom = max(cands)[1] if cands else None
-        _lib.profile_enable(dom is not None, only=dom, every=max(1, args.time_every))
+        _lib.profile_enable(dom is not None, only=dom, every=every)
     t0 = time.perf_counter()
     outs = run(args.steps)
     t_enq = time.perf_counter()
@@ -328,43 +439,62 @@ def main():
     kernels = _lib.profile_read() if dom else {}
     _lib.profile_enable(False)
 
-    (o_idx, o_val, splits, st_enc), (m_idx, m_val, m_count, st_mrg) = outs[-1]
-    nnz = int(splits.sum())
-    merged = int(m_count)
+    last = outs[-1]
+    nnz = [int(enc[2].sum()) for enc, _ in last]
+    merged = [int(mrg[2]) for _, mrg in last]
     flags = 0
-    for enc, mrg in outs:  # every step of the timed region must have gone through cleanly and agree
-        flags |= int(enc[3]) | int(mrg[3])
-        if int(enc[2].sum()) != nnz or int(mrg[2]) != merged:
-            print(f"bench.py: steps disagree on their result sizes (selected {int(enc[2].sum())} vs {nnz}, "
-                  f"merged {int(mrg[2])} vs {merged}, status {int(enc[3])} / {int(mrg[3])})", file=sys.stderr)
-            sys.exit(1)
+    for o in outs:  # every step of the timed region must have gone through cleanly and agree
+        for j, (enc, mrg) in enumerate(o):
+            flags |= int(enc[3]) | int(mrg[3])
+            if int(enc[2].sum()) != nnz[j] or int(mrg[2]) != merged[j]:
+                print(f"bench.py: steps disagree on their result sizes (bucket {j}: selected {int(enc[2].sum())} vs "
+                      f"{nnz[j]}, merged {int(mrg[2])} vs {merged[j]}, status {int(enc[3])} / {int(mrg[3])})", file=sys.stderr)
+                sys.exit(1)
     if flags:
         print("bench.py: device status " + _lib.describe_status(flags), file=sys.stderr)
         sys.exit(1)
 
     ms = (t1 - t0) * 1e3 / args.steps
-    value = n * esize / (ms * 1e-3) / 1e9
-    b_alg = workloads.algorithmic_bytes(n, esize, nnz, received, merged)
+    value = total_bytes / (ms * 1e-3) / 1e9
+    b_alg = sum(workloads.algorithmic_bytes(b.n, esize, nnz[j], flats[j][0].numel(), merged[j]) for j, b in enumerate(buckets))
+
+    # isolated steps (a step starts when the one before has finished), each bracketed by events: the median
+    # tells how a single bucket's latency compares with the pipelined rate above
+    lat = []
+    for i in range(min(args.steps, 20)):
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for s_ in side:
+            s_.wait_stream(main)
+        step(i)
+        for s_ in side:
+            main.wait_stream(s_)
+        e1.record()
+        torch.cuda.synchronize()
+        lat.append(e0.elapsed_time(e1))
+    lat.sort()
 
     # dominant kernel: the one with the largest summed duration among the
     # kernels that stream the dense gradient; its algorithmic bytes per launch
-    per_launch = {
-        "k_select_stage": n * esize + nnz * (4 + esize),
-        "k_select_compact": n * esize + nnz * (4 + esize),
-        "k_topk_hist": n * esize,
-    }
+    # (several buckets: the mean over the buckets' launches, all of which are timed)
+    sel_bytes = sum(b.n * esize + nnz[j] * (4 + esize) for j, b in enumerate(buckets)) / len(buckets)
+    per_launch = {"k_select_stage": sel_bytes, "k_select_compact": sel_bytes, "k_topk_hist": total_bytes / len(buckets)}
     roofline = None
     stage_ms = {name: round(total / args.steps, 4) for name, (total, _) in stages.items()}
     if dom in kernels:
         total_ms, launches = kernels[dom]
         avg_ms = total_ms / launches
         achieved = per_launch[dom] / (avg_ms * 1e-3) / 1e9
+        traffic = MEASURED_TRAFFIC.get((cfg.name, args.shrink, dom))
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                    "traffic": MEASURED_TRAFFIC.get((cfg.name, args.shrink, dom)),
+                    "traffic": traffic[0] if traffic else None, "traffic_source": traffic[1] if traffic else None,
                     "avg_launch_ms": round(avg_ms, 4), "launches_per_step": stages[dom][1] // args.steps,
                     "timed_launches": launches,
-                    "algorithmic_bytes_per_launch": per_launch[dom]}
+                    "algorithmic_bytes_per_launch": int(per_launch[dom]),
+                    "measured_read_ceiling_GBps": round(ceiling, 1) if ceiling else None,
+                    "frac_of_read_ceiling": round(achieved / ceiling, 4) if ceiling else None}
 
     line = {
         "metric": "encode+decode dense-gradient GB/s on 1 GPU; % of HBM roofline",
@@ -379,11 +509,15 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16" if grad.dtype == torch.bfloat16 else "f32",
         "data": "synthetic",
-        "config": {"workload": f"{cfg.name}: {cfg.note}", "elements": n, "partitions": P, "k": cfg.k,
-                   "selected": nnz, "received": received, "merged": merged, "peers": cfg.peers,
-                   "overlap": cfg.overlap, "shrink": args.shrink, "steps_in_flight": depth},
+        "config": {"workload": f"{cfg.name}: {cfg.note}", "elements": cfg.n, "partitions": P,
+                   "buckets": [{"name": b.name, "elements": b.n, "k": b.k, "selected": nnz[j],
+                                "received": flats[j][0].numel(), "merged": merged[j]} for j, b in enumerate(buckets)],
+                   "k": sum(b.k for b in buckets), "selected": sum(nnz), "received": received, "merged": sum(merged),
+                   "peers": cfg.peers, "overlap": cfg.overlap, "shrink": args.shrink, "steps_in_flight": depth,
+                   "input_copies": {"gradient": len(grad_sets[0]), "payloads": len(flat_sets[0])}},
         "path_algorithmic_GBps": round(b_alg / (ms * 1e-3) / 1e9, 2),
         "path_frac_of_hbm_peak": round(b_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "ms_per_step_isolated_median": round(lat[len(lat) // 2], 4),
         "host_enqueue_ms_per_step": round((t_enq - t0) * 1e3 / args.steps, 4),
         "stage_ms_per_step": stage_ms,
         "stage_ms_note": "from an untimed pass with every stage's events on; the timed region times only the "
@@ -391,11 +525,25 @@ def main():
         "roofline": roofline,
         "cpu_baseline": None,
     }
+    if cfg.name == "c4" or args.imbalance:
+        # per-bucket load, max / mean, of the hash partition (the split sizes) and of a plain range partition of
+        # the same indices (utils.py:66-88 is the reference's notion of skew)
+        enc = last[0][0]
+        count = nnz[0]
+        by_hash = enc[2].double()
+        by_range = torch.bincount(enc[0][:count].to(torch.int64) // -(-buckets[0].n // P), minlength=P).double()
+        line["bucket_imbalance"] = {"hash": round((by_hash.max() / by_hash.mean()).item(), 4),
+                                    "range": round((by_range.max() / by_range.mean()).item(), 4),
+                                    "what": "largest bucket / mean bucket over the P destinations"}
     if not args.no_cpu_baseline:
-        line["parity_vs_cpu_baseline"], line["cpu_baseline"] = cpu_baseline(cfg, grad, args.cpu_sample_div)
+        line["parity_vs_cpu_baseline"], line["cpu_baseline"] = cpu_baseline(
+            buckets, [gs[(args.steps - 1) % len(gs)] for gs in grad_sets],
+            [(list(torch.split(fs[(args.steps - 1) % len(fs)][0], [t.numel() for t in payloads[j][0]])),
+              list(torch.split(fs[(args.steps - 1) % len(fs)][1], [t.numel() for t in payloads[j][1]])))
+             for j, fs in enumerate(flat_sets)], last, args.cpu_sample_div)
     print(json.dumps(line))
     if line.get("parity_vs_cpu_baseline") and not line["parity_vs_cpu_baseline"]["ok"]:
-        print("bench.py: the HIP path and the CPU baseline disagree on the sample", file=sys.stderr)
+        print("bench.py: the HIP path and the CPU baseline disagree", file=sys.stderr)
         sys.exit(1)
 
 

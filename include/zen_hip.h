@@ -317,6 +317,15 @@ int zen_bucket_sort_pairs(uint32_t *keys, uint32_t *vals, int64_t max_count,
                           void *workspace, size_t workspace_bytes, int32_t *status, void *stream);
 
 /*
+ * Reads `bytes` bytes (16-byte aligned) with coalesced non-temporal 16-byte
+ * loads and does nothing else: the rate a read-only pass over a tensor can reach
+ * on the machine at hand, to set beside the published peak when a streaming
+ * kernel is judged.  *sink is a device word the kernel may write.  No counterpart
+ * in the reference; benchmarks time it.
+ */
+int zen_stream_read(const void *input, size_t bytes, uint32_t *sink, void *stream);
+
+/*
  * Per-kernel timing with HIP events recorded on the launch stream, for
  * benchmarks.  The reference's counterpart is its nvtx ranges
  * (tensor_load_balance.py:25-38, comm.py:66-144).  zen_profile_enable(1)
@@ -326,7 +335,7 @@ int zen_bucket_sort_pairs(uint32_t *keys, uint32_t *vals, int64_t max_count,
  * on the device: zen_profile_only(tag) limits the recording to one tag (a
  * negative tag lifts the limit), and zen_profile_every(n) to every n-th
  * launch of a tag, counted from zen_profile_enable (n = 1: all of them).
- * Process-wide, serialised by a mutex.
+ * Process-wide; with recording off a tagged launch site only reads a flag.
  */
 int zen_profile_enable(int on);
 int zen_profile_only(int tag);

@@ -66,12 +66,25 @@ def oracle_encode(oracle, cfg, grad, key=None):
 SHRUNK = [("c1", 1), ("c2", 16), ("c3", 64), ("c4", 128), ("c5", 32)]
 
 
+def bucket_views(cfg, grad):
+    """(bucket configuration, its stretch of the flat gradient) for every gradient bucket of a configuration
+    (c2 is handed over in two: the embedding as it is, the dense rest for the path to threshold)."""
+    from zen_repro_amd import workloads
+
+    return [(b, grad[b.offset:b.offset + b.n]) for b in workloads.buckets(cfg)]
+
+
 @pytest.mark.parametrize("mode", [0, 1])
 @pytest.mark.parametrize("name,shrink", SHRUNK)
 def test_shrunk_config_encode_is_bit_exact(zen, oracle, name, shrink, mode):
     from zen_repro_amd import workloads
 
-    cfg, grad = workloads.make(name, device="cuda", seed=0, shrink=shrink)
+    whole, flat = workloads.make(name, device="cuda", seed=0, shrink=shrink)
+    for cfg, grad in bucket_views(whole, flat):
+        check_shrunk_encode(zen, oracle, cfg, grad, mode)
+
+
+def check_shrunk_encode(zen, oracle, cfg, grad, mode):
     idx, val, splits, thr_out = encode(zen, cfg, grad, mode)
     key, idx_o, val_o, splits_o = oracle_encode(oracle, cfg, grad)
     count = int(splits.sum())
@@ -87,7 +100,14 @@ def test_shrunk_config_encode_is_bit_exact(zen, oracle, name, shrink, mode):
 def test_shrunk_config_merge_matches_oracle(zen, oracle, name, shrink):
     from zen_repro_amd import workloads
 
-    cfg, grad = workloads.make(name, device="cuda", seed=0, shrink=shrink)
+    whole, flat = workloads.make(name, device="cuda", seed=0, shrink=shrink)
+    for cfg, grad in bucket_views(whole, flat):
+        check_shrunk_merge(zen, oracle, cfg, grad)
+
+
+def check_shrunk_merge(zen, oracle, cfg, grad):
+    from zen_repro_amd import workloads
+
     nnz = cfg.k if cfg.k else int(torch.count_nonzero(grad))
     per_peer = max(1, nnz // cfg.partitions)
     idx_l, val_l, flat_idx, flat_val = workloads.peer_payloads(cfg, per_peer, device="cuda", seed=1)
@@ -114,17 +134,25 @@ def test_shrunk_config_merge_matches_oracle(zen, oracle, name, shrink):
 
 # ------------------------------------------------------------ full size
 
-FULL = ["c2", "c3", "c4", "c5"]
+FULL = [("c2", 0), ("c2", 1), ("c3", 0), ("c4", 0), ("c5", 0)]  # (configuration, gradient bucket)
+_made = {}
 
 
-@pytest.fixture(scope="module", params=FULL)
+@pytest.fixture(scope="module", params=FULL, ids=lambda p: f"{p[0]}.{p[1]}")
 def full(request, zen):
     from zen_repro_amd import workloads
 
-    cfg, grad = workloads.make(request.param, device="cuda", seed=0, shrink=1)
-    yield cfg, grad
-    del grad
-    torch.cuda.empty_cache()
+    name, which = request.param
+    if _made.get("name") != name:  # one configuration's tensor at a time
+        _made.clear()
+        torch.cuda.empty_cache()
+        _made["name"] = name
+        _made["made"] = workloads.make(name, device="cuda", seed=0, shrink=1)
+    whole, flat = _made["made"]
+    yield bucket_views(whole, flat)[which]
+    if (name, which) == FULL[-1]:
+        _made.clear()
+        torch.cuda.empty_cache()
 
 
 def test_full_config_encode_properties(zen, full):
@@ -164,6 +192,10 @@ def test_full_config_encode_properties(zen, full):
     by_hash, by_range = workloads.bucket_imbalance(idx, n, P)
     print(f"{cfg.name}: bucket max/mean hash {by_hash:.4f} range {by_range:.4f}")
     assert by_hash < (1.05 if cfg.name != "c5" else 1.2)  # 3072-long index runs are not spread perfectly by the cubic
+    if cfg.k and cfg.n > 1 << 24:  # a top-k of this size goes through the one-pass bucket-slab path
+        from zen_repro_amd import _lib
+
+        assert _lib.lib().zen_load_balance_path(n, n, _lib.dtype_code(grad), int(cfg.k * 1.25) + 4096, P, cfg.k, 0) == 2
     if cfg.name in ("c4", "c5"):
         assert by_range > 1.5 and by_range > 2 * by_hash
     # general mode (owner table like the reference) gives the same bytes

@@ -353,3 +353,34 @@ def test_table_and_merge_workspace_are_zero_again_after_every_call(zen, oracle):
         assert np.array_equal(m_val[:c].cpu().numpy().view(np.uint32), mv_o.view(np.uint32))
         ws = _lib.scratch.get(m_idx.device, "merge/0", 256, zero=True)
         assert int(ws[:L.zen_merge_zero_bytes()].count_nonzero()) == 0, r
+
+
+def test_load_balance_without_a_capacity_takes_the_slab_path(zen, oracle):
+    """TensorPartition.load_balance(tensor) as the reference calls it (tensor_load_balance.py:43): the capacity
+    it works out for itself keeps a bucket-sized, sparse tensor on the bucket-slab path, and the result is the
+    oracle's."""
+    from zen_repro_amd import _lib
+
+    L = _lib.lib()
+    n, P = 1 << 26, 16  # a 128 MB bf16 bucket (run_all.sh:22)
+    g_np = make_grad(oracle, n, 0.005, "bf16", seed=21)
+    grad = to_dev(g_np)
+    tp = zen.TensorPartition(P, 1, 3)
+    cap = tp._honest_capacity(grad, None, 0)
+    m, _ = tp.table_sizes(n)
+    assert cap < n // 100
+    assert L.zen_load_balance_path(n, m, _lib.BF16, cap, P, 0, _lib.MODE_FAST) == 2
+    assert L.zen_load_balance_workspace(n, m, _lib.BF16, cap, P) < 1 << 28
+    indices, values, splits = tp.load_balance(grad)
+    idx_o, val_o, splits_o, st_o = oracle.load_balance(g_np, P, 1, 3)
+    assert st_o == 0
+    assert np.array_equal(splits.cpu().numpy(), splits_o)
+    assert np.array_equal(torch.cat(indices).cpu().numpy(), idx_o)
+    assert np.array_equal(to_np(torch.cat(values)), val_o)
+    # with a threshold: the count that came with it sizes the call
+    thr = zen.topk_threshold(grad, 200_000)
+    assert tp._honest_capacity(grad, thr, 0) == int(thr[1].item()) + 1024
+    indices, values, splits = tp.load_balance(grad, thr=thr)
+    masked, kept = oracle.mask_dense(g_np, int(thr[0].item()))
+    idx_o, val_o, splits_o, st_o = oracle.load_balance(masked, P, 1, 3)
+    assert int(splits.sum()) == kept and np.array_equal(torch.cat(indices).cpu().numpy(), idx_o)

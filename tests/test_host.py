@@ -168,8 +168,17 @@ def test_workloads_small(name, shrink):
     nz = int(torch.count_nonzero(g))
     if name == "c3":
         assert nz > 0.99 * cfg.n and cfg.k == int(cfg.n * 0.005)
+    elif name == "c2":
+        # two gradient buckets: the embedding (row-sparse, taken as it is) and the dense rest (top 1 % by the path)
+        emb, rest = workloads.buckets(cfg)
+        assert emb.offset == 0 and rest.offset == emb.n and emb.n + rest.n == cfg.n
+        assert emb.k == 0 and rest.k == rest.n // 100
+        assert emb.n % cfg.partitions == 0 and rest.n % cfg.partitions == 0
+        assert 0 < int(torch.count_nonzero(g[:emb.n])) < 0.05 * emb.n
+        assert int(torch.count_nonzero(g[emb.n:])) > 0.99 * rest.n
     else:
         assert 0 < nz < 0.05 * cfg.n
+        assert workloads.buckets(cfg) == [cfg]
     if name == "c4":
         idx = torch.nonzero(g, as_tuple=True)[0]
         h, r = workloads.bucket_imbalance(idx, cfg.n, cfg.partitions)

@@ -74,6 +74,7 @@ def lib():
         "zen_sort_pairs": (i32, [vp, vp, i64, vp, i32, vp, sz, vp, vp]),
         "zen_bucket_sort_fits": (i32, [i64, ctypes.c_uint32]),
         "zen_bucket_sort_pairs": (i32, [vp, vp, i64, vp, ctypes.c_uint32, vp, sz, vp, vp]),
+        "zen_stream_read": (i32, [vp, sz, vp, vp]),
         "zen_profile_enable": (i32, [i32]),
         "zen_profile_only": (i32, [i32]),
         "zen_profile_every": (i32, [i32]),

@@ -60,7 +60,7 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Kernel timing tags (zen_profile.hip).  A ProfScope around a launch records
 // HIP events on the launch stream when profiling is enabled; otherwise it is
-// two branch instructions.
+// one relaxed load of a flag and a branch.
 enum ProfTag {
   kProfTopkHist = 0,
   kProfSelectCompact,
@@ -79,6 +79,8 @@ enum ProfTag {
   kProfSlabPlace,
   kProfMergeFeed,
   kProfMergeBucket,
+  kProfSampleHist,
+  kProfDecodeFused,
   kProfCount
 };
 

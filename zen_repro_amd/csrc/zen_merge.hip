@@ -121,20 +121,24 @@ __global__ __launch_bounds__(kMrgBlock) void k_merge_reduce(
 
 template <typename S>
 __global__ __launch_bounds__(256) void k_scatter_dense(const int32_t *__restrict__ idx, const float *__restrict__ sum,
-                                                       const int64_t *count, S *__restrict__ dense);
+                                                       const int64_t *count, S *__restrict__ dense, uint32_t dense_n);
+// The merged indices come out of workspace memory: after a merge that gave up (ZEN_STAT_INTERNAL, ZEN_STAT_RETRY)
+// some of them may never have been written, so none is trusted as an address without a look.
 template <>
 __global__ __launch_bounds__(256) void k_scatter_dense<uint32_t>(const int32_t *__restrict__ idx,
                                                                  const float *__restrict__ sum,
-                                                                 const int64_t *count, uint32_t *__restrict__ dense) {
+                                                                 const int64_t *count, uint32_t *__restrict__ dense,
+                                                                 uint32_t dense_n) {
   const int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
-  if (i < *count) dense[idx[i]] = __float_as_uint(sum[i]);
+  if (i < *count && (uint32_t)idx[i] < dense_n) dense[idx[i]] = __float_as_uint(sum[i]);
 }
 template <>
 __global__ __launch_bounds__(256) void k_scatter_dense<uint16_t>(const int32_t *__restrict__ idx,
                                                                  const float *__restrict__ sum,
-                                                                 const int64_t *count, uint16_t *__restrict__ dense) {
+                                                                 const int64_t *count, uint16_t *__restrict__ dense,
+                                                                 uint32_t dense_n) {
   const int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
-  if (i < *count) dense[idx[i]] = f32_to_bf16_rne(sum[i]);
+  if (i < *count && (uint32_t)idx[i] < dense_n) dense[idx[i]] = f32_to_bf16_rne(sum[i]);
 }
 
 // ---------------------------------------------------------- merge on bucket slabs
@@ -643,9 +647,11 @@ int zen_decode_dense(const void *idx, int idx64_in, const void *val, int dtype, 
   if (rc != ZEN_OK) return rc;
   const unsigned blocks = (unsigned)ceil_div(r, 256);
   if (dtype == ZEN_BF16)
-    k_scatter_dense<uint16_t><<<dim3(blocks), dim3(256), 0, s>>>(m_idx, m_val, m_count, static_cast<uint16_t *>(dense));
+    k_scatter_dense<uint16_t><<<dim3(blocks), dim3(256), 0, s>>>(m_idx, m_val, m_count, static_cast<uint16_t *>(dense),
+                                                                 (uint32_t)dense_n);
   else
-    k_scatter_dense<uint32_t><<<dim3(blocks), dim3(256), 0, s>>>(m_idx, m_val, m_count, static_cast<uint32_t *>(dense));
+    k_scatter_dense<uint32_t><<<dim3(blocks), dim3(256), 0, s>>>(m_idx, m_val, m_count, static_cast<uint32_t *>(dense),
+                                                                 (uint32_t)dense_n);
   ZEN_LAUNCH_CHECK("k_scatter_dense");
   return ZEN_OK;
 }

@@ -1,6 +1,7 @@
 // Optional per-kernel timing with HIP events recorded on the launch stream.
 // Off by default; when on, every tagged launch site records an event before
 // and after its kernel(s).  Reading a tag synchronises on its events.
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -15,7 +16,7 @@ struct Span {
 };
 
 std::mutex g_mu;
-bool g_on = false;
+std::atomic<bool> g_on{false};  // read without the mutex at every tagged launch site
 int g_only = -1;  // >= 0: only launches with this tag are timed
 int g_every = 1;  // of which every g_every-th one
 int64_t g_seen[kProfCount];  // launches per tag since recording began
@@ -38,7 +39,7 @@ const char *const kNames[kProfCount] = {
     "k_topk_hist", "k_select_compact", "k_insert_list", "k_final_key", "sort_pairs",
     "k_gather",    "k_merge_prep",     "k_merge_reduce", "k_compress", "k_insert_dense",
     "k_select_stage", "k_coarse_scatter+k_fine_scatter", "k_slab_sort", "k_slab_chains+classify", "k_slab_place",
-    "merge: k_coarse_scatter+k_fine_scatter", "k_merge_bucket",
+    "merge: k_coarse_scatter+k_fine_scatter", "k_merge_bucket", "k_sample_hist", "k_decode_fused",
 };
 
 void drop_spans() {  // the events go back to the spare list (a read has waited for them, or nobody will)
@@ -52,8 +53,9 @@ void drop_spans() {  // the events go back to the spare list (a read has waited 
 }  // namespace
 
 ProfScope::ProfScope(int tag, hipStream_t stream) : tag_(tag), stream_(stream), start_(nullptr), stop_(nullptr) {
+  if (!g_on.load(std::memory_order_relaxed)) return;  // off: host threads that enqueue side by side do not meet here
   std::lock_guard<std::mutex> lock(g_mu);
-  if (!g_on || (g_only >= 0 && tag != g_only)) return;
+  if (!g_on.load(std::memory_order_relaxed) || (g_only >= 0 && tag != g_only)) return;
   if (g_seen[tag]++ % g_every != 0) return;
   start_ = take_event();
   stop_ = start_ ? take_event() : nullptr;
@@ -79,9 +81,9 @@ extern "C" {
 int zen_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(zen::g_mu);
   zen::drop_spans();
-  zen::g_on = on != 0;
+  zen::g_on.store(on != 0, std::memory_order_relaxed);
   for (int64_t &c : zen::g_seen) c = 0;
-  while (zen::g_on && zen::g_spare.size() < zen::kSpareEvents) {
+  while (on != 0 && zen::g_spare.size() < zen::kSpareEvents) {
     hipEvent_t e = nullptr;
     if (hipEventCreate(&e) != hipSuccess) break;
     zen::g_spare.push_back(e);

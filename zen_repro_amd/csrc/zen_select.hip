@@ -1199,7 +1199,7 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
   if (blocks < 128) blocks = 128;
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
   {
-    ProfScope prof(kProfTopkHist, stream);
+    ProfScope prof(kProfSampleHist, stream);
     if (aligned)
       k_sample_hist<S, true><<<dim3((unsigned)blocks), dim3(kSampleBlock), 0, stream>>>(in, n, sample_log2, hist, rank,
                                                                                         thr_lo);
@@ -1286,7 +1286,47 @@ int topk_static_scratch(void **out) {
 
 }  // namespace
 
+namespace zen {
+namespace {
+
+// Reads `vecs` 16-byte vectors with coalesced non-temporal loads and does nothing else: what a read-only pass
+// over a tensor can reach on the machine at hand.  A workgroup reads kReadChunks consecutive chunks of 256
+// vectors (32 KB in a row; many short-lived workgroups, the arrangement that measured fastest for a bare
+// read).  sink receives a word only if the data XOR to a given value, which keeps the loads alive without a
+// store per thread.
+constexpr int kReadChunks = 8;
+__global__ __launch_bounds__(256) void k_stream_read(const u32x4 *__restrict__ in, size_t vecs, uint32_t *sink) {
+  uint32_t acc = 0;
+  const size_t base = (size_t)blockIdx.x * kReadChunks * 256 + threadIdx.x;
+  const size_t last = vecs - 1;
+  u32x4 q[kReadChunks];
+#pragma unroll
+  for (int i = 0; i < kReadChunks; ++i) {
+    const size_t at = base + (size_t)i * 256;
+    q[i] = __builtin_nontemporal_load(in + (at < last ? at : last));  // no branch around the loads
+  }
+#pragma unroll
+  for (int i = 0; i < kReadChunks; ++i) acc ^= q[i].x ^ q[i].y ^ q[i].z ^ q[i].w;
+  if (acc == 0x9e3779b9u) *sink = acc;
+}
+
+}  // namespace
+}  // namespace zen
+
 extern "C" {
+
+int zen_stream_read(const void *input, size_t bytes, uint32_t *sink, void *stream) {
+  using namespace zen;
+  if (!input || !sink || (reinterpret_cast<uintptr_t>(input) & 15u)) return fail(ZEN_EINVAL, "zen_stream_read: null or unaligned pointer");
+  const size_t vecs = bytes / 16;
+  if (vecs == 0) return ZEN_OK;
+  const size_t blocks = (vecs + (size_t)kReadChunks * 256 - 1) / ((size_t)kReadChunks * 256);
+  if (blocks > 0x7fffffffull) return fail(ZEN_EINVAL, "zen_stream_read: too large");
+  k_stream_read<<<dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const u32x4 *>(input), vecs, sink);
+  ZEN_LAUNCH_CHECK("k_stream_read");
+  return ZEN_OK;
+}
 
 size_t zen_topk_threshold_workspace(void) { return zen::topk_scratch_bytes(); }
 

@@ -1,6 +1,8 @@
 """Drop-in for the reference's extensions/cuda/functions.py: the two entry
 points `sparse_balance` and `hash_index`, same argument order and in-place
 semantics, backed by libzen_hip.so instead of the pybind CUDA module."""
+import threading
+
 import torch
 
 from . import _lib
@@ -32,13 +34,24 @@ def sparse_balance(tensor, memory, serial_memory, partitions, rehash):
         _lib.ptr(memory), memory.numel(), _lib.ptr(serial_memory), numel,
         _lib.ptr(offsets), partitions, rehash, _lib.ptr(status), _lib.stream_of(tensor.device))
     _lib.check(rc, "sparse_balance")
-    return _PendingStatus(status, offsets)
+    _last.pending = _PendingStatus(status, offsets)  # the call itself returns None, like the reference's
+
+
+_last = threading.local()
+
+
+def last_status():
+    """The calling thread's most recent sparse_balance: an object whose
+    check() synchronises and raises if the device flagged a condition (a serial
+    region that overflowed), with the status word and the final ticket counters
+    as attributes.  The reference has no such thing: it writes out of bounds."""
+    return getattr(_last, "pending", None)
 
 
 class _PendingStatus:
-    """What sparse_balance hands back instead of the reference's None: the
+    """Kept per host thread after every sparse_balance (see last_status): the
     device status word and final ticket counters, checked only on request so
-    the call itself stays asynchronous."""
+    the call itself stays asynchronous and returns None as the reference's does."""
 
     def __init__(self, status, offsets):
         self.status = status

@@ -4,7 +4,7 @@ one fused device pipeline (select, insert, slot-order compaction) instead of
 import torch
 
 from . import _lib
-from .functions import sparse_balance
+from .functions import last_status, sparse_balance
 
 
 class TensorPartition:
@@ -32,7 +32,8 @@ class TensorPartition:
         memory_size, serial_memory_size = self.table_sizes(tensor.numel())
         memory = torch.zeros(memory_size, dtype=torch.int32, device=tensor.device)
         serial_memory = torch.zeros(serial_memory_size, dtype=torch.int32, device=tensor.device)
-        sparse_balance(tensor, memory, serial_memory, self.partitions, rehash=self.rehash).check()
+        sparse_balance(tensor, memory, serial_memory, self.partitions, rehash=self.rehash)
+        last_status().check()
         return memory, serial_memory
 
     def get_sub_sparse_tensors(self, tensor, memory):
@@ -64,15 +65,32 @@ class TensorPartition:
         return pos, val.view(torch.int32)
 
     # ------------------------------------------------------- fused path
+    _MAX_TABLES = 4
+
     def _table(self, device, m, slot=0):
+        """The zeroed int32[m] table of (device, m, slot).  Gradient buckets of a
+        few different sizes come round again and again (the hook is called per
+        bucket, train.py:167-185), so a handful of tables is kept, least
+        recently used first out."""
         key = (torch.device(device), m, slot)
-        t = self._tables.get(key)
+        t = self._tables.pop(key, None)
         if t is None:
-            # one table per partitioner and slot: sizes rarely change
-            self._tables = {k: v for k, v in self._tables.items() if k[:2] == key[:2]}
+            while len(self._tables) >= self._MAX_TABLES:
+                self._tables.pop(next(iter(self._tables)))
             t = torch.zeros(m, dtype=torch.int32, device=device)
-            self._tables[key] = t
+        self._tables[key] = t  # most recently used last
         return t
+
+    def _honest_capacity(self, flat, thr, k):
+        """Room for the selection without guessing `numel` (which would take a
+        small selection off the bucket-slab path and size the workspace for the
+        whole tensor): from k, from the count the threshold came with, or from
+        a count of the nonzeros.  The last two read a device value."""
+        if k > 0:
+            return int(k) + int(k) // 4 + 4096  # ties at the threshold
+        if thr is not None:
+            return int(thr[1].item()) + 1024
+        return int(torch.count_nonzero(flat)) + 1024
 
     def load_balance_flat(self, tensor, thr=None, capacity=None, k=0, mode=_lib.MODE_FAST, thr_out=None, slot=0):
         """Fused path without host synchronisation.  Returns (indices int32
@@ -92,7 +110,9 @@ class TensorPartition:
         code = _lib.dtype_code(flat)
         m, _ = self.table_sizes(n)
         if capacity is None:
-            capacity = n
+            # no synchronisation here, so no count: the largest the library takes.  A caller that knows a bound
+            # should pass it (load_balance works one out): this default sizes everything for the whole tensor.
+            capacity = min(n, (1 << 29) - 1)
         dev = flat.device
         L = _lib.lib()
         out_idx = torch.empty(capacity, dtype=torch.int32, device=dev)
@@ -114,15 +134,25 @@ class TensorPartition:
         (tensor_load_balance.py:43-51).  The per-partition tensors are views of
         two contiguous buffers; slicing them needs the split sizes on the
         host, which is this call's only synchronisation."""
-        for mode in ((_lib.MODE_FAST, _lib.MODE_GENERAL) if mode is None else (mode,)):
-            out_idx, out_val, splits, status = self.load_balance_flat(tensor, thr, capacity, k, mode)
+        flat = tensor.reshape(-1)
+        n = flat.numel()
+        grow = capacity is None
+        if grow:
+            capacity = min(n, self._honest_capacity(flat, thr, k))
+        modes = [_lib.MODE_FAST, _lib.MODE_GENERAL] if mode is None else [mode]
+        while modes:
+            out_idx, out_val, splits, status = self.load_balance_flat(tensor, thr, capacity, k, modes[0])
             host = torch.cat([splits, status.to(torch.int64)]).tolist()
             bits = host[-1]
             if bits & (_lib.STAT_RETRY | _lib.STAT_INTERNAL):
                 # a declined or aborted call may leave entries and counters behind in the table
-                m, _ = self.table_sizes(tensor.numel())
+                m, _ = self.table_sizes(n)
                 self._table(tensor.device, m).zero_()
-            if not bits & _lib.STAT_RETRY:
+            if bits & _lib.STAT_RETRY:
+                modes.pop(0)
+            elif bits & _lib.STAT_CAPACITY and grow and capacity < n:
+                capacity = min(n, capacity * 4)  # more ties at the threshold than allowed for
+            else:
                 break
         if bits:
             raise RuntimeError("load_balance: " + _lib.describe_status(bits))

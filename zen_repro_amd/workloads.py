@@ -31,6 +31,19 @@ class Config:
     overlap: float
     k: int = 0            # > 0: exact top-k selection inside the timed path
     note: str = ""
+    offset: int = 0       # where this bucket starts in the flat gradient make() returns
+    parts: tuple = ()     # (name, offset, length, k) of the gradient buckets the tensor is handed over in
+                          # (empty: one bucket, the whole tensor)
+
+
+def buckets(cfg):
+    """The gradient buckets of a configuration, each as a Config of its own
+    (the reference's hook is called once per bucket, train.py:167-185, and
+    hashes each with the bucket's own length)."""
+    if not cfg.parts:
+        return [cfg]
+    return [Config(f"{cfg.name}/{name}", length, cfg.dtype, cfg.partitions, cfg.peers, cfg.overlap, k=k,
+                   note=cfg.note, offset=offset) for name, offset, length, k in cfg.parts]
 
 
 def _gen(seed, device):
@@ -63,13 +76,6 @@ def _row_sparse(rows, cols, active, s, gen, device, seed):
     return flat
 
 
-def _keep_topk(x, k):
-    """Zero everything below the k-th largest magnitude (data preparation for
-    configurations whose dense part arrives already thresholded)."""
-    thr = torch.topk(x.abs(), k, largest=True, sorted=False)[0].min()
-    return torch.where(x.abs() >= thr, x, torch.zeros((), dtype=x.dtype, device=x.device))
-
-
 def make(name, device="cuda", seed=0, shrink=1):
     """(Config, flat gradient tensor) for configuration c1..c5.  `shrink`
     divides the sizes (rows / elements) to get small parity-test cases."""
@@ -79,14 +85,16 @@ def make(name, device="cuda", seed=0, shrink=1):
         cfg = Config("c1", n, torch.float32, 4, 4, 0.2, k=n // 100, note="flat fp32 N(0,1e-3), top 1%")
         return cfg, _normal(n, gen, device)
     if name == "c2":
+        # two gradient buckets, as the hook would see them: the embedding (row-sparse, taken as it is) and the
+        # dense rest, whose top 1 % the path itself has to find
         rows, cols = 50257 // shrink, 768
         rest = 85842432 // shrink // 16 * 16
-        pad = (-(rows * cols + rest)) % 16
         emb = _row_sparse(rows, cols, max(1, 2048 // shrink), 1.1, gen, device, seed + 1)
-        dense = _keep_topk(_normal(rest + pad, gen, device), max(1, (rest + pad) // 100))
-        g = torch.cat([emb, dense])
+        g = torch.cat([emb, _normal(rest, gen, device)])
+        del emb
         cfg = Config("c2", g.numel(), torch.float32, 16, 16, 0.3,
-                     note="GPT-2-small: row-sparse embedding + top-1% dense rest, nonzero predicate")
+                     note="GPT-2-small: row-sparse embedding (nonzeros) + dense rest (top 1%)",
+                     parts=(("embedding", 0, rows * cols, 0), ("rest", rows * cols, rest, max(1, rest // 100))))
         return cfg, g
     if name == "c3":
         n = 743440384 // shrink // 16 * 16
