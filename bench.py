@@ -24,6 +24,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 MEASURED_TRAFFIC = {("c3", 1, "k_select_stage"): (1.519e9, "profiles/c3_select_stage_hbm_traffic.txt")}
 
 
+def note(msg):
+    """Progress line on stderr (a long CPU leg would otherwise look like a hang to whoever watches the run)."""
+    print(f"[bench {time.strftime('%H:%M:%S')}] {msg}", file=sys.stderr, flush=True)
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -67,6 +72,7 @@ def cpu_pass(buckets, grads, payloads, threads):
     total = {"select": 0.0, "partition": 0.0, "merge": 0.0}
     results = []
     for b, g, (idx_l, val_l) in zip(buckets, grads, payloads):
+        note(f"CPU pass over {b.name}: {b.n} elements, {threads} thread(s)")
         times, res = torch_path.timed_pass(g, b.k, b.partitions, idx_l, val_l)
         for key, sec in times.items():
             total[key] += sec
@@ -96,13 +102,14 @@ def cpu_baseline(buckets, grads_dev, payloads_dev, outs, div):
             sub = workloads.Config(b.name, n_s, b.dtype, b.partitions, b.peers, b.overlap, k=int(b.k * n_s / b.n) if b.k else 0)
             gs = g[:n_s].cpu()
             nnz_est = sub.k if sub.k else int(torch.count_nonzero(gs))
-            idx_l, val_l, _, _ = workloads.peer_payloads(sub, max(1, nnz_est // b.partitions), device=g.device, seed=1)
+            idx_l, val_l, _, _ = workloads.peer_payloads(sub, workloads.per_peer_entries(sub, nnz_est), device=g.device, seed=1)
             subs.append(sub)
             grads.append(gs)
             payloads.append(([t.cpu() for t in idx_l], [t.cpu() for t in val_l]))
         hip = hip_pass(subs, [g[:s.n] for g, s in zip(grads_dev, subs)],
                        [([t.to(grads_dev[0].device) for t in i], [t.to(grads_dev[0].device) for t in v]) for i, v in payloads])
     times, results = cpu_pass(subs, grads, payloads, all_threads)
+    note("checking the HIP outputs against the CPU pass")
     parity = parity_gate(subs, payloads, results, hip, "the last timed step's outputs" if div == 1 else
                          f"an untimed repeat on the first 1/{div} of every bucket")
     nbytes = sum(s.n * g.element_size() for s, g in zip(subs, grads))
@@ -125,11 +132,12 @@ def cpu_baseline(buckets, grads_dev, payloads_dev, outs, div):
         q = workloads.Config(s_.name, n_q, s_.dtype, s_.partitions, s_.peers, s_.overlap, k=int(s_.k * n_q / s_.n) if s_.k else 0)
         gq = g[:n_q]
         nnz_est = q.k if q.k else int(torch.count_nonzero(gq))
-        idx_l, val_l, _, _ = workloads.peer_payloads(q, max(1, nnz_est // q.partitions), device="cpu", seed=1)
+        idx_l, val_l, _, _ = workloads.peer_payloads(q, workloads.per_peer_entries(q, nnz_est), device="cpu", seed=1)
         q_subs.append(q)
         q_grads.append(gq)
         q_pay.append((idx_l, val_l))
     if q_subs:
+        note("one host thread on a quarter of the sample")
         t1, _ = cpu_pass(q_subs, q_grads, q_pay, 1)
         base["value_1thread"] = sum(q.n * g.element_size() for q, g in zip(q_subs, q_grads)) / sum(t1.values()) / 1e9
         base["sample_1thread"] = f"the first quarter of that sample ({sum(q.n for q in q_subs)} elements), one host thread"
@@ -332,6 +340,7 @@ def main():
         phase2_decode(args, dev)
         return
 
+    note(f"synthesising {args.config}")
     cfg, grad = workloads.make(args.config, device=dev, seed=0, shrink=args.shrink)
     esize, P = grad.element_size(), cfg.partitions
     buckets = workloads.buckets(cfg)  # the gradient buckets the tensor is handed over in (c2: two; else one)
@@ -345,7 +354,7 @@ def main():
         g = grad[b.offset:b.offset + b.n]
         nnz_guess = b.k if b.k else int(torch.count_nonzero(g))
         caps.append(int(b.k * 1.25) + 4096 if b.k else nnz_guess + 16)  # room for ties at the threshold
-        idx_l, val_l, flat_idx, flat_val = workloads.peer_payloads(b, max(1, nnz_guess // P), device=dev, seed=1)
+        idx_l, val_l, flat_idx, flat_val = workloads.peer_payloads(b, workloads.per_peer_entries(b, nnz_guess), device=dev, seed=1)
         grads.append(g)
         payloads.append((idx_l, val_l))
         flats.append((flat_idx, flat_val))
@@ -397,8 +406,10 @@ def main():
             main.wait_stream(s_)
         return outs
 
+    note("warm-up")
     run(args.warmup)
     torch.cuda.synchronize()
+    note("timing")
 
     # what a read-only pass over the gradient reaches on this box (plain non-temporal streaming loads)
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
@@ -536,6 +547,7 @@ def main():
                                     "range": round((by_range.max() / by_range.mean()).item(), 4),
                                     "what": "largest bucket / mean bucket over the P destinations"}
     if not args.no_cpu_baseline:
+        note(f"GPU part done: {ms:.4f} ms per step; CPU baseline next")
         line["parity_vs_cpu_baseline"], line["cpu_baseline"] = cpu_baseline(
             buckets, [gs[(args.steps - 1) % len(gs)] for gs in grad_sets],
             [(list(torch.split(fs[(args.steps - 1) % len(fs)][0], [t.numel() for t in payloads[j][0]])),

@@ -399,3 +399,69 @@ def test_bitmap_matches_packbits(oracle):
     assert np.array_equal(bm, np.packbits(mask, bitorder="little"))
     assert np.array_equal(oracle.bitmap_decode(mp, bm), pick)
     assert len(bm) == (len(mp) + 7) // 8
+
+
+def test_bitmap_of_indices_that_are_no_members(oracle):
+    """comm.py:61-63 looks every index up with torch.searchsorted (left side) and sets the bit at that
+    position, member or not: an index between two members marks the next member, one below the first member
+    marks the first, duplicates mark once, and a position past the end of the list is an error (torch's
+    index_put raises).  Pinned against numpy's and torch's searchsorted, not against the oracle's own loop."""
+    import torch
+
+    mp = np.array([3, 10, 11, 40, 41, 42, 100, 1000], np.int64)
+    idx = np.array([0, 3, 4, 9, 10, 12, 39, 43, 99, 100, 101, 999, 1000, 4, 4], np.int64)
+    pos = np.searchsorted(mp, idx, side="left")
+    assert np.array_equal(pos, torch.searchsorted(torch.from_numpy(mp), torch.from_numpy(idx)).numpy())
+    mask = np.zeros(len(mp), np.uint8)
+    mask[pos] = 1
+    bm = oracle.bitmap_encode(mp, idx)
+    assert np.array_equal(bm, np.packbits(mask, bitorder="little"))
+    # decoding gives members only: what was between members has become the next member
+    assert np.array_equal(oracle.bitmap_decode(mp, bm), mp[np.unique(pos)])
+    # one past the last member: no position in the list
+    with pytest.raises(IndexError):
+        oracle.bitmap_encode(mp, np.array([3, 1001], np.int64))
+    # random case, any order, many non-members
+    rng = np.random.default_rng(43)
+    mp = np.unique(rng.integers(0, 1 << 20, 5000)).astype(np.int64)
+    idx = rng.integers(0, int(mp[-1]) + 1, 3000).astype(np.int64)
+    mask = np.zeros(len(mp), np.uint8)
+    mask[np.searchsorted(mp, idx, side="left")] = 1
+    assert np.array_equal(oracle.bitmap_encode(mp, idx), np.packbits(mask, bitorder="little"))
+
+
+def test_selection_of_nan_gradients_is_by_bit_pattern(oracle):
+    """Where this build and the reference's torch ops part ways, written down: the selection compares
+    magnitude BIT PATTERNS, in which a NaN (exponent all ones, mantissa nonzero) ranks above infinity.
+    torch.topk also treats NaN as the largest value, so the threshold of train.py:81-82 becomes NaN as soon as
+    k reaches into the NaNs, and `tensor_abs >= threshold` (train.py:83) is then false everywhere: the
+    reference selects nothing, this build selects the NaNs and whatever else lies at or above the k-th
+    pattern.  Without NaNs among the k largest the two agree.  The nonzero predicate of the insert kernel
+    (float(x) != 0, functions_cuda_kernel.cu:100) counts NaN as nonzero in both."""
+    import torch
+
+    g = np.array([0.5, -2.0, np.nan, 1.0, -np.inf, 0.0, 3.0, -0.25, np.nan, 1e-3, -1e-3, 7.0, 0.125, -4.0, 2.5, 0.75],
+                 np.float32)
+    t = torch.from_numpy(g)
+    # k = 3 reaches two NaNs and the infinity
+    key = oracle.kth_key(g, 3)
+    assert key == 0x7F800000  # the pattern of infinity: the NaNs rank above it
+    masked, kept = oracle.mask_dense(g, key)
+    assert kept == 3 and np.isnan(masked[[2, 8]]).all() and masked[4] == -np.inf
+    thr = torch.topk(t.abs(), 3, largest=True, sorted=False)[0].min()
+    assert torch.isnan(thr) or thr == float("inf")  # torch: NaN is the largest, min() of the top 3 propagates it
+    ref = torch.where(t.abs() >= thr, t, torch.zeros(()))
+    assert int(torch.count_nonzero(ref)) <= 1  # the reference keeps (almost) nothing where this build keeps 3
+    # bf16 likewise
+    key16 = oracle.kth_key(oracle.f32_to_bf16_bits(g), 3)
+    assert key16 == 0x7F80
+    # no NaN among the k largest finite values: agreement with torch (k = 5 of the NaN-free tensor)
+    h = np.where(np.isnan(g), 0, g).astype(np.float32)
+    key = oracle.kth_key(h, 5)
+    th = torch.from_numpy(h)
+    thr = torch.topk(th.abs(), 5, largest=True, sorted=False)[0].min()
+    masked, kept = oracle.mask_dense(h, key)
+    assert np.array_equal(masked, torch.where(th.abs() >= thr, th, torch.zeros(())).numpy())
+    # the insert's predicate: NaN is nonzero, -0.0 is zero
+    mem, ser, off, st = oracle.sparse_balance(np.array([0.0, np.nan, -0.0, 1.0], np.float32), 4, 0, 1, 3)
+    assert sorted(int(x) for x in mem if x) == [1, 3]

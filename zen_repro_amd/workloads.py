@@ -136,6 +136,15 @@ def make(name, device="cuda", seed=0, shrink=1):
     raise ValueError(name)
 
 
+def per_peer_entries(cfg, nnz):
+    """Entries each of cfg.peers ranks sends to one destination when every rank selected about `nnz`: nnz / P,
+    but never more than the destination's index range can supply (the payloads hold distinct indices of one
+    partition, all but the shared fraction different from peer to peer)."""
+    distinct_per_entry = cfg.overlap + cfg.peers * (1.0 - cfg.overlap)
+    room = int((cfg.n // cfg.partitions) * 0.5 / distinct_per_entry)
+    return max(1, min(nnz // cfg.partitions, room))
+
+
 def peer_payloads(cfg, per_peer, dest=0, device="cuda", seed=1):
     """What `cfg.peers` ranks send to rank `dest`: per peer an (int32 indices,
     values) pair of `per_peer` entries whose partition is `dest`, a fraction
@@ -150,6 +159,8 @@ def peer_payloads(cfg, per_peer, dest=0, device="cuda", seed=1):
     n_pool = int(per_peer * cfg.overlap)
     n_own = per_peer - n_pool
     need = n_pool + cfg.peers * n_own
+    if need > 0.9 * npp:
+        raise ValueError(f"peer_payloads: {need} distinct indices wanted of a partition that has {npp}")
     have = torch.empty(0, dtype=torch.int64, device=device)
     while have.numel() < need:
         draw = torch.randint(1, n, (int((need - have.numel()) * parts * 1.25) + 4096,), generator=gen, device=device)
