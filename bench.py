@@ -247,10 +247,12 @@ def bitmap_codec(args, dev):
 
 
 def phase2_decode(args, dev):
-    """The second exchange's decode (comm.py:142-145): P ascending, pairwise disjoint shards of merged entries
-    (rank p's shard holds indices of hash partition p, as many as rank 0 merges in the main benchmark) into
-    the dense gradient.  One step = one decode_sparse_tensors(ascending=True) of the concatenated shards;
-    the result is checked against a plain assignment (the shards are disjoint)."""
+    """The second exchange's decode (comm.py:136-145): P pairwise disjoint shards of merged entries (rank p's
+    shard holds indices of hash partition p, as many as rank 0 merges in the main benchmark) into the dense
+    gradient.  Three ways, each checked against a plain assignment (the shards are disjoint): from the ranks'
+    bitmaps and value lists in one pass (decode_bitmaps_dense; the headline figure); from the bitmaps as the
+    reference does it, decode_bitmap for every rank and then decode_sparse_tensors; and from index lists
+    (method 2's exchange, decode_sparse_tensors(ascending=True))."""
     import torch
 
     from zen_repro_amd import LoadBalanceAllreduce, LocalGroup, workloads
@@ -265,43 +267,59 @@ def phase2_decode(args, dev):
     hash_index(part, P)
     per = max(1, int((cfg.k or n // 100) * 0.766))  # what a rank keeps after merging P payloads that overlap by a quarter
     gen = torch.Generator(device=dev).manual_seed(2)
-    idx, val = [], []
+    weights = torch.tensor([1, 2, 4, 8, 16, 32, 64, 128], dtype=torch.uint8, device=dev)
+    idx, val, bitmaps, members_of = [], [], [], []
     for p in range(P):
         members = torch.nonzero(part == p, as_tuple=True)[0]
         pick = torch.randperm(members.numel(), device=dev, generator=gen)[:per].sort().values
         idx.append(members[pick].contiguous())
         val.append((torch.randn(per, device=dev, generator=gen) * 1e-3).to(dtype))
-        del members, pick
+        bits = torch.zeros((members.numel() + 7) // 8 * 8, dtype=torch.uint8, device=dev)
+        bits[pick] = 1
+        bitmaps.append((bits.view(-1, 8) * weights).sum(1, dtype=torch.uint8))  # comm.py:79-83
+        members_of.append(members)
+        del pick, bits
     del part
     flat_i, flat_v = torch.cat(idx), torch.cat(val)
     sizes = [t.numel() for t in idx]
     views = list(torch.split(flat_i, sizes)), list(torch.split(flat_v, sizes))  # what an all-gather into one buffer leaves
-
-    def step():
-        return lba.decode_sparse_tensors(views[0], views[1], n, ascending=True)
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        dense = step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    flat_b = torch.cat(bitmaps)
+    bviews = list(torch.split(flat_b, [t.numel() for t in bitmaps]))
     want = torch.zeros(n, dtype=dtype, device=dev)
     want[flat_i] = flat_v
-    bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
-    if not torch.equal(dense.view(bits), want.view(bits)):
-        print("bench.py: the decoded dense tensor is not the shards' assignment", file=sys.stderr)
-        sys.exit(1)
+    bits_t = torch.int16 if dtype == torch.bfloat16 else torch.int32
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            dense = fn()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        if not torch.equal(dense.view(bits_t), want.view(bits_t)):
+            print("bench.py: the decoded dense tensor is not the shards' assignment", file=sys.stderr)
+            sys.exit(1)
+        return ms
+
+    ms_fused = timed(lambda: lba.decode_bitmaps_dense(bviews, views[1], n))
+    ms_lists = timed(lambda: lba.decode_sparse_tensors(views[0], views[1], n, ascending=True))
+    lba.mapping[n] = members_of  # what calculate_mapping returns (comm.py:52-56)
+    ms_two = timed(lambda: lba.decode_sparse_tensors(lba.decode_bitmap(bviews, n), views[1], n, ascending=True))
     r, s_ = flat_i.numel(), flat_v.element_size()
-    b_alg = r * (8 + s_) + n * s_
+    b_alg = flat_b.numel() + r * s_ + n * s_  # the bitmaps and the values in, the dense tensor out
     print(json.dumps({
-        "metric": "phase-2 decode: all ranks' merged shards into the dense gradient", "value": round(b_alg / (ms * 1e-3) / 1e9, 2),
-        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "metric": "phase-2 decode: all ranks' bitmaps and values into the dense gradient, one pass",
+        "value": round(b_alg / (ms_fused * 1e-3) / 1e9, 2),
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_fused, 4),
         "higher_is_better": True, "dtype": "bf16" if dtype == torch.bfloat16 else "f32", "data": "synthetic",
-        "config": {"workload": f"{cfg.name}: {cfg.note}", "elements": n, "shards": P, "entries": r},
-        "algorithmic_bytes": b_alg}))
+        "config": {"workload": f"{cfg.name}: {cfg.note}", "elements": n, "shards": P, "entries": r,
+                   "bitmap_bytes": flat_b.numel()},
+        "algorithmic_bytes": b_alg,
+        "frac_of_hbm_peak": round(b_alg / (ms_fused * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "ms_per_step_two_steps_from_bitmaps": round(ms_two, 4),
+        "ms_per_step_from_index_lists": round(ms_lists, 4)}))
 
 
 def main():

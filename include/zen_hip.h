@@ -288,6 +288,30 @@ int zen_decode_dense_sorted(const void *idx, int idx64_in, const void *val, int 
                             const int64_t *list_start, int nlists, void *dense, int64_t dense_n,
                             void *workspace, size_t workspace_bytes, int32_t *status, void *stream);
 
+/*
+ * The second exchange with bitmaps in one pass: every rank's bitmap (bit j of list p = the j-th index of
+ * partition p, comm.py:59-85) and value list straight into the dense gradient.  Replaces decode_bitmap for
+ * all ranks followed by decode_sparse_tensors (comm.py:87-99, 136-145) without the indices, the member lists
+ * (mapping) or a cleared dense tensor in between.
+ *   zen_bitmap_dense_dict builds, once per (numel, partitions), what stands in for the mapping the reference
+ * caches (comm.py:132-134): the partition id of every index (one byte) and per tile of 8192 indices the
+ * members of every partition below it (zen_bitmap_dense_dict_bytes bytes, 16-byte aligned).  members, if not
+ * NULL, is a HOST array that receives the partitions' list lengths (this synchronises on the stream).
+ *   zen_bitmap_dense: bitmaps / values hold the lists back to back, list p at byte bitmap_start[p] (of
+ * bitmap_start[p + 1] - bitmap_start[p] bytes) and element value_start[p]; both offset arrays are HOST arrays
+ * of partitions + 1 entries; at most 64 lists.  dense[t] = 0.0 + value for every index whose bit is set, 0
+ * elsewhere: what scatter_add_ into zeros leaves (comm.py:35-39; lists of different partitions never share an
+ * index).  Bits beyond a list's length are ignored (comm.py:97).  A bitmap shorter than its list, or more
+ * set bits than values, raises ZEN_STAT_BAD_INDEX (the reference raises an index error); the missing ones
+ * count as unset / zero.
+ */
+size_t zen_bitmap_dense_dict_bytes(int64_t numel, int partitions);
+int zen_bitmap_dense_dict(int64_t numel, int partitions, void *dict, int64_t *members, void *stream);
+size_t zen_bitmap_dense_workspace(int64_t numel, int partitions);
+int zen_bitmap_dense(const void *dict, int64_t numel, int partitions, const uint8_t *bitmaps,
+                     const int64_t *bitmap_start, const void *values, int dtype, const int64_t *value_start,
+                     void *dense, void *workspace, size_t workspace_bytes, int32_t *status, void *stream);
+
 /* --------------------------------------------------------------- utility */
 
 /*

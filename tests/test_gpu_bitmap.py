@@ -232,3 +232,110 @@ def test_sparse_allreduce_between_four_ranks(zen, method, dtype):
         tol = scale * (1e-6 if dtype == torch.float32 else 2.0 ** -7)
         assert bool((err <= tol).all())
         assert torch.equal(out, results[0])
+
+
+# ---------------------------------------------- bitmaps + values -> dense in one pass
+
+
+def _shards(oracle, n, P, frac, dtype, seed):
+    """Per rank: (members of its partition that are present, their values), as the merge of the first
+    exchange would leave them: ascending indices of partition p, nonzero values."""
+    rng = np.random.default_rng(seed)
+    mp = oracle.mapping(n, P)
+    idx, val = [], []
+    for p in range(P):
+        take = max(1, int(len(mp[p]) * frac))
+        pick = np.sort(rng.choice(mp[p], take, replace=False))
+        v = (rng.standard_normal(take) * 1e-3).astype(np.float32)
+        v[v == 0] = 1e-3
+        idx.append(pick)
+        val.append(oracle.f32_to_bf16_bits(v) if dtype == "bf16" else v)
+    return mp, idx, val
+
+
+def _dense_truth(oracle, n, idx, val):
+    """oracle.decode of all lists (fp32 accumulation, rounded once to the values' type)."""
+    flat_i, flat_v = np.concatenate(idx), np.concatenate(val)
+    f32 = oracle.decode(flat_i, flat_v, n, "f32acc")
+    return oracle.f32_to_bf16_bits(f32) if flat_v.dtype == np.uint16 else f32
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("n,P,frac", [
+    (1 << 16, 4, 0.05),
+    ((1 << 20) + 48, 16, 0.06),      # a last tile that is not full
+    (3000000, 3, 0.3),               # partitions not a power of two, n % 8192 != 0
+    (1 << 20, 64, 0.02),             # the most lists the kernel takes
+    (1 << 19, 2, 0.9),               # nearly every member present
+    (1003 * 7, 7, 0.5),              # below one tile per ... and n % P == 0 with odd sizes
+])
+def test_bitmaps_to_dense_in_one_pass_matches_oracle(zen, oracle, n, P, frac, dtype):
+    n = n // P * P
+    mp, idx, val = _shards(oracle, n, P, frac, dtype, seed=n + P)
+    bitmaps = [oracle.bitmap_encode(mp[p], idx[p]) for p in range(P)]
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P, 0), None, None)
+    got = lba.decode_bitmaps_dense([to_dev(b) for b in bitmaps], [to_dev(v) for v in val], n)
+    want = _dense_truth(oracle, n, idx, val)
+    assert got.numel() == n and np.array_equal(to_np(got), want)
+    # the two-step path of the reference (decode_bitmap, then decode_sparse_tensors) gives the same bytes
+    lba.mapping[n] = lba.calculate_mapping(n)
+    idx_lists = lba.decode_bitmap([to_dev(b) for b in bitmaps], n)
+    for p in range(P):
+        assert np.array_equal(to_np(idx_lists[p]), idx[p])
+    two_step = lba.decode_sparse_tensors(idx_lists, [to_dev(v) for v in val], n, ascending=True)
+    assert torch.equal(two_step.view(torch.int16 if dtype == "bf16" else torch.int32),
+                       got.view(torch.int16 if dtype == "bf16" else torch.int32))
+    # a second call on the cached dictionary, other data
+    mp, idx, val = _shards(oracle, n, P, frac / 2, dtype, seed=n + P + 1)
+    bitmaps = [oracle.bitmap_encode(mp[p], idx[p]) for p in range(P)]
+    got = lba.decode_bitmaps_dense([to_dev(b) for b in bitmaps], [to_dev(v) for v in val], n)
+    assert np.array_equal(to_np(got), _dense_truth(oracle, n, idx, val))
+
+
+def test_bitmaps_to_dense_edge_cases(zen, oracle):
+    n, P = 1 << 18, 8
+    mp, idx, val = _shards(oracle, n, P, 0.1, "f32", seed=3)
+    bitmaps = [oracle.bitmap_encode(mp[p], idx[p]) for p in range(P)]
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P, 0), None, None)
+    want = _dense_truth(oracle, n, idx, val)
+    # padding behind a bitmap (allgather_padding pads to the longest, DDPbackend.py:26-41; garbage bits past the
+    # list's length are ignored, comm.py:97) and lists that do not sit in one buffer
+    padded = [np.concatenate([b, np.full(5 + p, 0xFF, np.uint8)]) for p, b in enumerate(bitmaps)]
+    last_bits = [len(mp[p]) % 8 for p in range(P)]
+    for p in range(P):  # garbage in the unused bits of the last byte too
+        if last_bits[p]:
+            padded[p][len(bitmaps[p]) - 1] |= np.uint8((0xFF << last_bits[p]) & 0xFF)
+    got = lba.decode_bitmaps_dense([to_dev(b) for b in padded], [to_dev(v) for v in val], n)
+    assert np.array_equal(to_np(got), want)
+    # -0.0 among the values becomes +0.0, as 0 + (-0) does in scatter_add_; NaN stays
+    val2 = [v.copy() for v in val]
+    val2[0][0] = -0.0
+    val2[1][0] = np.nan
+    got = to_np(lba.decode_bitmaps_dense([to_dev(b) for b in bitmaps], [to_dev(v) for v in val2], n))
+    assert got.view(np.uint32)[idx[0][0]] == 0 and np.isnan(got[idx[1][0]])
+    # an empty list (no bit set, no values)
+    empty = [b.copy() for b in bitmaps]
+    empty[2][:] = 0
+    vals3 = [v if p != 2 else v[:0] for p, v in enumerate(val)]
+    got = to_np(lba.decode_bitmaps_dense([to_dev(b) for b in empty], [to_dev(v) for v in vals3], n))
+    want3 = want.copy()
+    want3[idx[2]] = 0
+    assert np.array_equal(got, want3)
+    # a bitmap shorter than its list, and fewer values than set bits: the reference raises an index error
+    short = [b if p != 1 else b[:-2] for p, b in enumerate(bitmaps)]
+    with pytest.raises(IndexError):
+        lba.decode_bitmaps_dense([to_dev(b) for b in short], [to_dev(v) for v in val], n)
+    fewer = [v if p != 3 else v[:-1] for p, v in enumerate(val)]
+    with pytest.raises(IndexError):
+        lba.decode_bitmaps_dense([to_dev(b) for b in bitmaps], [to_dev(v) for v in fewer], n)
+    # n % P != 0: some indices belong to no list (hash_index gives P for them, functions_cuda_kernel.cu:172-175)
+    n2, P2 = 100003, 4
+    part = oracle.hash_index(n2, P2)
+    mp2 = oracle.mapping(n2, P2)
+    rng = np.random.default_rng(8)
+    idx2 = [np.sort(rng.choice(m, len(m) // 3, replace=False)) for m in mp2]
+    val2 = [(rng.standard_normal(len(i)) * 1e-3).astype(np.float32) + 1.0 for i in idx2]
+    bm2 = [oracle.bitmap_encode(mp2[p], idx2[p]) for p in range(P2)]
+    lba2 = zen.LoadBalanceAllreduce(zen.LocalGroup(P2, 0), None, None)
+    got = to_np(lba2.decode_bitmaps_dense([to_dev(b) for b in bm2], [to_dev(v) for v in val2], n2))
+    assert np.array_equal(got, _dense_truth(oracle, n2, idx2, val2)) and (got[part == P2] == 0).all()

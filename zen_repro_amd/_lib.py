@@ -70,6 +70,11 @@ def lib():
         "zen_decode_dense": (i32, [vp, i32, vp, i32, i64, vp, i64, i32, vp, sz, vp, vp]),
         "zen_decode_dense_sorted_workspace": (sz, [i64, i32]),
         "zen_decode_dense_sorted": (i32, [vp, i32, vp, i32, ctypes.POINTER(ctypes.c_int64), i32, vp, i64, vp, sz, vp, vp]),
+        "zen_bitmap_dense_dict_bytes": (sz, [i64, i32]),
+        "zen_bitmap_dense_dict": (i32, [i64, i32, vp, ctypes.POINTER(ctypes.c_int64), vp]),
+        "zen_bitmap_dense_workspace": (sz, [i64, i32]),
+        "zen_bitmap_dense": (i32, [vp, i64, i32, vp, ctypes.POINTER(ctypes.c_int64), vp, i32,
+                                   ctypes.POINTER(ctypes.c_int64), vp, vp, sz, vp, vp]),
         "zen_sort_pairs_workspace": (sz, [i64]),
         "zen_sort_pairs": (i32, [vp, vp, i64, vp, i32, vp, sz, vp, vp]),
         "zen_bucket_sort_fits": (i32, [i64, ctypes.c_uint32]),

@@ -65,6 +65,7 @@ class LoadBalanceAllreduce:
         self.logger = logger
         self.mapping = {}
         self._bitmap_ranks = {}  # numel -> (mapping list of this rank, its rank table)
+        self._dense_dicts = {}   # numel -> dictionary of decode_bitmaps_dense
 
     def get_tensor_partition_obj(self, memory_scale, rehash):
         return TensorPartition(partitions=self.partitions, memory_scale=memory_scale, rehash=rehash)
@@ -284,6 +285,53 @@ class LoadBalanceAllreduce:
             raise RuntimeError("decode_bitmap: " + _lib.describe_status(host[-1]))
         return [out[:c] for out, c in zip(outs, host)]
 
+    def decode_bitmaps_dense(self, bitmap_indices, values_tensors, numel):
+        """decode_bitmap for every rank followed by decode_sparse_tensors
+        (comm.py:136-145) in one pass: bitmap_indices[i] / values_tensors[i] are
+        rank i's bitmap over partition i's index list and the values of its set
+        bits in order; returns the dense tensor of `numel` elements in the
+        values' dtype.  Neither the index lists nor self.mapping are needed: a
+        dictionary of one byte per index (each index's partition) is built on
+        first use of a `numel` and cached like the reference caches the mapping
+        (comm.py:132-134)."""
+        if len(bitmap_indices) != self.partitions or len(values_tensors) != self.partitions:
+            raise RuntimeError("decode_bitmaps_dense: one bitmap and one value list per rank")
+        for t in bitmap_indices:
+            _lib.require_gpu(t, "bitmap")
+            if t.dtype != torch.uint8:
+                raise RuntimeError("bitmap must be uint8")
+        L = _lib.lib()
+        dev = values_tensors[0].device
+        cached = self._dense_dicts.get(numel)
+        if cached is None:
+            nbytes = L.zen_bitmap_dense_dict_bytes(numel, self.partitions)
+            if nbytes == 0:
+                raise ValueError("decode_bitmaps_dense: at most 64 partitions, numel below 2^31")
+            cached = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            _lib.check(L.zen_bitmap_dense_dict(numel, self.partitions, _lib.ptr(cached), None, _lib.stream_of(dev)),
+                       "decode_bitmaps_dense")
+            self._dense_dicts[numel] = cached
+        bitmaps = self.stack_tensors(list(bitmap_indices))
+        values = self.stack_tensors(list(values_tensors))
+        _lib.require_gpu(values, "values")
+        P = self.partitions
+        bm_start = (ctypes.c_int64 * (P + 1))(0, *itertools.accumulate(int(t.numel()) for t in bitmap_indices))
+        v_start = (ctypes.c_int64 * (P + 1))(0, *itertools.accumulate(int(t.numel()) for t in values_tensors))
+        dense = torch.empty(numel, dtype=values.dtype, device=dev)
+        ws = _lib.scratch.get(dev, "bitmap_dense", L.zen_bitmap_dense_workspace(numel, P))
+        status = _lib.status_word(dev)
+        rc = L.zen_bitmap_dense(_lib.ptr(cached), numel, P, _lib.ptr(bitmaps), bm_start, _lib.ptr(values),
+                                _lib.dtype_code(values), v_start, _lib.ptr(dense), _lib.ptr(ws), ws.numel(),
+                                _lib.ptr(status), _lib.stream_of(dev))
+        _lib.check(rc, "decode_bitmaps_dense")
+        bits = int(status.item())  # the reference's masking and scatter_add_ raise on a mismatch, also a sync
+        if bits & _lib.STAT_BAD_INDEX:
+            raise IndexError("decode_bitmaps_dense: a bitmap is shorter than its partition's index list, or has "
+                             "more set bits than values came with it")
+        if bits:
+            raise RuntimeError("decode_bitmaps_dense: " + _lib.describe_status(bits))
+        return dense
+
     # ------------------------------------------------- the whole exchange
 
     def zen_sparse_comm(self, tensor, method):
@@ -321,7 +369,12 @@ class LoadBalanceAllreduce:
                 self.mapping[numel] = self.calculate_mapping(numel)
             bitmap_indices = self.encode_bitmap(sparse_indices, numel)
             bitmap_indices_gather = ddp.allgather_padding(bitmap_indices)
+            values_tensors = ddp.allgather_padding(sparse_values)
+            if self.partitions <= 64:
+                # decode_bitmap + decode_sparse_tensors (comm.py:140-145) in one pass, without the indices
+                return self.decode_bitmaps_dense(bitmap_indices_gather, values_tensors, numel)
             indices_tensors = self.decode_bitmap(bitmap_indices_gather, numel)
+            return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
         values_tensors = ddp.allgather_padding(sparse_values)
         return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
 
