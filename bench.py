@@ -46,6 +46,8 @@ def parse():
     ap.add_argument("--phase2-decode", action="store_true",
                     help="measure the decode of the second exchange instead (prints its own line)")
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
+    ap.add_argument("--no-prepare", action="store_true",
+                    help="do not take the next step's sample ahead on a stream of its own")
     ap.add_argument("--merge-follows", action="store_true",
                     help="with --depth: a step's merge runs on its encode's stream, after it")
     ap.add_argument("--depth", type=int, default=1,
@@ -398,7 +400,12 @@ def main():
     mrg_streams = [None if (args.one_stream or args.merge_follows) else torch.cuda.Stream(device=dev)
                    for _ in range(depth)]
 
-    def step(i):
+    # The sample that gives a top-k call its floor only needs the tensor: the next step's is taken ahead on a
+    # stream of its own, beside the current step's sort and placement, instead of in front of the next pass
+    # over the tensor (a hook that is called per bucket can do the same as soon as it holds the next bucket).
+    prep_stream = None if (args.one_stream or args.no_prepare) else torch.cuda.Stream(device=dev)
+
+    def step(i, more=True):
         slot = i % depth
         es, ms_ = enc_streams[slot], mrg_streams[slot]
         enc, mrg = [], []
@@ -406,20 +413,24 @@ def main():
             for j, b in enumerate(buckets):
                 g = grad_sets[j][i % len(grad_sets[j])]
                 enc.append(tp.load_balance_flat(g, None, caps[j], k=b.k, slot=slot))
+        if prep_stream is not None and more and depth == 1:
+            with torch.cuda.stream(prep_stream):
+                for j, b in enumerate(buckets):
+                    tp.prepare(grad_sets[j][(i + 1) % len(grad_sets[j])], b.k, caps[j], slot=slot)
         with torch.cuda.stream(ms_ if ms_ is not None else es):
             for j, b in enumerate(buckets):
                 fi, fv = flat_sets[j][i % len(flat_sets[j])]
                 mrg.append(lba.merge_sparse_flat(fi, fv, b.n, capacity=fi.numel(), slot=slot))
         return list(zip(enc, mrg))
 
-    side = enc_streams[1:] + [m for m in mrg_streams if m is not None]
+    side = enc_streams[1:] + [m for m in mrg_streams if m is not None] + ([prep_stream] if prep_stream is not None else [])
 
     def run(count):
         outs = []
         for s_ in side:
             s_.wait_stream(main)  # the inputs were produced on the main stream
         for i in range(count):
-            outs.append(step(i))
+            outs.append(step(i, more=i + 1 < count))
         for s_ in side:
             main.wait_stream(s_)
         return outs
@@ -496,7 +507,7 @@ def main():
         e0.record()
         for s_ in side:
             s_.wait_stream(main)
-        step(i)
+        step(i, more=False)
         for s_ in side:
             main.wait_stream(s_)
         e1.record()

@@ -55,6 +55,11 @@ extern "C" {
    returns ZEN_OK and raises neither ZEN_STAT_RETRY nor ZEN_STAT_INTERNAL (after those the caller clears
    them).  A workspace allocated zeroed and used for zen_merge only therefore needs no clearing at all. */
 #define ZEN_MODE_ZEROED 0x100
+/* OR-ed into the `mode` of zen_load_balance: zen_load_balance_prepare has run for this call (see there);
+   ZEN_MODE_SECOND names the second of its two sets of sampling memory. */
+#define ZEN_MODE_PREPARED 0x200
+#define ZEN_MODE_SECOND 0x400
+#define ZEN_MODE_DISCARD 0x800 /* zen_load_balance_prepare: drop a sample that no call will pick up */
 
 int zen_abi_version(void);
 
@@ -231,6 +236,22 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m,
                      int64_t capacity, int64_t *splits, int32_t *table, int mode,
                      void *workspace, size_t workspace_bytes,
                      int32_t *status, void *stream);
+
+/*
+ * The part of a top-k zen_load_balance call (k > 0, ZEN_MODE_FAST) that only needs the tensor: the sample
+ * that gives the one-pass selection its floor.  Taken ahead, on another stream, it runs beside whatever the
+ * main stream is still busy with (the previous gradient bucket's sort and placement, say) instead of in front
+ * of this call's pass over the tensor.  Same input, sizes, k, table and workspace as the zen_load_balance
+ * call that follows with mode | ZEN_MODE_PREPARED (that call must be ordered after this one: an event, a
+ * stream wait); `mode` is ZEN_MODE_FAST, with ZEN_MODE_SECOND for the second of two sets of sampling memory,
+ * which lets a caller prepare call i + 1 while call i (prepared with the other set) is in flight; a set may be
+ * prepared again once the call that used it has finished.  A sample that no call will pick up after all is
+ * dropped with mode | ZEN_MODE_DISCARD (same arguments; the table is not all zero before that).  On paths with
+ * nothing to take ahead the function does nothing and the flag is ignored.  No counterpart in the reference.
+ */
+int zen_load_balance_prepare(const void *input, int dtype, int64_t n, int64_t m, int partitions, int64_t k,
+                             int64_t capacity, int32_t *table, int mode, void *workspace,
+                             size_t workspace_bytes, void *stream);
 
 /*
  * Which implementation a zen_load_balance call with these sizes takes: 0 = owner table (the general

@@ -339,3 +339,85 @@ def test_bitmaps_to_dense_edge_cases(zen, oracle):
     lba2 = zen.LoadBalanceAllreduce(zen.LocalGroup(P2, 0), None, None)
     got = to_np(lba2.decode_bitmaps_dense([to_dev(b) for b in bm2], [to_dev(v) for v in val2], n2))
     assert np.array_equal(got, _dense_truth(oracle, n2, idx2, val2)) and (got[part == P2] == 0).all()
+
+
+# ---------------------------------------------------------- the DDP hook
+
+
+class _StubBucket:
+    """What the hook asks of a dist.GradBucket: its flat buffer (train.py:168)."""
+
+    def __init__(self, tensor):
+        self._t = tensor
+
+    def buffer(self):
+        return self._t
+
+
+def test_comm_hook_on_one_rank(zen, oracle):
+    """custom_comm_hook (train.py:167-183) with a stub bucket: the first call passes the bucket through, later
+    ones return a completed future holding the compressed bucket (one rank: no exchange, train.py:178); the
+    compression is the reference's sampled threshold with the sample positions given."""
+    n = 1 << 20
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    grad = (torch.randn(n, device="cuda", generator=gen) * 1e-3).to(torch.bfloat16)
+    sample = torch.randint(0, n, ((n + 99) // 100,), device="cuda", generator=gen)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(1, 0), None, None)
+    hook = zen.SparseCommHook(lba, top_k=5, method=3, tp_group=zen.LocalGroup(1, 0), sample_index=lambda numel: sample)
+    first = hook(None, _StubBucket(grad))
+    assert first.done() and first.value() is grad  # train.py:170-174
+    fut = hook(None, _StubBucket(grad))
+    assert isinstance(fut, torch.futures.Future) and fut.done()
+    out = fut.value()
+    hook.stream.synchronize()
+    # the reference's rule on the CPU: threshold = smallest of the top 5 % of the sampled magnitudes
+    g = grad.float().cpu()
+    s = g.abs()[sample.cpu()]
+    thr = torch.topk(s, s.numel() * 5 // 100, largest=True, sorted=False)[0].min()
+    want = torch.where(g.abs() >= thr, g, torch.zeros(())).to(torch.bfloat16)
+    assert out.dtype == grad.dtype and torch.equal(out.cpu().view(torch.int16), want.view(torch.int16))
+    # buckets of at most 4096 elements pass through (train.py:58-59)
+    small = grad[:4096].clone()
+    assert hook(None, _StubBucket(small)).value() is small
+
+
+def test_comm_hook_between_four_ranks(zen):
+    """The hook end to end with four ranks played by host threads: every rank's future holds the sum of all
+    ranks' compressed buckets (method 3: buckets exchanged, merged, sent round as bitmaps and decoded in one
+    pass)."""
+    P, n = 4, 1 << 20
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    grads = [(torch.randn(n, device="cuda", generator=gen) * 1e-3) for _ in range(P)]
+    samples = [torch.randint(0, n, ((n + 99) // 100,), device="cuda", generator=gen) for _ in range(P)]
+    ex = ThreadExchange(P)
+    results, compressed, errors = [None] * P, [None] * P, []
+
+    def run(rank):
+        try:
+            torch.cuda.set_device(0)
+            lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P, rank), None, None)
+            lba.ddp = ex.view(rank)
+            hook = zen.SparseCommHook(lba, top_k=2, method=3, tp_group=zen.LocalGroup(1, 0),
+                                      sample_index=lambda numel, r=rank: samples[r])
+            hook(None, _StubBucket(grads[rank]))  # the first call is passed through
+            compressed[rank] = zen.compress_with_allgather(2, grads[rank], zen.LocalGroup(1, 0), sample_index=samples[rank])
+            results[rank] = hook(None, _StubBucket(grads[rank])).value()
+            hook.stream.synchronize()
+            torch.cuda.current_stream().synchronize()
+        except BaseException as e:  # noqa: BLE001
+            errors.append((rank, repr(e)))
+            ex.barrier.abort()
+
+    threads = [threading.Thread(target=run, args=(r,)) for r in range(P)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    total = torch.stack([c.double() for c in compressed]).sum(dim=0)
+    scale = torch.stack([c.double().abs() for c in compressed]).sum(dim=0)
+    for r in range(P):
+        out = results[r]
+        assert out.numel() == n and torch.equal(out != 0, total != 0)
+        assert bool(((out.double() - total).abs() <= scale * 1e-6).all())
+        assert torch.equal(out, results[0])

@@ -384,3 +384,55 @@ def test_load_balance_without_a_capacity_takes_the_slab_path(zen, oracle):
     masked, kept = oracle.mask_dense(g_np, int(thr[0].item()))
     idx_o, val_o, splits_o, st_o = oracle.load_balance(masked, P, 1, 3)
     assert int(splits.sum()) == kept and np.array_equal(torch.cat(indices).cpu().numpy(), idx_o)
+
+
+def test_sample_taken_ahead_gives_the_same_result(zen, oracle):
+    """TensorPartition.prepare takes a top-k call's sample on another stream before the call: same bytes out
+    as without, over several calls in a row with the two sets of sampling memory in turn, also when a sample
+    is taken for a call that never comes (it is dropped), and the table is all zero afterwards."""
+    from zen_repro_amd import _lib
+
+    n, P = 1 << 25, 16
+    rng = np.random.default_rng(31)
+    side = torch.cuda.Stream()
+    tp = zen.TensorPartition(P, 1, 3)
+    grads, wants = [], []
+    for i in range(3):
+        g_np = oracle.f32_to_bf16_bits((rng.standard_normal(n) * 1e-3).astype(np.float32))
+        k = n // 200 + 1000 * i
+        key = oracle.kth_key(g_np, k)
+        masked, kept = oracle.mask_dense(g_np, key)
+        grads.append((to_dev(g_np), k, int(k * 1.25) + 4096))
+        wants.append(oracle.load_balance(masked, P, 1, 3))
+    torch.cuda.synchronize()
+    m, _ = tp.table_sizes(n)
+    assert _lib.lib().zen_load_balance_path(n, m, _lib.BF16, grads[0][2], P, grads[0][1], _lib.MODE_FAST) == 2
+
+    def check(out, want):
+        idx, val, splits, st = out
+        idx_o, val_o, splits_o, st_o = want
+        assert int(st.item()) == 0 and st_o == 0
+        total = int(splits.sum())
+        assert np.array_equal(splits.cpu().numpy(), splits_o)
+        assert np.array_equal(idx[:total].cpu().numpy(), idx_o) and np.array_equal(to_np(val[:total]), val_o)
+
+    # call i's sample is taken while call i - 1 is still being enqueued / running
+    with torch.cuda.stream(side):
+        tp.prepare(*grads[0])
+    outs = []
+    for i in range(6):
+        g, k, cap = grads[i % 3]
+        outs.append(tp.load_balance_flat(g, None, cap, k=k))
+        if i + 1 < 6:
+            with torch.cuda.stream(side):
+                tp.prepare(*grads[(i + 1) % 3])
+    for i, out in enumerate(outs):
+        check(out, wants[i % 3])
+    # a sample for a call that does not come: the next call (other tensor) drops it and samples for itself
+    with torch.cuda.stream(side):
+        tp.prepare(*grads[1])
+    g, k, cap = grads[2]
+    check(tp.load_balance_flat(g, None, cap, k=k), wants[2])
+    check(tp.load_balance_flat(grads[0][0], None, grads[0][2], k=grads[0][1]), wants[0])
+    torch.cuda.synchronize()
+    assert int(tp._table(g.device, m).count_nonzero()) == 0

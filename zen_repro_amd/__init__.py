@@ -6,3 +6,4 @@ from .functions import hash_index, last_status, sparse_balance  # noqa: F401
 from .tensor_load_balance import TensorPartition  # noqa: F401
 from .comm import LoadBalanceAllreduce, LocalGroup  # noqa: F401
 from .compress import compress, compress_with_allgather, topk_threshold  # noqa: F401
+from .hook import SparseCommHook  # noqa: F401

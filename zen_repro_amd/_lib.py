@@ -13,6 +13,7 @@ OK, EINVAL, EHIP, EWORKSPACE = 0, -1, -2, -3
 STAT_SERIAL_OVERFLOW, STAT_CAPACITY, STAT_INTERNAL, STAT_BAD_INDEX, STAT_RETRY = 1, 2, 4, 8, 16
 MODE_FAST, MODE_GENERAL = 0, 1
 MODE_ZEROED = 0x100  # zen_merge: the head of the workspace is zero (and stays so)
+MODE_PREPARED, MODE_SECOND, MODE_DISCARD = 0x200, 0x400, 0x800  # zen_load_balance: the sample was taken ahead (zen_load_balance_prepare)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # ZEN_HIP_LIB names another build of the library (a debug build, a build with other compile-time settings)
@@ -61,6 +62,7 @@ def lib():
         "zen_select": (i32, [vp, i32, i64, vp, vp, i32, vp, i64, vp, vp, sz, vp, vp]),
         "zen_load_balance_workspace": (sz, [i64, i64, i32, i64, i32]),
         "zen_load_balance": (i32, [vp, i32, i64, i64, i32, i32, vp, i64, vp, vp, vp, i64, vp, vp, i32, vp, sz, vp, vp]),
+        "zen_load_balance_prepare": (i32, [vp, i32, i64, i64, i32, i64, i64, vp, i32, vp, sz, vp]),
         "zen_load_balance_path": (i32, [i64, i64, i32, i64, i32, i64, i32]),
         "zen_merge_workspace": (sz, [i64, i64]),
         "zen_merge_path": (i32, [i64, i64, i32]),

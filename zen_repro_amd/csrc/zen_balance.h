@@ -140,6 +140,9 @@ struct SlabBalanceArgs {
   uint32_t hash_log2;
   void *workspace;            // slab_balance_bytes(...)
   int32_t *status;
+  int prepared = 0;           // 1 / 2: the sampled floor of the first / second set is there already (zen_load_balance_prepare)
+  bool only_prepare = false;  // take the sample for that set and nothing else
+  bool discard = false;       // with only_prepare: clear the set's sampling memory instead (a sample nobody picks up)
 };
 bool slab_balance_fits(int64_t n, int64_t m, int partitions, int dtype, int64_t capacity, int64_t k, SlabGeom *geo);
 size_t slab_balance_bytes(int64_t m, int partitions, int dtype, int64_t capacity);

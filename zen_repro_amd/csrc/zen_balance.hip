@@ -373,9 +373,55 @@ size_t zen_load_balance_workspace(int64_t n, int64_t m, int dtype, int64_t capac
 }
 
 int zen_load_balance_path(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions, int64_t k, int mode) {
+  mode &= 0xff;
   if (mode != ZEN_MODE_FAST || partitions <= 0 || m <= 0 || m % partitions != 0) return 0;
   if (zen::slab_balance_fits(n, m, partitions, dtype, capacity, k, nullptr)) return 2;
   return m >= 4096 ? 1 : 0;
+}
+
+namespace {
+
+// the head of the table belongs to the hash map; the megabyte behind it is left to the slab path's counters
+uint32_t slab_hash_log2(int64_t m) {
+  uint32_t log2 = 0;
+  while (log2 < 24 && (16ull << log2) + (1ull << 20) <= (uint64_t)m * sizeof(int32_t)) ++log2;
+  return log2;
+}
+
+}  // namespace
+
+int zen_load_balance_prepare(const void *input, int dtype, int64_t n, int64_t m, int partitions, int64_t k,
+                             int64_t capacity, int32_t *table, int mode, void *workspace, size_t workspace_bytes,
+                             void *stream) {
+  using namespace zen;
+  if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_load_balance_prepare: bad dtype");
+  if (n <= 0 || n > 0x7fffffffll || m <= 0 || m > 0x7fffffffll || partitions <= 0 || partitions > 65535 ||
+      m % partitions != 0 || capacity <= 0 || capacity > 0x1fffffffll || k < 0 || k > n)
+    return fail(ZEN_EINVAL, "zen_load_balance_prepare: sizes as for zen_load_balance");
+  if (!input || !table || !workspace) return fail(ZEN_EINVAL, "zen_load_balance_prepare: null pointer");
+  if (workspace_bytes < zen_load_balance_workspace(n, m, dtype, capacity, partitions))
+    return fail(ZEN_EWORKSPACE, "zen_load_balance_prepare: workspace too small");
+  const int second = (mode & ZEN_MODE_SECOND) != 0;
+  if ((mode & 0xff) != ZEN_MODE_FAST || k == 0 || (reinterpret_cast<uintptr_t>(table) & 7u) != 0 ||
+      !slab_balance_fits(n, m, partitions, dtype, capacity, k, nullptr))
+    return ZEN_OK;  // nothing to take ahead on the other paths
+  SlabBalanceArgs sa{};
+  sa.input = input;
+  sa.dtype = dtype;
+  sa.n = n;
+  sa.g.m = (uint32_t)m;
+  sa.g.npp = (uint32_t)(m / partitions);
+  sa.g.levels = 3;
+  sa.partitions = partitions;
+  sa.k = k;
+  sa.capacity = capacity;
+  sa.hash = reinterpret_cast<unsigned long long *>(table);
+  sa.hash_log2 = slab_hash_log2(m);
+  sa.workspace = workspace;
+  sa.prepared = second ? 2 : 1;
+  sa.only_prepare = true;
+  sa.discard = (mode & ZEN_MODE_DISCARD) != 0;
+  return slab_load_balance(sa, static_cast<hipStream_t>(stream));
 }
 
 int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
@@ -383,6 +429,8 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
                      int64_t capacity, int64_t *splits, int32_t *table, int mode, void *workspace,
                      size_t workspace_bytes, int32_t *status, void *stream) {
   using namespace zen;
+  const int prepared = (mode & ZEN_MODE_PREPARED) ? ((mode & ZEN_MODE_SECOND) ? 2 : 1) : 0;
+  mode &= ~(ZEN_MODE_PREPARED | ZEN_MODE_SECOND);
   if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_load_balance: bad dtype");
   if (mode != ZEN_MODE_FAST && mode != ZEN_MODE_GENERAL) return fail(ZEN_EINVAL, "zen_load_balance: bad mode");
   if (n <= 0 || n > 0x7fffffffll || m <= 0 || m > 0x7fffffffll || partitions <= 0 || partitions > 65535 ||
@@ -418,12 +466,10 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
     sa.capacity = capacity;
     sa.splits = splits;
     sa.hash = reinterpret_cast<unsigned long long *>(table);
-    // the map takes the head of the table; the megabyte behind it is left to the path's counters
-    uint32_t log2 = 0;
-    while (log2 < 24 && (16ull << log2) + (1ull << 20) <= (uint64_t)m * sizeof(int32_t)) ++log2;
-    sa.hash_log2 = log2;
+    sa.hash_log2 = slab_hash_log2(m);
     sa.workspace = workspace;
     sa.status = status;
+    sa.prepared = prepared;
     return slab_load_balance(sa, s);
   }
   BalancePlan p = plan_balance(workspace, n, m, dtype, capacity);

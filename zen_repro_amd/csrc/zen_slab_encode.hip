@@ -680,12 +680,14 @@ __global__ __launch_bounds__(kSlabBlock) void k_slab_place(SlabGeom geo, SlabTab
 
 struct SlabPlan {
   SlabTables tb;
-  uint32_t *sample_hist;  // sampled floor histogram (+ finished-block count)
+  uint32_t *sample_hist[2];  // sampled floor histogram (+ finished-block count); two sets, so that the sample of
+                             // the next call can be taken (zen_load_balance_prepare) while this call still runs
   uint32_t *cand_hist;
   uint32_t *ticket;
   CoarseGeom cg;
   FeedBuffers feed;
-  uint32_t *thr;          // [0..1] exact threshold + count, [2..3] sampled floor, [4] candidates above the k-th's bin
+  uint32_t *thr;          // [0..1] exact threshold + count, [2..3] sampled floor, [4] candidates above the k-th's bin,
+                          // [6..7] sampled floor of the second set
   uint32_t *refine_hist;  // fp32: histogram of the threshold's last 16 bits (+ finished-workgroup count)
   size_t state_bytes;     // of the zero-between-calls memory
   size_t bytes;           // of the workspace
@@ -697,7 +699,8 @@ SlabPlan plan_slab(void *workspace, void *state, const SlabGeom &geo, int partit
   const size_t B = geo.nbuckets;
   {
     Carver cv(state);
-    p.sample_hist = cv.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
+    p.sample_hist[0] = cv.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
+    p.sample_hist[1] = cv.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
     p.cand_hist = cv.take<uint32_t>((size_t)kCandHistWords);
     p.ticket = cv.take<uint32_t>(select_stage_ticket_words());
     p.tb.cursor = cv.take<uint32_t>(B * kCursorPad);
@@ -710,7 +713,7 @@ SlabPlan plan_slab(void *workspace, void *state, const SlabGeom &geo, int partit
     p.state_bytes = cv.used;
   }
   Carver cv(workspace);
-  p.thr = cv.take<uint32_t>(8);
+  p.thr = cv.take<uint32_t>(16);
   p.cg = coarse_geometry(geo, list_cap);
   p.feed.coarse_words = cv.take<uint32_t>(feed_coarse_words(p.cg, 2));
   p.tb.bucket_lo = cv.take<uint32_t>(B);
@@ -821,17 +824,31 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
   sc.ticket = p.ticket;
   sc.status = a.status;
   int rc;
+  const int set = a.prepared == 2 ? 1 : 0;
+  uint32_t *floor = p.thr + 2 + 4 * set;
+  if (a.only_prepare) {
+    if (a.discard) {  // a sample nobody will pick up: its histogram goes back to zero
+      launch_fill<uint32_t>(p.sample_hist[set], 0u, sampled_floor_zero_bytes() / sizeof(uint32_t), s);
+      ZEN_LAUNCH_CHECK("slab: discard a sample");
+      return ZEN_OK;
+    }
+    // the sample alone: the floor stays in the workspace until the call proper picks it up
+    if (a.k > 0) return topk_sampled_floor(a.input, a.dtype, a.n, a.k, floor, p.sample_hist[set], s, true);
+    return ZEN_OK;
+  }
   if (a.k > 0) {
     // one pass: everything at or above a floor estimated from a sample goes to the slabs, the exact
     // threshold is read off the candidates' histogram and applied when the buckets are sorted
-    if ((rc = topk_sampled_floor(a.input, a.dtype, a.n, a.k, p.thr + 2, p.sample_hist, s, true)) != ZEN_OK) return rc;
-    sc.thr = p.thr + 2;
+    if (!a.prepared &&
+        (rc = topk_sampled_floor(a.input, a.dtype, a.n, a.k, floor, p.sample_hist[set], s, true)) != ZEN_OK)
+      return rc;
+    sc.thr = floor;
     sc.cand_hist = p.cand_hist;
     sc.pick_k = a.k;
     sc.pick_thr = p.thr;
     sc.pick_above = p.thr + 4;
     sc.thr_copy = refine ? nullptr : a.thr_out;  // fp32: the threshold is not final yet
-    sc.clear = p.sample_hist;  // the sample kernel is through with its histogram
+    sc.clear = p.sample_hist[set];  // the sample kernel is through with its histogram
     sc.clear_words = (uint32_t)(sampled_floor_zero_bytes() / sizeof(uint32_t));
   }
   if ((rc = select_stage_slabs(sc, s)) != ZEN_OK) return rc;

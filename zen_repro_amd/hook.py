@@ -1,0 +1,56 @@
+"""The DDP communication hook of the reference's training driver
+(train.py:158-185) as a callable object: same arguments, same return value (a
+completed torch.futures.Future holding the tensor), same steps in the same
+order.  The exchanges belong to the LoadBalanceAllreduce's `ddp` backend, which
+this package does not ship: with a group of one rank (or no backend) the hook
+returns the compressed bucket, as the reference does when dp_group.size() == 1
+(train.py:178)."""
+import torch
+
+from .compress import compress_with_allgather
+
+
+class SparseCommHook:
+    """custom_comm_hook(state, bucket) of train.py:167-183.
+
+    load_balance_allreduce  the LoadBalanceAllreduce of the data-parallel group
+    top_k                   args.top_k: per cent of the sample kept (train.py:176)
+    method                  args.method: 1, 2 or 3 (comm.py:101-146)
+    tp_group                the group whose ranks share a threshold (train.py:176)
+    all_gather              callable(sample) -> samples of every rank of tp_group
+                            (dist.all_gather_into_tensor in the reference,
+                            train.py:63-64); needed only when tp_group has more
+                            than one rank
+    stream                  the side stream the path runs on (train.py:165);
+                            default priority
+    The first call passes the bucket through untouched (train.py:170-174)."""
+
+    def __init__(self, load_balance_allreduce, top_k, method, tp_group, all_gather=None, stream=None,
+                 sample_index=None):
+        self.lba = load_balance_allreduce
+        self.top_k = top_k
+        self.method = method
+        self.tp_group = tp_group
+        self.all_gather = all_gather
+        self.stream = stream if stream is not None else torch.cuda.Stream()
+        self.sample_index = sample_index  # callable(numel) -> int64 sample positions; None: drawn like the reference
+        self.skip = True
+
+    def __call__(self, state, bucket):
+        tensors = bucket.buffer()
+        future = torch.futures.Future()
+        if self.skip:
+            future.set_result(tensors)
+            self.skip = False
+            return future
+        with torch.cuda.stream(self.stream):
+            index = self.sample_index(tensors.numel()) if self.sample_index is not None else None
+            tensors_compressed = compress_with_allgather(self.top_k, tensors, self.tp_group, sample_index=index,
+                                                         all_gather=self.all_gather)
+            tensors = tensors_compressed
+            if self.lba.process_group.size() > 1 and getattr(self.lba, "ddp", None) is not None:
+                tensors = self.lba.zen_sparse_comm(tensors_compressed, self.method)
+        # like the reference, the future is completed at once: whoever consumes the result does so in the
+        # stream order of `self.stream` (train.py:181)
+        future.set_result(tensors)
+        return future

@@ -1,6 +1,8 @@
 """Drop-in for the reference's tensor_load_balance.py.  `load_balance` runs as
 one fused device pipeline (select, insert, slot-order compaction) instead of
 2P boolean-mask compactions with a host sync each."""
+import ctypes
+
 import torch
 
 from . import _lib
@@ -17,6 +19,7 @@ class TensorPartition:
         self.rehash = rehash
         self.device = torch.cuda.current_device()
         self._tables = {}
+        self._ahead = {}  # (device, slot) -> samples taken ahead of their calls (prepare)
 
     # ------------------------------------------------------------ sizes
     def table_sizes(self, numel):
@@ -92,6 +95,54 @@ class TensorPartition:
             return int(thr[1].item()) + 1024
         return int(torch.count_nonzero(flat)) + 1024
 
+    def _ahead_state(self, device, slot):
+        # "next": the set of sampling memory the next prepare takes (the second first: a call that samples for
+        # itself uses the first); "free": per set, the event after the last call that used it; "pending":
+        # samples taken and not yet picked up by their calls
+        key = (torch.device(device).index, slot)
+        state = self._ahead.get(key)
+        if state is None:
+            state = self._ahead[key] = {"next": 1, "free": [None, None], "pending": []}
+        return state
+
+    def prepare(self, tensor, k, capacity, slot=0):
+        """Takes the sample of a coming load_balance_flat(tensor, None, capacity,
+        k=k, slot=slot) ahead, on the CURRENT stream, which may be another one
+        than the call's: the sample then runs beside whatever the call's stream
+        is still busy with (the previous bucket's sort and placement) instead of
+        in front of the pass over the tensor.  The tensor must be ready in the
+        current stream's order.  The call that follows finds the sample by
+        itself (same tensor, k, capacity and slot) and waits for it; two samples
+        per slot can be ahead of their calls.  Where there is nothing to take
+        ahead (k == 0, small tensors) this does nothing."""
+        _lib.require_gpu(tensor, "input")
+        flat = tensor.reshape(-1)
+        n = flat.numel()
+        code = _lib.dtype_code(flat)
+        m, _ = self.table_sizes(n)
+        dev = flat.device
+        L = _lib.lib()
+        if k <= 0 or L.zen_load_balance_path(n, m, code, capacity, self.partitions, k, _lib.MODE_FAST) != 2:
+            return
+        state = self._ahead_state(dev, slot)
+        if len(state["pending"]) >= 2:
+            return  # both sets are spoken for
+        which = state["next"]
+        state["next"] ^= 1
+        stream = torch.cuda.current_stream(dev)
+        if state["free"][which] is not None:
+            stream.wait_event(state["free"][which])  # the call that used this set last has finished
+        nbytes = L.zen_load_balance_workspace(n, m, code, capacity, self.partitions)
+        ws = _lib.scratch.get(dev, f"load_balance/{slot}", nbytes)
+        table = self._table(dev, m, slot)
+        rc = L.zen_load_balance_prepare(_lib.ptr(flat), code, n, m, self.partitions, int(k), capacity, _lib.ptr(table),
+                                        _lib.MODE_FAST | (_lib.MODE_SECOND if which else 0), _lib.ptr(ws), ws.numel(),
+                                        _lib.stream_of(dev))
+        _lib.check(rc, "load_balance prepare")
+        done = torch.cuda.Event()
+        done.record(stream)
+        state["pending"].append((flat.data_ptr(), n, int(k), capacity, ws.data_ptr(), which, done))
+
     def load_balance_flat(self, tensor, thr=None, capacity=None, k=0, mode=_lib.MODE_FAST, thr_out=None, slot=0):
         """Fused path without host synchronisation.  Returns (indices int32
         [capacity], values [capacity], splits int64[P] on device, status int32[1]
@@ -122,11 +173,40 @@ class TensorPartition:
         nbytes = L.zen_load_balance_workspace(n, m, code, capacity, self.partitions)
         ws = _lib.scratch.get(dev, f"load_balance/{slot}", nbytes)
         table = self._table(dev, m, slot)
+        # a sample taken ahead for this very call (prepare)?
+        state = self._ahead_state(dev, slot)
+        ahead = None
+        if state["pending"]:
+            ahead = state["pending"].pop(0)
+            if ahead[:5] != (flat.data_ptr(), n, int(k), capacity, ws.data_ptr()) or mode != _lib.MODE_FAST or thr is not None:
+                # not for this call: its histogram is cleared again (with the arguments it was taken with) and
+                # the call samples for itself
+                cur = torch.cuda.current_stream(dev)
+                cur.wait_event(ahead[6])
+                a_ptr, a_n, a_k, a_cap, a_ws, a_which, _ = ahead
+                a_m, _ = self.table_sizes(a_n)
+                _lib.check(L.zen_load_balance_prepare(
+                    ctypes.c_void_p(a_ptr), code, a_n, a_m, self.partitions, a_k, a_cap,
+                    _lib.ptr(self._table(dev, a_m, slot)), _lib.MODE_FAST | _lib.MODE_DISCARD |
+                    (_lib.MODE_SECOND if a_which else 0), ctypes.c_void_p(a_ws), ws.numel(), _lib.stream_of(dev)),
+                    "load_balance discard")
+                ahead = None
+        flags = 0
+        if ahead is not None:
+            torch.cuda.current_stream(dev).wait_event(ahead[6])
+            flags = _lib.MODE_PREPARED | (_lib.MODE_SECOND if ahead[5] else 0)
         rc = L.zen_load_balance(
             _lib.ptr(flat), code, n, m, self.partitions, self.rehash, _lib.ptr(thr), int(k), _lib.ptr(thr_out),
-            _lib.ptr(out_idx), _lib.ptr(out_val), capacity, _lib.ptr(splits), _lib.ptr(table), mode,
+            _lib.ptr(out_idx), _lib.ptr(out_val), capacity, _lib.ptr(splits), _lib.ptr(table), mode | flags,
             _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
         _lib.check(rc, "load_balance")
+        if k > 0:
+            # whichever set of sampling memory this call used (a call that samples for itself uses the first)
+            # is free again once it has finished
+            used = ahead[5] if ahead is not None else 0
+            free = torch.cuda.Event()
+            free.record(torch.cuda.current_stream(dev))
+            state["free"][used] = free
         return out_idx, out_val, splits, status
 
     def load_balance(self, tensor, thr=None, capacity=None, k=0, mode=None):
