@@ -315,8 +315,9 @@ int zen_decode_dense_sorted(const void *idx, int idx64_in, const void *val, int 
  * all ranks followed by decode_sparse_tensors (comm.py:87-99, 136-145) without the indices, the member lists
  * (mapping) or a cleared dense tensor in between.
  *   zen_bitmap_dense_dict builds, once per (numel, partitions), what stands in for the mapping the reference
- * caches (comm.py:132-134): the partition id of every index (one byte) and per tile of 8192 indices the
- * members of every partition below it (zen_bitmap_dense_dict_bytes bytes, 16-byte aligned).  members, if not
+ * caches (comm.py:132-134): per tile of 8192 indices the places of the tile's indices ordered by partition (16
+ * bits each) and the members of every partition below the tile (zen_bitmap_dense_dict_bytes bytes, a little
+ * over two per element, 16-byte aligned).  members, if not
  * NULL, is a HOST array that receives the partitions' list lengths (this synchronises on the stream).
  *   zen_bitmap_dense: bitmaps / values hold the lists back to back, list p at byte bitmap_start[p] (of
  * bitmap_start[p + 1] - bitmap_start[p] bytes) and element value_start[p]; both offset arrays are HOST arrays

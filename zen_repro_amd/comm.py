@@ -291,8 +291,9 @@ class LoadBalanceAllreduce:
         rank i's bitmap over partition i's index list and the values of its set
         bits in order; returns the dense tensor of `numel` elements in the
         values' dtype.  Neither the index lists nor self.mapping are needed: a
-        dictionary of one byte per index (each index's partition) is built on
-        first use of a `numel` and cached like the reference caches the mapping
+        dictionary of two bytes per element (per tile of the dense tensor, the
+        places of its indices ordered by partition) is built on first use of a
+        `numel` and cached like the reference caches the mapping
         (comm.py:132-134)."""
         if len(bitmap_indices) != self.partitions or len(values_tensors) != self.partitions:
             raise RuntimeError("decode_bitmaps_dense: one bitmap and one value list per rank")
