@@ -55,6 +55,10 @@ def parse():
                          "(1 = a step starts when the previous one has finished)")
     ap.add_argument("--rotate", type=int, default=16,
                     help="at most this many copies of the inputs, used in turn (as many as make 512 MB)")
+    ap.add_argument("--graph", action="store_true",
+                    help="capture a step (encode, and the merge on its second stream) into a HIP graph per input copy "
+                         "and time replays: what a caller gets who hands the library's calls to a graph, without "
+                         "the host's share of every launch (matters for small buckets)")
     ap.add_argument("--imbalance", action="store_true", help="report the per-bucket load imbalance (always for c4)")
     ap.add_argument("--time-every", type=int, default=2,
                     help="in the timed region every n-th launch of the roofline kernel carries HIP events")
@@ -394,7 +398,7 @@ def main():
     # per bucket), and nothing in bucket i+1 depends on bucket i: with --depth 2 consecutive steps alternate
     # between two sets of streams, workspaces and tables ("slots"), so the long, memory-bound select of one
     # step runs next to the short, latency-bound kernels of the other.  All streams have default priority.
-    depth = 1 if args.one_stream else max(1, args.depth)
+    depth = 1 if (args.one_stream or args.graph) else max(1, args.depth)
     main = torch.cuda.current_stream(dev)
     enc_streams = [main] + [torch.cuda.Stream(device=dev) for _ in range(depth - 1)]
     mrg_streams = [None if (args.one_stream or args.merge_follows) else torch.cuda.Stream(device=dev)
@@ -403,11 +407,13 @@ def main():
     # The sample that gives a top-k call its floor only needs the tensor: the next step's is taken ahead on a
     # stream of its own, beside the current step's sort and placement, instead of in front of the next pass
     # over the tensor (a hook that is called per bucket can do the same as soon as it holds the next bucket).
-    prep_stream = None if (args.one_stream or args.no_prepare) else torch.cuda.Stream(device=dev)
+    prep_stream = None if (args.one_stream or args.no_prepare or args.graph) else torch.cuda.Stream(device=dev)
 
-    def step(i, more=True):
+    def step(i, more=True, es=None):
         slot = i % depth
-        es, ms_ = enc_streams[slot], mrg_streams[slot]
+        ms_ = mrg_streams[slot]
+        if es is None:
+            es = enc_streams[slot]
         enc, mrg = [], []
         with torch.cuda.stream(es):
             for j, b in enumerate(buckets):
@@ -471,13 +477,52 @@ def main():
         cands = [(stages[name][0], name) for name in streaming if name in stages]
         dom = max(cands)[1] if cands else None
         _lib.profile_enable(dom is not None, only=dom, every=every)
-    t0 = time.perf_counter()
-    outs = run(args.steps)
-    t_enq = time.perf_counter()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    kernels = _lib.profile_read() if dom else {}
-    _lib.profile_enable(False)
+    if args.graph:
+        # one graph per combination of input copies; a replay is the whole step: the encode on the graph's
+        # stream, the merge forked onto the second stream and joined again
+        _lib.profile_enable(False)
+        lens = [len(gs) for gs in grad_sets] + [len(fs) for fs in flat_sets]
+        rounds = max(lens)  # graph r reads copy r % len of every input
+        cap = torch.cuda.Stream(device=dev)
+        graphs, graph_outs = [], []
+        for r in range(rounds):
+            g_ = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g_, stream=cap):
+                cur = torch.cuda.current_stream(dev)
+                _lib.zeros.fresh(dev)  # this graph's status words and counts: a block of its own, zeroed by the graph
+                if mrg_streams[0] is not None:
+                    mrg_streams[0].wait_stream(cur)
+                    with torch.cuda.stream(mrg_streams[0]):
+                        _lib.zeros.fresh(dev)
+                graph_outs.append(step(r, more=False, es=cur))
+                if mrg_streams[0] is not None:
+                    cur.wait_stream(mrg_streams[0])
+            graphs.append(g_)
+        _lib.zeros.fresh(dev)
+        with torch.cuda.stream(cap):
+            _lib.zeros.fresh(dev)
+        if mrg_streams[0] is not None:
+            with torch.cuda.stream(mrg_streams[0]):
+                _lib.zeros.fresh(dev)  # later eager calls must not take pieces of a graph's block
+        for r in range(min(rounds, args.warmup)):
+            graphs[r].replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            graphs[i % rounds].replay()
+        t_enq = time.perf_counter()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        outs = [graph_outs[(args.steps - 1 - j) % rounds] for j in range(min(rounds, args.steps))][::-1]  # last: the last replay's
+        kernels = {dom: stages[dom]} if dom else {}  # the roofline kernel's duration: from the pass with events above
+    else:
+        t0 = time.perf_counter()
+        outs = run(args.steps)
+        t_enq = time.perf_counter()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        kernels = _lib.profile_read() if dom else {}
+        _lib.profile_enable(False)
 
     last = outs[-1]
     nnz = [int(enc[2].sum()) for enc, _ in last]
@@ -536,6 +581,8 @@ def main():
                     "measured_read_ceiling_GBps": round(ceiling, 1) if ceiling else None,
                     "frac_of_read_ceiling": round(achieved / ceiling, 4) if ceiling else None}
 
+    if roofline and args.graph:
+        roofline["timed_in"] = "the untimed pass with every stage's events on (graph replays carry no events)"
     line = {
         "metric": "encode+decode dense-gradient GB/s on 1 GPU; % of HBM roofline",
         "value": round(value, 2),
@@ -553,7 +600,7 @@ def main():
                    "buckets": [{"name": b.name, "elements": b.n, "k": b.k, "selected": nnz[j],
                                 "received": flats[j][0].numel(), "merged": merged[j]} for j, b in enumerate(buckets)],
                    "k": sum(b.k for b in buckets), "selected": sum(nnz), "received": received, "merged": sum(merged),
-                   "peers": cfg.peers, "overlap": cfg.overlap, "shrink": args.shrink, "steps_in_flight": depth,
+                   "peers": cfg.peers, "overlap": cfg.overlap, "shrink": args.shrink, "steps_in_flight": depth, "replayed_from_graph": bool(args.graph),
                    "input_copies": {"gradient": len(grad_sets[0]), "payloads": len(flat_sets[0])}},
         "path_algorithmic_GBps": round(b_alg / (ms * 1e-3) / 1e9, 2),
         "path_frac_of_hbm_peak": round(b_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),

@@ -198,6 +198,17 @@ class ZeroPool:
         return entry[0][at:at + nbytes].view(dtype)
 
 
+    def fresh(self, device):
+        """Forget the current stream's block: the next piece comes from a new one.  Call this at the start of
+        every HIP graph capture: the block made inside the capture, fill included, then belongs to that graph
+        alone (its replays put its own status words and counts back to zero and nobody else's)."""
+        dev = torch.device(device)
+        index = dev.index if dev.index is not None else torch.cuda.current_device()
+        blocks = getattr(self._local, "blocks", None)
+        if blocks is not None:
+            blocks.pop((index, torch.cuda.current_stream(dev).cuda_stream), None)
+
+
 zeros = ZeroPool()
 
 

@@ -18,7 +18,10 @@
 namespace zen {
 namespace {
 
-constexpr int kFdTile = 8192;
+#ifndef ZEN_FD_TILE
+#define ZEN_FD_TILE 8192
+#endif
+constexpr int kFdTile = ZEN_FD_TILE;
 constexpr int kFdBlock = 512;
 constexpr int kFdPer = kFdTile / kFdBlock;   // consecutive indices per thread (16)
 constexpr int kFdMaxLists = 64;
@@ -209,8 +212,8 @@ __device__ inline uint32_t fd_value<uint32_t>(uint32_t v) {
 // threads take one SET bit each: its member's place in the tile is one entry of the dictionary, the value goes
 // there, into a copy of the tile in LDS that is written out once.  The next tile's table entries are asked for
 // while this tile is worked on.
-constexpr int kFdValStage = 1024;  // values of a tile kept in LDS (tiles with more set bits fetch the rest one by one)
-constexpr int kFdHitStage = 1024;  // set bits of a tile listed at a time
+constexpr int kFdValStage = kFdTile / 8;  // values of a tile kept in LDS (tiles with more set bits fetch the rest one by one)
+constexpr int kFdHitStage = kFdTile / 8;  // set bits of a tile listed at a time
 constexpr int kFdBytesPer = (kFdMaxBytes + kFdBlock - 1) / kFdBlock;  // 3
 constexpr int kFdValsPer = kFdValStage / kFdBlock;                    // 2
 #ifndef ZEN_FD_MIN_WAVES
