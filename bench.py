@@ -48,10 +48,12 @@ def parse():
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
     ap.add_argument("--no-prepare", action="store_true",
                     help="do not take the next step's sample ahead on a stream of its own")
-    ap.add_argument("--merge-follows", action="store_true",
-                    help="with --depth: a step's merge runs on its encode's stream, after it")
-    ap.add_argument("--depth", type=int, default=1,
-                    help="gradient buckets in flight: step i+1 is enqueued on its own streams next to step i "
+    ap.add_argument("--merge-beside", action="store_true",
+                    help="with --depth 2 or more: a step's merge runs on a stream of its own beside its encode "
+                         "(default there: on its encode's stream, after it; at --depth 1 it always runs beside)")
+    ap.add_argument("--depth", type=int, default=2,
+                    help="steps in flight: step i+1 is enqueued on its own stream next to step i, as a training "
+                         "step hands over one gradient bucket after the other "
                          "(1 = a step starts when the previous one has finished)")
     ap.add_argument("--rotate", type=int, default=16,
                     help="at most this many copies of the inputs, used in turn (as many as make 512 MB)")
@@ -393,15 +395,17 @@ def main():
     pay_bytes = sum(fi.numel() * (4 + esize) for fi, _ in flats)
     flat_sets = [[(fi, fv)] + [(fi.clone(), fv.clone()) for _ in range(copies_of(pay_bytes) - 1)] for fi, fv in flats]
 
-    # The merge of the received payloads does not depend on this rank's own encode, so it runs on a second
-    # stream.  A training step hands over one gradient bucket after the other (train.py:167-185 is called
-    # per bucket), and nothing in bucket i+1 depends on bucket i: with --depth 2 consecutive steps alternate
-    # between two sets of streams, workspaces and tables ("slots"), so the long, memory-bound select of one
-    # step runs next to the short, latency-bound kernels of the other.  All streams have default priority.
+    # A training step hands over one gradient bucket after the other (train.py:167-185 is called per bucket),
+    # and nothing in bucket i+1 depends on bucket i: by default two consecutive steps are in flight, alternating
+    # between two streams, workspaces and tables ("slots"), each step's merge behind its encode on the step's
+    # own stream, so that the long, memory-bound select of one step runs next to the short, latency-bound
+    # kernels of the other.  At --depth 1 a step starts when the one before has finished, and its merge, which
+    # does not depend on its encode, runs beside it on a second stream.  All streams have default priority.
     depth = 1 if (args.one_stream or args.graph) else max(1, args.depth)
     main = torch.cuda.current_stream(dev)
     enc_streams = [main] + [torch.cuda.Stream(device=dev) for _ in range(depth - 1)]
-    mrg_streams = [None if (args.one_stream or args.merge_follows) else torch.cuda.Stream(device=dev)
+    merge_follows = depth > 1 and not args.merge_beside
+    mrg_streams = [None if (args.one_stream or merge_follows) else torch.cuda.Stream(device=dev)
                    for _ in range(depth)]
 
     # The sample that gives a top-k call its floor only needs the tensor: the next step's is taken ahead on a
@@ -600,7 +604,8 @@ def main():
                    "buckets": [{"name": b.name, "elements": b.n, "k": b.k, "selected": nnz[j],
                                 "received": flats[j][0].numel(), "merged": merged[j]} for j, b in enumerate(buckets)],
                    "k": sum(b.k for b in buckets), "selected": sum(nnz), "received": received, "merged": sum(merged),
-                   "peers": cfg.peers, "overlap": cfg.overlap, "shrink": args.shrink, "steps_in_flight": depth, "replayed_from_graph": bool(args.graph),
+                   "peers": cfg.peers, "overlap": cfg.overlap, "shrink": args.shrink, "steps_in_flight": depth, "merge_runs": "behind its step's encode" if (merge_follows or args.one_stream) else "beside its step's encode",
+                   "replayed_from_graph": bool(args.graph),
                    "input_copies": {"gradient": len(grad_sets[0]), "payloads": len(flat_sets[0])}},
         "path_algorithmic_GBps": round(b_alg / (ms * 1e-3) / 1e9, 2),
         "path_frac_of_hbm_peak": round(b_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),

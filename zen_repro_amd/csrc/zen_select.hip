@@ -1100,7 +1100,10 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   if (subs > 0x3fffffff) return fail(ZEN_EINVAL, "select_stage: tensor too large");
   // three workgroups per compute unit (measured: two are 10 % slower, four no faster); their LDS, 60 KB per
   // unit, leaves room for another stream's kernels next to this long one
-  int64_t blocks = (int64_t)device_cus() * 3;
+#ifndef ZEN_STAGE_WGS
+#define ZEN_STAGE_WGS 3
+#endif
+  int64_t blocks = (int64_t)device_cus() * ZEN_STAGE_WGS;
   const int64_t least = ceil_div(subs, kStageSmall);
   if (blocks > least) blocks = least;
   // seven eighths of the tensor in counter-free tiles, the rest through tickets (measured on 1.5 GB: all
