@@ -436,3 +436,72 @@ def test_sample_taken_ahead_gives_the_same_result(zen, oracle):
     check(tp.load_balance_flat(grads[0][0], None, grads[0][2], k=grads[0][1]), wants[0])
     torch.cuda.synchronize()
     assert int(tp._table(g.device, m).count_nonzero()) == 0
+
+
+def test_step_replayed_from_a_captured_graph(zen, oracle):
+    """An encode (fused top-k) and a merge captured into a HIP graph, the merge forked onto a second stream:
+    every replay, with eager calls on the same workspaces and a synchronisation in between, leaves the bytes
+    the eager call leaves (the calls record kernels only: nothing a replay would skip or do twice)."""
+    from zen_repro_amd import _lib
+
+    n, P = 1 << 25, 16
+    rng = np.random.default_rng(41)
+    g_np = oracle.f32_to_bf16_bits((rng.standard_normal(n) * 1e-3).astype(np.float32))
+    k = n // 200
+    cap = int(k * 1.25) + 4096
+    key = oracle.kth_key(g_np, k)
+    masked, _ = oracle.mask_dense(g_np, key)
+    idx_o, val_o, splits_o, st_o = oracle.load_balance(masked, P, 1, 3)
+    per_peer = k // P
+    peers_i = [rng.choice(n - 1, per_peer, replace=False).astype(np.int32) + 1 for _ in range(P)]
+    flat_i = np.concatenate(peers_i)
+    flat_v = oracle.f32_to_bf16_bits((rng.standard_normal(flat_i.size) * 1e-3).astype(np.float32))
+    want_i, want_v = oracle.merge_sparse(flat_i, flat_v, n)
+    grad, fi, fv = to_dev(g_np), to_dev(flat_i), to_dev(flat_v)
+    tp = zen.TensorPartition(P, 1, 3)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P), None, None)
+    m, _ = tp.table_sizes(n)
+    assert _lib.lib().zen_load_balance_path(n, m, _lib.BF16, cap, P, k, _lib.MODE_FAST) == 2
+    assert _lib.lib().zen_merge_path(flat_i.size, n, _lib.MODE_FAST) == 2
+
+    def check(enc, mrg):
+        idx, val, splits, st = enc
+        m_idx, m_val, m_count, m_st = mrg
+        assert int(st.item()) == 0 and int(m_st.item()) == 0
+        total = int(splits.sum())
+        assert np.array_equal(splits.cpu().numpy(), splits_o)
+        assert np.array_equal(idx[:total].cpu().numpy(), idx_o) and np.array_equal(to_np(val[:total]), val_o)
+        u = int(m_count.item())
+        assert u == len(want_i) and np.array_equal(m_idx[:u].cpu().numpy(), want_i.astype(np.int32))
+        assert np.array_equal(m_val[:u].cpu().numpy().view(np.uint32), want_v.view(np.uint32))
+
+    def eager():
+        return (tp.load_balance_flat(grad, None, cap, k=k),
+                lba.merge_sparse_flat(fi, fv, n, capacity=flat_i.size))
+
+    check(*eager())  # also makes the workspaces, outside the capture
+    torch.cuda.synchronize()
+    side, cap_stream = torch.cuda.Stream(), torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=cap_stream):
+        cur = torch.cuda.current_stream()
+        _lib.zeros.fresh(grad.device)
+        side.wait_stream(cur)
+        enc = tp.load_balance_flat(grad, None, cap, k=k)
+        with torch.cuda.stream(side):
+            _lib.zeros.fresh(grad.device)
+            mrg = lba.merge_sparse_flat(fi, fv, n, capacity=flat_i.size)
+        cur.wait_stream(side)
+    _lib.zeros.fresh(grad.device)
+    for s_ in (side, cap_stream):
+        with torch.cuda.stream(s_):
+            _lib.zeros.fresh(grad.device)
+    for _ in range(3):
+        enc[0].fill_(-1)
+        mrg[0].fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        check(enc, mrg)
+        check(*eager())  # the same tables and workspaces, between two replays
+        torch.cuda.synchronize()
+    assert int(tp._table(grad.device, m).count_nonzero()) == 0
