@@ -158,6 +158,18 @@ struct SlabSortSharedT<true> {
   uint32_t bad;
 };
 
+// The same sharing of memory without the queue (the queue's code costs slab_rank registers).
+struct SlabSortSharedNoQueue {
+  static constexpr bool kQueue = false;
+  uint32_t key[kSlabCap];
+  union {
+    uint32_t tie[kSlabCap];
+    uint32_t cnt[kSlabSubs + 1];
+  };
+  uint32_t scan[kSlabMaxBlock / 64 + 1];
+  uint32_t bad;
+};
+
 static_assert(kSlabSubs + 1 <= kSlabCap, "the counters fit under the ties");
 using SlabSortShared = SlabSortSharedT<false>;
 

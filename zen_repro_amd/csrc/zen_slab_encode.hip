@@ -193,7 +193,9 @@ constexpr int kSortItems = kSlabCap / kSortBlock;
 
 template <typename S>
 __global__ __launch_bounds__(kSortBlock, 8) void k_slab_sort(SlabGeom geo, SlabTables tb, int32_t *status) {
-  __shared__ SlabSortShared sh;
+  // the ties take the place of the counters once the ranks are known: with 32-bit values the kernel would
+  // otherwise need 88 KB of LDS, one workgroup to a compute unit instead of two
+  __shared__ SlabSortSharedNoQueue sh;
   __shared__ S s_val[kSlabCap];
   __shared__ uint32_t s_lost, s_base;
   const uint32_t b = blockIdx.x;
@@ -243,9 +245,10 @@ __global__ __launch_bounds__(kSortBlock, 8) void k_slab_sort(SlabGeom geo, SlabT
   // every thread has read the slab's fill count (slab_rank synchronised); this workgroup was its only reader
   if (threadIdx.x == 0) tb.cursor[b * kCursorPad] = 0;
   // the counters hold where every narrow range starts in the sorted bucket: every kSlabIndexStep-th goes to
-  // the index (before the counters' memory is used for the list of losers below)
+  // the index (before the counters' memory is used for the ties below)
   for (int j = threadIdx.x; j < kSlabIndexLen; j += kSortBlock)
     tb.sub_index[(size_t)b * kSlabIndexLen + j] = (uint16_t)sh.cnt[sub_place<kSortBlock>((uint32_t)j * kSlabIndexStep)];
+  __syncthreads();
 #pragma unroll
   for (int i = 0; i < kSortItems; ++i) {
     if (live & (1u << i)) {
@@ -274,16 +277,26 @@ __global__ __launch_bounds__(kSortBlock, 8) void k_slab_sort(SlabGeom geo, SlabT
   }
   __syncthreads();
   // In a run of equal slots the first entry has the smallest index: the slot's level-1 owner.  The others
-  // lost level 1.  Their places in the sorted slab are collected in sh.cnt (a bucket has at most kSlabSubs
-  // of them, else the call is declined).
-  for (uint32_t p = threadIdx.x; p < n; p += kSortBlock) {
-    const uint32_t k = sh.key[p];
-    const bool lost = p > 0 && sh.key[p - 1] == k;
-    tb.slab_idx[base + p] = (int32_t)(sh.tie[p] | (lost ? kRemovedBit : 0u));
-    slab_val[base + p] = s_val[p];  // every thread has read its records: in place is safe
-    if (lost) {
+  // lost level 1.  Their places in the sorted slab are collected where the slots were, once every thread has
+  // looked at those (a bucket has at most kSlabSubs of them, else the call is declined).
+  uint32_t lost_mask = 0;
+#pragma unroll 1
+  for (int i = 0; i < kSortItems; ++i) {
+    const uint32_t p = threadIdx.x + (uint32_t)i * kSortBlock;
+    if (p < n) {
+      const uint32_t k = sh.key[p];
+      const bool lost = p > 0 && sh.key[p - 1] == k;
+      tb.slab_idx[base + p] = (int32_t)(sh.tie[p] | (lost ? kRemovedBit : 0u));
+      slab_val[base + p] = s_val[p];  // every thread has read its records: in place is safe
+      lost_mask |= lost ? 1u << i : 0u;
+    }
+  }
+  __syncthreads();
+#pragma unroll 1
+  for (int i = 0; i < kSortItems; ++i) {
+    if (lost_mask & (1u << i)) {
       const uint32_t at = atomicAdd(&s_lost, 1u);
-      if (at < (uint32_t)kSlabSubs) sh.cnt[at] = p;
+      if (at < (uint32_t)kSlabSubs) sh.key[at] = threadIdx.x + (uint32_t)i * kSortBlock;
     }
   }
   __syncthreads();
@@ -300,7 +313,7 @@ __global__ __launch_bounds__(kSortBlock, 8) void k_slab_sort(SlabGeom geo, SlabT
   __syncthreads();
   for (uint32_t i = threadIdx.x; i < lost_n; i += kSortBlock) {
     const uint32_t at = s_base + i;
-    const uint32_t p = sh.cnt[i];
+    const uint32_t p = sh.key[i];
     if (at < tb.log_cap) {
       tb.log_t[at] = sh.tie[p];
       tb.log_v[at] = (uint32_t)s_val[p];
