@@ -75,7 +75,7 @@ class TensorPartition:
         few different sizes come round again and again (the hook is called per
         bucket, train.py:167-185), so a handful of tables is kept, least
         recently used first out."""
-        key = (torch.device(device), m, slot)
+        key = (device if isinstance(device, torch.device) else torch.device(device), m, slot)
         t = self._tables.pop(key, None)
         if t is None:
             while len(self._tables) >= self._MAX_TABLES:
@@ -95,13 +95,16 @@ class TensorPartition:
             return int(thr[1].item()) + 1024
         return int(torch.count_nonzero(flat)) + 1024
 
-    def _ahead_state(self, device, slot):
+    def _ahead_state(self, device, slot, create=False):
         # "next": the set of sampling memory the next prepare takes (the second first: a call that samples for
         # itself uses the first); "free": per set, the event after the last call that used it; "pending":
         # samples taken and not yet picked up by their calls
-        key = (torch.device(device).index, slot)
+        key = (_lib.device_index(device), slot)
         state = self._ahead.get(key)
-        if state is None:
+        if state is None and create:
+            # Calls made before the first prepare left no events behind (a call only keeps this book once
+            # samples are taken ahead for its slot): wait for them all, once.
+            torch.cuda.synchronize(device)
             state = self._ahead[key] = {"next": 1, "free": [None, None], "pending": []}
         return state
 
@@ -124,7 +127,7 @@ class TensorPartition:
         L = _lib.lib()
         if k <= 0 or L.zen_load_balance_path(n, m, code, capacity, self.partitions, k, _lib.MODE_FAST) != 2:
             return
-        state = self._ahead_state(dev, slot)
+        state = self._ahead_state(dev, slot, create=True)
         if len(state["pending"]) >= 2:
             return  # both sets are spoken for
         which = state["next"]
@@ -174,9 +177,9 @@ class TensorPartition:
         ws = _lib.scratch.get(dev, f"load_balance/{slot}", nbytes)
         table = self._table(dev, m, slot)
         # a sample taken ahead for this very call (prepare)?
-        state = self._ahead_state(dev, slot)
+        state = self._ahead_state(dev, slot)  # None: no sample was ever taken ahead for this slot
         ahead = None
-        if state["pending"]:
+        if state is not None and state["pending"]:
             ahead = state["pending"].pop(0)
             if ahead[:5] != (flat.data_ptr(), n, int(k), capacity, ws.data_ptr()) or mode != _lib.MODE_FAST or thr is not None:
                 # not for this call: its histogram is cleared again (with the arguments it was taken with) and
@@ -200,7 +203,7 @@ class TensorPartition:
             _lib.ptr(out_idx), _lib.ptr(out_val), capacity, _lib.ptr(splits), _lib.ptr(table), mode | flags,
             _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
         _lib.check(rc, "load_balance")
-        if k > 0:
+        if k > 0 and state is not None:
             # whichever set of sampling memory this call used (a call that samples for itself uses the first)
             # is free again once it has finished
             used = ahead[5] if ahead is not None else 0
