@@ -57,6 +57,9 @@ def parse():
                          "(1 = a step starts when the previous one has finished)")
     ap.add_argument("--rotate", type=int, default=16,
                     help="at most this many copies of the inputs, used in turn (as many as make 512 MB)")
+    ap.add_argument("--near-threshold", action="store_true",
+                    help="top-k steps are handed the threshold key the warm-up found for their bucket (in training: "
+                         "the previous iteration's) and take no sample: one kernel less per bucket")
     ap.add_argument("--graph", action="store_true",
                     help="capture a step (encode, and the merge on its second stream) into a HIP graph per input copy "
                          "and time replays: what a caller gets who hands the library's calls to a graph, without "
@@ -411,7 +414,12 @@ def main():
     # The sample that gives a top-k call its floor only needs the tensor: the next step's is taken ahead on a
     # stream of its own, beside the current step's sort and placement, instead of in front of the next pass
     # over the tensor (a hook that is called per bucket can do the same as soon as it holds the next bucket).
-    prep_stream = None if (args.one_stream or args.no_prepare or args.graph) else torch.cuda.Stream(device=dev)
+    prep_stream = (None if (args.one_stream or args.no_prepare or args.graph or args.near_threshold)
+                   else torch.cuda.Stream(device=dev))
+
+    warm_thr = [torch.zeros(2, dtype=torch.int32, device=dev) for _ in buckets]
+    near_keys = [None for _ in buckets]
+    warm = False
 
     def step(i, more=True, es=None):
         slot = i % depth
@@ -422,7 +430,8 @@ def main():
         with torch.cuda.stream(es):
             for j, b in enumerate(buckets):
                 g = grad_sets[j][i % len(grad_sets[j])]
-                enc.append(tp.load_balance_flat(g, None, caps[j], k=b.k, slot=slot))
+                enc.append(tp.load_balance_flat(g, None, caps[j], k=b.k, slot=slot, thr_out=warm_thr[j] if warm else None,
+                                                near=near_keys[j]))
         if prep_stream is not None and more and depth == 1:
             with torch.cuda.stream(prep_stream):
                 for j, b in enumerate(buckets):
@@ -446,8 +455,12 @@ def main():
         return outs
 
     note("warm-up")
-    run(args.warmup)
+    warm = True
+    run(max(1, args.warmup))
     torch.cuda.synchronize()
+    warm = False
+    if args.near_threshold:
+        near_keys = [warm_thr[j].clone() if b.k else None for j, b in enumerate(buckets)]
     note("timing")
 
     # what a read-only pass over the gradient reaches on this box (plain non-temporal streaming loads)
@@ -606,6 +619,7 @@ def main():
                    "k": sum(b.k for b in buckets), "selected": sum(nnz), "received": received, "merged": sum(merged),
                    "peers": cfg.peers, "overlap": cfg.overlap, "shrink": args.shrink, "steps_in_flight": depth, "merge_runs": "behind its step's encode" if (merge_follows or args.one_stream) else "beside its step's encode",
                    "replayed_from_graph": bool(args.graph),
+                   "topk_sample": "none: the warm-up's threshold key is handed over" if args.near_threshold else "taken in every step",
                    "input_copies": {"gradient": len(grad_sets[0]), "payloads": len(flat_sets[0])}},
         "path_algorithmic_GBps": round(b_alg / (ms * 1e-3) / 1e9, 2),
         "path_frac_of_hbm_peak": round(b_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),

@@ -60,6 +60,12 @@ extern "C" {
 #define ZEN_MODE_PREPARED 0x200
 #define ZEN_MODE_SECOND 0x400
 #define ZEN_MODE_DISCARD 0x800 /* zen_load_balance_prepare: drop a sample that no call will pick up */
+/* OR-ed into the `mode` of zen_load_balance with k > 0: thr[0] is a key close to the k-th largest magnitude, for
+   example what an earlier call on a gradient of the same kind wrote to thr_out.  The call then takes no sample:
+   it lists everything from a little below that key (4/128 of its power of two) and picks the exact k-th
+   largest among those.  If fewer than k elements qualify, or far too many, ZEN_STAT_RETRY is raised as when a
+   sample misleads.  Paths that do not sample ignore the key. */
+#define ZEN_MODE_FLOOR 0x1000
 
 int zen_abi_version(void);
 
@@ -210,8 +216,8 @@ int zen_select(const void *input, int dtype, int64_t n, const uint32_t *thr,
  * thr != NULL or k > 0, compress (train.py:75-84) in front of it.
  * Selection: thr == NULL and k == 0: the nonzero elements; thr != NULL: key >=
  * max(thr[0], 1); k > 0: the k largest magnitudes, ties at the k-th kept (thr
- * must be NULL; thr_out, if not NULL, receives that key and the number
- * selected).  In ZEN_MODE_FAST the k-th largest is found with one pass over
+ * must be NULL unless ZEN_MODE_FLOOR says what it is; thr_out, if not NULL,
+ * receives that key and the number selected).  In ZEN_MODE_FAST the k-th largest is found with one pass over
  * the tensor (sampled floor, exact refinement among the candidates); if the
  * sample misleads, ZEN_STAT_RETRY is raised and nothing valid is produced.
  * Output: out_idx / out_val hold partition 0's entries, then partition 1's,

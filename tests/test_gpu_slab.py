@@ -505,3 +505,58 @@ def test_step_replayed_from_a_captured_graph(zen, oracle):
         check(*eager())  # the same tables and workspaces, between two replays
         torch.cuda.synchronize()
     assert int(tp._table(grad.device, m).count_nonzero()) == 0
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_threshold_of_an_earlier_call_replaces_the_sample(zen, oracle, dtype):
+    """load_balance_flat(..., k, near=thr_out of an earlier call): no sample kernel, same bytes out, on the
+    same gradient and on gradients a few per cent larger and smaller; a key that is far off (the gradient
+    halved or doubled) makes the call decline (STAT_RETRY) or still gives the exact answer, never a wrong one."""
+    from zen_repro_amd import _lib
+
+    n, P = 1 << 24, 16
+    rng = np.random.default_rng(53)
+    base = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    k = n // 200
+    cap = int(k * 1.25) + 4096
+    tp = zen.TensorPartition(P, 1, 3)
+    m, _ = tp.table_sizes(n)
+    code = _lib.BF16 if dtype == "bf16" else _lib.F32
+    assert _lib.lib().zen_load_balance_path(n, m, code, cap, P, k, _lib.MODE_FAST) == 2
+
+    def bits(x):
+        return oracle.f32_to_bf16_bits(x) if dtype == "bf16" else x
+
+    def want(g_np):
+        key = oracle.kth_key(g_np, k)
+        masked, _ = oracle.mask_dense(g_np, key)
+        return key, oracle.load_balance(masked, P, 1, 3)
+
+    g0 = bits(base)
+    thr_out = torch.zeros(2, dtype=torch.int32, device="cuda")
+    g0_dev = to_dev(g0)
+    dev = g0_dev.device
+    first = tp.load_balance_flat(g0_dev, None, cap, k=k, thr_out=thr_out)
+    key0, w0 = want(g0)
+    assert int(first[3].item()) == 0 and int(thr_out[0].item()) == key0
+    near = thr_out.clone()
+    exact = 0
+    for scale in (1.0, 1.02, 0.98, 0.5, 2.0):
+        g_np = bits((base * np.float32(scale)).astype(np.float32))
+        key, (idx_o, val_o, splits_o, st_o) = want(g_np)
+        thr_now = torch.zeros(2, dtype=torch.int32, device="cuda")
+        idx, val, splits, st = tp.load_balance_flat(to_dev(g_np), None, cap, k=k, thr_out=thr_now, near=near)
+        status = int(st.item())
+        if status & (_lib.STAT_RETRY | _lib.STAT_INTERNAL):
+            assert scale in (0.5, 2.0), f"declined at scale {scale}"
+            tp._table(dev, m).zero_()  # a declined call leaves the table for its caller to clear
+            continue
+        assert status == 0 and st_o == 0
+        total = int(splits.sum())
+        assert int(thr_now[0].item()) == key
+        assert np.array_equal(splits.cpu().numpy(), splits_o)
+        assert np.array_equal(idx[:total].cpu().numpy(), idx_o) and np.array_equal(to_np(val[:total]), val_o)
+        exact += 1
+    assert exact >= 3
+    torch.cuda.synchronize()
+    assert int(tp._table(dev, m).count_nonzero()) == 0

@@ -140,6 +140,7 @@ struct SlabBalanceArgs {
   uint32_t hash_log2;
   void *workspace;            // slab_balance_bytes(...)
   int32_t *status;
+  const uint32_t *near_key = nullptr;  // optional, k > 0: a key close to the k-th largest (no sample is taken)
   int prepared = 0;           // 1 / 2: the sampled floor of the first / second set is there already (zen_load_balance_prepare)
   bool only_prepare = false;  // take the sample for that set and nothing else
   bool discard = false;       // with only_prepare: clear the set's sampling memory instead (a sample nobody picks up)

@@ -430,7 +430,13 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
                      size_t workspace_bytes, int32_t *status, void *stream) {
   using namespace zen;
   const int prepared = (mode & ZEN_MODE_PREPARED) ? ((mode & ZEN_MODE_SECOND) ? 2 : 1) : 0;
-  mode &= ~(ZEN_MODE_PREPARED | ZEN_MODE_SECOND);
+  const uint32_t *near_key = nullptr;
+  if (mode & ZEN_MODE_FLOOR) {
+    if (k <= 0 || !thr) return fail(ZEN_EINVAL, "zen_load_balance: ZEN_MODE_FLOOR needs k > 0 and the key in thr");
+    near_key = thr;
+    thr = nullptr;  // paths that take no sample have no use for it
+  }
+  mode &= ~(ZEN_MODE_PREPARED | ZEN_MODE_SECOND | ZEN_MODE_FLOOR);
   if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_load_balance: bad dtype");
   if (mode != ZEN_MODE_FAST && mode != ZEN_MODE_GENERAL) return fail(ZEN_EINVAL, "zen_load_balance: bad mode");
   if (n <= 0 || n > 0x7fffffffll || m <= 0 || m > 0x7fffffffll || partitions <= 0 || partitions > 65535 ||
@@ -469,7 +475,8 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
     sa.hash_log2 = slab_hash_log2(m);
     sa.workspace = workspace;
     sa.status = status;
-    sa.prepared = prepared;
+    sa.prepared = near_key ? 0 : prepared;
+    sa.near_key = near_key;
     return slab_load_balance(sa, s);
   }
   BalancePlan p = plan_balance(workspace, n, m, dtype, capacity);

@@ -102,6 +102,7 @@ struct StageArgs {
   int dtype = ZEN_F32;
   int64_t n = 0;
   const uint32_t *thr = nullptr;
+  uint32_t floor_margin = 0;        // what is taken off thr[0] (a key near the threshold, not a floor below it)
   SlabGeom geo;                     // buckets of the level-1 hash slots
   CoarseGeom cg;
   uint32_t *coarse_cursor = nullptr;

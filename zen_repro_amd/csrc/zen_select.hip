@@ -843,7 +843,7 @@ template <typename S, bool ALIGNED>
 __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
     const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, StageSlabs out, uint32_t *ticket,
     StageSched sch, uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *pick_above,
-    uint32_t *thr_copy, uint32_t *clear, uint32_t clear_words, int32_t *status) {
+    uint32_t *thr_copy, uint32_t *clear, uint32_t clear_words, uint32_t floor_margin, int32_t *status) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kSub = kSelBlock * kSelVecs * V;
   constexpr int kWaves = kSelBlock / 64;
@@ -862,6 +862,7 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
   if (hist)
     for (int i = threadIdx.x; i < kCandBins; i += kSelBlock) s_hist[i] = 0;
   uint32_t floor_key = thr ? thr[0] : 1u;
+  floor_key = floor_key > floor_margin ? floor_key - floor_margin : 1u;
   if (floor_key == 0) floor_key = 1u;  // zeros are never selected
   if (floor_key > KeyOf<S>::kMask) floor_key = KeyOf<S>::kMask + 1u;  // nothing qualifies
   const int wave = threadIdx.x >> 6;
@@ -1119,11 +1120,11 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   if (aligned)
     k_select_stage<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
         in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.pick_above, a.thr_copy,
-        a.clear, a.clear_words, a.status);
+        a.clear, a.clear_words, a.floor_margin, a.status);
   else
     k_select_stage<S, false><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
         in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.pick_above, a.thr_copy,
-        a.clear, a.clear_words, a.status);
+        a.clear, a.clear_words, a.floor_margin, a.status);
   ZEN_LAUNCH_CHECK("k_select_stage");
   return ZEN_OK;
 }

@@ -870,10 +870,17 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
   if (a.k > 0) {
     // one pass: everything at or above a floor estimated from a sample goes to the slabs, the exact
     // threshold is read off the candidates' histogram and applied when the buckets are sorted
-    if (!a.prepared &&
-        (rc = topk_sampled_floor(a.input, a.dtype, a.n, a.k, floor, p.sample_hist[set], s, true)) != ZEN_OK)
-      return rc;
-    sc.thr = floor;
+    if (a.near_key) {
+      // the caller knows about where the threshold lies (an earlier call's): everything from 4/128 of a power
+      // of two below that key is a candidate, no sample
+      sc.thr = a.near_key;
+      sc.floor_margin = a.dtype == ZEN_BF16 ? 4u : 4u << 16;
+    } else {
+      if (!a.prepared &&
+          (rc = topk_sampled_floor(a.input, a.dtype, a.n, a.k, floor, p.sample_hist[set], s, true)) != ZEN_OK)
+        return rc;
+      sc.thr = floor;
+    }
     sc.cand_hist = p.cand_hist;
     sc.pick_k = a.k;
     sc.pick_thr = p.thr;

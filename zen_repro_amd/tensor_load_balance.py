@@ -146,15 +146,20 @@ class TensorPartition:
         done.record(stream)
         state["pending"].append((flat.data_ptr(), n, int(k), capacity, ws.data_ptr(), which, done))
 
-    def load_balance_flat(self, tensor, thr=None, capacity=None, k=0, mode=_lib.MODE_FAST, thr_out=None, slot=0):
+    def load_balance_flat(self, tensor, thr=None, capacity=None, k=0, mode=_lib.MODE_FAST, thr_out=None, slot=0,
+                          near=None):
         """Fused path without host synchronisation.  Returns (indices int32
         [capacity], values [capacity], splits int64[P] on device, status int32[1]
         on device); the first splits.sum() entries are valid, partition-major.
         Selection: `k` > 0 keeps the k largest magnitudes (ties kept; `thr_out`,
         an int32[2] device tensor, receives the threshold key and the count);
         else `thr` is the device tensor written by topk_threshold; else the
-        nonzeros.  A status with STAT_RETRY (fast mode only) means the call
-        must be repeated with mode=MODE_GENERAL; load_balance does that.
+        nonzeros.  With `k`, `near` may be a device tensor whose first word is
+        a key close to the threshold, e.g. the `thr_out` of the previous call
+        on this gradient bucket: the call then takes no sample (one kernel
+        less) and raises STAT_RETRY if the key was too far off.  A status with
+        STAT_RETRY (fast mode only) means the call must be repeated (without
+        `near`, or with mode=MODE_GENERAL); load_balance does that.
         Calls that may be in flight at the same time (different streams, e.g.
         one gradient bucket's encode next to the previous bucket's) must use
         different `slot` numbers: a slot owns its workspace and its table."""
@@ -181,7 +186,8 @@ class TensorPartition:
         ahead = None
         if state is not None and state["pending"]:
             ahead = state["pending"].pop(0)
-            if ahead[:5] != (flat.data_ptr(), n, int(k), capacity, ws.data_ptr()) or mode != _lib.MODE_FAST or thr is not None:
+            if (ahead[:5] != (flat.data_ptr(), n, int(k), capacity, ws.data_ptr()) or mode != _lib.MODE_FAST
+                    or thr is not None or near is not None):
                 # not for this call: its histogram is cleared again (with the arguments it was taken with) and
                 # the call samples for itself
                 cur = torch.cuda.current_stream(dev)
@@ -198,6 +204,8 @@ class TensorPartition:
         if ahead is not None:
             torch.cuda.current_stream(dev).wait_event(ahead[6])
             flags = _lib.MODE_PREPARED | (_lib.MODE_SECOND if ahead[5] else 0)
+        if near is not None and k > 0 and thr is None:
+            thr, flags = near, flags | _lib.MODE_FLOOR
         rc = L.zen_load_balance(
             _lib.ptr(flat), code, n, m, self.partitions, self.rehash, _lib.ptr(thr), int(k), _lib.ptr(thr_out),
             _lib.ptr(out_idx), _lib.ptr(out_val), capacity, _lib.ptr(splits), _lib.ptr(table), mode | flags,
