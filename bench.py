@@ -427,19 +427,29 @@ def main():
         if es is None:
             es = enc_streams[slot]
         enc, mrg = [], []
-        with torch.cuda.stream(es):
+
+        def encode():
             for j, b in enumerate(buckets):
                 g = grad_sets[j][i % len(grad_sets[j])]
                 enc.append(tp.load_balance_flat(g, None, caps[j], k=b.k, slot=slot, thr_out=warm_thr[j] if warm else None,
                                                 near=near_keys[j]))
+
+        def merge():
+            for j, b in enumerate(buckets):
+                fi, fv = flat_sets[j][i % len(flat_sets[j])]
+                mrg.append(lba.merge_sparse_flat(fi, fv, b.n, capacity=fi.numel(), slot=slot))
+
+        with torch.cuda.stream(es):
+            encode()
+            if ms_ is None:
+                merge()  # behind the encode, on its stream
         if prep_stream is not None and more and depth == 1:
             with torch.cuda.stream(prep_stream):
                 for j, b in enumerate(buckets):
                     tp.prepare(grad_sets[j][(i + 1) % len(grad_sets[j])], b.k, caps[j], slot=slot)
-        with torch.cuda.stream(ms_ if ms_ is not None else es):
-            for j, b in enumerate(buckets):
-                fi, fv = flat_sets[j][i % len(flat_sets[j])]
-                mrg.append(lba.merge_sparse_flat(fi, fv, b.n, capacity=fi.numel(), slot=slot))
+        if ms_ is not None:
+            with torch.cuda.stream(ms_):
+                merge()
         return list(zip(enc, mrg))
 
     side = enc_streams[1:] + [m for m in mrg_streams if m is not None] + ([prep_stream] if prep_stream is not None else [])
