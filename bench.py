@@ -51,10 +51,12 @@ def parse():
     ap.add_argument("--merge-beside", action="store_true",
                     help="with --depth 2 or more: a step's merge runs on a stream of its own beside its encode "
                          "(default there: on its encode's stream, after it; at --depth 1 it always runs beside)")
-    ap.add_argument("--depth", type=int, default=2,
-                    help="steps in flight: step i+1 is enqueued on its own stream next to step i, as a training "
-                         "step hands over one gradient bucket after the other "
-                         "(1 = a step starts when the previous one has finished)")
+    ap.add_argument("--depth", type=int, default=1,
+                    help="steps in flight in the timed region: 1 = a step starts when the previous one has finished "
+                         "(its merge runs beside its encode on a second stream), so that a kernel's events time "
+                         "that kernel; 2 or more: step i+1 is enqueued on its own stream next to step i, as a "
+                         "training step hands over one gradient bucket after the other (the default run reports "
+                         "that rate too, as two_steps_in_flight)")
     ap.add_argument("--rotate", type=int, default=16,
                     help="at most this many copies of the inputs, used in turn (as many as make 512 MB)")
     ap.add_argument("--near-threshold", action="store_true",
@@ -67,6 +69,9 @@ def parse():
     ap.add_argument("--imbalance", action="store_true", help="report the per-bucket load imbalance (always for c4)")
     ap.add_argument("--time-every", type=int, default=2,
                     help="in the timed region every n-th launch of the roofline kernel carries HIP events")
+    ap.add_argument("--stage-steps", type=int, default=20,
+                    help="steps of the untimed pass with every stage's events on (the stage table; it also tells "
+                         "which kernel is the roofline kernel)")
     ap.add_argument("--no-kernel-timing", action="store_true",
                     help="leave the HIP-event kernel timers off during the timed region")
     return ap.parse_args()
@@ -398,12 +403,13 @@ def main():
     pay_bytes = sum(fi.numel() * (4 + esize) for fi, _ in flats)
     flat_sets = [[(fi, fv)] + [(fi.clone(), fv.clone()) for _ in range(copies_of(pay_bytes) - 1)] for fi, fv in flats]
 
-    # A training step hands over one gradient bucket after the other (train.py:167-185 is called per bucket),
-    # and nothing in bucket i+1 depends on bucket i: by default two consecutive steps are in flight, alternating
-    # between two streams, workspaces and tables ("slots"), each step's merge behind its encode on the step's
-    # own stream, so that the long, memory-bound select of one step runs next to the short, latency-bound
-    # kernels of the other.  At --depth 1 a step starts when the one before has finished, and its merge, which
-    # does not depend on its encode, runs beside it on a second stream.  All streams have default priority.
+    # By default a step starts when the one before has finished, and its merge, which does not depend on its
+    # encode, runs beside it on a second stream.  A training step hands over one gradient bucket after the
+    # other (train.py:167-185 is called per bucket), and nothing in bucket i+1 depends on bucket i: with
+    # --depth 2 two consecutive steps are in flight, alternating between two streams, workspaces and tables
+    # ("slots"), each step's merge behind its encode on the step's own stream, so that the long, memory-bound
+    # select of one step runs next to the short, latency-bound kernels of the other (a kernel's events then
+    # also time its wait for room on the chip).  All streams have default priority.
     depth = 1 if (args.one_stream or args.graph) else max(1, args.depth)
     main = torch.cuda.current_stream(dev)
     enc_streams = [main] + [torch.cuda.Stream(device=dev) for _ in range(depth - 1)]
@@ -498,7 +504,8 @@ def main():
     every = 1 if len(buckets) > 1 else max(1, args.time_every)  # several buckets: every launch, or one bucket's only
     if not args.no_kernel_timing:
         _lib.profile_enable(True)
-        run(args.steps)
+        stage_steps = max(1, args.stage_steps)
+        run(stage_steps)
         torch.cuda.synchronize()
         stages = _lib.profile_read()
         cands = [(stages[name][0], name) for name in streaming if name in stages]
@@ -587,13 +594,41 @@ def main():
         lat.append(e0.elapsed_time(e1))
     lat.sort()
 
+    # the rate with two steps in flight (see --depth), when the timed region above ran one at a time
+    two = None
+    if depth == 1 and not args.one_stream and not args.graph:
+        torch.cuda.synchronize()
+        second = torch.cuda.Stream(device=dev)
+
+        def pipelined(count):
+            second.wait_stream(main)
+            for i in range(count):
+                with torch.cuda.stream(second if i % 2 else main):
+                    for j, b in enumerate(buckets):
+                        tp.load_balance_flat(grad_sets[j][i % len(grad_sets[j])], None, caps[j], k=b.k, slot=i % 2,
+                                             near=near_keys[j])
+                    for j, b in enumerate(buckets):
+                        fi, fv = flat_sets[j][i % len(flat_sets[j])]
+                        lba.merge_sparse_flat(fi, fv, b.n, capacity=fi.numel(), slot=i % 2)
+            main.wait_stream(second)
+
+        pipelined(4)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        pipelined(args.steps)
+        torch.cuda.synchronize()
+        ms2 = (time.perf_counter() - t2) * 1e3 / args.steps
+        two = {"ms_per_step": round(ms2, 4), "value": round(total_bytes / (ms2 * 1e-3) / 1e9, 2), "unit": "GB/s",
+               "path_frac_of_hbm_peak": round(b_alg / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+               "what": "the same steps with two in flight on two streams, a step's merge behind its encode (--depth 2)"}
+
     # dominant kernel: the one with the largest summed duration among the
     # kernels that stream the dense gradient; its algorithmic bytes per launch
     # (several buckets: the mean over the buckets' launches, all of which are timed)
     sel_bytes = sum(b.n * esize + nnz[j] * (4 + esize) for j, b in enumerate(buckets)) / len(buckets)
     per_launch = {"k_select_stage": sel_bytes, "k_select_compact": sel_bytes, "k_topk_hist": total_bytes / len(buckets)}
     roofline = None
-    stage_ms = {name: round(total / args.steps, 4) for name, (total, _) in stages.items()}
+    stage_ms = {name: round(total / stage_steps, 4) for name, (total, _) in stages.items()} if stages else {}
     if dom in kernels:
         total_ms, launches = kernels[dom]
         avg_ms = total_ms / launches
@@ -602,7 +637,7 @@ def main():
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                     "traffic": traffic[0] if traffic else None, "traffic_source": traffic[1] if traffic else None,
-                    "avg_launch_ms": round(avg_ms, 4), "launches_per_step": stages[dom][1] // args.steps,
+                    "avg_launch_ms": round(avg_ms, 4), "launches_per_step": stages[dom][1] // stage_steps,
                     "timed_launches": launches,
                     "algorithmic_bytes_per_launch": int(per_launch[dom]),
                     "measured_read_ceiling_GBps": round(ceiling, 1) if ceiling else None,
@@ -634,6 +669,7 @@ def main():
         "path_algorithmic_GBps": round(b_alg / (ms * 1e-3) / 1e9, 2),
         "path_frac_of_hbm_peak": round(b_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "ms_per_step_isolated_median": round(lat[len(lat) // 2], 4),
+        "two_steps_in_flight": two,
         "host_enqueue_ms_per_step": round((t_enq - t0) * 1e3 / args.steps, 4),
         "stage_ms_per_step": stage_ms,
         "stage_ms_note": "from an untimed pass with every stage's events on; the timed region times only the "
