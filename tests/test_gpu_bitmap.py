@@ -381,10 +381,12 @@ def test_comm_hook_on_one_rank(zen, oracle):
     assert hook(None, _StubBucket(small)).value() is small
 
 
-def test_comm_hook_between_four_ranks(zen):
+@pytest.mark.parametrize("method,fused", [(3, True), (3, False), (2, True), (1, True)])
+def test_comm_hook_between_four_ranks(zen, method, fused):
     """The hook end to end with four ranks played by host threads: every rank's future holds the sum of all
     ranks' compressed buckets (method 3: buckets exchanged, merged, sent round as bitmaps and decoded in one
-    pass)."""
+    pass), whether the threshold is handed to the all-reduce (fused) or applied to a copy of the bucket first
+    as in the reference."""
     P, n = 4, 1 << 20
     gen = torch.Generator(device="cuda").manual_seed(5)
     grads = [(torch.randn(n, device="cuda", generator=gen) * 1e-3) for _ in range(P)]
@@ -397,8 +399,8 @@ def test_comm_hook_between_four_ranks(zen):
             torch.cuda.set_device(0)
             lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P, rank), None, None)
             lba.ddp = ex.view(rank)
-            hook = zen.SparseCommHook(lba, top_k=2, method=3, tp_group=zen.LocalGroup(1, 0),
-                                      sample_index=lambda numel, r=rank: samples[r])
+            hook = zen.SparseCommHook(lba, top_k=2, method=method, tp_group=zen.LocalGroup(1, 0),
+                                      sample_index=lambda numel, r=rank: samples[r], fused=fused)
             hook(None, _StubBucket(grads[rank]))  # the first call is passed through
             compressed[rank] = zen.compress_with_allgather(2, grads[rank], zen.LocalGroup(1, 0), sample_index=samples[rank])
             results[rank] = hook(None, _StubBucket(grads[rank])).value()

@@ -335,24 +335,42 @@ class LoadBalanceAllreduce:
 
     # ------------------------------------------------- the whole exchange
 
-    def zen_sparse_comm(self, tensor, method):
+    def zen_sparse_comm(self, tensor, method, thr=None, capacity=None):
         """The reference's driver of one sparse all-reduce (comm.py:101-150):
         method 1 = all-gather of (indices, values); 2 = load balance, exchange of
         the buckets, merge, all-gather of the merged indices; 3 = as 2 with the
         indices travelling as bitmaps.  The exchanges themselves belong to
         `self.ddp`, an object with the reference backend's allgather /
         allgather_padding / alltoallv (DDPbackend.py:13-41, 71-81); this build
-        ships none, so the attribute has to be set by the caller."""
+        ships none, so the attribute has to be set by the caller.
+        The reference is handed a tensor that compress has thresholded already;
+        with `thr` (the device tensor topk_threshold returns) the tensor is the
+        gradient as it is and everything below that magnitude counts as zero:
+        the masked copy and the pass that reads it again fall away.  `capacity`
+        then says how many elements are expected to pass."""
         ddp = getattr(self, "ddp", None)
         if ddp is None:
             raise RuntimeError("zen_sparse_comm needs a communication backend in self.ddp")
         numel = tensor.numel()
         if method == 1:
-            sparse_indices, sparse_values = self.encode_sparse_tensor(tensor)
+            if thr is None:
+                sparse_indices, sparse_values = self.encode_sparse_tensor(tensor)
+            else:
+                _lib.require_gpu(tensor, "input")
+                room = capacity
+                while True:
+                    try:
+                        sparse_indices, sparse_values, _ = _select(tensor, thr, idx64=True, capacity=room)
+                        break
+                    except RuntimeError:
+                        if room is None or room >= numel:
+                            raise
+                        room = min(numel, room * 4)  # more passed the threshold than the estimate allowed for
             indices_tensors = ddp.allgather_padding(sparse_indices)
             values_tensors = ddp.allgather_padding(sparse_values)
             return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
-        indices, values, splits = self.tensor_partition.load_balance(tensor)
+        indices, values, splits = self.tensor_partition.load_balance(tensor, thr=thr, capacity=capacity,
+                                                                     grow=True if thr is not None else None)
         gather_splits = ddp.allgather(splits)
         indices_tensors = ddp.alltoallv(indices, gather_splits)
         values_tensors = ddp.alltoallv(values, gather_splits)

@@ -64,16 +64,15 @@ def compress(top_k, tensor, sample_index=None):
     return mask_below(flat, thr).view_as(tensor)
 
 
-def compress_with_allgather(top_k, tensor, pg_group, sample_index=None, all_gather=None):
-    """The reference's compress_with_allgather (train.py:56-73): as compress,
-    but the threshold is the (n_all*top_k//100)-th largest magnitude among
-    the 1 % samples of every rank of pg_group.  `all_gather(sample)` returns
-    the samples of all ranks as one tensor (the reference calls
-    dist.all_gather_into_tensor there); this build ships no exchange, so it
-    has to be passed in for groups of more than one rank."""
+def threshold_with_allgather(top_k, tensor, pg_group, sample_index=None, all_gather=None):
+    """The threshold compress_with_allgather applies (train.py:56-71), as the
+    device tensor topk_threshold returns, without the masked copy of the
+    tensor: for callers that hand it on to the load balance, which selects
+    while it reads the tensor anyway.  None for tensors of at most 4096
+    elements (they pass through uncompressed, train.py:58-59)."""
     numel = tensor.numel()
     if numel <= 4096:
-        return tensor
+        return None
     flat = tensor.reshape(-1)
     if sample_index is None:
         sample_index = torch.randint(0, numel, (math.ceil(0.01 * numel),), device=tensor.device)
@@ -89,5 +88,17 @@ def compress_with_allgather(top_k, tensor, pg_group, sample_index=None, all_gath
     k = samples.numel() * top_k // 100
     if k < 1:
         raise RuntimeError("compress_with_allgather: top-k of the samples is empty")
-    thr = topk_threshold(samples.contiguous(), k)
-    return mask_below(flat, thr).view_as(tensor)
+    return topk_threshold(samples.contiguous(), k)
+
+
+def compress_with_allgather(top_k, tensor, pg_group, sample_index=None, all_gather=None):
+    """The reference's compress_with_allgather (train.py:56-73): as compress,
+    but the threshold is the (n_all*top_k//100)-th largest magnitude among
+    the 1 % samples of every rank of pg_group.  `all_gather(sample)` returns
+    the samples of all ranks as one tensor (the reference calls
+    dist.all_gather_into_tensor there); this build ships no exchange, so it
+    has to be passed in for groups of more than one rank."""
+    thr = threshold_with_allgather(top_k, tensor, pg_group, sample_index, all_gather)
+    if thr is None:
+        return tensor
+    return mask_below(tensor.reshape(-1), thr).view_as(tensor)

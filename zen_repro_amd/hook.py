@@ -7,7 +7,7 @@ returns the compressed bucket, as the reference does when dp_group.size() == 1
 (train.py:178)."""
 import torch
 
-from .compress import compress_with_allgather
+from .compress import mask_below, threshold_with_allgather
 
 
 class SparseCommHook:
@@ -23,10 +23,16 @@ class SparseCommHook:
                             than one rank
     stream                  the side stream the path runs on (train.py:165);
                             default priority
+    fused                   False: the reference's steps one by one (the bucket
+                            is thresholded into a dense copy, the all-reduce
+                            reads that copy); True (default): the threshold is
+                            handed to the all-reduce, which selects while it
+                            reads the bucket: same result, two passes over the
+                            bucket fewer
     The first call passes the bucket through untouched (train.py:170-174)."""
 
     def __init__(self, load_balance_allreduce, top_k, method, tp_group, all_gather=None, stream=None,
-                 sample_index=None):
+                 sample_index=None, fused=True):
         self.lba = load_balance_allreduce
         self.top_k = top_k
         self.method = method
@@ -34,6 +40,7 @@ class SparseCommHook:
         self.all_gather = all_gather
         self.stream = stream if stream is not None else torch.cuda.Stream()
         self.sample_index = sample_index  # callable(numel) -> int64 sample positions; None: drawn like the reference
+        self.fused = fused
         self.skip = True
 
     def __call__(self, state, bucket):
@@ -45,11 +52,20 @@ class SparseCommHook:
             return future
         with torch.cuda.stream(self.stream):
             index = self.sample_index(tensors.numel()) if self.sample_index is not None else None
-            tensors_compressed = compress_with_allgather(self.top_k, tensors, self.tp_group, sample_index=index,
-                                                         all_gather=self.all_gather)
-            tensors = tensors_compressed
-            if self.lba.process_group.size() > 1 and getattr(self.lba, "ddp", None) is not None:
-                tensors = self.lba.zen_sparse_comm(tensors_compressed, self.method)
+            thr = threshold_with_allgather(self.top_k, tensors, self.tp_group, sample_index=index,
+                                           all_gather=self.all_gather)
+            exchange = self.lba.process_group.size() > 1 and getattr(self.lba, "ddp", None) is not None
+            if thr is None:  # a small bucket: not compressed (train.py:58-59)
+                if exchange:
+                    tensors = self.lba.zen_sparse_comm(tensors, self.method)
+            elif exchange and self.fused:
+                # about top_k per cent of the bucket pass the sampled threshold; the call grows its buffers if more do
+                room = int(tensors.numel() * self.top_k / 100 * 1.5) + 4096
+                tensors = self.lba.zen_sparse_comm(tensors, self.method, thr=thr, capacity=min(room, tensors.numel()))
+            else:
+                tensors = mask_below(tensors.reshape(-1), thr).view_as(tensors)
+                if exchange:
+                    tensors = self.lba.zen_sparse_comm(tensors, self.method)
         # like the reference, the future is completed at once: whoever consumes the result does so in the
         # stream order of `self.stream` (train.py:181)
         future.set_result(tensors)

@@ -220,15 +220,19 @@ class TensorPartition:
             state["free"][used] = free
         return out_idx, out_val, splits, status
 
-    def load_balance(self, tensor, thr=None, capacity=None, k=0, mode=None):
+    def load_balance(self, tensor, thr=None, capacity=None, k=0, mode=None, grow=None):
         """Returns (indices[P], values[P], splits) like the reference
         (tensor_load_balance.py:43-51).  The per-partition tensors are views of
         two contiguous buffers; slicing them needs the split sizes on the
-        host, which is this call's only synchronisation."""
+        host, which is this call's only synchronisation.  Without a `capacity`
+        one is worked out and the call is repeated with four times as much
+        when the selection turns out larger; `grow=True` asks for the same
+        with a capacity that is the caller's estimate."""
         flat = tensor.reshape(-1)
         n = flat.numel()
-        grow = capacity is None
-        if grow:
+        if grow is None:
+            grow = capacity is None
+        if capacity is None:
             capacity = min(n, self._honest_capacity(flat, thr, k))
         modes = [_lib.MODE_FAST, _lib.MODE_GENERAL] if mode is None else [mode]
         while modes:
