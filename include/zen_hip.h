@@ -66,6 +66,10 @@ extern "C" {
    largest among those.  If fewer than k elements qualify, or far too many, ZEN_STAT_RETRY is raised as when a
    sample misleads.  Paths that do not sample ignore the key. */
 #define ZEN_MODE_FLOOR 0x1000
+/* zen_load_balance, zen_merge, zen_decode_dense: with ZEN_MODE_FAST, stay off the path for up to a few million
+   entries (at most 256 wide buckets, one resident workgroup each, whose launches the library keeps from
+   overlapping on a device) and take the bucket-slab path wherever that fits.  Results are the same. */
+#define ZEN_MODE_SLABS 0x2000
 
 int zen_abi_version(void);
 

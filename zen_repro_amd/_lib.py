@@ -15,6 +15,7 @@ MODE_FAST, MODE_GENERAL = 0, 1
 MODE_ZEROED = 0x100  # zen_merge: the head of the workspace is zero (and stays so)
 MODE_PREPARED, MODE_SECOND, MODE_DISCARD = 0x200, 0x400, 0x800  # zen_load_balance: the sample was taken ahead (zen_load_balance_prepare)
 MODE_FLOOR = 0x1000  # zen_load_balance with k > 0: thr holds a key close to the threshold, no sample is taken
+MODE_SLABS = 0x2000  # fast mode without the wide-bucket path (bucket slabs where they fit)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # ZEN_HIP_LIB names another build of the library (a debug build, a build with other compile-time settings)

@@ -148,6 +148,15 @@ struct SlabBalanceArgs {
 bool slab_balance_fits(int64_t n, int64_t m, int partitions, int dtype, int64_t capacity, int64_t k, SlabGeom *geo);
 size_t slab_balance_bytes(int64_t m, int partitions, int dtype, int64_t capacity);
 int slab_load_balance(const SlabBalanceArgs &a, hipStream_t stream);
+int slab_prepare(const SlabBalanceArgs &a, hipStream_t stream);  // only_prepare, whichever of the two paths the call takes
+size_t slab_state_offset(uint32_t hash_log2);  // where the zero-between-calls counters start in the caller's table
+
+// Load balance on wide buckets (zen_wide_encode.hip): select and one resident kernel, for selections of a few
+// million entries at most on a chip of `cus` compute units.
+bool wide_balance_fits(int64_t m, int partitions, int64_t capacity, int64_t k, int cus, SlabGeom *geo);
+size_t wide_balance_bytes(int64_t m, int partitions, int dtype, int64_t capacity, int cus);
+int wide_load_balance(const SlabBalanceArgs &a, size_t state_offset, hipStream_t stream);
+int wide_device_cus();  // compute units of the current device (0: no device)
 
 size_t resolve_scratch_bytes(int64_t list_cap, uint64_t key_limit);  // key_limit = P * (m / P + 1) + 1
 int resolve_and_place(const ResolveArgs &a, hipStream_t stream);

@@ -369,12 +369,18 @@ size_t zen_load_balance_workspace(int64_t n, int64_t m, int dtype, int64_t capac
   if (n <= 0 || m <= 0 || capacity < 0) return 0;
   const size_t general = zen::plan_balance(nullptr, n, m, dtype, capacity).bytes;
   const size_t slabs = partitions > 0 && m % partitions == 0 ? zen::slab_balance_bytes(m, partitions, dtype, capacity) : 0;
-  return general > slabs ? general : slabs;
+  const size_t wide = partitions > 0 && m % partitions == 0
+                          ? zen::wide_balance_bytes(m, partitions, dtype, capacity, zen::wide_device_cus())
+                          : 0;
+  const size_t fast = slabs > wide ? slabs : wide;
+  return general > fast ? general : fast;
 }
 
 int zen_load_balance_path(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions, int64_t k, int mode) {
+  const bool slabs_only = (mode & ZEN_MODE_SLABS) != 0;
   mode &= 0xff;
   if (mode != ZEN_MODE_FAST || partitions <= 0 || m <= 0 || m % partitions != 0) return 0;
+  if (!slabs_only && zen::wide_balance_fits(m, partitions, capacity, k, zen::wide_device_cus(), nullptr)) return 3;
   if (zen::slab_balance_fits(n, m, partitions, dtype, capacity, k, nullptr)) return 2;
   return m >= 4096 ? 1 : 0;
 }
@@ -403,7 +409,8 @@ int zen_load_balance_prepare(const void *input, int dtype, int64_t n, int64_t m,
     return fail(ZEN_EWORKSPACE, "zen_load_balance_prepare: workspace too small");
   const int second = (mode & ZEN_MODE_SECOND) != 0;
   if ((mode & 0xff) != ZEN_MODE_FAST || k == 0 || (reinterpret_cast<uintptr_t>(table) & 7u) != 0 ||
-      !slab_balance_fits(n, m, partitions, dtype, capacity, k, nullptr))
+      (!slab_balance_fits(n, m, partitions, dtype, capacity, k, nullptr) &&
+       !wide_balance_fits(m, partitions, capacity, k, wide_device_cus(), nullptr)))
     return ZEN_OK;  // nothing to take ahead on the other paths
   SlabBalanceArgs sa{};
   sa.input = input;
@@ -421,7 +428,7 @@ int zen_load_balance_prepare(const void *input, int dtype, int64_t n, int64_t m,
   sa.prepared = second ? 2 : 1;
   sa.only_prepare = true;
   sa.discard = (mode & ZEN_MODE_DISCARD) != 0;
-  return slab_load_balance(sa, static_cast<hipStream_t>(stream));
+  return slab_prepare(sa, static_cast<hipStream_t>(stream));
 }
 
 int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
@@ -436,7 +443,8 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
     near_key = thr;
     thr = nullptr;  // paths that take no sample have no use for it
   }
-  mode &= ~(ZEN_MODE_PREPARED | ZEN_MODE_SECOND | ZEN_MODE_FLOOR);
+  const bool slabs_only = (mode & ZEN_MODE_SLABS) != 0;
+  mode &= ~(ZEN_MODE_PREPARED | ZEN_MODE_SECOND | ZEN_MODE_FLOOR | ZEN_MODE_SLABS);
   if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_load_balance: bad dtype");
   if (mode != ZEN_MODE_FAST && mode != ZEN_MODE_GENERAL) return fail(ZEN_EINVAL, "zen_load_balance: bad mode");
   if (n <= 0 || n > 0x7fffffffll || m <= 0 || m > 0x7fffffffll || partitions <= 0 || partitions > 65535 ||
@@ -455,8 +463,10 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
   const int64_t spp = n / partitions / 10;  // tensor_load_balance.py:18
   const uint32_t drop_key = (uint32_t)partitions * (g.npp + 1u);
   const int bits = ceil_log2_u64(drop_key);
-  if (mode == ZEN_MODE_FAST && (reinterpret_cast<uintptr_t>(table) & 7u) == 0 &&
-      slab_balance_fits(n, m, partitions, dtype, capacity, k, nullptr)) {
+  const bool wide = mode == ZEN_MODE_FAST && !slabs_only && (reinterpret_cast<uintptr_t>(table) & 7u) == 0 &&
+                    wide_balance_fits(m, partitions, capacity, k, wide_device_cus(), nullptr);
+  if (wide || (mode == ZEN_MODE_FAST && (reinterpret_cast<uintptr_t>(table) & 7u) == 0 &&
+               slab_balance_fits(n, m, partitions, dtype, capacity, k, nullptr))) {
     SlabBalanceArgs sa;
     sa.input = input;
     sa.dtype = dtype;
@@ -477,6 +487,7 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
     sa.status = status;
     sa.prepared = near_key ? 0 : prepared;
     sa.near_key = near_key;
+    if (wide) return wide_load_balance(sa, slab_state_offset(sa.hash_log2), s);
     return slab_load_balance(sa, s);
   }
   BalancePlan p = plan_balance(workspace, n, m, dtype, capacity);

@@ -81,6 +81,9 @@ enum ProfTag {
   kProfMergeBucket,
   kProfSampleHist,
   kProfDecodeFused,
+  kProfWideTail,
+  kProfWideScatter,
+  kProfWideMerge,
   kProfCount
 };
 

@@ -40,6 +40,7 @@ const char *const kNames[kProfCount] = {
     "k_gather",    "k_merge_prep",     "k_merge_reduce", "k_compress", "k_insert_dense",
     "k_select_stage", "k_coarse_scatter+k_fine_scatter", "k_slab_sort", "k_slab_chains+classify", "k_slab_place",
     "merge: k_coarse_scatter+k_fine_scatter", "k_merge_bucket", "k_sample_hist", "k_decode_fused",
+    "k_wide_tail", "k_wide_scatter", "k_wide_merge",
 };
 
 void drop_spans() {  // the events go back to the spare list (a read has waited for them, or nobody will)

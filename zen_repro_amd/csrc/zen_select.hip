@@ -735,30 +735,39 @@ __device__ inline uint32_t pick_elem<uint32_t>(const uint4 (&q)[kSelVecs], int o
   return pick_word(q, off);
 }
 
-// Where the candidates go.
+// Where the candidates go: the coarse slabs of zen_slab_feed.h (two word planes: index, value), or straight to
+// wide buckets (zen_wide.h; three planes: index, level-1 slot, value).  Either way a destination is kept in
+// kCoarseSplit parts with a cursor each.
 struct StageSlabs {
   SlabGeom geo;
-  CoarseGeom cg;
-  uint32_t *cursor;  // coarse cursors
-  uint32_t *words;   // word planes of the coarse slabs
+  CoarseGeom cg;     // wide: groups = buckets, per = 1, cap = entries per part
+  uint32_t *cursor;  // part cursors
+  uint32_t *words;   // word planes
+  uint32_t wide;
 };
 
+constexpr int kStageDstMax = 256;  // destinations of a flush, at most (one counter per thread)
+static_assert(kStageDstMax == kSelBlock && kCoarseMax <= kStageDstMax, "a thread per destination");
+
 struct StageFlushShared {
-  uint32_t cnt[kCoarseMax], pref[kCoarseMax + 1], gbase[kCoarseMax];
-  uint8_t dst[kScatStage];
+  uint32_t cnt[kStageDstMax], pref[kStageDstMax + 1], gbase[kStageDstMax];
+  uint32_t scan[kSelBlock / 64 + 1];
+  uint16_t dst[kScatStage];
 };
 
 // Called by the whole block after a barrier made the staged entries visible.  What k_coarse_scatter does for
-// a list, done for the staged candidates: every entry finds its coarse slab (from the level-1 hash slot of
-// its index), the stage is put in slab order in place, every slab's run is reserved with one atomic and
-// consecutive lanes write consecutive places.  Element 0 is not handed on (index 0 is never transmitted:
-// 0 is the table's empty marker, tensor_load_balance.py:31), but counts in the histogram.
+// a list, done for the staged candidates: every entry finds its destination (from the level-1 hash slot of
+// its index), the stage is put in destination order in place, every destination's run is reserved with one
+// atomic and consecutive lanes write consecutive places.  Element 0 is not handed on (index 0 is never
+// transmitted: 0 is the table's empty marker, tensor_load_balance.py:31), but counts in the histogram.
 template <typename S>
 __device__ inline void stage_flush(uint32_t count, int32_t *st_idx, S *st_val, StageFlushShared &fl,
                                    uint32_t *s_hist, uint32_t floor_key, const StageSlabs &out, int32_t *status) {
   constexpr int kPer = kScatStage / kSelBlock;
-  static_assert(kScatStage % kSelBlock == 0 && kCoarseMax <= 64, "flush layout");
-  if (threadIdx.x < kCoarseMax) fl.cnt[threadIdx.x] = 0;
+  constexpr uint32_t kNoDst = 0xffffu;
+  static_assert(kScatStage % kSelBlock == 0, "flush layout");
+  const uint32_t ndst = out.cg.groups;
+  fl.cnt[threadIdx.x] = 0;
   __syncthreads();
   const uint32_t part = blockIdx.x % kCoarseSplit;
   uint32_t t[kPer], d[kPer], r[kPer];
@@ -766,7 +775,7 @@ __device__ inline void stage_flush(uint32_t count, int32_t *st_idx, S *st_val, S
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
     const uint32_t e = threadIdx.x + i * kSelBlock;
-    d[i] = 0xffu;
+    d[i] = kNoDst;
     t[i] = r[i] = 0;
     v[i] = 0;
     if (e < count) {
@@ -779,44 +788,47 @@ __device__ inline void stage_flush(uint32_t count, int32_t *st_idx, S *st_val, S
       if (t[i] != 0) {
         uint32_t rem;
         const uint32_t bucket = out.geo.bucket_of(out.geo.mod_m(poly(t[i]) + kSeed1));
-        d[i] = SlabGeom::div_small(bucket, out.cg.per, out.cg.inv_per, &rem);
+        d[i] = out.wide ? bucket : SlabGeom::div_small(bucket, out.cg.per, out.cg.inv_per, &rem);
         r[i] = atomicAdd(&fl.cnt[d[i]], 1u);
       }
     }
   }
   __syncthreads();
-  if (threadIdx.x < 64) {
-    const uint32_t c = threadIdx.x < kCoarseMax ? fl.cnt[threadIdx.x] : 0u;
-    const uint32_t incl = wave_inclusive_scan(c);
-    if (threadIdx.x < kCoarseMax) {
-      fl.pref[threadIdx.x] = incl - c;
+  {
+    const uint32_t c = threadIdx.x < ndst ? fl.cnt[threadIdx.x] : 0u;
+    uint32_t total;
+    const uint32_t before = block_exclusive_scan<uint32_t, kSelBlock>(c, fl.scan, &total);
+    if (threadIdx.x < ndst) {
+      fl.pref[threadIdx.x] = before;
       fl.gbase[threadIdx.x] = c ? atomicAdd(&out.cursor[(threadIdx.x * kCoarseSplit + part) * kCoarsePad], c) : 0u;
     }
-    if (threadIdx.x == kCoarseMax - 1) fl.pref[kCoarseMax] = incl;
+    if (threadIdx.x == 0) fl.pref[ndst] = total;
   }
   __syncthreads();  // every thread holds its entries in registers: the stage is reordered in place
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
-    if (d[i] != 0xffu) {
+    if (d[i] != kNoDst) {
       const uint32_t p = fl.pref[d[i]] + r[i];
       st_idx[p] = (int32_t)t[i];
       st_val[p] = v[i];
-      fl.dst[p] = (uint8_t)d[i];
+      fl.dst[p] = (uint16_t)d[i];
     }
   }
   __syncthreads();
-  const uint32_t total = fl.pref[kCoarseMax];
-  const size_t plane = (size_t)out.cg.groups * kCoarseSplit * out.cg.cap;
-  S *val_plane = reinterpret_cast<S *>(out.words + plane);
+  const uint32_t total = fl.pref[ndst];
+  const size_t plane = (size_t)ndst * kCoarseSplit * out.cg.cap;
+  S *val_plane = reinterpret_cast<S *>(out.words + (out.wide ? 2 : 1) * plane);
   for (uint32_t p = threadIdx.x; p < total; p += kSelBlock) {
     const uint32_t g = fl.dst[p];
     const uint32_t at = fl.gbase[g] + (p - fl.pref[g]);
     if (at < out.cg.cap) {
       const size_t o = (size_t)(g * kCoarseSplit + part) * out.cg.cap + at;
-      out.words[o] = (uint32_t)st_idx[p];
+      const uint32_t idx = (uint32_t)st_idx[p];
+      out.words[o] = idx;
+      if (out.wide) out.words[plane + o] = out.geo.mod_m(poly(idx) + kSeed1);  // hashed again: cheaper than staging it
       val_plane[o] = st_val[p];
     } else {
-      atomicOr(status, ZEN_STAT_RETRY);  // a coarse slab is full: the general path answers
+      atomicOr(status, ZEN_STAT_RETRY);  // a slab is full: another path answers
     }
   }
   __syncthreads();
@@ -1115,7 +1127,7 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   sch.ticket_tiles = (uint32_t)ceil_div(subs - (int64_t)sch.fixed_subs, kStageSmall);
   const S *in = static_cast<const S *>(a.in);
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0 && a.n >= V;
-  const StageSlabs out{a.geo, a.cg, a.coarse_cursor, a.coarse_words};
+  const StageSlabs out{a.geo, a.cg, a.coarse_cursor, a.coarse_words, a.wide ? 1u : 0u};
   ProfScope prof(kProfSelectStage, stream);
   if (aligned)
     k_select_stage<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(

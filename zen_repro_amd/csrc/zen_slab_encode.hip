@@ -26,6 +26,7 @@
 #include "zen_hashmap.h"
 #include "zen_slab.h"
 #include "zen_slab_feed.h"
+#include "zen_refine.h"
 
 namespace zen {
 namespace {
@@ -96,92 +97,6 @@ struct EncodeSink {
     raw_val[at] = (S)w[1];
   }
 };
-
-// --------------------------------------------- fp32: the threshold's last 16 bits
-
-constexpr int kRefineBins = 65536;
-constexpr int kRefineBlock = 512;
-
-// The candidates' histogram resolves the 15 leading bits of an fp32 key: after the select kernel thr[0] is
-// the lowest key of the bin the k-th largest lies in, thr[1] the number of candidates at or above it and
-// *above the number in the bins above.  This kernel histograms the low 16 key bits of the candidates of that
-// bin (they sit in the coarse slabs; element 0, which is never handed on, is looked at in the tensor), and the
-// workgroup that finishes last replaces thr[0..1] by the exact key and the number of elements at or above it.
-// Grid: any number of workgroups, which take the parts of the coarse slabs in turn.  hist: kRefineBins + 1 zeroed words.
-__global__ __launch_bounds__(kRefineBlock) void k_refine_threshold(CoarseGeom cg,
-                                                                   const uint32_t *__restrict__ coarse_cursor,
-                                                                   const uint32_t *__restrict__ coarse_words,
-                                                                   const uint32_t *__restrict__ dense,
-                                                                   uint32_t *thr, const uint32_t *above, uint32_t k,
-                                                                   uint32_t *hist, uint32_t *thr_copy, int32_t *status) {
-  __shared__ uint32_t s_scan[kRefineBlock / 64 + 1];
-  __shared__ bool s_last;
-  const uint32_t base = thr[0];
-  const size_t plane = (size_t)cg.groups * kCoarseSplit * cg.cap;
-  const uint32_t parts = cg.groups * (uint32_t)kCoarseSplit;
-  // a workgroup takes several parts: every workgroup ends with an atomic on one counter, and a thousand of
-  // those stand in line for 11 us
-  for (uint32_t part = blockIdx.x; part < parts; part += gridDim.x) {
-    uint32_t count = coarse_cursor[part * kCoarsePad];
-    if (count > cg.cap) count = cg.cap;
-    const uint32_t *vals = coarse_words + plane + (size_t)part * cg.cap;
-    for (uint32_t e = threadIdx.x; e < count; e += kRefineBlock) {
-      const uint32_t d = (vals[e] & KeyOf<uint32_t>::kMask) - base;
-      if (d < (uint32_t)kRefineBins) atomicAdd(&hist[d], 1u);
-    }
-  }
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    const uint32_t key0 = dense[0] & KeyOf<uint32_t>::kMask;  // counted by the select kernel if it was a candidate
-    if (key0 - base < (uint32_t)kRefineBins) atomicAdd(&hist[key0 - base], 1u);  // base is at or above the floor
-  }
-  wait_global_acks();
-  __syncthreads();
-  if (threadIdx.x == 0) s_last = atomicAdd(&hist[kRefineBins], 1u) == gridDim.x - 1u;
-  __syncthreads();
-  if (!s_last) return;
-  // from the top down: thread t owns the kPer bins below kRefineBins - t * kPer.  The counts were raised
-  // by atomics in memory and this workgroup has not looked at them before: once the cache lines it may
-  // hold are dropped, plain 16-byte loads see them all, and many of them are in flight together (one
-  // uncached load after the other took 50 us here)
-  constexpr int kPer = kRefineBins / kRefineBlock;
-  static_assert(kPer % 4 == 0, "a thread's bins are read four at a time");
-  const uint32_t hi = (uint32_t)kRefineBins - threadIdx.x * (uint32_t)kPer;
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-  uint32_t mine = 0;
-  {
-    const uint4 *own = reinterpret_cast<const uint4 *>(hist + (hi - (uint32_t)kPer));
-#pragma unroll 8
-    for (int j = 0; j < kPer / 4; ++j) {
-      const uint4 q = own[j];
-      mine += q.x + q.y + q.z + q.w;
-    }
-  }
-  uint32_t total;
-  uint32_t before = block_exclusive_scan<uint32_t, kRefineBlock>(mine, s_scan, &total);
-  const uint32_t over = above[0];
-  const uint32_t need = k > over ? k - over : 1u;  // rank inside the bin, from the top
-  if (total < need) {
-    if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);  // the two histograms disagree: let the general mode answer
-    return;
-  }
-  if (before < need && need <= before + mine) {
-    const uint4 *own = reinterpret_cast<const uint4 *>(hist + (hi - (uint32_t)kPer));
-    for (int j = 1; j <= kPer; ++j) {
-      const uint4 q = own[(kPer - j) >> 2];  // the bin hi - j, in the lines read above
-      const uint32_t w = (uint32_t)(kPer - j) & 3u;
-      const uint32_t c = w == 0 ? q.x : w == 1 ? q.y : w == 2 ? q.z : q.w;
-      if (before < need && need <= before + c) {
-        thr[0] = base + hi - (uint32_t)j;
-        thr[1] = over + before + c;
-        if (thr_copy) {
-          thr_copy[0] = base + hi - (uint32_t)j;
-          thr_copy[1] = over + before + c;
-        }
-      }
-      before += c;
-    }
-  }
-}
 
 // ------------------------------------------------------------ sort a bucket
 
@@ -819,7 +734,7 @@ size_t slab_balance_bytes(int64_t m, int partitions, int dtype, int64_t capacity
 
 // The hash map takes the first 8 << hash_log2 bytes of the caller's table (at most half of it: zen_load_balance
 // sizes the map so); the counters sit behind it.
-static size_t slab_state_offset(uint32_t hash_log2) { return align_up((size_t)8 << hash_log2, 256); }
+size_t slab_state_offset(uint32_t hash_log2) { return align_up((size_t)8 << hash_log2, 256); }
 
 bool slab_balance_fits(int64_t n, int64_t m, int partitions, int dtype, int64_t capacity, int64_t k, SlabGeom *geo) {
   (void)n;
@@ -831,6 +746,28 @@ bool slab_balance_fits(int64_t n, int64_t m, int partitions, int dtype, int64_t 
   // counters less than 1 MB
   if (geo) *geo = g;
   return true;
+}
+
+// The sample of a coming call, or the clearing of one nobody will pick up.  The sampling memory and the floor
+// sit at the head of the zero-between-calls memory and of the workspace whatever the geometry and the path.
+int slab_prepare(const SlabBalanceArgs &a, hipStream_t s) {
+  char *state = reinterpret_cast<char *>(a.hash) + slab_state_offset(a.hash_log2);
+  Carver cs(state);
+  uint32_t *sample_hist[2];
+  sample_hist[0] = cs.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
+  sample_hist[1] = cs.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
+  Carver cw(a.workspace);
+  uint32_t *thr = cw.take<uint32_t>(16);
+  const int set = a.prepared == 2 ? 1 : 0;
+  uint32_t *floor = thr + 2 + 4 * set;
+  if (a.discard) {  // a sample nobody will pick up: its histogram goes back to zero
+    launch_fill<uint32_t>(sample_hist[set], 0u, sampled_floor_zero_bytes() / sizeof(uint32_t), s);
+    ZEN_LAUNCH_CHECK("slab: discard a sample");
+    return ZEN_OK;
+  }
+  // the sample alone: the floor stays in the workspace until the call proper picks it up
+  if (a.k > 0) return topk_sampled_floor(a.input, a.dtype, a.n, a.k, floor, sample_hist[set], s, true);
+  return ZEN_OK;
 }
 
 int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
@@ -857,16 +794,7 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
   int rc;
   const int set = a.prepared == 2 ? 1 : 0;
   uint32_t *floor = p.thr + 2 + 4 * set;
-  if (a.only_prepare) {
-    if (a.discard) {  // a sample nobody will pick up: its histogram goes back to zero
-      launch_fill<uint32_t>(p.sample_hist[set], 0u, sampled_floor_zero_bytes() / sizeof(uint32_t), s);
-      ZEN_LAUNCH_CHECK("slab: discard a sample");
-      return ZEN_OK;
-    }
-    // the sample alone: the floor stays in the workspace until the call proper picks it up
-    if (a.k > 0) return topk_sampled_floor(a.input, a.dtype, a.n, a.k, floor, p.sample_hist[set], s, true);
-    return ZEN_OK;
-  }
+  if (a.only_prepare) return slab_prepare(a, s);
   if (a.k > 0) {
     // one pass: everything at or above a floor estimated from a sample goes to the slabs, the exact
     // threshold is read off the candidates' histogram and applied when the buckets are sorted
@@ -893,7 +821,7 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
   if (refine) {
     const uint32_t refine_parts = p.cg.groups * (uint32_t)kCoarseSplit;
     k_refine_threshold<<<dim3(refine_parts < 128u ? refine_parts : 128u), dim3(kRefineBlock), 0, s>>>(
-        p.cg, p.feed.coarse_cursor, p.feed.coarse_words, static_cast<const uint32_t *>(a.input), p.thr,
+        p.cg, 1, p.feed.coarse_cursor, p.feed.coarse_words, static_cast<const uint32_t *>(a.input), p.thr,
         p.thr + 4, (uint32_t)a.k, p.refine_hist, a.thr_out, a.status);
     ZEN_LAUNCH_CHECK("k_refine_threshold");
   }

@@ -125,7 +125,7 @@ class TensorPartition:
         m, _ = self.table_sizes(n)
         dev = flat.device
         L = _lib.lib()
-        if k <= 0 or L.zen_load_balance_path(n, m, code, capacity, self.partitions, k, _lib.MODE_FAST) != 2:
+        if k <= 0 or L.zen_load_balance_path(n, m, code, capacity, self.partitions, k, _lib.MODE_FAST) not in (2, 3):
             return
         state = self._ahead_state(dev, slot, create=True)
         if len(state["pending"]) >= 2:
