@@ -63,78 +63,52 @@ inline uint32_t wide_part_cap(const SlabGeom &geo, int64_t list_cap) {
   return (uint32_t)((share + share / 4 + 1024 + 63) / 64 * 64);
 }
 
-// The parts of a bucket's slab as one sequence of records: where record j of the sequence sits.
-struct WideParts {
-  uint32_t cum[kWideSplit + 1];  // records in the parts before part q
-  uint32_t first;                // number of the bucket's first part
-  uint32_t cap;                  // entries a part holds
-  __device__ inline uint32_t total() const { return cum[kWideSplit]; }
-  __device__ inline size_t place(uint32_t j) const {
-    uint32_t q = 0, base = 0;
-#pragma unroll
-    for (int i = 1; i < kWideSplit; ++i) {
-      const bool past = j >= cum[i];
-      q += past;
-      base = past ? cum[i] : base;
-    }
-    return (size_t)(first + q) * cap + (j - base);
-  }
-};
-
-// Reads the part counts of bucket b (clamped to the parts' capacity: the producer flagged the overflow).
-__device__ inline WideParts wide_parts(const uint32_t *cursor, uint32_t b, uint32_t cap) {
-  WideParts p;
-  p.first = b * kWideSplit;
-  p.cap = cap;
-  uint32_t c[kWideSplit];
-#pragma unroll
-  for (int q = 0; q < kWideSplit; ++q) c[q] = cursor[(b * kWideSplit + q) * kWidePad];
-  p.cum[0] = 0;
-#pragma unroll
-  for (int q = 0; q < kWideSplit; ++q) p.cum[q + 1] = p.cum[q] + (c[q] < cap ? c[q] : cap);
-  return p;
-}
-
-// Counters of the narrow ranges: 16 bits each, two to a word, with a zero in front of the first (the end of
-// "range -1"), so that range s spans [cnt[s - 1], cnt[s]) once the counters have become running ends.
+// Counters of the narrow ranges: 16 bits each, two to a word.  Thread t of the workgroup owns ranges
+// 16 t .. 16 t + 15 when the counts become running sums; range s is kept at place (s % 16) * 1024 + s / 16, so
+// that the lanes of a wave then walk through consecutive halfwords (and the atomics of the counting steps, on
+// ranges that a hash picks, spread over the banks whatever the layout).
 struct alignas(16) WideCounters {
-  uint32_t pad[4];                 // cnt16[-8 .. -1]: stays zero
-  uint32_t word[kWideSubs / 2];    // cnt16[0 .. kWideSubs)
-  __device__ inline uint16_t *cnt16() { return reinterpret_cast<uint16_t *>(word); }
+  uint32_t word[kWideSubs / 2];
+  static_assert(kWideSubs == 16 * kWideBlock, "sixteen ranges per thread");
+  __device__ static inline uint32_t place(uint32_t sub) { return ((sub & 15u) << 10) | (sub >> 4); }
+  __device__ inline const uint16_t *half() const { return reinterpret_cast<const uint16_t *>(word); }
   __device__ inline void clear() {
-    uint32_t *all = reinterpret_cast<uint32_t *>(this);
-    for (int i = threadIdx.x; i < kWideSubs / 2 + 4; i += kWideBlock) all[i] = 0;
+    for (int i = threadIdx.x; i < kWideSubs / 2; i += kWideBlock) word[i] = 0;
   }
-  __device__ inline void count(uint32_t sub) { atomicAdd(&word[sub >> 1], 1u << (16 * (sub & 1u))); }
+  __device__ inline void count(uint32_t sub) {
+    const uint32_t p = place(sub);
+    atomicAdd(&word[p >> 1], 1u << (16 * (p & 1u)));
+  }
   // takes the next place of range `sub` (after starts() the counters are running cursors)
   __device__ inline uint32_t take(uint32_t sub) {
-    const uint32_t sh = 16 * (sub & 1u);
-    return (atomicAdd(&word[sub >> 1], 1u << sh) >> sh) & 0xffffu;
+    const uint32_t p = place(sub), sh = 16 * (p & 1u);
+    return (atomicAdd(&word[p >> 1], 1u << sh) >> sh) & 0xffffu;
   }
-  // Counts -> exclusive starts, by the whole workgroup (thread t owns ranges 16 t .. 16 t + 15); returns the
-  // number of records counted.  smem: kWideBlock / 64 + 1 words.
-  __device__ inline uint32_t starts(uint32_t *smem) {
-    static_assert(kWideSubs == 16 * kWideBlock, "sixteen ranges per thread");
-    uint4 *mine = reinterpret_cast<uint4 *>(word) + 2 * threadIdx.x;
-    const uint4 a = mine[0], b = mine[1];
-    const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-    uint32_t sum = 0;
+  // once every record has taken its place the counter of range s holds where the range ends
+  __device__ inline uint32_t end_of(uint32_t sub) const { return half()[place(sub)]; }
+  __device__ inline uint32_t start_of(uint32_t sub) const { return sub ? half()[place(sub - 1u)] : 0u; }
+  // Counts -> exclusive starts, by the whole workgroup; returns the number of records counted and sets *big
+  // (a word of LDS, zero before) if any range holds more than `limit` of them; the caller may read *big once
+  // it has synchronised.  smem: kWideBlock / 64 + 1 words.
+  __device__ inline uint32_t starts(uint32_t *smem, uint32_t limit, uint32_t *big) {
+    uint16_t *h = reinterpret_cast<uint16_t *>(word);
+    uint32_t c[16];
+    uint32_t sum = 0, over = 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) sum += (w[i] & 0xffffu) + (w[i] >> 16);
-    uint32_t total;
-    uint32_t run = block_exclusive_scan<uint32_t, kWideBlock>(sum, smem, &total);
-    uint32_t o[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t lo = run;
-      run += w[i] & 0xffffu;
-      const uint32_t hi = run;
-      run += w[i] >> 16;
-      o[i] = (lo & 0xffffu) | (hi << 16);
+    for (int e = 0; e < 16; ++e) {
+      c[e] = h[e * kWideBlock + threadIdx.x];
+      sum += c[e];
+      over |= c[e] > limit;
     }
+    uint32_t total;
+    if (over) *big = 1u;
+    uint32_t run = block_exclusive_scan<uint32_t, kWideBlock>(sum, smem, &total);
     if (total <= 0xffffu) {  // more than the counters hold: the caller gives up anyway
-      mine[0] = make_uint4(o[0], o[1], o[2], o[3]);
-      mine[1] = make_uint4(o[4], o[5], o[6], o[7]);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        h[e * kWideBlock + threadIdx.x] = (uint16_t)run;
+        run += c[e];
+      }
     }
     return total;
   }

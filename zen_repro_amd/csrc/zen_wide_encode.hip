@@ -85,43 +85,46 @@ int wide_device_cus() {
 
 namespace {
 
-constexpr int kWideItems = 20;                          // raw records per thread (candidates below the threshold included)
-constexpr int kWideRaw = kWideBlock * kWideItems;       // raw records per bucket, at most
+constexpr int kWideRounds = 3;                          // a part of a bucket's slab is read in rounds of kWideBlock records
+constexpr int kWideItems = kWideSplit * kWideRounds;    // raw records per thread (candidates below the threshold included)
+constexpr int kWidePartMax = kWideBlock * kWideRounds;  // raw records of one part, at most
 constexpr int kWideMove = 1024;                         // entries that may move into one bucket from elsewhere
 constexpr int kWideRemoved = 1024;                      // entries of a bucket that may lose their level-1 slot
+constexpr int kWideQueue = (2 * kWideMove + kWideMove + kWideRemoved) / 2;  // records set aside while ranking
+constexpr int kWideLanes = 4;                           // records a thread handles per step of the ranking loops
 constexpr int kWideGroupLimit = 512;                    // records in one narrow range: bounds the rank loop
 constexpr int kWideIndexStep = 4;                       // every 4th narrow range has its first sorted place written down
 constexpr int kWideIndexLen = kWideSubs / kWideIndexStep;
 constexpr int kWideCtrPad = 8;                          // words between two per-partition counters
+constexpr int kWideSteps = kWideSplit * kWideRounds / 4;  // = kWideItems / kWideLanes
+constexpr int kWideProbeLimit = 512;                    // probes in the map before it counts as full
 constexpr uint32_t kInvalid = 0xffffffffu;
-static_assert(kWideRaw <= (1 << 15) && kWideCap <= kWideRaw, "raw places in 15 bits");
+// a record's raw place: part * 4096 + place inside the part
+static_assert(kWidePartMax <= 4096 && kWideSplit * 4096 <= (1 << 15), "raw places in 15 bits");
 static_assert(kWideMove <= kWideBlock && kWideRemoved <= kWideBlock, "one entry per thread");
+static_assert(kWideSplit % 4 == 0, "steps of four records");
+static_assert(kWideMove < (1 << 12) && kWideRemoved < (1 << 12), "two counts in one word");
 
 struct WideTables {
   // zero between calls (kept in the caller's zero table, behind the hash map)
   uint32_t *cursor;            // [B * kWideSplit * kWidePad] part cursors
   uint32_t *gbar;              // [P * kWidePad] barrier counters of the partitions' workgroups
+  uint32_t *pdone;             // [P * kWidePad] workgroups of the partition that have finished
   uint32_t *log_n;             // [P * kWideCtrPad] entries that lost level 1, per partition
   uint32_t *dlog_n;            // [P * kWideCtrPad] level-1 owners pushed out by a level-2/3 prober, per partition
-  uint32_t *serial_n;          // [P * kWideCtrPad] entries that found no slot
-  uint32_t *movein_n;          // [B] entries whose final slot lies in the bucket but whose level-1 slot does not own it
-  uint32_t *dl_n;              // [B] owners pushed out of the bucket
   unsigned long long *desc;    // [B] what every bucket contributes to the output (flag + count)
   uint32_t *done;              // [1] workgroups that have finished
-  Counters *ctr;
+  Counters *ctr;               // [P] (the claims of the partition's map)
   // workspace
   uint32_t *words;             // [3][B * kWideSplit * part_cap] raw candidates: index, level-1 slot, value
   uint32_t *slab_idx;          // [B * kWideCap] sorted indices (| kRemovedBit: lost level 1)
   uint32_t *sub_index;         // [B * kWideIndexLen] first sorted place of narrow range 4 j, and of 4 j + 4 in the high half
-  uint32_t *bucket_n;          // [B] sorted records
-  uint32_t *bucket_lo;         // [B] smallest level-1 slot
   uint32_t *log_t, *log_cell;  // [P * log_cap] losers; the map cell each ends in (kNone: none)
-  uint32_t *dlog_t, *dlog_cell;
-  uint32_t *mv_slot, *mv_idx;  // [B * kWideMove]
-  uint32_t *dl_pos;            // [B * kWideRemoved] sorted places of the owners pushed out
+  uint32_t *dlog_t, *dlog_cell, *dlog_at;  // the same for the owners pushed out, and bucket << 16 | sorted place of each
   uint32_t *ser_idx;           // [P * kSlabSerialCap]
   uint32_t part_cap;
   uint32_t log_cap;            // per partition
+  uint32_t map_log2;           // cells of one partition's map
   int partitions;
 };
 
@@ -135,25 +138,53 @@ struct WideShared {
     WideCounters cnt;
     S val[kWideCap];          // the sorted values
   };
-  uint32_t mk[kWideMove];     // slots of the moved-in entries
-  uint32_t mi[kWideMove];     // their indices
-  uint32_t mp[kWideMove];     // sorted place in front of which each slips in, by ascending slot
-  uint32_t rm[kWideRemoved];  // losers' indices while they are logged, then the sorted places of the removed entries
+  union {
+    struct {
+      uint32_t mk[kWideMove];     // slots of the moved-in entries
+      uint32_t mi[kWideMove];     // their indices
+      uint32_t mp[kWideMove];     // sorted place in front of which each slips in, by ascending slot
+      uint32_t rm[kWideRemoved];  // losers' indices while they are logged, then the sorted places of the removed entries
+    };
+    struct {                      // while ranking: the records set aside
+      uint32_t q_word[kWideQueue];   // the record's word, then its rank (| kRemovedBit)
+      uint32_t q_range[kWideQueue];  // where its narrow range starts | where it ends << 16
+    };
+  };
   int32_t delta[kWideCap / 64];
   uint32_t scan[kWideBlock / 64 + 1];
   uint64_t scan64[kWideBlock / 64 + 1];
-  uint32_t lo, lost_n, nrm, base, flag;
+  uint32_t lo, lost_n, nrm, mv_n, ser_n, base, flag, big;
 };
 
 __device__ inline unsigned long long cell_fresh(const unsigned long long *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// map_min (zen_hashmap.h) with one trip to memory where the slot is met for the first time: the cell is
+// claimed with a compare-and-swap straight away, and the count of claims is raised without waiting for it (a
+// map that fills up shows in the length of the probe sequences instead).
+__device__ inline uint32_t map_min_claim(unsigned long long *cells, uint32_t log2, uint32_t slot, uint32_t t,
+                                         Counters *ctr, bool *full) {
+  const uint32_t mask = (1u << log2) - 1u;
+  const unsigned long long mine = ((unsigned long long)(slot + 1u) << 32) | t;
+  uint32_t h = cell_home(slot, log2);
+  for (uint32_t probes = 0; probes <= mask && probes < (uint32_t)kWideProbeLimit; ++probes, h = (h + 1u) & mask) {
+    const unsigned long long cur = atomicCAS(&cells[h], 0ull, mine);
+    if (cur == 0ull) {
+      atomicAdd(&ctr->claims, 1u);
+      return kNone;
+    }
+    if ((uint32_t)(cur >> 32) == slot + 1u) return (uint32_t)atomicMin(&cells[h], mine);
+  }
+  *full = true;
+  return 0u;  // pretend a smaller index owns it: the chain moves on and the call is retried anyway
+}
+
 // map_find while other workgroups of the running kernel have been writing the map.
 __device__ inline uint32_t map_find_fresh(const unsigned long long *cells, uint32_t log2, uint32_t slot, uint32_t *cell_out) {
   const uint32_t mask = (1u << log2) - 1u;
   uint32_t h = cell_home(slot, log2);
-  for (uint32_t probes = 0; probes <= mask; ++probes, h = (h + 1u) & mask) {
+  for (uint32_t probes = 0; probes <= mask && probes < (uint32_t)kWideProbeLimit; ++probes, h = (h + 1u) & mask) {
     const unsigned long long cur = cell_fresh(&cells[h]);
     if (cur == 0ull) return kNone;
     if ((uint32_t)(cur >> 32) == slot + 1u) {
@@ -171,13 +202,11 @@ __device__ inline uint32_t map_find_fresh(const unsigned long long *cells, uint3
 __device__ inline uint32_t wide_head(const SlabGeom &geo, const WideTables &tb, uint32_t slot, uint32_t *place_out,
                                      uint32_t *bucket_out) {
   const uint32_t b = geo.bucket_of(slot);
-  const uint32_t n = load_agent(&tb.bucket_n[b]);
-  const uint32_t lo = load_agent(&tb.bucket_lo[b]);
-  const uint32_t j = ((slot - lo) >> geo.sub_shift) / (uint32_t)kWideIndexStep;
+  const uint32_t j = ((slot - geo.first_key(b)) >> geo.sub_shift) / (uint32_t)kWideIndexStep;
   if (j >= (uint32_t)kWideIndexLen) return kNone;
   const uint32_t w = load_agent(&tb.sub_index[(size_t)b * kWideIndexLen + j]);
-  uint32_t p = w & 0xffffu, end = w >> 16;
-  if (end > n) end = n;
+  uint32_t p = w & 0xffffu;
+  const uint32_t end = w >> 16;
   const uint32_t *idx = tb.slab_idx + (size_t)b * kWideCap;
   for (; p < end; p += 4) {
     uint32_t t[4];
@@ -198,10 +227,17 @@ __device__ inline uint32_t wide_head(const SlabGeom &geo, const WideTables &tb, 
   return kNone;
 }
 
+#ifdef ZEN_WIDE_TIMING
+__device__ unsigned long long g_wide_dbg[256 * 32];
+#define WIDE_MARK(k) do { if (threadIdx.x == 0) g_wide_dbg[blockIdx.x * 32 + (k)] = wall_clock64(); } while (0)
+#else
+#define WIDE_MARK(k) do { } while (0)
+#endif
+
 template <typename S>
 __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g, WideTables tb,
                                                           const uint32_t *__restrict__ filter,
-                                                          unsigned long long *cells, uint32_t log2, int64_t spp,
+                                                          unsigned long long *cells, int64_t spp,
                                                           const S *__restrict__ dense, int32_t *__restrict__ out_idx,
                                                           S *__restrict__ out_val, uint32_t capacity,
                                                           int64_t *__restrict__ splits, uint32_t *clear,
@@ -210,156 +246,260 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
   const uint32_t b = blockIdx.x, B = geo.nbuckets, bpp = geo.bpp;
   const uint32_t part = b / bpp;
   const uint32_t tid = threadIdx.x;
+  WIDE_MARK(0);
   // counters of the kernels before this one that nobody needs any more: back to zero, a slice per workgroup
   for (uint32_t i = b * kWideBlock + tid; i < clear_words; i += B * kWideBlock) clear[i] = 0;
   if (tid == 0) {
     sh.lo = geo.first_key(b);
-    sh.lost_n = 0;
-    sh.nrm = 0;
+    sh.lost_n = sh.nrm = sh.mv_n = sh.ser_n = sh.big = 0;
   }
   sh.cnt.clear();
-  const WideParts parts = wide_parts(tb.cursor, b, tb.part_cap);
-  uint32_t n_raw = parts.total();
+  // the bucket's candidates sit in kWideSplit parts; item r * kWideSplit + q of a thread is the record at
+  // place tid + r * kWideBlock of part q
+  uint32_t pcount[kWideSplit];
+  uint32_t longest = 0;
+#pragma unroll
+  for (int q = 0; q < kWideSplit; ++q) {
+    pcount[q] = tb.cursor[(b * kWideSplit + q) * kWidePad];
+    if (pcount[q] > tb.part_cap) pcount[q] = tb.part_cap;  // the producer flagged the overflow
+    longest = pcount[q] > longest ? pcount[q] : longest;
+  }
   bool declined = false;
-  if (n_raw > (uint32_t)kWideRaw) {  // more candidates than the workgroup looks at: another path answers
+  if (longest > (uint32_t)kWidePartMax) {  // more candidates than the workgroup looks at: another path answers
     declined = true;
-    n_raw = 0;
+#pragma unroll
+    for (int q = 0; q < kWideSplit; ++q) pcount[q] = 0;
+    longest = 0;
   }
   const uint32_t thr_key = filter ? filter[0] : 0u;
   const size_t plane = (size_t)B * kWideSplit * tb.part_cap;
-  const uint32_t *idx_plane = tb.words;
-  const uint32_t *slot_plane = tb.words + plane;
-  const S *val_plane = reinterpret_cast<const S *>(tb.words + 2 * plane);
+  const uint32_t *idx_plane = tb.words + (size_t)b * kWideSplit * tb.part_cap;
+  const uint32_t *slot_plane = idx_plane + plane;
+  const S *val_plane = reinterpret_cast<const S *>(tb.words + 2 * plane) + (size_t)b * kWideSplit * tb.part_cap;
   __syncthreads();
   const uint32_t lo = sh.lo;
   const int shift = geo.sub_shift;
   const uint32_t low_mask = (1u << shift) - 1u;
 
-  // ---- the bucket's candidates: slot offsets in registers; loads in no branch, so that all are in flight
+  // ---- slot offsets in registers; loads in no branch (places past a part's end are pulled back onto its
+  // first record), so that all are in flight together
   uint32_t off[kWideItems];
 #pragma unroll
-  for (int i = 0; i < kWideItems; ++i) {
-    const uint32_t j = tid + (uint32_t)i * kWideBlock;
-    const size_t at = parts.place(j < n_raw ? j : 0u);
-    const uint32_t slot = slot_plane[at];
-    const S v = val_plane[at];
-    const bool keep = j < n_raw && (v & KeyOf<S>::kMask) >= thr_key;
-    off[i] = keep ? slot - lo : kInvalid;
+  for (int r = 0; r < kWideRounds; ++r) {
+#pragma unroll
+    for (int q = 0; q < kWideSplit; ++q) off[r * kWideSplit + q] = kInvalid;
+    if ((uint32_t)r * kWideBlock < longest) {
+#pragma unroll
+      for (int q = 0; q < kWideSplit; ++q) {
+        const uint32_t e = tid + (uint32_t)r * kWideBlock;
+        const size_t at = (size_t)q * tb.part_cap + (e < pcount[q] ? e : 0u);
+        const uint32_t slot = slot_plane[at];
+        const S v = val_plane[at];
+        const bool keep = e < pcount[q] && (v & KeyOf<S>::kMask) >= thr_key;
+        off[r * kWideSplit + q] = keep ? slot - lo : kInvalid;
+      }
+    }
   }
+  WIDE_MARK(1);
 #pragma unroll
   for (int i = 0; i < kWideItems; ++i)
     if (off[i] != kInvalid) sh.cnt.count(off[i] >> shift);
   __syncthreads();
-  uint32_t n;
-  {
-    // a narrow range that holds hundreds of records (keys piled on a few values) would keep the rank loop busy
-    // for too long: declined as well
-    const uint16_t *c16 = sh.cnt.cnt16();
-    uint32_t big = 0;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) big |= c16[tid * 16 + e] > (uint32_t)kWideGroupLimit;
-    if (big) sh.lost_n = 1;  // any nonzero value: read back below, then put back to zero
-    n = sh.cnt.starts(sh.scan);
-  }
+  // a narrow range that holds hundreds of records (keys piled on a few values) would keep the rank loop busy
+  // for too long: declined as well
+  uint32_t n = sh.cnt.starts(sh.scan, (uint32_t)kWideGroupLimit, &sh.big);
   __syncthreads();
-  if (n > (uint32_t)kWideCap || sh.lost_n) {
+  if (n > (uint32_t)kWideCap || sh.big) {
     declined = true;
     __syncthreads();
     sh.cnt.clear();
-    if (tid == 0) sh.lost_n = 0;
 #pragma unroll
     for (int i = 0; i < kWideItems; ++i) off[i] = kInvalid;
     n = 0;
     __syncthreads();
   }
   if (declined && tid == 0) atomicOr(status, ZEN_STAT_RETRY);
+  // From here on a thread's records are worked through in kWideSteps steps of kWideLanes records, by a loop
+  // whose body always handles the first kWideLanes registers of the set and then rotates the set: with the
+  // body written out for all records the kernel's code no longer fits the instruction cache, and every
+  // workgroup runs it just once.
+  auto rotate = [](uint32_t (&a)[kWideItems]) {
+    uint32_t head[kWideLanes];
 #pragma unroll
-  for (int i = 0; i < kWideItems; ++i) {
-    if (off[i] != kInvalid) {
-      const uint32_t p = sh.cnt.take(off[i] >> shift);
-      sh.word[p] = ((off[i] & low_mask) << 15) | (tid + (uint32_t)i * kWideBlock);
-    }
-  }
-  __syncthreads();
-  // rank = records of the bucket with a smaller (slot, index): the records of the narrow ranges before it,
-  // plus those of its own range with a smaller slot, plus (rare) those with its slot and a smaller index
-  uint32_t rk[kWideItems];
-  {
-    const uint16_t *c16 = sh.cnt.cnt16();
+    for (int k = 0; k < kWideLanes; ++k) head[k] = a[k];
 #pragma unroll
-    for (int i = 0; i < kWideItems; ++i) {
-      rk[i] = kInvalid;
-      if (off[i] != kInvalid) {
-        const uint32_t sub = off[i] >> shift;
-        const uint32_t g1 = c16[sub], g0 = c16[(int)sub - 1];
-        const uint32_t j = tid + (uint32_t)i * kWideBlock;
-        const uint32_t key = off[i] & low_mask;
-        const uint32_t my = (key << 15) | j;
-        uint32_t less = 0, twins = 0;
-        for (uint32_t u = g0; u < g1; u += 4) {
-          const uint32_t last = g1 - 1u;
-          uint32_t a[4];
+    for (int i = 0; i + kWideLanes < kWideItems; ++i) a[i] = a[i + kWideLanes];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) a[q] = sh.word[u + q < last ? u + q : last];
+    for (int k = 0; k < kWideLanes; ++k) a[kWideItems - kWideLanes + k] = head[k];
+  };
+  // raw place of the record in lane k of step s: part * 4096 + place inside the part
+  auto raw_place = [&](int s, int k) {
+    constexpr int kPer = kWideSplit / kWideLanes;  // steps per round
+    return (uint32_t)((s % kPer) * kWideLanes + k) * 4096u + tid + (uint32_t)(s / kPer) * kWideBlock;
+  };
+  // steps of rounds that no part of the slab reaches hold nothing: the loops stop short of them
+  const int steps = longest == 0 ? 0 : (int)((longest + kWideBlock - 1) / kWideBlock) * (kWideSplit / kWideLanes);
+#pragma unroll 1
+  for (int s = 0; s < kWideSteps; ++s) {
+    if (s < steps) {
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            if (u + q < g1) {
-              less += (a[q] >> 15) < key;
-              twins += (a[q] >> 15) == key && a[q] != my;
-            }
-          }
+      for (int k = 0; k < kWideLanes; ++k) {
+        if (off[k] != kInvalid) {
+          const uint32_t p = sh.cnt.take(off[k] >> shift);
+          sh.word[p] = ((off[k] & low_mask) << 15) | raw_place(s, k);
         }
-        uint32_t lost = 0;
-        if (twins) {  // another candidate with this very slot: the smaller index comes first
-          const uint32_t mine = idx_plane[parts.place(j)];
-          for (uint32_t u = g0; u < g1; ++u) {
-            const uint32_t w = sh.word[u];
-            if ((w >> 15) == key && w != my) lost += idx_plane[parts.place(w & 0x7fffu)] < mine;
-          }
-        }
-        rk[i] = (g0 + less + lost) | (lost ? kRemovedBit : 0u);
       }
     }
+    rotate(off);
   }
   __syncthreads();
+  WIDE_MARK(2);
+  // rank = records of the bucket with a smaller (slot, index): the records of the narrow ranges before it,
+  // plus those of its own range with a smaller slot, plus (rare) those with its slot and a smaller index.
+  // A round's eight records at a time: first where every record's range starts and ends, then the range's
+  // first three words of each (most ranges hold no more), all in flight together.
+  uint32_t rk[kWideItems];
+  auto raw_at = [&](uint32_t j) { return (size_t)(j >> 12) * tb.part_cap + (j & 4095u); };
+#pragma unroll
+  for (int i = 0; i < kWideItems; ++i) rk[i] = kInvalid;
+#pragma unroll 1
+  for (int s = 0; s < kWideSteps; ++s) {
+    constexpr int kAhead = 4;
+    uint32_t out[kWideLanes];
+#pragma unroll
+    for (int k = 0; k < kWideLanes; ++k) out[k] = kInvalid;
+    if (s < steps) {
+    uint32_t g0[kWideLanes], g1[kWideLanes], a[kWideLanes][kAhead];
+#pragma unroll
+    for (int k = 0; k < kWideLanes; ++k) {
+      const uint32_t sub = off[k] != kInvalid ? off[k] >> shift : 0u;
+      g0[k] = sh.cnt.start_of(sub);
+      g1[k] = sh.cnt.end_of(sub);
+    }
+#pragma unroll
+    for (int k = 0; k < kWideLanes; ++k) {
+      const uint32_t last = g1[k] > g0[k] ? g1[k] - 1u : g0[k];
+#pragma unroll
+      for (int e = 0; e < kAhead; ++e) a[k][e] = sh.word[g0[k] + e < last ? g0[k] + e : last];
+    }
+#pragma unroll
+    for (int k = 0; k < kWideLanes; ++k) {
+      if (off[k] != kInvalid) {
+        const uint32_t key = off[k] & low_mask;
+        const uint32_t my = (key << 15) | raw_place(s, k);
+        uint32_t less = 0, twins = 0;
+#pragma unroll
+        for (int e = 0; e < kAhead; ++e) {
+          if (g0[k] + e < g1[k]) {
+            less += (a[k][e] >> 15) < key;
+            twins += (a[k][e] >> 15) == key && a[k][e] != my;
+          }
+        }
+        uint32_t x = g0[k] + less;
+        if (twins || g1[k] - g0[k] > (uint32_t)kAhead) {
+          // A range of more than kAhead records, or another candidate with this very slot (the smaller
+          // index then comes first, and comparing indices takes trips to memory): a wave would wait for
+          // every lane that has one of these, at every record.  They are set aside and settled afterwards,
+          // one per thread.
+          const uint32_t at = atomicAdd(&sh.lost_n, 1u);
+          if (at < (uint32_t)kWideQueue) {
+            sh.q_word[at] = my;
+            sh.q_range[at] = g0[k] | (g1[k] << 16);
+            x = kRemovedBit | at;  // pending: place in the queue
+          }
+        }
+        out[k] = x;
+      }
+    }
+    }
+    rotate(off);
+    rotate(rk);  // the step's ranks enter at the end: after the last step rank i belongs to record i
+#pragma unroll
+    for (int k = 0; k < kWideLanes; ++k) rk[kWideItems - kWideLanes + k] = out[k];
+    WIDE_MARK(16 + s);
+  }
+  WIDE_MARK(22);
+  __syncthreads();
+  {
+    WIDE_MARK(23);
+    uint32_t pending = sh.lost_n;
+    if (pending > (uint32_t)kWideQueue) {
+      if (tid == 0) atomicOr(status, ZEN_STAT_RETRY);
+      pending = kWideQueue;
+    }
+    for (uint32_t e = tid; e < pending; e += kWideBlock) {
+      const uint32_t my = sh.q_word[e], key = my >> 15;
+      const uint32_t g0 = sh.q_range[e] & 0xffffu, g1 = sh.q_range[e] >> 16;
+      uint32_t less = 0, twins = 0;
+      for (uint32_t u = g0; u < g1; ++u) {
+        const uint32_t w = sh.word[u];
+        less += (w >> 15) < key;
+        twins += (w >> 15) == key && w != my;
+      }
+      uint32_t lost = 0;
+      if (twins) {
+        const uint32_t mine = idx_plane[raw_at(my & 0x7fffu)];
+        for (uint32_t u = g0; u < g1; ++u) {
+          const uint32_t w = sh.word[u];
+          if ((w >> 15) == key && w != my) lost += idx_plane[raw_at(w & 0x7fffu)] < mine;
+        }
+      }
+      sh.q_word[e] = (g0 + less + lost) | (lost ? kRemovedBit : 0u);  // the entry's thread is its only reader
+    }
+    WIDE_MARK(24);
+    __syncthreads();
+    WIDE_MARK(25);
+#pragma unroll
+    for (int i = 0; i < kWideItems; ++i)
+      if (rk[i] != kInvalid && (rk[i] & kRemovedBit)) rk[i] = sh.q_word[rk[i] & kIndexMask];
+    __syncthreads();  // the queue's memory serves other lists from here on
+    if (tid == 0) sh.lost_n = 0;
+  }
+  __syncthreads();
+  WIDE_MARK(3);
   // the narrow ranges' first places go to memory for the other workgroups' look-ups before the values take
   // the counters' place
-  {
-    const uint16_t *c16 = sh.cnt.cnt16();
-    for (uint32_t j = tid; j < (uint32_t)kWideIndexLen; j += kWideBlock) {
-      const uint32_t s0 = j * kWideIndexStep;
-      store_agent(&tb.sub_index[(size_t)b * kWideIndexLen + j],
-                  (uint32_t)c16[(int)s0 - 1] | ((uint32_t)c16[s0 + kWideIndexStep - 1] << 16));
-    }
+  for (uint32_t j = tid; j < (uint32_t)kWideIndexLen; j += kWideBlock) {
+    const uint32_t s0 = j * kWideIndexStep;
+    store_agent(&tb.sub_index[(size_t)b * kWideIndexLen + j],
+                sh.cnt.start_of(s0) | (sh.cnt.end_of(s0 + kWideIndexStep - 1) << 16));
   }
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < kWideItems; ++i) {
-    const uint32_t j = tid + (uint32_t)i * kWideBlock;
-    const size_t at = parts.place(rk[i] != kInvalid ? j : 0u);
-    const uint32_t t = idx_plane[at];
-    const S v = val_plane[at];
-    if (rk[i] != kInvalid) {
-      const uint32_t r = rk[i] & kIndexMask;
-      sh.idx[r] = t | (rk[i] & kRemovedBit);
-      sh.val[r] = v;
-      if (rk[i] & kRemovedBit) {
-        const uint32_t q = atomicAdd(&sh.lost_n, 1u);
-        if (q < (uint32_t)kWideRemoved) sh.rm[q] = t;
+  for (int r = 0; r < kWideRounds; ++r) {
+    if ((uint32_t)r * kWideBlock < longest) {
+      uint32_t t[kWideSplit];
+      S v[kWideSplit];
+#pragma unroll
+      for (int q = 0; q < kWideSplit; ++q) {
+        const uint32_t e = tid + (uint32_t)r * kWideBlock;
+        const size_t at = (size_t)q * tb.part_cap + (rk[r * kWideSplit + q] != kInvalid ? e : 0u);
+        t[q] = idx_plane[at];
+        v[q] = val_plane[at];
+      }
+#pragma unroll
+      for (int q = 0; q < kWideSplit; ++q) {
+        const uint32_t x = rk[r * kWideSplit + q];
+        if (x != kInvalid) {
+          const uint32_t p = x & kIndexMask;
+          sh.idx[p] = t[q] | (x & kRemovedBit);
+          sh.val[p] = v[q];
+          if (x & kRemovedBit) {
+            const uint32_t at = atomicAdd(&sh.lost_n, 1u);
+            if (at < (uint32_t)kWideRemoved) sh.rm[at] = t[q];
+          }
+        }
       }
     }
   }
   __syncthreads();
+  WIDE_MARK(4);
   uint32_t lost_n = sh.lost_n;
   if (lost_n > (uint32_t)kWideRemoved) {
     if (tid == 0) atomicOr(status, ZEN_STAT_RETRY);
     lost_n = kWideRemoved;
   }
-  if (tid == 0) {
-    store_agent(&tb.bucket_n[b], n);
-    store_agent(&tb.bucket_lo[b], lo);
-    sh.base = lost_n ? atomicAdd(&tb.log_n[part * kWideCtrPad], lost_n) : 0u;
-  }
+  if (tid == 0) sh.base = lost_n ? atomicAdd(&tb.log_n[part * kWideCtrPad], lost_n) : 0u;
   for (uint32_t p = tid; p < n; p += kWideBlock) store_agent(&tb.slab_idx[(size_t)b * kWideCap + p], sh.idx[p]);
   __syncthreads();
   for (uint32_t i = tid; i < lost_n; i += kWideBlock) {
@@ -370,13 +510,18 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
       atomicOr(status, ZEN_STAT_RETRY);
   }
   uint32_t *gbar = &tb.gbar[part * kWidePad];
+  WIDE_MARK(5);
   group_barrier(gbar, bpp, 1, status);
+  WIDE_MARK(6);
 
-  // ---- levels 2 and 3 for the partition's losers
-  const uint32_t lane_of_group = (b - part * bpp) * kWideBlock + tid, group_threads = bpp * kWideBlock;
+  // ---- levels 2 and 3 for the partition's losers: loser i is the business of workgroup i % bpp, thread
+  // i / bpp (more than bpp * 1024 of them: in rounds)
+  unsigned long long *pcells = cells + ((size_t)part << tb.map_log2);
+  Counters *pctr = &tb.ctr[part];
+  const uint32_t local = b - part * bpp;
   uint32_t losers = load_agent(&tb.log_n[part * kWideCtrPad]);
   if (losers > tb.log_cap) losers = tb.log_cap;
-  for (uint32_t i = lane_of_group; i < losers; i += group_threads) {
+  for (uint32_t i = tid * bpp + local; i < losers; i += bpp * kWideBlock) {
     uint32_t cur = load_agent(&tb.log_t[(size_t)part * tb.log_cap + i]);
     int lv = 1;
     bool full = false;
@@ -393,7 +538,7 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
         ++lv;
         continue;
       }
-      const uint32_t old = map_min(cells, log2, slot, cur, tb.ctr, &full);
+      const uint32_t old = map_min_claim(pcells, tb.map_log2, slot, cur, pctr, &full);
       if (full) {
         atomicOr(status, ZEN_STAT_RETRY);
         break;
@@ -405,16 +550,13 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
       if (old == kNone) {
         // first level-2/3 prober of this slot: its level-1 owner (a larger index, if any) is pushed out
         if (head == kNone) break;
-        const uint32_t at = atomicAdd(&tb.dl_n[head_bucket], 1u);
-        if (at < (uint32_t)kWideRemoved)
-          store_agent(&tb.dl_pos[(size_t)head_bucket * kWideRemoved + at], head_place);
-        else
+        const uint32_t at = atomicAdd(&tb.dlog_n[part * kWideCtrPad], 1u);
+        if (at < tb.log_cap) {
+          store_agent(&tb.dlog_t[(size_t)part * tb.log_cap + at], head);
+          store_agent(&tb.dlog_at[(size_t)part * tb.log_cap + at], (head_bucket << 16) | head_place);
+        } else {
           atomicOr(status, ZEN_STAT_RETRY);
-        const uint32_t at2 = atomicAdd(&tb.dlog_n[part * kWideCtrPad], 1u);
-        if (at2 < tb.log_cap)
-          store_agent(&tb.dlog_t[(size_t)part * tb.log_cap + at2], head);
-        else
-          atomicOr(status, ZEN_STAT_RETRY);
+        }
         cur = head;
         lv = 1;
         continue;
@@ -427,60 +569,60 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
       lv = lw + 1;
     }
   }
+  WIDE_MARK(7);
   group_barrier(gbar, bpp, 2, status);
+  WIDE_MARK(8);
 
-  // ---- final place of every logged entry: the level-2/3 slot it holds in the map, or the serial list
-  {
-    uint32_t pushed = load_agent(&tb.dlog_n[part * kWideCtrPad]);
-    if (pushed > tb.log_cap) pushed = tb.log_cap;
-    for (uint32_t i = lane_of_group; i < losers + pushed; i += group_threads) {
-      const bool first = i < losers;
-      const size_t at_log = (size_t)part * tb.log_cap + (first ? i : i - losers);
-      const uint32_t t = load_agent(first ? &tb.log_t[at_log] : &tb.dlog_t[at_log]);
-      uint32_t prt = 0, cell = kNone, slot = kNone;
-      for (int lv = 1; lv < g.levels && slot == kNone; ++lv) {
-        const uint32_t s = probe_slot(g, t, lv, &prt);
-        uint32_t at = 0;
-        if (map_find_fresh(cells, log2, s, &at) == t) {
-          slot = s;
-          cell = at;
-        }
-      }
-      store_agent(first ? &tb.log_cell[at_log] : &tb.dlog_cell[at_log], cell);
-      if (slot != kNone) {
-        const uint32_t b2 = geo.bucket_of(slot);
-        const uint32_t at = atomicAdd(&tb.movein_n[b2], 1u);
-        if (at < (uint32_t)kWideMove) {
-          store_agent(&tb.mv_slot[(size_t)b2 * kWideMove + at], slot);
-          store_agent(&tb.mv_idx[(size_t)b2 * kWideMove + at], t);
-        } else {
-          atomicOr(status, ZEN_STAT_RETRY);
-        }
-      } else {
-        const uint32_t at = atomicAdd(&tb.serial_n[part * kWideCtrPad], 1u);
-        if (at < (uint32_t)kSlabSerialCap)
-          store_agent(&tb.ser_idx[(size_t)part * kSlabSerialCap + at], t);
-        else  // more than the partition's serial region holds is an overflow; more than this path carries, a retry
-          atomicOr(status, (int64_t)at >= spp ? ZEN_STAT_SERIAL_OVERFLOW : ZEN_STAT_RETRY);
+  // ---- every workgroup of the partition looks at every logged entry: where it finally sits (the level-2/3
+  // slot it holds in the map, or nowhere), and keeps what concerns its bucket: entries whose final slot lies
+  // in it move in, its own owners that were pushed out drop out; the partition's last bucket also gathers the
+  // entries that found no slot
+  const bool last_of_part = local == bpp - 1;
+  uint32_t pushed = load_agent(&tb.dlog_n[part * kWideCtrPad]);
+  if (pushed > tb.log_cap) pushed = tb.log_cap;
+  for (uint32_t i = tid; i < losers + pushed; i += kWideBlock) {
+    const bool first = i < losers;
+    const size_t at_log = (size_t)part * tb.log_cap + (first ? i : i - losers);
+    const uint32_t t = load_agent(first ? &tb.log_t[at_log] : &tb.dlog_t[at_log]);
+    const uint32_t from = first ? 0u : load_agent(&tb.dlog_at[at_log]);
+    if (!first && (from >> 16) == b && (from & 0xffffu) < n) sh.idx[from & 0xffffu] |= kRemovedBit;  // pushed out once
+    uint32_t prt = 0, cell = kNone, slot = kNone;
+    for (int lv = 1; lv < g.levels && slot == kNone; ++lv) {
+      const uint32_t s = probe_slot(g, t, lv, &prt);
+      uint32_t at = 0;
+      if (map_find_fresh(pcells, tb.map_log2, s, &at) == t) {
+        slot = s;
+        cell = at;
       }
     }
-  }
-  group_barrier(gbar, bpp, 3, status);
-
-  // ---- place: the sorted bucket is almost its part of the output already
-  uint32_t pushed_n = load_agent(&tb.dl_n[b]);
-  if (pushed_n > (uint32_t)kWideRemoved) pushed_n = kWideRemoved;
-  if (tid < pushed_n) {
-    const uint32_t p = load_agent(&tb.dl_pos[(size_t)b * kWideRemoved + tid]);
-    if (p < n) sh.idx[p] |= kRemovedBit;  // places are distinct: a slot's owner is pushed out once
-  }
-  uint32_t mv_n = load_agent(&tb.movein_n[b]);
-  if (mv_n > (uint32_t)kWideMove) mv_n = kWideMove;
-  if (tid < mv_n) {
-    sh.mk[tid] = load_agent(&tb.mv_slot[(size_t)b * kWideMove + tid]);
-    sh.mi[tid] = load_agent(&tb.mv_idx[(size_t)b * kWideMove + tid]);
+    if (i % bpp == local) store_agent(first ? &tb.log_cell[at_log] : &tb.dlog_cell[at_log], cell);
+    if (slot != kNone) {
+      if (geo.bucket_of(slot) == b) {
+        const uint32_t at = atomicAdd(&sh.mv_n, 1u);
+        if (at < (uint32_t)kWideMove) {
+          sh.mk[at] = slot;
+          sh.mi[at] = t;
+        }
+      }
+    } else if (last_of_part) {
+      const uint32_t at = atomicAdd(&sh.ser_n, 1u);
+      if (at < (uint32_t)kSlabSerialCap) store_agent(&tb.ser_idx[(size_t)part * kSlabSerialCap + at], t);
+    }
   }
   __syncthreads();
+  WIDE_MARK(9);
+  uint32_t mv_n = sh.mv_n;
+  if (mv_n > (uint32_t)kWideMove) {
+    if (tid == 0) atomicOr(status, ZEN_STAT_RETRY);
+    mv_n = kWideMove;
+  }
+  const uint32_t serial_raw = sh.ser_n;
+  uint32_t serial = serial_raw;
+  if (serial > (uint32_t)kSlabSerialCap) {
+    // more than the partition's serial region holds is an overflow; more than this path carries, a retry
+    if (tid == 0) atomicOr(status, (int64_t)kSlabSerialCap >= spp ? ZEN_STAT_SERIAL_OVERFLOW : ZEN_STAT_RETRY);
+    serial = kSlabSerialCap;
+  }
   for (uint32_t p = tid; p < n; p += kWideBlock) {
     if (sh.idx[p] & kRemovedBit) {
       const uint32_t at = atomicAdd(&sh.nrm, 1u);
@@ -493,9 +635,14 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
     if (tid == 0) atomicOr(status, ZEN_STAT_RETRY);
     rm_n = kWideRemoved;
   }
+  // what the bucket contributes is known: published at once, so that the later buckets find it while this
+  // one still works out its places
+  const uint32_t own_n = n - rm_n + mv_n;  // survivors + moved-in
+  if (tid == 0) desc_store(&tb.desc[b], kDescAggregate | (uint64_t)(own_n + serial));
   {
     // the removed places in ascending order; moved-in entry j: its slot's rank among the moved-in slots (they
-    // are distinct: a slot has one owner) and the sorted place in front of which it slips in
+    // are distinct: a slot has one owner) and the sorted place in front of which it slips in (a bisection of
+    // the bucket, whose slots are hashed again)
     uint32_t x = 0, xr = 0;
     if (tid < rm_n) {
       x = sh.rm[tid];
@@ -505,27 +652,19 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
     if (tid < mv_n) {
       const uint32_t k = sh.mk[tid];
       for (uint32_t u = 0; u < mv_n; ++u) mj += sh.mk[u] < k;
-      const uint32_t j = ((k - lo) >> shift) / (uint32_t)kWideIndexStep;
-      const uint32_t w = j < (uint32_t)kWideIndexLen ? load_agent(&tb.sub_index[(size_t)b * kWideIndexLen + j]) : n | (n << 16);
-      uint32_t p = w & 0xffffu, end = w >> 16;
-      if (end > n) end = n;
-      mplace = p;
-      for (; p < end; ++p) mplace += geo.mod_m(poly(sh.idx[p] & kIndexMask) + kSeed1) < k;
+      uint32_t p0 = 0, p1 = n;
+      while (p0 < p1) {
+        const uint32_t mid = p0 + ((p1 - p0) >> 1);
+        if (geo.mod_m(poly(sh.idx[mid] & kIndexMask) + kSeed1) < k) p0 = mid + 1; else p1 = mid;
+      }
+      mplace = p0;
     }
     __syncthreads();
     if (tid < rm_n) sh.rm[xr] = x;
     if (tid < mv_n) sh.mp[mj] = mplace;
     __syncthreads();
-    // what the bucket contributes, and where it starts: the sum of what the earlier buckets publish (every
-    // workgroup of the launch is resident; the wait is bounded all the same)
-    const bool last_of_part = b % bpp == bpp - 1;
-    uint32_t serial = 0, serial_raw = 0;
-    if (last_of_part) {
-      serial_raw = load_agent(&tb.serial_n[part * kWideCtrPad]);
-      serial = serial_raw > (uint32_t)kSlabSerialCap ? (uint32_t)kSlabSerialCap : serial_raw;
-    }
-    const uint32_t own_n = n - rm_n + mv_n;  // survivors + moved-in
-    if (tid == 0) desc_store(&tb.desc[b], kDescAggregate | (uint64_t)(own_n + serial));
+    // where the bucket starts: the sum of what the earlier buckets publish (every workgroup of the launch is
+    // resident; the wait is bounded all the same)
     uint64_t before = 0;  // low half: entries of all earlier buckets; high half: of the partition's earlier buckets
     if (tid < b) {
       uint64_t d = desc_load(&tb.desc[tid]);
@@ -541,12 +680,16 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
       const uint64_t v = d & 0xffffffffull;
       before = v | (tid >= part * bpp ? v << 32 : 0ull);
     }
+    WIDE_MARK(10);
     uint64_t sums;
     block_exclusive_scan<uint64_t, kWideBlock>(before, sh.scan64, &sums);
     const uint32_t out_base = (uint32_t)sums, in_part = (uint32_t)(sums >> 32);
     // Most stretches of 64 consecutive sorted places contain neither a removed entry nor the place where a
     // moved-in entry slips in: all their entries move by the same amount, found once per stretch.
-    constexpr int32_t kNoDelta = INT32_MIN;
+    // Per stretch of 64 consecutive sorted places: how many moved-in entries slip in at or before its first
+    // place and how many removed entries lie before it (12 bits each), and whether that holds for the whole
+    // stretch (most contain neither a removed entry nor a place where an entry slips in).
+    constexpr uint32_t kSame = 1u << 31;
     for (uint32_t c = tid; c * 64u < n; c += kWideBlock) {
       const uint32_t p0 = c * 64u, p1 = p0 + 63u < n ? p0 + 63u : n - 1u;
       uint32_t mv0 = 0, mv1 = 0, r0 = 0, r1 = 0;
@@ -558,19 +701,25 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
         r0 = lower_bound_u32(sh.rm, rm_n, p0);
         r1 = lower_bound_u32(sh.rm, rm_n, p1);
       }
-      sh.delta[c] = (mv0 == mv1 && r0 == r1) ? (int32_t)(mv0 - r0) : kNoDelta;
+      sh.delta[c] = (int32_t)(mv0 | (r0 << 12) | ((mv0 == mv1 && r0 == r1) ? kSame : 0u));
     }
     __syncthreads();
+    WIDE_MARK(11);
+#pragma unroll 4
     for (uint32_t p = tid; p < n; p += kWideBlock) {
       const uint32_t t = sh.idx[p];
+      const S v = sh.val[p];
+      const uint32_t d = (uint32_t)sh.delta[p >> 6];
       if (!(t & kRemovedBit)) {
-        int32_t delta = sh.delta[p >> 6];
-        if (delta == kNoDelta)
-          delta = (int32_t)((mv_n ? upper_bound_u32(sh.mp, mv_n, p) : 0u) - (rm_n ? lower_bound_u32(sh.rm, rm_n, p) : 0u));
-        const uint32_t pos = out_base + p + (uint32_t)delta;
+        uint32_t mv = d & 0xfffu, r = (d >> 12) & 0xfffu;
+        if (!(d & kSame)) {  // a few steps from the stretch's first place
+          while (mv < mv_n && sh.mp[mv] <= p) ++mv;
+          while (r < rm_n && sh.rm[r] < p) ++r;
+        }
+        const uint32_t pos = out_base + p + mv - r;
         if (pos < capacity) {
           out_idx[pos] = (int32_t)t;
-          out_val[pos] = sh.val[p];
+          out_val[pos] = v;
         }
       }
     }
@@ -604,43 +753,41 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
       if (out_base + own_n + serial > capacity) atomicOr(status, ZEN_STAT_CAPACITY);
     }
   }
+  WIDE_MARK(12);
 
-  // ---- the workgroup that finishes last leaves the borrowed memory as it was: the map's cells and every
-  // counter back at zero
+  // ---- the borrowed memory goes back as it was.  This workgroup was the only reader of its part cursors;
+  // the partition's workgroup that finishes last (all of them are through with the map and the logs then)
+  // empties the cells the partition holds and clears its counters; the launch's last workgroup clears what
+  // the buckets published.
+  if (tid < (uint32_t)kWideSplit) tb.cursor[(b * kWideSplit + tid) * kWidePad] = 0;
   wait_global_acks();
   __syncthreads();
-  if (tid == 0) sh.flag = atomicAdd(tb.done, 1u) == B - 1u;
+  if (tid == 0) {
+    const uint32_t here = atomicAdd(&tb.pdone[part * kWidePad], 1u), all = atomicAdd(tb.done, 1u);
+    sh.flag = (here == bpp - 1u ? 1u : 0u) | (all == B - 1u ? 2u : 0u);
+  }
   __syncthreads();
-  if (!sh.flag) return;
-  const uint32_t P = (uint32_t)tb.partitions;
-  for (uint32_t q = 0; q < P; ++q) {
-    uint32_t nl = load_agent(&tb.log_n[q * kWideCtrPad]), nd = load_agent(&tb.dlog_n[q * kWideCtrPad]);
-    if (nl > tb.log_cap) nl = tb.log_cap;
-    if (nd > tb.log_cap) nd = tb.log_cap;
-    // every occupied cell ends with the index that finally holds its slot, and that index recorded the cell
-    for (uint32_t i = tid; i < nl + nd; i += kWideBlock) {
-      const size_t at = (size_t)q * tb.log_cap + (i < nl ? i : i - nl);
-      const uint32_t cell = load_agent(i < nl ? &tb.log_cell[at] : &tb.dlog_cell[at]);
-      if (cell != kNone) cells[cell] = 0ull;
+  WIDE_MARK(13);
+  if (sh.flag & 1u) {
+    // every occupied cell ends with the index that finally holds its slot, and that index's cell was recorded
+    for (uint32_t i = tid; i < losers + pushed; i += kWideBlock) {
+      const size_t at = (size_t)part * tb.log_cap + (i < losers ? i : i - losers);
+      const uint32_t cell = load_agent(i < losers ? &tb.log_cell[at] : &tb.dlog_cell[at]);
+      if (cell != kNone) pcells[cell] = 0ull;
+    }
+    if (tid == 0) {
+      tb.gbar[part * kWidePad] = 0;
+      tb.pdone[part * kWidePad] = 0;
+      tb.log_n[part * kWideCtrPad] = 0;
+      tb.dlog_n[part * kWideCtrPad] = 0;
+      pctr->logged = pctr->losers = pctr->claims = pctr->displaced = 0;
     }
   }
-  __syncthreads();
-  for (uint32_t i = tid; i < B * kWideSplit; i += kWideBlock) tb.cursor[i * kWidePad] = 0;
-  for (uint32_t i = tid; i < P; i += kWideBlock) {
-    tb.gbar[i * kWidePad] = 0;
-    tb.log_n[i * kWideCtrPad] = 0;
-    tb.dlog_n[i * kWideCtrPad] = 0;
-    tb.serial_n[i * kWideCtrPad] = 0;
+  if (sh.flag & 2u) {
+    for (uint32_t i = tid; i < B; i += kWideBlock) tb.desc[i] = 0ull;
+    if (tid == 0) *tb.done = 0;
   }
-  for (uint32_t i = tid; i < B; i += kWideBlock) {
-    tb.movein_n[i] = 0;
-    tb.dl_n[i] = 0;
-    tb.desc[i] = 0ull;
-  }
-  if (tid == 0) {
-    *tb.done = 0;
-    tb.ctr->logged = tb.ctr->losers = tb.ctr->claims = tb.ctr->displaced = 0;
-  }
+  WIDE_MARK(14);
 }
 
 struct WidePlan {
@@ -665,14 +812,12 @@ WidePlan plan_wide(void *workspace, void *state, const SlabGeom &geo, int partit
     p.ticket = cv.take<uint32_t>(select_stage_ticket_words());
     p.tb.cursor = cv.take<uint32_t>(B * kWideSplit * kWidePad);
     p.tb.gbar = cv.take<uint32_t>(P * kWidePad);
+    p.tb.pdone = cv.take<uint32_t>(P * kWidePad);
     p.tb.log_n = cv.take<uint32_t>(P * kWideCtrPad);
     p.tb.dlog_n = cv.take<uint32_t>(P * kWideCtrPad);
-    p.tb.serial_n = cv.take<uint32_t>(P * kWideCtrPad);
-    p.tb.movein_n = cv.take<uint32_t>(B);
-    p.tb.dl_n = cv.take<uint32_t>(B);
     p.tb.desc = cv.take<unsigned long long>(B);
     p.tb.done = cv.take<uint32_t>(1);
-    p.tb.ctr = cv.take<Counters>(1);
+    p.tb.ctr = cv.take<Counters>(P);
     p.refine_hist = cv.take<uint32_t>(dtype == ZEN_BF16 ? 1 : (size_t)kRefineBins + 1);
     p.state_bytes = cv.used;
   }
@@ -686,16 +831,12 @@ WidePlan plan_wide(void *workspace, void *state, const SlabGeom &geo, int partit
   p.tb.words = cv.take<uint32_t>((size_t)3 * B * kWideSplit * p.tb.part_cap);
   p.tb.slab_idx = cv.take<uint32_t>(B * kWideCap);
   p.tb.sub_index = cv.take<uint32_t>(B * kWideIndexLen);
-  p.tb.bucket_n = cv.take<uint32_t>(B);
-  p.tb.bucket_lo = cv.take<uint32_t>(B);
   p.tb.log_cap = (uint32_t)(list_cap / 4 / (int64_t)P + 1024);
   p.tb.log_t = cv.take<uint32_t>(P * p.tb.log_cap);
   p.tb.log_cell = cv.take<uint32_t>(P * p.tb.log_cap);
   p.tb.dlog_t = cv.take<uint32_t>(P * p.tb.log_cap);
   p.tb.dlog_cell = cv.take<uint32_t>(P * p.tb.log_cap);
-  p.tb.mv_slot = cv.take<uint32_t>(B * kWideMove);
-  p.tb.mv_idx = cv.take<uint32_t>(B * kWideMove);
-  p.tb.dl_pos = cv.take<uint32_t>(B * kWideRemoved);
+  p.tb.dlog_at = cv.take<uint32_t>(P * p.tb.log_cap);
   p.tb.ser_idx = cv.take<uint32_t>(P * kSlabSerialCap);
   p.tb.partitions = partitions;
   p.bytes = cv.used;
@@ -729,6 +870,11 @@ int wide_load_balance(const SlabBalanceArgs &a, size_t state_offset, hipStream_t
   WidePlan p = plan_wide(a.workspace, state, geo, a.partitions, a.dtype, list_capacity(a.capacity));
   if (state_offset + p.state_bytes > (size_t)a.g.m * sizeof(int32_t))
     return fail(ZEN_EINVAL, "wide_load_balance: table too small for the counters");
+  // the map is cut into one part per partition (a partition's chains never leave its slots), so that a
+  // partition's workgroups can empty their part as soon as they are through with it
+  const int part_bits = ceil_log2_u64((uint64_t)a.partitions - 1u);
+  if ((int)a.hash_log2 < part_bits + 8) return fail(ZEN_EINVAL, "wide_load_balance: table too small for the map");
+  p.tb.map_log2 = a.hash_log2 - (uint32_t)part_bits;
   const bool refine = a.k > 0 && a.dtype == ZEN_F32;
   StageArgs sc;
   sc.in = a.input;
@@ -779,11 +925,11 @@ int wide_load_balance(const SlabBalanceArgs &a, size_t state_offset, hipStream_t
     ProfScope prof(kProfWideTail, s);
     if (a.dtype == ZEN_BF16)
       k_wide_tail<uint16_t><<<dim3(geo.nbuckets), dim3(kWideBlock), 0, s>>>(
-          geo, a.g, p.tb, filter, a.hash, a.hash_log2, a.spp, static_cast<const uint16_t *>(a.input), a.out_idx,
+          geo, a.g, p.tb, filter, a.hash, a.spp, static_cast<const uint16_t *>(a.input), a.out_idx,
           static_cast<uint16_t *>(a.out_val), (uint32_t)a.capacity, a.splits, clear, clear_words, a.status);
     else
       k_wide_tail<uint32_t><<<dim3(geo.nbuckets), dim3(kWideBlock), 0, s>>>(
-          geo, a.g, p.tb, filter, a.hash, a.hash_log2, a.spp, static_cast<const uint32_t *>(a.input), a.out_idx,
+          geo, a.g, p.tb, filter, a.hash, a.spp, static_cast<const uint32_t *>(a.input), a.out_idx,
           static_cast<uint32_t *>(a.out_val), (uint32_t)a.capacity, a.splits, clear, clear_words, a.status);
     ZEN_LAUNCH_CHECK("k_wide_tail");
   }
@@ -796,3 +942,9 @@ int wide_load_balance(const SlabBalanceArgs &a, size_t state_offset, hipStream_t
 }
 
 }  // namespace zen
+
+#ifdef ZEN_WIDE_TIMING
+extern "C" int zen_wide_debug_read(unsigned long long *host) {
+  return hipMemcpyFromSymbol(host, HIP_SYMBOL(zen::g_wide_dbg), sizeof(unsigned long long) * 256 * 32) == hipSuccess ? 0 : -1;
+}
+#endif
