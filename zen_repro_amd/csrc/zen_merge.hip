@@ -7,8 +7,17 @@
 #include "zen_common.h"
 #include "zen_slab.h"
 #include "zen_slab_feed.h"
+#include "zen_wide.h"
 
 namespace zen {
+
+// zen_wide_merge.hip
+bool wide_merge_fits(int64_t r, int64_t dense_n, int cus, SlabGeom *geo);
+size_t wide_merge_bytes(int64_t r, int64_t dense_n, int cus);
+int wide_merge(const void *idx, int idx64_in, const void *val, int dtype, int64_t r, int64_t dense_n, void *out_idx,
+               int idx64_out, float *out_val, int64_t capacity, int64_t *out_count, unsigned long long *scan,
+               uint32_t *cursor, void *rest, int cus, int32_t *status, hipStream_t s);
+
 namespace {
 
 constexpr int kMrgBlock = 512;
@@ -493,6 +502,8 @@ MergePlan plan_merge(void *workspace, int64_t r, int64_t dense_n) {
     const size_t slabs = plan_slab_merge(nullptr, geo, r).bytes;
     if (slabs > p.bytes) p.bytes = slabs;
   }
+  const size_t wide = wide_merge_bytes(r, dense_n, wide_device_cus());
+  if (wide && kMergeZeroBytes + wide > p.bytes) p.bytes = kMergeZeroBytes + wide;
   return p;
 }
 
@@ -501,8 +512,22 @@ int merge_launch(const void *idx, int idx64_in, const S *val, int64_t r, int64_t
                  int idx64_out, float *out_val, int64_t capacity, int64_t *out_count, int mode, void *workspace,
                  int32_t *status, hipStream_t s) {
   const bool zeroed = (mode & ZEN_MODE_ZEROED) != 0;
-  mode &= ~ZEN_MODE_ZEROED;
+  const bool slabs_only = (mode & ZEN_MODE_SLABS) != 0;
+  mode &= ~(ZEN_MODE_ZEROED | ZEN_MODE_SLABS);
   SlabGeom geo;
+  if (mode == ZEN_MODE_FAST && !slabs_only && wide_merge_fits(r, dense_n, wide_device_cus(), nullptr)) {
+    // the zero region at the head of the workspace: the prefix state first, the cursors behind it
+    Carver cv(workspace);
+    unsigned long long *scan = cv.take<unsigned long long>(scan_words((int64_t)kSlabMaxBuckets));
+    uint32_t *cursor = cv.take<uint32_t>(feed_coarse_cursor_words());
+    if (!zeroed) {
+      launch_fill<unsigned long long>(scan, 0ull, kMergeZeroBytes / sizeof(unsigned long long), s);
+      ZEN_LAUNCH_CHECK("merge: clear prefix state");
+    }
+    return wide_merge(idx, idx64_in, val, sizeof(S) == 2 ? ZEN_BF16 : ZEN_F32, r, dense_n, out_idx, idx64_out, out_val,
+                      capacity, out_count, scan, cursor, static_cast<char *>(workspace) + kMergeZeroBytes,
+                      wide_device_cus(), status, s);
+  }
   if (mode == ZEN_MODE_FAST && slab_merge_fits(r, dense_n, &geo)) {
     if (idx64_in)
       return slab_merge_launch(geo, static_cast<const int64_t *>(idx), val, r, dense_n, out_idx, idx64_out, out_val,
@@ -555,7 +580,8 @@ int merge_launch(const void *idx, int idx64_in, const S *val, int64_t r, int64_t
 
 int merge_check(const void *idx, const void *val, int dtype, int64_t r, int64_t dense_n, int mode, const char **why) {
   if (dtype != ZEN_F32 && dtype != ZEN_BF16) { *why = "bad dtype"; return ZEN_EINVAL; }
-  if ((mode & ~ZEN_MODE_ZEROED) != ZEN_MODE_FAST && (mode & ~ZEN_MODE_ZEROED) != ZEN_MODE_GENERAL) {
+  if ((mode & ~(ZEN_MODE_ZEROED | ZEN_MODE_SLABS)) != ZEN_MODE_FAST &&
+      (mode & ~(ZEN_MODE_ZEROED | ZEN_MODE_SLABS)) != ZEN_MODE_GENERAL) {
     *why = "bad mode";
     return ZEN_EINVAL;
   }
@@ -580,8 +606,10 @@ size_t zen_merge_workspace(int64_t r, int64_t dense_n) {
 size_t zen_merge_zero_bytes(void) { return zen::kMergeZeroBytes; }
 
 int zen_merge_path(int64_t r, int64_t dense_n, int mode) {
-  mode &= ~ZEN_MODE_ZEROED;
+  const bool slabs_only = (mode & ZEN_MODE_SLABS) != 0;
+  mode &= ~(ZEN_MODE_ZEROED | ZEN_MODE_SLABS);
   if (mode != ZEN_MODE_FAST || r <= 0 || dense_n <= 0) return 0;
+  if (!slabs_only && zen::wide_merge_fits(r, dense_n, zen::wide_device_cus(), nullptr)) return 3;
   if (zen::slab_merge_fits(r, dense_n, nullptr)) return 2;
   return zen::bucket_sort_fits(r, (uint32_t)dense_n) ? 1 : 0;
 }
