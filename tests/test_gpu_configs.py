@@ -195,7 +195,7 @@ def test_full_config_encode_properties(zen, full):
     if cfg.k and cfg.n > 1 << 24:  # a top-k of this size goes through the one-pass bucket-slab path
         from zen_repro_amd import _lib
 
-        assert _lib.lib().zen_load_balance_path(n, n, _lib.dtype_code(grad), int(cfg.k * 1.25) + 4096, P, cfg.k, 0) == 2
+        assert _lib.lib().zen_load_balance_path(n, n, _lib.dtype_code(grad), int(cfg.k * 1.25) + 4096, P, cfg.k, 0) in (2, 3)
     if cfg.name in ("c4", "c5"):
         assert by_range > 1.5 and by_range > 2 * by_hash
     # general mode (owner table like the reference) gives the same bytes

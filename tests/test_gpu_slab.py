@@ -13,6 +13,35 @@ from gpu_util import make_grad, to_dev, to_np
 pytestmark = pytest.mark.gpu
 
 SLAB = 2
+WIDE = 3
+FLAGS = 0  # OR-ed into the fast mode of every call and path query of this module (set per run, below)
+
+
+@pytest.fixture(scope="module", autouse=True, params=["wide", "slabs"])
+def fast_path(request):
+    """Every test of this module runs twice: on the wide buckets (where the sizes suit them) and with
+    MODE_SLABS, which keeps the calls on the bucket slabs."""
+    global FLAGS
+    import zen_repro_amd
+    from zen_repro_amd import _lib
+
+    FLAGS = _lib.MODE_SLABS if request.param == "slabs" else 0
+    zen_repro_amd.TensorPartition.fast_flags = FLAGS
+    zen_repro_amd.LoadBalanceAllreduce.fast_flags = FLAGS
+    yield request.param
+    FLAGS = 0
+    zen_repro_amd.TensorPartition.fast_flags = 0
+    zen_repro_amd.LoadBalanceAllreduce.fast_flags = 0
+
+
+def on_fast_path(code):
+    """Whether a zen_*_path answer is the path this run is about: the bucket slabs with MODE_SLABS, else the
+    wide buckets (sizes that take the bucket slabs either way are covered by the other run)."""
+    if FLAGS:
+        return code == SLAB
+    if code == SLAB:
+        pytest.skip("these sizes take the bucket slabs with or without MODE_SLABS: covered by the other run")
+    return code == WIDE
 
 
 @pytest.fixture(scope="module")
@@ -29,7 +58,7 @@ def lb_path(zen, n, P, dtype, capacity, k=0, mode=0, scale=1):
     from zen_repro_amd import _lib
 
     m = int(n * scale // P * P)
-    return _lib.lib().zen_load_balance_path(n, m, 1 if dtype == "bf16" else 0, capacity, P, k, mode)
+    return _lib.lib().zen_load_balance_path(n, m, 1 if dtype == "bf16" else 0, capacity, P, k, mode | FLAGS)
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
@@ -49,7 +78,7 @@ def test_slab_load_balance_bit_exact(zen, oracle, n, P, density, rehash, dtype):
     idx_o, val_o, splits_o, st_o = oracle.load_balance(g, P, 1, rehash)
     assert st_o == 0
     capacity = int(len(idx_o) * 1.1) + 1024
-    assert lb_path(zen, n, P, dtype, capacity) == SLAB
+    assert on_fast_path(lb_path(zen, n, P, dtype, capacity))
     tp = zen.TensorPartition(P, 1, rehash)
     d = to_dev(g)
     for rep in range(2):  # the second call finds the borrowed table zero again
@@ -75,7 +104,7 @@ def test_slab_load_balance_odd_length_unaligned_and_empty(zen, oracle, dtype):
     idx_o, val_o, splits_o, st_o = oracle.load_balance(g, P, 1, 3)
     assert st_o == 0
     capacity = len(idx_o) + 2048
-    assert lb_path(zen, n, P, dtype, capacity) == SLAB
+    assert on_fast_path(lb_path(zen, n, P, dtype, capacity))
     buf = to_dev(np.concatenate([g[:3], g]))
     d = buf[3:]
     assert d.data_ptr() % 16 != 0
@@ -108,7 +137,7 @@ def test_slab_load_balance_declines_and_general_mode_takes_over(zen, oracle):
     idx_o, val_o, splits_o, st_o = oracle.load_balance(g, P, 1, 1)
     assert st_o == 0
     capacity = int(len(idx_o) * 1.1) + 1024
-    assert lb_path(zen, n, P, "bf16", capacity) == SLAB
+    assert on_fast_path(lb_path(zen, n, P, "bf16", capacity))
     tp = zen.TensorPartition(P, 1, 1)
     d = to_dev(g)
     _, _, _, status = tp.load_balance_flat(d, capacity=capacity, mode=_lib.MODE_FAST)
@@ -128,7 +157,7 @@ def test_slab_load_balance_too_many_candidates_declines(zen, oracle):
     n, P = 1 << 23, 8
     g = make_grad(oracle, n, 0.05, "f32", seed=5)
     capacity = 1 << 16  # about a sixth of the nonzeros
-    assert lb_path(zen, n, P, "f32", capacity) == SLAB
+    assert on_fast_path(lb_path(zen, n, P, "f32", capacity))
     tp = zen.TensorPartition(P, 1, 3)
     _, _, _, status = tp.load_balance_flat(to_dev(g), capacity=capacity, mode=_lib.MODE_FAST)
     assert status.item() & (_lib.STAT_RETRY | _lib.STAT_CAPACITY)
@@ -155,7 +184,7 @@ def test_slab_load_balance_fused_topk_fp32(zen, oracle):
     idx_o, val_o, splits_o, st_o = oracle.load_balance(masked, P, 1, 3)
     assert st_o == 0 and 0 not in idx_o
     capacity = int(1.25 * k) + 4096
-    assert lb_path(zen, n, P, "f32", capacity, k=k) == SLAB
+    assert on_fast_path(lb_path(zen, n, P, "f32", capacity, k=k))
     tp = zen.TensorPartition(P, 1, 3)
     d = to_dev(x)
     thr_out = torch.zeros(2, dtype=torch.int32, device="cuda")
@@ -183,7 +212,7 @@ def test_slab_load_balance_threshold_given(zen, oracle):
     d = to_dev(g)
     thr = zen.topk_threshold(d, k)
     capacity = kept + 4096
-    assert lb_path(zen, n, P, "bf16", capacity) == SLAB
+    assert on_fast_path(lb_path(zen, n, P, "bf16", capacity))
     tp = zen.TensorPartition(P, 1, 3)
     oi, ov, splits, status = tp.load_balance_flat(d, thr=thr, capacity=capacity)
     assert status.item() == 0 and np.array_equal(to_np(splits), splits_o)
@@ -199,7 +228,7 @@ def test_two_slots_in_flight_give_the_same_answer(zen, oracle):
     d = to_dev(g)
     k = n // 200
     capacity = int(1.3 * k) + 4096
-    assert lb_path(zen, n, P, "bf16", capacity, k=k) == SLAB
+    assert on_fast_path(lb_path(zen, n, P, "bf16", capacity, k=k))
     tp = zen.TensorPartition(P, 1, 3)
     lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P), None, None)
     mi = to_dev(rng.integers(1, n, 400000).astype(np.int32))
@@ -259,7 +288,7 @@ def test_slab_merge_bit_exact(zen, oracle, n, peers, per_peer, overlap, dtype, i
     rng = np.random.default_rng(n % 1000 + peers)
     ci, cv = payloads(oracle, rng, n, peers, per_peer, overlap, dtype)
     ci = ci.astype(np.int64 if idx64 else np.int32)
-    assert _lib.lib().zen_merge_path(len(ci), n, _lib.MODE_FAST) == SLAB
+    assert on_fast_path(_lib.lib().zen_merge_path(len(ci), n, _lib.MODE_FAST | FLAGS))
     want_i, want_v = oracle.merge_sparse(ci, cv, n)
     lba = zen.LoadBalanceAllreduce(zen.LocalGroup(peers), None, None)
     gi, gv, cnt, st = lba.merge_sparse_flat(to_dev(ci), to_dev(cv), n, idx64=idx64, mode=_lib.MODE_FAST)
@@ -284,7 +313,7 @@ def test_slab_merge_bad_indices_cancellation_and_pile_up(zen, oracle):
     val[1000:1100] = -val[0:100]
     idx[5000] = -7                        # out of range on both sides
     idx[5001] = n
-    assert _lib.lib().zen_merge_path(len(idx), n, _lib.MODE_FAST) == SLAB
+    assert on_fast_path(_lib.lib().zen_merge_path(len(idx), n, _lib.MODE_FAST | FLAGS))
     lba = zen.LoadBalanceAllreduce(zen.LocalGroup(4), None, None)
     gi, gv, cnt, st = lba.merge_sparse_flat(to_dev(idx), to_dev(val), n, idx64=True, mode=_lib.MODE_FAST)
     assert st.item() == _lib.STAT_BAD_INDEX
@@ -328,7 +357,7 @@ def test_table_and_merge_workspace_are_zero_again_after_every_call(zen, oracle):
         else:
             masked, cap = x_np, int(np.count_nonzero(x)) + 1024
         m, _ = tp.table_sizes(n)
-        assert L.zen_load_balance_path(n, m, _lib.dtype_code(grad), cap, P, k, _lib.MODE_FAST) == 2
+        assert on_fast_path(L.zen_load_balance_path(n, m, _lib.dtype_code(grad), cap, P, k, _lib.MODE_FAST | FLAGS))
         idx, val, splits, st = tp.load_balance_flat(grad, None, cap, k=k)
         idx_o, val_o, splits_o, st_o = oracle.load_balance(masked, P, 1, 3)
         assert int(st.item()) == 0 and st_o == 0
@@ -344,7 +373,7 @@ def test_table_and_merge_workspace_are_zero_again_after_every_call(zen, oracle):
         idx = rng.integers(1, dense_n, r).astype(np.int32)
         idx[rng.integers(0, r, r // 3)] = idx[rng.integers(0, r, r // 3)]  # duplicates
         val = (rng.standard_normal(r) * 1e-3).astype(np.float32)
-        assert L.zen_merge_path(r, dense_n, _lib.MODE_FAST) == 2
+        assert on_fast_path(L.zen_merge_path(r, dense_n, _lib.MODE_FAST | FLAGS))
         m_idx, m_val, count, st = lba.merge_sparse_flat(to_dev(idx), to_dev(val), dense_n)
         assert int(st.item()) == 0
         mi_o, mv_o = oracle.merge_sparse(idx, val, dense_n)
@@ -369,7 +398,7 @@ def test_load_balance_without_a_capacity_takes_the_slab_path(zen, oracle):
     cap = tp._honest_capacity(grad, None, 0)
     m, _ = tp.table_sizes(n)
     assert cap < n // 100
-    assert L.zen_load_balance_path(n, m, _lib.BF16, cap, P, 0, _lib.MODE_FAST) == 2
+    assert on_fast_path(L.zen_load_balance_path(n, m, _lib.BF16, cap, P, 0, _lib.MODE_FAST | FLAGS))
     assert L.zen_load_balance_workspace(n, m, _lib.BF16, cap, P) < 1 << 28
     indices, values, splits = tp.load_balance(grad)
     idx_o, val_o, splits_o, st_o = oracle.load_balance(g_np, P, 1, 3)
@@ -406,7 +435,7 @@ def test_sample_taken_ahead_gives_the_same_result(zen, oracle):
         wants.append(oracle.load_balance(masked, P, 1, 3))
     torch.cuda.synchronize()
     m, _ = tp.table_sizes(n)
-    assert _lib.lib().zen_load_balance_path(n, m, _lib.BF16, grads[0][2], P, grads[0][1], _lib.MODE_FAST) == 2
+    assert on_fast_path(_lib.lib().zen_load_balance_path(n, m, _lib.BF16, grads[0][2], P, grads[0][1], _lib.MODE_FAST | FLAGS))
 
     def check(out, want):
         idx, val, splits, st = out
@@ -461,8 +490,8 @@ def test_step_replayed_from_a_captured_graph(zen, oracle):
     tp = zen.TensorPartition(P, 1, 3)
     lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P), None, None)
     m, _ = tp.table_sizes(n)
-    assert _lib.lib().zen_load_balance_path(n, m, _lib.BF16, cap, P, k, _lib.MODE_FAST) == 2
-    assert _lib.lib().zen_merge_path(flat_i.size, n, _lib.MODE_FAST) == 2
+    assert on_fast_path(_lib.lib().zen_load_balance_path(n, m, _lib.BF16, cap, P, k, _lib.MODE_FAST | FLAGS))
+    assert on_fast_path(_lib.lib().zen_merge_path(flat_i.size, n, _lib.MODE_FAST | FLAGS))
 
     def check(enc, mrg):
         idx, val, splits, st = enc
@@ -522,7 +551,7 @@ def test_threshold_of_an_earlier_call_replaces_the_sample(zen, oracle, dtype):
     tp = zen.TensorPartition(P, 1, 3)
     m, _ = tp.table_sizes(n)
     code = _lib.BF16 if dtype == "bf16" else _lib.F32
-    assert _lib.lib().zen_load_balance_path(n, m, code, cap, P, k, _lib.MODE_FAST) == 2
+    assert on_fast_path(_lib.lib().zen_load_balance_path(n, m, code, cap, P, k, _lib.MODE_FAST | FLAGS))
 
     def bits(x):
         return oracle.f32_to_bf16_bits(x) if dtype == "bf16" else x

@@ -111,7 +111,7 @@ class LoadBalanceAllreduce:
             if not int(status.item()):  # the reference's scatter_add_ raises on a bad index, also a sync
                 return dense
         ws = _lib.scratch.get(dev, "decode", L.zen_decode_dense_workspace(r, alltoall_dense_size))
-        for mode in (_lib.MODE_FAST, _lib.MODE_GENERAL):
+        for mode in self._fast_then_general():
             status = _lib.status_word(dev)
             rc = L.zen_decode_dense(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(values),
                                     _lib.dtype_code(values), r, _lib.ptr(dense), alltoall_dense_size, mode,
@@ -123,6 +123,15 @@ class LoadBalanceAllreduce:
         if bits:
             raise RuntimeError("decode_sparse_tensors: " + _lib.describe_status(bits))
         return dense
+
+    # OR-ed into the mode of every fast-mode call (_lib.MODE_SLABS keeps the calls off the wide buckets)
+    fast_flags = 0
+
+    def _fast_then_general(self):
+        """The modes a call that may be declined (STAT_RETRY) goes through: the fast mode, the fast mode on the
+        bucket slabs alone, the general mode."""
+        fast = _lib.MODE_FAST | self.fast_flags
+        return [fast] + ([_lib.MODE_FAST | _lib.MODE_SLABS] if not fast & _lib.MODE_SLABS else []) + [_lib.MODE_GENERAL]
 
     def encode_sparse_tensor(self, tensor):
         """(ascending int64 indices of the nonzeros, their values), comm.py:47-50."""
@@ -149,6 +158,8 @@ class LoadBalanceAllreduce:
         r = indices.numel()
         if capacity is None:
             capacity = r
+        if (mode & 0xff) == _lib.MODE_FAST:
+            mode |= self.fast_flags
         out_idx = torch.empty(capacity, dtype=torch.int64 if idx64 else torch.int32, device=dev)
         out_val = torch.empty(capacity, dtype=torch.float32, device=dev)
         count = _lib.zeros.take(dev, 1, torch.int64)
@@ -174,7 +185,7 @@ class LoadBalanceAllreduce:
 
     def merge_sparse(self, indices_tensors, values_tensors, dense_size):
         """Synchronising form of merge_sparse_flat: (int64 indices, fp32 sums)."""
-        for mode in (_lib.MODE_FAST, _lib.MODE_GENERAL):
+        for mode in self._fast_then_general():
             idx, val, count, status = self.merge_sparse_flat(indices_tensors, values_tensors, dense_size,
                                                              idx64=True, mode=mode)
             host = torch.cat([count, status.to(torch.int64)]).tolist()

@@ -35,13 +35,28 @@ constexpr int kWsBlock = 512;
 constexpr int kWsItems = 8;
 constexpr int kWsBatch = kWsBlock * kWsItems;  // list entries per workgroup
 
+// A record in a bucket's slab is one 64-bit word: the index's offset from the bucket's first index (below
+// 2^23) in bits 0-22, the arrival number (below 2^25) in bits 23-47 and, for bf16, the value in bits 48-63;
+// fp32 values travel in a word plane of their own.  One store per record, and a run of sixteen fills a line.
+constexpr uint32_t kWmOffBits = 23, kWmArrBits = 25;
 struct WideSlabs {
   uint32_t *cursor;    // [nbuckets * kWideSplit * kWmPad], zero before the scatter; the bucket's workgroup puts them back
-  uint32_t *idx;       // [nbuckets * kWideSplit * part_cap]
-  uint32_t *arr;       // arrival numbers
-  void *val;           // values in their own type
+  uint2 *rec;          // [nbuckets * kWideSplit * part_cap]
+  uint32_t *val32;     // fp32 values (unused for bf16)
   uint32_t part_cap;
 };
+__device__ inline uint2 wm_pack(uint32_t off, uint32_t arr, uint32_t val16) {
+  return make_uint2(off | (arr << kWmOffBits), (arr >> (32 - kWmOffBits)) | (val16 << 16));
+}
+__device__ inline uint32_t wm_off(uint2 r) { return r.x & ((1u << kWmOffBits) - 1u); }
+__device__ inline uint32_t wm_arr(uint2 r) { return (r.x >> kWmOffBits) | ((r.y & 0xffffu) << (32 - kWmOffBits)); }
+
+#ifdef ZEN_WIDE_TIMING
+__device__ unsigned long long g_wm_dbg[1024 * 16];
+#define WM_MARK(k) do { if (threadIdx.x == 0 && blockIdx.x < 1024) g_wm_dbg[blockIdx.x * 16 + (k)] = wall_clock64(); } while (0)
+#else
+#define WM_MARK(k) do { } while (0)
+#endif
 
 template <typename I, typename S>
 __global__ __launch_bounds__(kWsBlock) void k_wide_scatter(SlabGeom geo, const I *__restrict__ idx,
@@ -50,13 +65,21 @@ __global__ __launch_bounds__(kWsBlock) void k_wide_scatter(SlabGeom geo, const I
   __shared__ uint32_t s_cnt[kWideMaxBuckets], s_pref[kWideMaxBuckets + 1], s_gbase[kWideMaxBuckets];
   __shared__ uint32_t s_scan[kWsBlock / 64 + 1];
   __shared__ uint32_t s_idx[kWsBatch];
+  // 32 KB of LDS in all: five workgroups share a compute unit and the whole grid is resident in one round (the
+  // values do not pass through LDS for that reason: they are fetched again when the record is written)
   __shared__ uint16_t s_from[kWsBatch];  // place inside the batch (the arrival number, and where the value is)
-  __shared__ uint16_t s_dst[kWsBatch];
+  __shared__ uint8_t s_dst[kWsBatch];
+  static_assert(kWideMaxBuckets <= 256, "a destination in a byte");
+  __shared__ uint32_t s_lo[kWideMaxBuckets];  // the buckets' first indices (a 64-bit division each)
   const uint32_t batch = blockIdx.x * (uint32_t)kWsBatch;
   const uint32_t part = blockIdx.x % kWideSplit;
   const uint32_t nb = geo.nbuckets;
-  if (threadIdx.x < (uint32_t)kWideMaxBuckets) s_cnt[threadIdx.x] = 0;
+  if (threadIdx.x < (uint32_t)kWideMaxBuckets) {
+    s_cnt[threadIdx.x] = 0;
+    s_lo[threadIdx.x] = threadIdx.x < nb ? geo.first_key(threadIdx.x) : 0u;
+  }
   __syncthreads();
+  WM_MARK(0);
   uint32_t k[kWsItems], d[kWsItems], rank[kWsItems];
 #pragma unroll
   for (int i = 0; i < kWsItems; ++i) {
@@ -73,10 +96,12 @@ __global__ __launch_bounds__(kWsBlock) void k_wide_scatter(SlabGeom geo, const I
       }
     }
   }
+  WM_MARK(1);
 #pragma unroll
   for (int i = 0; i < kWsItems; ++i)
     if (d[i] != kInvalid) rank[i] = atomicAdd(&s_cnt[d[i]], 1u);
   __syncthreads();
+  WM_MARK(2);
   {
     const uint32_t c = threadIdx.x < nb ? s_cnt[threadIdx.x] : 0u;
     uint32_t total;
@@ -88,31 +113,36 @@ __global__ __launch_bounds__(kWsBlock) void k_wide_scatter(SlabGeom geo, const I
     if (threadIdx.x == 0) s_pref[nb] = total;
   }
   __syncthreads();
+  WM_MARK(3);
 #pragma unroll
   for (int i = 0; i < kWsItems; ++i) {
     if (d[i] != kInvalid) {
       const uint32_t p = s_pref[d[i]] + rank[i];
       s_idx[p] = k[i];
       s_from[p] = (uint16_t)(threadIdx.x + i * kWsBlock);
-      s_dst[p] = (uint16_t)d[i];
+      s_dst[p] = (uint8_t)d[i];
     }
   }
   __syncthreads();
+  WM_MARK(4);
   const uint32_t total = s_pref[nb];
-  S *out_val = static_cast<S *>(out.val);
+#pragma unroll 2
   for (uint32_t p = threadIdx.x; p < total; p += kWsBlock) {
     const uint32_t g = s_dst[p];
     const uint32_t at = s_gbase[g] + (p - s_pref[g]);
     if (at < out.part_cap) {
       const size_t o = (size_t)(g * kWideSplit + part) * out.part_cap + at;
       const uint32_t e = batch + s_from[p];
-      out.idx[o] = s_idx[p];
-      out.arr[o] = e;
-      out_val[o] = val[e];  // a workgroup's 4096 arrival numbers are consecutive: these loads hit what it has just read
+      const S v = val[e];  // a workgroup's 4096 arrival numbers are consecutive: these loads hit what it has just read
+      out.rec[o] = wm_pack(s_idx[p] - s_lo[g], e, sizeof(S) == 2 ? (uint32_t)v : 0u);
+      if (sizeof(S) == 4) out.val32[o] = (uint32_t)v;
     } else {
       atomicOr(status, ZEN_STAT_RETRY);  // a slab is full: another path answers
     }
   }
+  WM_MARK(5);
+  wait_global_acks();
+  WM_MARK(6);
 }
 
 // ------------------------------------------------------------ a bucket
@@ -165,9 +195,8 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_merge(SlabGeom geo, WideSla
     for (int q = 0; q < kWideSplit; ++q) pcount[q] = 0;
     longest = 0;
   }
-  const uint32_t *idx_plane = in.idx + (size_t)b * kWideSplit * in.part_cap;
-  const uint32_t *arr_plane = in.arr + (size_t)b * kWideSplit * in.part_cap;
-  const S *val_plane = static_cast<const S *>(in.val) + (size_t)b * kWideSplit * in.part_cap;
+  const uint2 *rec_plane = in.rec + (size_t)b * kWideSplit * in.part_cap;
+  const uint32_t *val_plane = in.val32 + (size_t)b * kWideSplit * in.part_cap;
   const int shift = geo.sub_shift;
   const uint32_t low_mask = (1u << shift) - 1u;
 
@@ -183,8 +212,8 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_merge(SlabGeom geo, WideSla
       for (int q = 0; q < kWideSplit; ++q) {
         const uint32_t e = tid + (uint32_t)r * kWideBlock;
         const size_t at = (size_t)q * in.part_cap + (e < pcount[q] ? e : 0u);
-        const uint32_t off = idx_plane[at] - lo;
-        const uint32_t arr = arr_plane[at];
+        const uint2 rec = rec_plane[at];
+        const uint32_t off = wm_off(rec), arr = wm_arr(rec);
         if (e < pcount[q]) {
           w[r * kWideSplit + q] = ((off & low_mask) << tie_bits) | arr;
           ps[r * kWideSplit + q] = off >> shift;  // the narrow range, for now
@@ -322,18 +351,19 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_merge(SlabGeom geo, WideSla
 #pragma unroll
   for (int r = 0; r < kWmRounds; ++r) {
     if ((uint32_t)r * kWideBlock < longest) {
-      S v[kWideSplit];
+      uint32_t v[kWideSplit];
 #pragma unroll
       for (int q = 0; q < kWideSplit; ++q) {
         const uint32_t e = tid + (uint32_t)r * kWideBlock;
-        v[q] = val_plane[(size_t)q * in.part_cap + (rk[r * kWideSplit + q] != kInvalid ? e : 0u)];
+        const size_t at = (size_t)q * in.part_cap + (rk[r * kWideSplit + q] != kInvalid ? e : 0u);
+        v[q] = sizeof(S) == 2 ? rec_plane[at].y >> 16 : val_plane[at];
       }
 #pragma unroll
       for (int q = 0; q < kWideSplit; ++q) {
         const int i = r * kWideSplit + q;
         if (rk[i] != kInvalid) {
           sh.key[rk[i]] = ((ps[i] >> 14) << shift) | (w[i] >> tie_bits);
-          sh.val[rk[i]] = KeyOf<S>::to_f32(v[q]);
+          sh.val[rk[i]] = KeyOf<S>::to_f32((S)v[q]);
         }
       }
     }
@@ -448,6 +478,8 @@ bool wide_merge_fits(int64_t r, int64_t dense_n, int cus, SlabGeom *geo) {
   SlabGeom g;
   if (r < (1 << 15) || r > 0x7ffffffell || cus <= 0 || !wide_geometry(dense_n, 1, r, cus, &g)) return false;
   if (g.sub_shift + ceil_log2_u64((uint64_t)r) > 32) return false;  // (index inside a narrow range, arrival number) must fit a word
+  // a slab record carries the index's offset inside its bucket and the arrival number in fixed fields
+  if ((uint64_t)g.sub_shift + 14 > kWmOffBits || (uint64_t)r >= (1ull << kWmArrBits)) return false;
   if (geo) *geo = g;
   return true;
 }
@@ -459,7 +491,7 @@ size_t wide_merge_bytes(int64_t r, int64_t dense_n, int cus) {
   SlabGeom geo;
   if (!wide_merge_fits(r, dense_n, cus, &geo)) return 0;
   const size_t entries = (size_t)geo.nbuckets * kWideSplit * wide_merge_part_cap(geo, r);
-  return 3 * align_up(entries * sizeof(uint32_t), 256);
+  return align_up(entries * sizeof(uint2), 256) + align_up(entries * sizeof(uint32_t), 256);
 }
 
 // scan: zeroed prefix state for 256 buckets (descriptors, ticket, finished count); cursor: kCoarseCursorWords
@@ -473,9 +505,8 @@ static int wide_merge_typed(const SlabGeom &geo, const I_in *idx, const S *val, 
   const size_t entries = (size_t)geo.nbuckets * kWideSplit * slabs.part_cap;
   Carver cv(rest);
   slabs.cursor = cursor;
-  slabs.idx = cv.take<uint32_t>(entries);
-  slabs.arr = cv.take<uint32_t>(entries);
-  slabs.val = cv.take<uint32_t>(entries);
+  slabs.rec = cv.take<uint2>(entries);
+  slabs.val32 = cv.take<uint32_t>(entries);
   {
     ProfScope prof(kProfWideScatter, s);
     k_wide_scatter<I_in, S><<<dim3((unsigned)ceil_div(r, kWsBatch)), dim3(kWsBlock), 0, s>>>(
@@ -517,3 +548,9 @@ int wide_merge(const void *idx, int idx64_in, const void *val, int dtype, int64_
 }
 
 }  // namespace zen
+
+#ifdef ZEN_WIDE_TIMING
+extern "C" int zen_wm_debug_read(unsigned long long *host) {
+  return hipMemcpyFromSymbol(host, HIP_SYMBOL(zen::g_wm_dbg), sizeof(unsigned long long) * 1024 * 16) == hipSuccess ? 0 : -1;
+}
+#endif

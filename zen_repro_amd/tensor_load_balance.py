@@ -13,6 +13,9 @@ class TensorPartition:
     """Same constructor and methods as the reference class
     (tensor_load_balance.py:5-51)."""
 
+    # OR-ed into the mode of every fast-mode call (_lib.MODE_SLABS keeps the calls off the wide buckets)
+    fast_flags = 0
+
     def __init__(self, partitions, memory_scale, rehash):
         self.partitions = partitions
         self.memory_scale = memory_scale
@@ -125,7 +128,8 @@ class TensorPartition:
         m, _ = self.table_sizes(n)
         dev = flat.device
         L = _lib.lib()
-        if k <= 0 or L.zen_load_balance_path(n, m, code, capacity, self.partitions, k, _lib.MODE_FAST) not in (2, 3):
+        if k <= 0 or L.zen_load_balance_path(n, m, code, capacity, self.partitions, k,
+                                             _lib.MODE_FAST | self.fast_flags) not in (2, 3):
             return
         state = self._ahead_state(dev, slot, create=True)
         if len(state["pending"]) >= 2:
@@ -172,6 +176,8 @@ class TensorPartition:
             # no synchronisation here, so no count: the largest the library takes.  A caller that knows a bound
             # should pass it (load_balance works one out): this default sizes everything for the whole tensor.
             capacity = min(n, (1 << 29) - 1)
+        if (mode & 0xff) == _lib.MODE_FAST:
+            mode |= self.fast_flags
         dev = flat.device
         L = _lib.lib()
         out_idx = torch.empty(capacity, dtype=torch.int32, device=dev)
@@ -186,7 +192,7 @@ class TensorPartition:
         ahead = None
         if state is not None and state["pending"]:
             ahead = state["pending"].pop(0)
-            if (ahead[:5] != (flat.data_ptr(), n, int(k), capacity, ws.data_ptr()) or mode != _lib.MODE_FAST
+            if (ahead[:5] != (flat.data_ptr(), n, int(k), capacity, ws.data_ptr()) or (mode & 0xff) != _lib.MODE_FAST
                     or thr is not None or near is not None):
                 # not for this call: its histogram is cleared again (with the arguments it was taken with) and
                 # the call samples for itself
@@ -234,7 +240,9 @@ class TensorPartition:
             grow = capacity is None
         if capacity is None:
             capacity = min(n, self._honest_capacity(flat, thr, k))
-        modes = [_lib.MODE_FAST, _lib.MODE_GENERAL] if mode is None else [mode]
+        fast = _lib.MODE_FAST | self.fast_flags
+        modes = ([fast] + ([_lib.MODE_FAST | _lib.MODE_SLABS] if not fast & _lib.MODE_SLABS else []) +
+                 [_lib.MODE_GENERAL]) if mode is None else [mode]
         while modes:
             out_idx, out_val, splits, status = self.load_balance_flat(tensor, thr, capacity, k, modes[0])
             host = torch.cat([splits, status.to(torch.int64)]).tolist()
