@@ -45,6 +45,9 @@ def parse():
                     help="measure the bitmap index codec of the second exchange instead (prints its own line)")
     ap.add_argument("--phase2-decode", action="store_true",
                     help="measure the decode of the second exchange instead (prints its own line)")
+    ap.add_argument("--separate-calls", action="store_true",
+                    help="one library call for the encode and one for the merge instead of one per bucket for both "
+                         "(zen_encode_merge); the kernels and streams are the same")
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
     ap.add_argument("--no-prepare", action="store_true",
                     help="do not take the next step's sample ahead on a stream of its own")
@@ -410,6 +413,7 @@ def main():
     # ("slots"), each step's merge behind its encode on the step's own stream, so that the long, memory-bound
     # select of one step runs next to the short, latency-bound kernels of the other (a kernel's events then
     # also time its wait for room on the chip).  All streams have default priority.
+    fused = not (args.separate_calls or args.graph)
     depth = 1 if (args.one_stream or args.graph) else max(1, args.depth)
     main = torch.cuda.current_stream(dev)
     enc_streams = [main] + [torch.cuda.Stream(device=dev) for _ in range(depth - 1)]
@@ -445,15 +449,28 @@ def main():
                 fi, fv = flat_sets[j][i % len(flat_sets[j])]
                 mrg.append(lba.merge_sparse_flat(fi, fv, b.n, capacity=fi.numel(), slot=slot))
 
+        def both():
+            for j, b in enumerate(buckets):
+                g = grad_sets[j][i % len(grad_sets[j])]
+                fi, fv = flat_sets[j][i % len(flat_sets[j])]
+                e_, m_ = lba.encode_merge_flat(tp, g, caps[j], b.k, fi, fv, b.n, slot=slot,
+                                               thr_out=warm_thr[j] if warm else None, near=near_keys[j],
+                                               merge_stream=ms_)
+                enc.append(e_)
+                mrg.append(m_)
+
         with torch.cuda.stream(es):
-            encode()
-            if ms_ is None:
-                merge()  # behind the encode, on its stream
+            if fused:
+                both()
+            else:
+                encode()
+                if ms_ is None:
+                    merge()  # behind the encode, on its stream
         if prep_stream is not None and more and depth == 1:
             with torch.cuda.stream(prep_stream):
                 for j, b in enumerate(buckets):
                     tp.prepare(grad_sets[j][(i + 1) % len(grad_sets[j])], b.k, caps[j], slot=slot)
-        if ms_ is not None:
+        if ms_ is not None and not fused:
             with torch.cuda.stream(ms_):
                 merge()
         return list(zip(enc, mrg))
@@ -604,6 +621,12 @@ def main():
             second.wait_stream(main)
             for i in range(count):
                 with torch.cuda.stream(second if i % 2 else main):
+                    if fused:
+                        for j, b in enumerate(buckets):
+                            fi, fv = flat_sets[j][i % len(flat_sets[j])]
+                            lba.encode_merge_flat(tp, grad_sets[j][i % len(grad_sets[j])], caps[j], b.k, fi, fv, b.n,
+                                                  slot=i % 2, near=near_keys[j])
+                        continue
                     for j, b in enumerate(buckets):
                         tp.load_balance_flat(grad_sets[j][i % len(grad_sets[j])], None, caps[j], k=b.k, slot=i % 2,
                                              near=near_keys[j])
@@ -662,7 +685,8 @@ def main():
                    "buckets": [{"name": b.name, "elements": b.n, "k": b.k, "selected": nnz[j],
                                 "received": flats[j][0].numel(), "merged": merged[j]} for j, b in enumerate(buckets)],
                    "k": sum(b.k for b in buckets), "selected": sum(nnz), "received": received, "merged": sum(merged),
-                   "peers": cfg.peers, "overlap": cfg.overlap, "shrink": args.shrink, "steps_in_flight": depth, "merge_runs": "behind its step's encode" if (merge_follows or args.one_stream) else "beside its step's encode",
+                   "peers": cfg.peers, "overlap": cfg.overlap, "shrink": args.shrink, "steps_in_flight": depth, "calls_per_bucket": 1 if fused else 2,
+                   "merge_runs": "behind its step's encode" if (merge_follows or args.one_stream) else "beside its step's encode",
                    "replayed_from_graph": bool(args.graph),
                    "topk_sample": "none: the warm-up's threshold key is handed over" if args.near_threshold else "taken in every step",
                    "input_copies": {"gradient": len(grad_sets[0]), "payloads": len(flat_sets[0])}},

@@ -56,7 +56,8 @@ extern "C" {
    them).  A workspace allocated zeroed and used for zen_merge only therefore needs no clearing at all. */
 #define ZEN_MODE_ZEROED 0x100
 /* OR-ed into the `mode` of zen_load_balance: zen_load_balance_prepare has run for this call (see there);
-   ZEN_MODE_SECOND names the second of its two sets of sampling memory. */
+   ZEN_MODE_SECOND names the second of the two sets of sampling memory (without ZEN_MODE_PREPARED: the call takes
+   its own sample in that set, e.g. because the first holds the sample of another call that is still to come). */
 #define ZEN_MODE_PREPARED 0x200
 #define ZEN_MODE_SECOND 0x400
 #define ZEN_MODE_DISCARD 0x800 /* zen_load_balance_prepare: drop a sample that no call will pick up */
@@ -292,6 +293,52 @@ int zen_merge(const void *idx, int idx64_in, const void *val, int dtype,
               void *out_idx, int idx64_out, float *out_val, int64_t capacity,
               int64_t *out_count, int mode, void *workspace, size_t workspace_bytes,
               int32_t *status, void *stream);
+
+/*
+ * One step of the path in one call: zen_load_balance of the rank's own gradient and zen_merge of the entries it
+ * received, with the arguments of those two calls (the received values have the gradient's type `dtype`).
+ * Replaces the two halves of LoadBalanceAllreduce.zen_sparse_comm around the first exchange (comm.py:118-127:
+ * load_balance before it, decode_sparse_tensors + encode_sparse_tensor after it) for a caller that holds the
+ * received entries of the previous bucket while it encodes the next one.  The encode is enqueued on `stream`,
+ * the merge on `merge_stream` (NULL: on `stream`, behind the encode); results and status words are those of
+ * the two calls.  No counterpart in the reference: it exists so that a hook crosses the language boundary once
+ * per bucket.
+ */
+typedef struct zen_encode_merge_args {
+  /* zen_load_balance */
+  const void *input;
+  int dtype;
+  int64_t n, m;
+  int partitions, rehash;
+  const uint32_t *thr;
+  int64_t k;
+  uint32_t *thr_out;
+  int32_t *out_idx;
+  void *out_val;
+  int64_t capacity;
+  int64_t *splits;
+  int32_t *table;
+  int mode;
+  void *workspace;
+  size_t workspace_bytes;
+  int32_t *status;
+  /* zen_merge */
+  const void *recv_idx;
+  int recv_idx64;
+  const void *recv_val;
+  int64_t r, dense_n;
+  void *merged_idx;
+  int merged_idx64;
+  float *merged_val;
+  int64_t merged_capacity;
+  int64_t *merged_count;
+  int merge_mode;
+  void *merge_workspace;
+  size_t merge_workspace_bytes;
+  int32_t *merge_status;
+  void *stream, *merge_stream;
+} zen_encode_merge_args;
+int zen_encode_merge(const zen_encode_merge_args *args);
 
 /*
  * dense[0..dense_n) = 0, then dense[idx[j]] += val[j] with fp32 accumulation

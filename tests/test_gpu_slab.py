@@ -457,12 +457,27 @@ def test_sample_taken_ahead_gives_the_same_result(zen, oracle):
                 tp.prepare(*grads[(i + 1) % 3])
     for i, out in enumerate(outs):
         check(out, wants[i % 3])
-    # a sample for a call that does not come: the next call (other tensor) drops it and samples for itself
+    # a sample whose call comes later: the calls in between (other buckets on the same slot) leave it alone and
+    # sample for themselves, in the other set of sampling memory
     with torch.cuda.stream(side):
         tp.prepare(*grads[1])
     g, k, cap = grads[2]
     check(tp.load_balance_flat(g, None, cap, k=k), wants[2])
     check(tp.load_balance_flat(grads[0][0], None, grads[0][2], k=grads[0][1]), wants[0])
+    state = tp._ahead_state(g.device, 0)
+    assert len(state["pending"]) == 1
+    check(tp.load_balance_flat(grads[1][0], None, grads[1][2], k=grads[1][1]), wants[1])
+    assert not state["pending"]
+    # both sets hold samples of calls still to come and a third bucket turns up: the older sample gives way
+    with torch.cuda.stream(side):
+        tp.prepare(*grads[1])
+        tp.prepare(*grads[2])
+    assert len(state["pending"]) == 2
+    check(tp.load_balance_flat(grads[0][0], None, grads[0][2], k=grads[0][1]), wants[0])
+    assert len(state["pending"]) == 1
+    check(tp.load_balance_flat(grads[1][0], None, grads[1][2], k=grads[1][1]), wants[1])  # samples again
+    check(tp.load_balance_flat(g, None, cap, k=k), wants[2])                                # picks its sample up
+    assert not state["pending"]
     torch.cuda.synchronize()
     assert int(tp._table(g.device, m).count_nonzero()) == 0
 
@@ -589,3 +604,44 @@ def test_threshold_of_an_earlier_call_replaces_the_sample(zen, oracle, dtype):
     assert exact >= 3
     torch.cuda.synchronize()
     assert int(tp._table(dev, m).count_nonzero()) == 0
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_encode_and_merge_in_one_call(zen, oracle, dtype):
+    """encode_merge_flat (zen_encode_merge) against the two calls it stands for, bit for bit: a top-k bucket and
+    the entries received for it, twice in a row (the second call finds every counter where the first left it),
+    then with a sample taken ahead, and with the merge on a stream of its own."""
+    from zen_repro_amd import _lib
+
+    n, P, k = 1 << 25, 16, (1 << 25) // 100
+    g = make_grad(oracle, n, 1.0, dtype, seed=31)
+    rng = np.random.default_rng(5)
+    ci, cv = payloads(oracle, rng, n, P, 20000, 0.25, dtype)
+    ci = ci.astype(np.int32)
+    cap = int(k * 1.25) + 4096
+    d, di, dv = to_dev(g), to_dev(ci), to_dev(cv)
+    tp = zen.TensorPartition(P, 1, 3)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P), None, None)
+    e0 = tp.load_balance_flat(d, None, cap, k=k, slot=1)
+    m0 = lba.merge_sparse_flat(di, dv, n, slot=1)
+    torch.cuda.synchronize()
+    assert e0[3].item() == 0 and m0[3].item() == 0
+    total, cnt = int(e0[2].sum()), int(m0[2])
+    side = torch.cuda.Stream()
+
+    def same(e, m):
+        torch.cuda.synchronize()
+        assert e[3].item() == 0 and m[3].item() == 0
+        assert torch.equal(e[2], e0[2]) and int(m[2]) == cnt
+        assert torch.equal(e[0][:total], e0[0][:total]) and torch.equal(to_dev(to_np(e[1][:total])), to_dev(to_np(e0[1][:total])))
+        assert torch.equal(m[0][:cnt], m0[0][:cnt]) and torch.equal(m[1][:cnt].view(torch.int32), m0[1][:cnt].view(torch.int32))
+
+    for rep in range(2):
+        same(*lba.encode_merge_flat(tp, d, cap, k, di, dv, n))
+    tp.prepare(d, k, cap)
+    same(*lba.encode_merge_flat(tp, d, cap, k, di, dv, n))
+    side.wait_stream(torch.cuda.current_stream())
+    same(*lba.encode_merge_flat(tp, d, cap, k, di, dv, n, merge_stream=side))
+    torch.cuda.current_stream().wait_stream(side)
+    m, _ = oracle.table_sizes(n, P, 1)
+    assert not tp._table(d.device, m).any()

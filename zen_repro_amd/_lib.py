@@ -24,6 +24,22 @@ LIB_PATH = os.environ.get("ZEN_HIP_LIB") or os.path.join(_HERE, "csrc", "libzen_
 _lib = None
 
 
+class EncodeMergeArgs(ctypes.Structure):
+    """zen_encode_merge_args of include/zen_hip.h."""
+    _vp, _i32, _i64, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
+    _fields_ = [
+        ("input", _vp), ("dtype", _i32), ("n", _i64), ("m", _i64), ("partitions", _i32), ("rehash", _i32),
+        ("thr", _vp), ("k", _i64), ("thr_out", _vp), ("out_idx", _vp), ("out_val", _vp), ("capacity", _i64),
+        ("splits", _vp), ("table", _vp), ("mode", _i32), ("workspace", _vp), ("workspace_bytes", _sz),
+        ("status", _vp),
+        ("recv_idx", _vp), ("recv_idx64", _i32), ("recv_val", _vp), ("r", _i64), ("dense_n", _i64),
+        ("merged_idx", _vp), ("merged_idx64", _i32), ("merged_val", _vp), ("merged_capacity", _i64),
+        ("merged_count", _vp), ("merge_mode", _i32), ("merge_workspace", _vp), ("merge_workspace_bytes", _sz),
+        ("merge_status", _vp),
+        ("stream", _vp), ("merge_stream", _vp),
+    ]
+
+
 def build():
     """Compile libzen_hip.so for gfx950 with hipcc (cross-compiles without a GPU)."""
     import subprocess
@@ -70,6 +86,7 @@ def lib():
         "zen_merge_path": (i32, [i64, i64, i32]),
         "zen_merge_zero_bytes": (sz, []),
         "zen_merge": (i32, [vp, i32, vp, i32, i64, i64, vp, i32, vp, i64, vp, i32, vp, sz, vp, vp]),
+        "zen_encode_merge": (i32, [ctypes.POINTER(EncodeMergeArgs)]),
         "zen_decode_dense_workspace": (sz, [i64, i64]),
         "zen_decode_dense": (i32, [vp, i32, vp, i32, i64, vp, i64, i32, vp, sz, vp, vp]),
         "zen_decode_dense_sorted_workspace": (sz, [i64, i32]),

@@ -176,6 +176,60 @@ class LoadBalanceAllreduce:
         _lib.check(rc, "merge_sparse")
         return out_idx, out_val, count, status
 
+    def encode_merge_flat(self, partition, tensor, capacity, k, recv_indices, recv_values, dense_size, slot=0,
+                          thr_out=None, near=None, merge_stream=None):
+        """One bucket's step in one call of the library: partition.load_balance_flat(tensor, None, capacity,
+        k=k, slot=slot, thr_out=thr_out, near=near) of the rank's own gradient and merge_sparse_flat(recv_indices,
+        recv_values, dense_size, slot=slot) of the entries it received, whose values have the gradient's type.
+        Returns the two calls' tuples.  Everything is enqueued on the current stream unless `merge_stream` (a
+        torch stream in whose order the received entries are ready) takes the merge.  A sample taken ahead with
+        partition.prepare() is picked up as load_balance_flat would."""
+        from .tensor_load_balance import TensorPartition  # noqa: F401 (the type of `partition`)
+
+        _lib.require_gpu(tensor, "input")
+        flat = tensor.reshape(-1)
+        indices = self.stack_tensors(recv_indices)
+        values = self.stack_tensors(recv_values)
+        _lib.require_gpu(indices, "indices")
+        _lib.require_gpu(values, "values")
+        assert values.dtype == flat.dtype, "received values must have the gradient's type"
+        dev = flat.device
+        L = _lib.lib()
+        n, r = flat.numel(), indices.numel()
+        code = _lib.dtype_code(flat)
+        m, _ = partition.table_sizes(n)
+        P = partition.partitions
+        mode = _lib.MODE_FAST | partition.fast_flags
+        out_idx = torch.empty(capacity, dtype=torch.int32, device=dev)
+        out_val = torch.empty(capacity, dtype=flat.dtype, device=dev)
+        m_idx = torch.empty(r, dtype=torch.int32, device=dev)
+        m_val = torch.empty(r, dtype=torch.float32, device=dev)
+        small = _lib.zeros.take(dev, P + 2, torch.int64)  # split sizes, merged count, the two status words
+        splits, count = small[:P], small[P:P + 1]
+        status2 = small[P + 1:P + 2].view(torch.int32)
+        status, m_status = status2[0:1], status2[1:2]
+        ws = _lib.scratch.get(dev, f"load_balance/{slot}", L.zen_load_balance_workspace(n, m, code, capacity, P))
+        mws = _lib.scratch.get(dev, f"merge/{slot}", L.zen_merge_workspace(r, dense_size), zero=True)
+        table = partition._table(dev, m, slot)
+        flags, used = partition._take_ahead(flat, n, int(k), capacity, ws, slot, mode, None, near)
+        thr = None
+        if near is not None and k > 0:
+            thr, flags = near, flags | _lib.MODE_FLOOR
+        a = _lib.EncodeMergeArgs(
+            flat.data_ptr(), code, n, m, P, partition.rehash, thr.data_ptr() if thr is not None else None, int(k),
+            thr_out.data_ptr() if thr_out is not None else None, out_idx.data_ptr(), out_val.data_ptr(), capacity,
+            splits.data_ptr(), table.data_ptr(), mode | flags, ws.data_ptr(), ws.numel(), status.data_ptr(),
+            indices.data_ptr(), int(indices.dtype == torch.int64), values.data_ptr(), r, dense_size,
+            m_idx.data_ptr(), 0, m_val.data_ptr(), r, count.data_ptr(),
+            _lib.MODE_FAST | self.fast_flags | _lib.MODE_ZEROED, mws.data_ptr(), mws.numel(), m_status.data_ptr(),
+            _lib.stream_handle(dev), merge_stream.cuda_stream if merge_stream is not None else None)
+        rc = L.zen_encode_merge(ctypes.byref(a))
+        if rc != _lib.OK:
+            mws[:L.zen_merge_zero_bytes()].zero_()
+        _lib.check(rc, "encode_merge")
+        partition._after_call(dev, slot, int(k), used)
+        return (out_idx, out_val, splits, status), (m_idx, m_val, count, m_status)
+
     def reset_merge_workspace(self, device, slot=0):
         """After a merge_sparse_flat whose status carried STAT_RETRY or
         STAT_INTERNAL: clears the head of the slot's workspace again."""

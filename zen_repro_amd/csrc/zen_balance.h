@@ -142,6 +142,7 @@ struct SlabBalanceArgs {
   int32_t *status;
   const uint32_t *near_key = nullptr;  // optional, k > 0: a key close to the k-th largest (no sample is taken)
   int prepared = 0;           // 1 / 2: the sampled floor of the first / second set is there already (zen_load_balance_prepare)
+  bool second = false;        // the call's sample uses the second set of sampling memory (always so with prepared == 2)
   bool only_prepare = false;  // take the sample for that set and nothing else
   bool discard = false;       // with only_prepare: clear the set's sampling memory instead (a sample nobody picks up)
 };
@@ -157,6 +158,7 @@ bool wide_balance_fits(int64_t m, int partitions, int64_t capacity, int64_t k, i
 size_t wide_balance_bytes(int64_t m, int partitions, int dtype, int64_t capacity, int cus);
 int wide_load_balance(const SlabBalanceArgs &a, size_t state_offset, hipStream_t stream);
 int wide_device_cus();  // compute units of the current device (0: no device)
+
 
 size_t resolve_scratch_bytes(int64_t list_cap, uint64_t key_limit);  // key_limit = P * (m / P + 1) + 1
 int resolve_and_place(const ResolveArgs &a, hipStream_t stream);

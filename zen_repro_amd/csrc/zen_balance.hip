@@ -426,6 +426,7 @@ int zen_load_balance_prepare(const void *input, int dtype, int64_t n, int64_t m,
   sa.hash_log2 = slab_hash_log2(m);
   sa.workspace = workspace;
   sa.prepared = second ? 2 : 1;
+  sa.second = second != 0;
   sa.only_prepare = true;
   sa.discard = (mode & ZEN_MODE_DISCARD) != 0;
   return slab_prepare(sa, static_cast<hipStream_t>(stream));
@@ -437,6 +438,7 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
                      size_t workspace_bytes, int32_t *status, void *stream) {
   using namespace zen;
   const int prepared = (mode & ZEN_MODE_PREPARED) ? ((mode & ZEN_MODE_SECOND) ? 2 : 1) : 0;
+  const bool second_set = (mode & ZEN_MODE_SECOND) != 0;
   const uint32_t *near_key = nullptr;
   if (mode & ZEN_MODE_FLOOR) {
     if (k <= 0 || !thr) return fail(ZEN_EINVAL, "zen_load_balance: ZEN_MODE_FLOOR needs k > 0 and the key in thr");
@@ -486,6 +488,7 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
     sa.workspace = workspace;
     sa.status = status;
     sa.prepared = near_key ? 0 : prepared;
+    sa.second = second_set;
     sa.near_key = near_key;
     if (wide) return wide_load_balance(sa, slab_state_offset(sa.hash_log2), s);
     return slab_load_balance(sa, s);
@@ -579,6 +582,18 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
         static_cast<uint32_t *>(out_val), splits, status);
   ZEN_LAUNCH_CHECK("k_splits_serial");
   return ZEN_OK;
+}
+
+int zen_encode_merge(const zen_encode_merge_args *a) {
+  using namespace zen;
+  if (!a) return fail(ZEN_EINVAL, "zen_encode_merge: null pointer");
+  const int rc = zen_load_balance(a->input, a->dtype, a->n, a->m, a->partitions, a->rehash, a->thr, a->k, a->thr_out,
+                                  a->out_idx, a->out_val, a->capacity, a->splits, a->table, a->mode, a->workspace,
+                                  a->workspace_bytes, a->status, a->stream);
+  if (rc != ZEN_OK) return rc;
+  return zen_merge(a->recv_idx, a->recv_idx64, a->recv_val, a->dtype, a->r, a->dense_n, a->merged_idx, a->merged_idx64,
+                   a->merged_val, a->merged_capacity, a->merged_count, a->merge_mode, a->merge_workspace,
+                   a->merge_workspace_bytes, a->merge_status, a->merge_stream ? a->merge_stream : a->stream);
 }
 
 }  // extern "C"

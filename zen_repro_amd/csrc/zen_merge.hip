@@ -11,13 +11,6 @@
 
 namespace zen {
 
-// zen_wide_merge.hip
-bool wide_merge_fits(int64_t r, int64_t dense_n, int cus, SlabGeom *geo);
-size_t wide_merge_bytes(int64_t r, int64_t dense_n, int cus);
-int wide_merge(const void *idx, int idx64_in, const void *val, int dtype, int64_t r, int64_t dense_n, void *out_idx,
-               int idx64_out, float *out_val, int64_t capacity, int64_t *out_count, unsigned long long *scan,
-               uint32_t *cursor, void *rest, int cus, int32_t *status, hipStream_t s);
-
 namespace {
 
 constexpr int kMrgBlock = 512;
@@ -524,9 +517,12 @@ int merge_launch(const void *idx, int idx64_in, const S *val, int64_t r, int64_t
       launch_fill<unsigned long long>(scan, 0ull, kMergeZeroBytes / sizeof(unsigned long long), s);
       ZEN_LAUNCH_CHECK("merge: clear prefix state");
     }
-    return wide_merge(idx, idx64_in, val, sizeof(S) == 2 ? ZEN_BF16 : ZEN_F32, r, dense_n, out_idx, idx64_out, out_val,
-                      capacity, out_count, scan, cursor, static_cast<char *>(workspace) + kMergeZeroBytes,
-                      wide_device_cus(), status, s);
+    WideList list;
+    if (!wide_merge_list(idx, idx64_in, val, r, dense_n, cursor, static_cast<char *>(workspace) + kMergeZeroBytes,
+                         wide_device_cus(), status, &list))
+      return fail(ZEN_EINVAL, "zen_merge: sizes do not suit the wide buckets");
+    return wide_merge(list, sizeof(S) == 2 ? ZEN_BF16 : ZEN_F32, false, out_idx, idx64_out, out_val, capacity, out_count,
+                      scan, s);
   }
   if (mode == ZEN_MODE_FAST && slab_merge_fits(r, dense_n, &geo)) {
     if (idx64_in)

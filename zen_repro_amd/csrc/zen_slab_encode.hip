@@ -758,7 +758,7 @@ int slab_prepare(const SlabBalanceArgs &a, hipStream_t s) {
   sample_hist[1] = cs.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
   Carver cw(a.workspace);
   uint32_t *thr = cw.take<uint32_t>(16);
-  const int set = a.prepared == 2 ? 1 : 0;
+  const int set = (a.prepared == 2 || a.second) ? 1 : 0;
   uint32_t *floor = thr + 2 + 4 * set;
   if (a.discard) {  // a sample nobody will pick up: its histogram goes back to zero
     launch_fill<uint32_t>(sample_hist[set], 0u, sampled_floor_zero_bytes() / sizeof(uint32_t), s);
@@ -792,7 +792,7 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
   sc.ticket = p.ticket;
   sc.status = a.status;
   int rc;
-  const int set = a.prepared == 2 ? 1 : 0;
+  const int set = (a.prepared == 2 || a.second) ? 1 : 0;
   uint32_t *floor = p.thr + 2 + 4 * set;
   if (a.only_prepare) return slab_prepare(a, s);
   if (a.k > 0) {

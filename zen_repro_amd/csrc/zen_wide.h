@@ -146,6 +146,131 @@ __device__ inline uint32_t load_agent(const uint32_t *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+
+// ------------------------------------------------------- received entries -> wide buckets (merge side)
+//
+// A record in a bucket's slab is one 64-bit word: the index's offset from the bucket's first index (below
+// 2^23) in bits 0-22, the arrival number (below 2^25) in bits 23-47 and, for bf16, the value in bits 48-63;
+// fp32 values travel in a word plane of their own.  One store per record, and a run of eight fills a line.
+constexpr uint32_t kWmOffBits = 23, kWmArrBits = 25;
+constexpr int kWmPad = 8;  // words between two part cursors
+struct WideSlabs {
+  uint32_t *cursor;    // [nbuckets * kWideSplit * kWmPad], zero before the scatter; the bucket's workgroup puts them back
+  uint2 *rec;          // [nbuckets * kWideSplit * part_cap]
+  uint32_t *val32;     // fp32 values (unused for bf16)
+  uint32_t part_cap;
+};
+__device__ inline uint2 wm_pack(uint32_t off, uint32_t arr, uint32_t val16) {
+  return make_uint2(off | (arr << kWmOffBits), (arr >> (32 - kWmOffBits)) | (val16 << 16));
+}
+__device__ inline uint32_t wm_off(uint2 r) { return r.x & ((1u << kWmOffBits) - 1u); }
+__device__ inline uint32_t wm_arr(uint2 r) { return (r.x >> kWmOffBits) | ((r.y & 0xffffu) << (32 - kWmOffBits)); }
+
+// What a workgroup of BLOCK threads needs in LDS to scatter a batch of BLOCK * ITEMS list entries.
+template <int BLOCK, int ITEMS>
+struct WideScatterShared {
+  uint32_t cnt[kWideMaxBuckets], pref[kWideMaxBuckets + 1], gbase[kWideMaxBuckets];
+  uint32_t lo[kWideMaxBuckets];  // the buckets' first indices (a 64-bit division each)
+  uint32_t scan[BLOCK / 64 + 1];
+  uint32_t idx[BLOCK * ITEMS];
+  uint16_t from[BLOCK * ITEMS];  // place inside the batch (the arrival number, and where the value is)
+  uint8_t dst[BLOCK * ITEMS];
+  static_assert(kWideMaxBuckets <= 256 && BLOCK * ITEMS <= 65536, "a destination in a byte, a place in a halfword");
+};
+
+// The list of received entries the scatter works on.
+struct WideList {
+  SlabGeom geo;        // buckets over the index range [0, dense_n)
+  const void *idx;     // int32 or int64
+  const void *val;     // values in the type S of the caller's template
+  uint32_t r, dense_n;
+  int idx64;
+  WideSlabs out;
+  int32_t *status;     // BAD_INDEX, RETRY
+};
+
+// Called by the whole workgroup once before its first batch: the buckets' first indices.
+template <int BLOCK, int ITEMS>
+__device__ inline void wide_scatter_prepare(const WideList &a, WideScatterShared<BLOCK, ITEMS> &sh) {
+  for (uint32_t b = threadIdx.x; b < (uint32_t)kWideMaxBuckets; b += BLOCK)
+    sh.lo[b] = b < a.geo.nbuckets ? a.geo.first_key(b) : 0u;
+  __syncthreads();
+}
+
+// Batch number `batch` of the list (BLOCK * ITEMS entries) goes to the buckets' slabs: the workgroup orders
+// the entries by bucket in LDS, reserves one run per bucket behind the cursor of part `part` and writes the
+// runs with consecutive lanes on consecutive records.  Entries whose index lies outside [0, dense_n) are
+// skipped and flagged.  Ends with a barrier.
+template <typename S, int BLOCK, int ITEMS>
+__device__ inline void wide_scatter_batch(const WideList &a, uint32_t batch, uint32_t part,
+                                          WideScatterShared<BLOCK, ITEMS> &sh) {
+  constexpr uint32_t kNone = 0xffffffffu;
+  const uint32_t first = batch * (uint32_t)(BLOCK * ITEMS);
+  const uint32_t nb = a.geo.nbuckets;
+  const S *val = static_cast<const S *>(a.val);
+  for (uint32_t b = threadIdx.x; b < (uint32_t)kWideMaxBuckets; b += BLOCK) sh.cnt[b] = 0;
+  __syncthreads();
+  uint32_t k[ITEMS], d[ITEMS], rank[ITEMS];
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t e = first + threadIdx.x + i * BLOCK;
+    d[i] = kNone;
+    k[i] = rank[i] = 0;
+    if (e < a.r) {
+      const int64_t v = a.idx64 ? static_cast<const int64_t *>(a.idx)[e] : (int64_t)static_cast<const int32_t *>(a.idx)[e];
+      if (v < 0 || v >= (int64_t)a.dense_n) {
+        atomicOr(a.status, ZEN_STAT_BAD_INDEX);  // skipped, like everything behind the good ones in the general path
+      } else {
+        k[i] = (uint32_t)v;
+        d[i] = a.geo.bucket_of(k[i]);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i)
+    if (d[i] != kNone) rank[i] = atomicAdd(&sh.cnt[d[i]], 1u);
+  __syncthreads();
+  uint32_t total = 0;
+  for (uint32_t b0 = 0; b0 < (uint32_t)kWideMaxBuckets; b0 += BLOCK) {  // one turn unless BLOCK < 256
+    const uint32_t b = b0 + threadIdx.x;
+    const uint32_t c = b < nb ? sh.cnt[b] : 0u;
+    uint32_t turn;
+    const uint32_t before = total + block_exclusive_scan<uint32_t, BLOCK>(c, sh.scan, &turn);
+    if (b < nb) {
+      sh.pref[b] = before;
+      sh.gbase[b] = c ? atomicAdd(&a.out.cursor[(b * kWideSplit + part) * kWmPad], c) : 0u;
+    }
+    total += turn;
+  }
+  if (threadIdx.x == 0) sh.pref[nb] = total;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    if (d[i] != kNone) {
+      const uint32_t p = sh.pref[d[i]] + rank[i];
+      sh.idx[p] = k[i];
+      sh.from[p] = (uint16_t)(threadIdx.x + i * BLOCK);
+      sh.dst[p] = (uint8_t)d[i];
+    }
+  }
+  __syncthreads();
+#pragma unroll 2
+  for (uint32_t p = threadIdx.x; p < total; p += BLOCK) {
+    const uint32_t g = sh.dst[p];
+    const uint32_t at = sh.gbase[g] + (p - sh.pref[g]);
+    if (at < a.out.part_cap) {
+      const size_t o = (size_t)(g * kWideSplit + part) * a.out.part_cap + at;
+      const uint32_t e = first + sh.from[p];
+      const S v = val[e];  // the batch's arrival numbers are consecutive: these loads hit what it has just read
+      a.out.rec[o] = wm_pack(sh.idx[p] - sh.lo[g], e, sizeof(S) == 2 ? (uint32_t)v : 0u);
+      if (sizeof(S) == 4) a.out.val32[o] = (uint32_t)v;
+    } else {
+      atomicOr(a.status, ZEN_STAT_RETRY);  // a slab is full: another path answers
+    }
+  }
+  __syncthreads();
+}
+
 // Launches that need all their workgroups resident at once must not be dispatched side by side (each could
 // end up holding a part of the chip and waiting for the rest): the host keeps them in line with an event per
 // device.  wide_line_enter makes `stream` wait for the last such launch, wide_line_leave records the new one.
@@ -153,5 +278,13 @@ __device__ inline uint32_t load_agent(const uint32_t *p) {
 int wide_line_enter(hipStream_t stream);
 int wide_line_leave(hipStream_t stream);
 int wide_device_cus();
+
+// zen_wide_merge.hip
+bool wide_merge_fits(int64_t r, int64_t dense_n, int cus, SlabGeom *geo);
+size_t wide_merge_bytes(int64_t r, int64_t dense_n, int cus);
+bool wide_merge_list(const void *idx, int idx64_in, const void *val, int64_t r, int64_t dense_n, uint32_t *cursor,
+                     void *rest, int cus, int32_t *status, WideList *list);
+int wide_merge(const WideList &list, int dtype, bool scattered, void *out_idx, int idx64_out, float *out_val,
+               int64_t capacity, int64_t *out_count, unsigned long long *scan, hipStream_t s);
 
 }  // namespace zen

@@ -889,7 +889,7 @@ int wide_load_balance(const SlabBalanceArgs &a, size_t state_offset, hipStream_t
   sc.ticket = p.ticket;
   sc.status = a.status;
   int rc;
-  const int set = a.prepared == 2 ? 1 : 0;
+  const int set = (a.prepared == 2 || a.second) ? 1 : 0;
   uint32_t *floor = p.thr + 2 + 4 * set;
   if (a.k > 0) {
     if (a.near_key) {

@@ -14,7 +14,6 @@
 namespace zen {
 namespace {
 
-constexpr int kWmPad = 8;                                  // words between two part cursors
 constexpr uint32_t kWmCursorWords = kWideMaxBuckets * kWideSplit * kWmPad;
 static_assert(kWmCursorWords <= kCoarseCursorWords, "the cursors fit the zero region of the slab path's coarse cursors");
 constexpr int kWmRounds = 3;                               // a part of a bucket's slab is read in rounds of kWideBlock records
@@ -35,114 +34,13 @@ constexpr int kWsBlock = 512;
 constexpr int kWsItems = 8;
 constexpr int kWsBatch = kWsBlock * kWsItems;  // list entries per workgroup
 
-// A record in a bucket's slab is one 64-bit word: the index's offset from the bucket's first index (below
-// 2^23) in bits 0-22, the arrival number (below 2^25) in bits 23-47 and, for bf16, the value in bits 48-63;
-// fp32 values travel in a word plane of their own.  One store per record, and a run of sixteen fills a line.
-constexpr uint32_t kWmOffBits = 23, kWmArrBits = 25;
-struct WideSlabs {
-  uint32_t *cursor;    // [nbuckets * kWideSplit * kWmPad], zero before the scatter; the bucket's workgroup puts them back
-  uint2 *rec;          // [nbuckets * kWideSplit * part_cap]
-  uint32_t *val32;     // fp32 values (unused for bf16)
-  uint32_t part_cap;
-};
-__device__ inline uint2 wm_pack(uint32_t off, uint32_t arr, uint32_t val16) {
-  return make_uint2(off | (arr << kWmOffBits), (arr >> (32 - kWmOffBits)) | (val16 << 16));
-}
-__device__ inline uint32_t wm_off(uint2 r) { return r.x & ((1u << kWmOffBits) - 1u); }
-__device__ inline uint32_t wm_arr(uint2 r) { return (r.x >> kWmOffBits) | ((r.y & 0xffffu) << (32 - kWmOffBits)); }
-
-#ifdef ZEN_WIDE_TIMING
-__device__ unsigned long long g_wm_dbg[1024 * 16];
-#define WM_MARK(k) do { if (threadIdx.x == 0 && blockIdx.x < 1024) g_wm_dbg[blockIdx.x * 16 + (k)] = wall_clock64(); } while (0)
-#else
-#define WM_MARK(k) do { } while (0)
-#endif
-
-template <typename I, typename S>
-__global__ __launch_bounds__(kWsBlock) void k_wide_scatter(SlabGeom geo, const I *__restrict__ idx,
-                                                           const S *__restrict__ val, uint32_t r, uint32_t dense_n,
-                                                           WideSlabs out, int32_t *status) {
-  __shared__ uint32_t s_cnt[kWideMaxBuckets], s_pref[kWideMaxBuckets + 1], s_gbase[kWideMaxBuckets];
-  __shared__ uint32_t s_scan[kWsBlock / 64 + 1];
-  __shared__ uint32_t s_idx[kWsBatch];
-  // 32 KB of LDS in all: five workgroups share a compute unit and the whole grid is resident in one round (the
-  // values do not pass through LDS for that reason: they are fetched again when the record is written)
-  __shared__ uint16_t s_from[kWsBatch];  // place inside the batch (the arrival number, and where the value is)
-  __shared__ uint8_t s_dst[kWsBatch];
-  static_assert(kWideMaxBuckets <= 256, "a destination in a byte");
-  __shared__ uint32_t s_lo[kWideMaxBuckets];  // the buckets' first indices (a 64-bit division each)
-  const uint32_t batch = blockIdx.x * (uint32_t)kWsBatch;
-  const uint32_t part = blockIdx.x % kWideSplit;
-  const uint32_t nb = geo.nbuckets;
-  if (threadIdx.x < (uint32_t)kWideMaxBuckets) {
-    s_cnt[threadIdx.x] = 0;
-    s_lo[threadIdx.x] = threadIdx.x < nb ? geo.first_key(threadIdx.x) : 0u;
-  }
-  __syncthreads();
-  WM_MARK(0);
-  uint32_t k[kWsItems], d[kWsItems], rank[kWsItems];
-#pragma unroll
-  for (int i = 0; i < kWsItems; ++i) {
-    const uint32_t e = batch + threadIdx.x + i * kWsBlock;
-    d[i] = kInvalid;
-    k[i] = rank[i] = 0;
-    if (e < r) {
-      const I v = idx[e];
-      if (v < 0 || (uint64_t)v >= (uint64_t)dense_n) {
-        atomicOr(status, ZEN_STAT_BAD_INDEX);  // skipped, like everything behind the good ones in the general path
-      } else {
-        k[i] = (uint32_t)v;
-        d[i] = geo.bucket_of(k[i]);
-      }
-    }
-  }
-  WM_MARK(1);
-#pragma unroll
-  for (int i = 0; i < kWsItems; ++i)
-    if (d[i] != kInvalid) rank[i] = atomicAdd(&s_cnt[d[i]], 1u);
-  __syncthreads();
-  WM_MARK(2);
-  {
-    const uint32_t c = threadIdx.x < nb ? s_cnt[threadIdx.x] : 0u;
-    uint32_t total;
-    const uint32_t before = block_exclusive_scan<uint32_t, kWsBlock>(c, s_scan, &total);
-    if (threadIdx.x < nb) {
-      s_pref[threadIdx.x] = before;
-      s_gbase[threadIdx.x] = c ? atomicAdd(&out.cursor[(threadIdx.x * kWideSplit + part) * kWmPad], c) : 0u;
-    }
-    if (threadIdx.x == 0) s_pref[nb] = total;
-  }
-  __syncthreads();
-  WM_MARK(3);
-#pragma unroll
-  for (int i = 0; i < kWsItems; ++i) {
-    if (d[i] != kInvalid) {
-      const uint32_t p = s_pref[d[i]] + rank[i];
-      s_idx[p] = k[i];
-      s_from[p] = (uint16_t)(threadIdx.x + i * kWsBlock);
-      s_dst[p] = (uint8_t)d[i];
-    }
-  }
-  __syncthreads();
-  WM_MARK(4);
-  const uint32_t total = s_pref[nb];
-#pragma unroll 2
-  for (uint32_t p = threadIdx.x; p < total; p += kWsBlock) {
-    const uint32_t g = s_dst[p];
-    const uint32_t at = s_gbase[g] + (p - s_pref[g]);
-    if (at < out.part_cap) {
-      const size_t o = (size_t)(g * kWideSplit + part) * out.part_cap + at;
-      const uint32_t e = batch + s_from[p];
-      const S v = val[e];  // a workgroup's 4096 arrival numbers are consecutive: these loads hit what it has just read
-      out.rec[o] = wm_pack(s_idx[p] - s_lo[g], e, sizeof(S) == 2 ? (uint32_t)v : 0u);
-      if (sizeof(S) == 4) out.val32[o] = (uint32_t)v;
-    } else {
-      atomicOr(status, ZEN_STAT_RETRY);  // a slab is full: another path answers
-    }
-  }
-  WM_MARK(5);
-  wait_global_acks();
-  WM_MARK(6);
+template <typename S>
+__global__ __launch_bounds__(kWsBlock) void k_wide_scatter(WideList list) {
+  // 32 KB of LDS: five workgroups share a compute unit and the whole grid is resident in one round (the values
+  // do not pass through LDS for that reason: they are fetched again when the record is written)
+  __shared__ WideScatterShared<kWsBlock, kWsItems> sh;
+  wide_scatter_prepare(list, sh);
+  wide_scatter_batch<S>(list, blockIdx.x, blockIdx.x % kWideSplit, sh);
 }
 
 // ------------------------------------------------------------ a bucket
@@ -494,12 +392,12 @@ size_t wide_merge_bytes(int64_t r, int64_t dense_n, int cus) {
   return align_up(entries * sizeof(uint2), 256) + align_up(entries * sizeof(uint32_t), 256);
 }
 
-// scan: zeroed prefix state for 256 buckets (descriptors, ticket, finished count); cursor: kCoarseCursorWords
-// zeroed words; rest: wide_merge_bytes(...) bytes.  Both zero regions are zero again when the launches end.
-template <typename I_in, typename S>
-static int wide_merge_typed(const SlabGeom &geo, const I_in *idx, const S *val, int64_t r, int64_t dense_n,
-                            void *out_idx, int idx64_out, float *out_val, int64_t capacity, int64_t *out_count,
-                            unsigned long long *scan, uint32_t *cursor, void *rest, int32_t *status, hipStream_t s) {
+// The received entries as the scatter wants them: cursor: kCoarseCursorWords zeroed words (zero again when
+// k_wide_merge has run); rest: wide_merge_bytes(...) bytes.  False if the sizes do not suit the wide buckets.
+bool wide_merge_list(const void *idx, int idx64_in, const void *val, int64_t r, int64_t dense_n, uint32_t *cursor,
+                     void *rest, int cus, int32_t *status, WideList *list) {
+  SlabGeom geo;
+  if (!wide_merge_fits(r, dense_n, cus, &geo)) return false;
   WideSlabs slabs;
   slabs.part_cap = wide_merge_part_cap(geo, r);
   const size_t entries = (size_t)geo.nbuckets * kWideSplit * slabs.part_cap;
@@ -507,50 +405,52 @@ static int wide_merge_typed(const SlabGeom &geo, const I_in *idx, const S *val, 
   slabs.cursor = cursor;
   slabs.rec = cv.take<uint2>(entries);
   slabs.val32 = cv.take<uint32_t>(entries);
-  {
+  list->geo = geo;
+  list->idx = idx;
+  list->val = val;
+  list->r = (uint32_t)r;
+  list->dense_n = (uint32_t)dense_n;
+  list->idx64 = idx64_in;
+  list->out = slabs;
+  list->status = status;
+  return true;
+}
+
+uint32_t wide_scatter_batches(const WideList &list, int batch) { return (uint32_t)ceil_div((int64_t)list.r, batch); }
+
+// The two launches (one if the entries are in the buckets' slabs already: `scattered`).  scan: zeroed prefix
+// state for 256 buckets (descriptors, ticket, finished count), zero again when the launch ends.
+int wide_merge(const WideList &list, int dtype, bool scattered, void *out_idx, int idx64_out, float *out_val,
+               int64_t capacity, int64_t *out_count, unsigned long long *scan, hipStream_t s) {
+  if (!scattered) {
     ProfScope prof(kProfWideScatter, s);
-    k_wide_scatter<I_in, S><<<dim3((unsigned)ceil_div(r, kWsBatch)), dim3(kWsBlock), 0, s>>>(
-        geo, idx, val, (uint32_t)r, (uint32_t)dense_n, slabs, status);
+    if (dtype == ZEN_BF16)
+      k_wide_scatter<uint16_t><<<dim3(wide_scatter_batches(list, kWsBatch)), dim3(kWsBlock), 0, s>>>(list);
+    else
+      k_wide_scatter<uint32_t><<<dim3(wide_scatter_batches(list, kWsBatch)), dim3(kWsBlock), 0, s>>>(list);
     ZEN_LAUNCH_CHECK("k_wide_scatter");
   }
-  const ScanState st = scan_state(scan, (int64_t)geo.nbuckets);
-  const int tie_bits = ceil_log2_u64((uint64_t)r);  // arrival numbers are < r
+  const ScanState st = scan_state(scan, (int64_t)list.geo.nbuckets);
+  const int tie_bits = ceil_log2_u64((uint64_t)list.r);  // arrival numbers are < r
   ProfScope prof(kProfWideMerge, s);
-  if (idx64_out)
-    k_wide_merge<int64_t, S><<<dim3(geo.nbuckets), dim3(kWideBlock), 0, s>>>(
-        geo, slabs, static_cast<int64_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
-  else
-    k_wide_merge<int32_t, S><<<dim3(geo.nbuckets), dim3(kWideBlock), 0, s>>>(
-        geo, slabs, static_cast<int32_t *>(out_idx), out_val, capacity, st, tie_bits, out_count, status);
+  const dim3 grid(list.geo.nbuckets), block(kWideBlock);
+  if (dtype == ZEN_BF16) {
+    if (idx64_out)
+      k_wide_merge<int64_t, uint16_t><<<grid, block, 0, s>>>(list.geo, list.out, static_cast<int64_t *>(out_idx), out_val,
+                                                             capacity, st, tie_bits, out_count, list.status);
+    else
+      k_wide_merge<int32_t, uint16_t><<<grid, block, 0, s>>>(list.geo, list.out, static_cast<int32_t *>(out_idx), out_val,
+                                                             capacity, st, tie_bits, out_count, list.status);
+  } else {
+    if (idx64_out)
+      k_wide_merge<int64_t, uint32_t><<<grid, block, 0, s>>>(list.geo, list.out, static_cast<int64_t *>(out_idx), out_val,
+                                                             capacity, st, tie_bits, out_count, list.status);
+    else
+      k_wide_merge<int32_t, uint32_t><<<grid, block, 0, s>>>(list.geo, list.out, static_cast<int32_t *>(out_idx), out_val,
+                                                             capacity, st, tie_bits, out_count, list.status);
+  }
   ZEN_LAUNCH_CHECK("k_wide_merge");
   return ZEN_OK;
 }
 
-int wide_merge(const void *idx, int idx64_in, const void *val, int dtype, int64_t r, int64_t dense_n, void *out_idx,
-               int idx64_out, float *out_val, int64_t capacity, int64_t *out_count, unsigned long long *scan,
-               uint32_t *cursor, void *rest, int cus, int32_t *status, hipStream_t s) {
-  SlabGeom geo;
-  if (!wide_merge_fits(r, dense_n, cus, &geo)) return fail(ZEN_EINVAL, "wide_merge: sizes do not suit the wide buckets");
-  if (dtype == ZEN_BF16) {
-    const uint16_t *v = static_cast<const uint16_t *>(val);
-    if (idx64_in)
-      return wide_merge_typed(geo, static_cast<const int64_t *>(idx), v, r, dense_n, out_idx, idx64_out, out_val,
-                              capacity, out_count, scan, cursor, rest, status, s);
-    return wide_merge_typed(geo, static_cast<const int32_t *>(idx), v, r, dense_n, out_idx, idx64_out, out_val,
-                            capacity, out_count, scan, cursor, rest, status, s);
-  }
-  const uint32_t *v = static_cast<const uint32_t *>(val);
-  if (idx64_in)
-    return wide_merge_typed(geo, static_cast<const int64_t *>(idx), v, r, dense_n, out_idx, idx64_out, out_val,
-                            capacity, out_count, scan, cursor, rest, status, s);
-  return wide_merge_typed(geo, static_cast<const int32_t *>(idx), v, r, dense_n, out_idx, idx64_out, out_val, capacity,
-                          out_count, scan, cursor, rest, status, s);
-}
-
 }  // namespace zen
-
-#ifdef ZEN_WIDE_TIMING
-extern "C" int zen_wm_debug_read(unsigned long long *host) {
-  return hipMemcpyFromSymbol(host, HIP_SYMBOL(zen::g_wm_dbg), sizeof(unsigned long long) * 1024 * 16) == hipSuccess ? 0 : -1;
-}
-#endif

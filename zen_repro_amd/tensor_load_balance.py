@@ -99,16 +99,16 @@ class TensorPartition:
         return int(torch.count_nonzero(flat)) + 1024
 
     def _ahead_state(self, device, slot, create=False):
-        # "next": the set of sampling memory the next prepare takes (the second first: a call that samples for
-        # itself uses the first); "free": per set, the event after the last call that used it; "pending":
-        # samples taken and not yet picked up by their calls
+        # "free": per set of sampling memory, the event after the last call that used it; "pending": samples
+        # taken and not yet picked up by their calls (tensor, size, k, capacity, workspace, set, event, type,
+        # workspace bytes)
         key = (_lib.device_index(device), slot)
         state = self._ahead.get(key)
         if state is None and create:
             # Calls made before the first prepare left no events behind (a call only keeps this book once
             # samples are taken ahead for its slot): wait for them all, once.
             torch.cuda.synchronize(device)
-            state = self._ahead[key] = {"next": 1, "free": [None, None], "pending": []}
+            state = self._ahead[key] = {"free": [None, None], "pending": []}
         return state
 
     def prepare(self, tensor, k, capacity, slot=0):
@@ -132,10 +132,10 @@ class TensorPartition:
                                              _lib.MODE_FAST | self.fast_flags) not in (2, 3):
             return
         state = self._ahead_state(dev, slot, create=True)
-        if len(state["pending"]) >= 2:
+        busy = {entry[5] for entry in state["pending"]}
+        if len(busy) >= 2:
             return  # both sets are spoken for
-        which = state["next"]
-        state["next"] ^= 1
+        which = 1 if 1 not in busy else 0  # the second first: a call that samples for itself prefers the first
         stream = torch.cuda.current_stream(dev)
         if state["free"][which] is not None:
             stream.wait_event(state["free"][which])  # the call that used this set last has finished
@@ -143,12 +143,69 @@ class TensorPartition:
         ws = _lib.scratch.get(dev, f"load_balance/{slot}", nbytes)
         table = self._table(dev, m, slot)
         rc = L.zen_load_balance_prepare(_lib.ptr(flat), code, n, m, self.partitions, int(k), capacity, _lib.ptr(table),
-                                        _lib.MODE_FAST | (_lib.MODE_SECOND if which else 0), _lib.ptr(ws), ws.numel(),
+                                        _lib.MODE_FAST | self.fast_flags | (_lib.MODE_SECOND if which else 0),
+                                        _lib.ptr(ws), ws.numel(),
                                         _lib.stream_of(dev))
         _lib.check(rc, "load_balance prepare")
         done = torch.cuda.Event()
         done.record(stream)
-        state["pending"].append((flat.data_ptr(), n, int(k), capacity, ws.data_ptr(), which, done))
+        state["pending"].append((flat.data_ptr(), n, int(k), capacity, ws.data_ptr(), which, done, code, ws.numel()))
+
+    def _take_ahead(self, flat, n, k, capacity, ws, slot, mode, thr, near):
+        """The sample taken ahead for the call that is about to be made, if there is one: (mode flags that tell
+        the library, the set of sampling memory the call will use).  Samples taken for other calls stay where
+        they are; one that its bucket will never pick up (same tensor and size, other arguments) is dropped."""
+        dev = flat.device
+        state = self._ahead_state(dev, slot)  # None: no sample was ever taken ahead for this slot
+        if state is None or k <= 0:
+            return 0, 0
+        L = _lib.lib()
+        want = (flat.data_ptr(), n, k, capacity, ws.data_ptr())
+        ahead = None
+        for i, entry in enumerate(state["pending"]):
+            if entry[:5] == want:
+                ahead = state["pending"].pop(i)
+                break
+        usable = (mode & 0xff) == _lib.MODE_FAST and thr is None and near is None
+        cur = torch.cuda.current_stream(dev)
+        if ahead is not None and not usable:
+            # taken for this very call, which will not use it: its histogram is cleared again
+            self._discard(ahead, slot, dev)
+            ahead = None
+        if ahead is not None:
+            cur.wait_event(ahead[6])
+            return _lib.MODE_PREPARED | (_lib.MODE_SECOND if ahead[5] else 0), ahead[5]
+        # the call samples for itself, in a set no pending sample sits in (and whose last user has finished)
+        busy = {entry[5] for entry in state["pending"]}
+        which = 0 if 0 not in busy else 1
+        if which in busy:
+            # both sets hold samples of other buckets: the older one gives way
+            old = state["pending"].pop(0)
+            self._discard(old, slot, dev)
+            which = old[5]
+        if state["free"][which] is not None:
+            cur.wait_event(state["free"][which])
+        return (_lib.MODE_SECOND if which else 0), which
+
+    def _discard(self, entry, slot, dev):
+        """Clears the sampling memory of a sample nobody will pick up (with the arguments it was taken with)."""
+        L = _lib.lib()
+        a_ptr, a_n, a_k, a_cap, a_ws, a_which, a_done, a_code, a_bytes = entry
+        torch.cuda.current_stream(dev).wait_event(a_done)
+        a_m, _ = self.table_sizes(a_n)
+        _lib.check(L.zen_load_balance_prepare(
+            ctypes.c_void_p(a_ptr), a_code, a_n, a_m, self.partitions, a_k, a_cap,
+            _lib.ptr(self._table(dev, a_m, slot)), _lib.MODE_FAST | self.fast_flags | _lib.MODE_DISCARD |
+            (_lib.MODE_SECOND if a_which else 0), ctypes.c_void_p(a_ws), a_bytes, _lib.stream_of(dev)),
+            "load_balance discard")
+
+    def _after_call(self, dev, slot, k, used):
+        """The set of sampling memory a top-k call used is free again once the call has finished."""
+        state = self._ahead_state(dev, slot)
+        if k > 0 and state is not None:
+            free = torch.cuda.Event()
+            free.record(torch.cuda.current_stream(dev))
+            state["free"][used] = free
 
     def load_balance_flat(self, tensor, thr=None, capacity=None, k=0, mode=_lib.MODE_FAST, thr_out=None, slot=0,
                           near=None):
@@ -187,29 +244,7 @@ class TensorPartition:
         nbytes = L.zen_load_balance_workspace(n, m, code, capacity, self.partitions)
         ws = _lib.scratch.get(dev, f"load_balance/{slot}", nbytes)
         table = self._table(dev, m, slot)
-        # a sample taken ahead for this very call (prepare)?
-        state = self._ahead_state(dev, slot)  # None: no sample was ever taken ahead for this slot
-        ahead = None
-        if state is not None and state["pending"]:
-            ahead = state["pending"].pop(0)
-            if (ahead[:5] != (flat.data_ptr(), n, int(k), capacity, ws.data_ptr()) or (mode & 0xff) != _lib.MODE_FAST
-                    or thr is not None or near is not None):
-                # not for this call: its histogram is cleared again (with the arguments it was taken with) and
-                # the call samples for itself
-                cur = torch.cuda.current_stream(dev)
-                cur.wait_event(ahead[6])
-                a_ptr, a_n, a_k, a_cap, a_ws, a_which, _ = ahead
-                a_m, _ = self.table_sizes(a_n)
-                _lib.check(L.zen_load_balance_prepare(
-                    ctypes.c_void_p(a_ptr), code, a_n, a_m, self.partitions, a_k, a_cap,
-                    _lib.ptr(self._table(dev, a_m, slot)), _lib.MODE_FAST | _lib.MODE_DISCARD |
-                    (_lib.MODE_SECOND if a_which else 0), ctypes.c_void_p(a_ws), ws.numel(), _lib.stream_of(dev)),
-                    "load_balance discard")
-                ahead = None
-        flags = 0
-        if ahead is not None:
-            torch.cuda.current_stream(dev).wait_event(ahead[6])
-            flags = _lib.MODE_PREPARED | (_lib.MODE_SECOND if ahead[5] else 0)
+        flags, used = self._take_ahead(flat, n, int(k), capacity, ws, slot, mode, thr, near)
         if near is not None and k > 0 and thr is None:
             thr, flags = near, flags | _lib.MODE_FLOOR
         rc = L.zen_load_balance(
@@ -217,13 +252,7 @@ class TensorPartition:
             _lib.ptr(out_idx), _lib.ptr(out_val), capacity, _lib.ptr(splits), _lib.ptr(table), mode | flags,
             _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
         _lib.check(rc, "load_balance")
-        if k > 0 and state is not None:
-            # whichever set of sampling memory this call used (a call that samples for itself uses the first)
-            # is free again once it has finished
-            used = ahead[5] if ahead is not None else 0
-            free = torch.cuda.Event()
-            free.record(torch.cuda.current_stream(dev))
-            state["free"][used] = free
+        self._after_call(dev, slot, int(k), used)
         return out_idx, out_val, splits, status
 
     def load_balance(self, tensor, thr=None, capacity=None, k=0, mode=None, grow=None):
