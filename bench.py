@@ -10,6 +10,7 @@ times, the CPU baseline on the same workload and whether the HIP path reproduced
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--shrink S]
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -17,11 +18,51 @@ import time
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
-# HBM bytes per launch of the dominant kernel on the full c3 workload, from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by what the same counters read
-# for a plain 1 GiB copy, and the summary that holds the figures.  Other
-# workloads report null.
-MEASURED_TRAFFIC = {("c3", 1, "k_select_stage"): (1.519e9, "profiles/c3_select_stage_hbm_traffic.txt")}
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by what the
+# same counters read for a plain 1 GiB copy: the summaries under profiles/ that hold such figures, by
+# (configuration, --shrink).  A summary names the kernel sources it was measured on (a digest of the library's
+# source files); a figure measured on other sources is not reported.
+TRAFFIC_PROFILES = {("c3", 1): "profiles/c3_select_stage_hbm_traffic.txt"}
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def kernel_sources_digest():
+    """sha256 over the library's source files (names and contents, in name order)."""
+    import glob
+    import hashlib
+
+    h = hashlib.sha256()
+    files = sorted(glob.glob(os.path.join(HERE, "zen_repro_amd", "csrc", "*.hip")) +
+                   glob.glob(os.path.join(HERE, "zen_repro_amd", "csrc", "*.h")) +
+                   glob.glob(os.path.join(HERE, "include", "*.h")))
+    for f in files:
+        h.update(os.path.basename(f).encode() + b"\0")
+        h.update(open(f, "rb").read())
+    return h.hexdigest()
+
+
+def measured_traffic(config, shrink, kernel):
+    """(bytes per launch or None, where it comes from or why it is missing) for `kernel` on this workload: read
+    from the summary's header lines '# kernel_sources_sha256: <digest>' and
+    '# traffic_bytes_per_launch <kernel>: <bytes>'."""
+    rel = TRAFFIC_PROFILES.get((config, shrink))
+    if rel is None:
+        return None, None
+    try:
+        text = open(os.path.join(HERE, rel)).read()
+    except OSError:
+        return None, f"{rel} is missing"
+    digest = value = None
+    for ln in text.splitlines():
+        if ln.startswith("# kernel_sources_sha256:"):
+            digest = ln.split(":", 1)[1].strip()
+        elif ln.startswith(f"# traffic_bytes_per_launch {kernel}:"):
+            value = float(ln.split(":", 1)[1].strip())
+    if value is None or digest is None:
+        return None, f"{rel} holds no figure for {kernel}"
+    if digest != kernel_sources_digest():
+        return None, f"{rel} was measured on other kernel sources (digest {digest[:12]}): not reported"
+    return value, rel
 
 
 def note(msg):
@@ -75,6 +116,8 @@ def parse():
     ap.add_argument("--stage-steps", type=int, default=20,
                     help="steps of the untimed pass with every stage's events on (the stage table; it also tells "
                          "which kernel is the roofline kernel)")
+    ap.add_argument("--no-reference-bucket", action="store_true",
+                    help="leave out the sub-record for one bucket of a training run's size (c3 only)")
     ap.add_argument("--no-kernel-timing", action="store_true",
                     help="leave the HIP-event kernel timers off during the timed region")
     return ap.parse_args()
@@ -341,6 +384,90 @@ def phase2_decode(args, dev):
         "ms_per_step_from_index_lists": round(ms_lists, 4)}))
 
 
+def reference_bucket(dev, steps, warmup):
+    """The step on ONE gradient bucket of the size a training run hands over (the c3 tensor cut in twelve:
+    61,953,360 bf16 elements, the 0.5 % largest kept, P = 16): one call of the library per step, the next step's
+    sample taken ahead, the merge beside the encode; then the same with two steps in flight."""
+    import torch
+
+    from zen_repro_amd import LoadBalanceAllreduce, LocalGroup, TensorPartition, _lib, workloads
+
+    cfg, grad = workloads.make("c3", device=dev, seed=0, shrink=12)
+    b = workloads.buckets(cfg)[0]
+    esize, P = grad.element_size(), cfg.partitions
+    cap = int(b.k * 1.25) + 4096
+    _, _, fi, fv = workloads.peer_payloads(b, workloads.per_peer_entries(b, b.k), device=dev, seed=1)
+    copies = max(1, -(-(512 << 20) // (b.n * esize)))  # more bytes than the last-level cache holds
+    grads = [grad] + [grad.clone() for _ in range(copies - 1)]
+    tp = TensorPartition(P, 1, 3)
+    lba = LoadBalanceAllreduce(LocalGroup(P), None, None)
+    main = torch.cuda.current_stream(dev)
+    second, beside, ahead = (torch.cuda.Stream(device=dev) for _ in range(3))
+
+    def run(count, depth, marks=None):
+        outs = []
+        for s_ in (second, beside, ahead):
+            s_.wait_stream(main)
+        for i in range(count):
+            es = second if (depth == 2 and i % 2) else main
+            with torch.cuda.stream(es):
+                outs.append(lba.encode_merge_flat(tp, grads[i % copies], cap, b.k, fi, fv, b.n, slot=i % depth,
+                                                  merge_stream=beside if depth == 1 else None))
+            if depth == 1 and i + 1 < count:
+                with torch.cuda.stream(ahead):
+                    tp.prepare(grads[(i + 1) % copies], b.k, cap, slot=0)
+            if marks is not None:
+                marks.append(torch.cuda.Event(enable_timing=True))
+                marks[-1].record(es)
+        for s_ in (second, beside, ahead):
+            main.wait_stream(s_)
+        return outs
+
+    rec = {"elements": b.n, "k": b.k, "partitions": P, "dtype": "bf16"}
+    for depth in (1, 2):
+        run(max(1, warmup), depth)
+        torch.cuda.synchronize()
+        _lib.profile_enable(True)
+        run(4, depth)
+        torch.cuda.synchronize()
+        launches = sum(v[1] for v in _lib.profile_read().values()) // 4
+        _lib.profile_enable(False)
+        t0 = time.perf_counter()
+        outs = run(steps, depth)
+        t_enq = time.perf_counter()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        marks = []
+        run(max(21, min(steps, 60)) + depth, depth, marks)
+        torch.cuda.synchronize()
+        per = sorted(marks[i].elapsed_time(marks[i + depth]) / depth for i in range(len(marks) - depth))
+        call_us = None
+        if depth == 1:
+            # what the one call of the library costs the host: the last step's call again, a hundred times, timed
+            # until the last one returns (nothing waits for the device; the results are the same every time)
+            a = lba.last_encode_merge_args
+            L = _lib.lib()
+            t2 = time.perf_counter()
+            for _ in range(100):
+                L.zen_encode_merge(ctypes.byref(a))
+            call_us = (time.perf_counter() - t2) * 1e4
+            torch.cuda.synchronize()
+        (_, _, splits, st), (_, _, count, mst) = outs[-1]
+        if int(st) | int(mst):
+            print("bench.py: reference bucket: device status " + _lib.describe_status(int(st) | int(mst)), file=sys.stderr)
+            sys.exit(1)
+        b_alg = workloads.algorithmic_bytes(b.n, esize, int(splits.sum()), fi.numel(), int(count))
+        rec["one_step_at_a_time" if depth == 1 else "two_steps_in_flight"] = {
+            "ms_per_step": round(ms, 4), "ms_per_step_device_median": round(per[len(per) // 2], 4),
+            "value": round(b.n * esize / (ms * 1e-3) / 1e9, 2), "unit": "GB/s",
+            "path_frac_of_hbm_peak": round(b_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "host_enqueue_ms_per_step": round((t_enq - t0) * 1e3 / steps, 4), "kernel_launches_per_step": launches}
+        if call_us is not None:
+            rec["library_call_host_ms"] = round(call_us / 1e3, 4)
+    rec["selected"], rec["received"], rec["merged"] = int(splits.sum()), fi.numel(), int(count)
+    return rec
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -477,12 +604,15 @@ def main():
 
     side = enc_streams[1:] + [m for m in mrg_streams if m is not None] + ([prep_stream] if prep_stream is not None else [])
 
-    def run(count):
+    def run(count, marks=None):
         outs = []
         for s_ in side:
             s_.wait_stream(main)  # the inputs were produced on the main stream
         for i in range(count):
             outs.append(step(i, more=i + 1 < count))
+            if marks is not None:  # where the step's encode stream stands once the step is enqueued
+                marks.append(torch.cuda.Event(enable_timing=True))
+                marks[-1].record(enc_streams[i % depth])
         for s_ in side:
             main.wait_stream(s_)
         return outs
@@ -575,6 +705,18 @@ def main():
         kernels = _lib.profile_read() if dom else {}
         _lib.profile_enable(False)
 
+    # The same steps once more with an event behind each: the median of the per-step device times does not move
+    # with a slow first step or a hiccup of the host as the mean above does.
+    device_ms = None
+    if not args.graph:
+        marks = []
+        run(max(21, min(args.steps, 60)) + depth, marks)
+        torch.cuda.synchronize()
+        per = sorted(marks[i].elapsed_time(marks[i + depth]) / depth for i in range(len(marks) - depth))
+        device_ms = {"median": round(per[len(per) // 2], 4), "min": round(per[0], 4), "max": round(per[-1], 4),
+                     "steps": len(per),
+                     "what": "time between the ends of consecutive steps' encodes on the device, back to back, untimed pass"}
+
     last = outs[-1]
     nnz = [int(enc[2].sum()) for enc, _ in last]
     merged = [int(mrg[2]) for _, mrg in last]
@@ -656,10 +798,10 @@ def main():
         total_ms, launches = kernels[dom]
         avg_ms = total_ms / launches
         achieved = per_launch[dom] / (avg_ms * 1e-3) / 1e9
-        traffic = MEASURED_TRAFFIC.get((cfg.name, args.shrink, dom))
+        traffic = measured_traffic(cfg.name, args.shrink, dom)
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                    "traffic": traffic[0] if traffic else None, "traffic_source": traffic[1] if traffic else None,
+                    "traffic": traffic[0], "traffic_source": traffic[1],
                     "avg_launch_ms": round(avg_ms, 4), "launches_per_step": stages[dom][1] // stage_steps,
                     "timed_launches": launches,
                     "algorithmic_bytes_per_launch": int(per_launch[dom]),
@@ -692,6 +834,10 @@ def main():
                    "input_copies": {"gradient": len(grad_sets[0]), "payloads": len(flat_sets[0])}},
         "path_algorithmic_GBps": round(b_alg / (ms * 1e-3) / 1e9, 2),
         "path_frac_of_hbm_peak": round(b_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "ms_per_step_device_median": device_ms["median"] if device_ms else None,
+        "path_frac_of_hbm_peak_at_median": (round(b_alg / (device_ms["median"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+                                            if device_ms else None),
+        "per_step_device_ms": device_ms,
         "ms_per_step_isolated_median": round(lat[len(lat) // 2], 4),
         "two_steps_in_flight": two,
         "host_enqueue_ms_per_step": round((t_enq - t0) * 1e3 / args.steps, 4),
@@ -701,6 +847,9 @@ def main():
         "roofline": roofline,
         "cpu_baseline": None,
     }
+    if cfg.name == "c3" and args.shrink == 1 and not (args.no_reference_bucket or args.graph or args.one_stream):
+        note("one bucket of a training run's size")
+        line["reference_bucket"] = reference_bucket(dev, args.steps, args.warmup)
     if cfg.name == "c4" or args.imbalance:
         # per-bucket load, max / mean, of the hash partition (the split sizes) and of a plain range partition of
         # the same indices (utils.py:66-88 is the reference's notion of skew)

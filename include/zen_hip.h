@@ -177,6 +177,23 @@ int zen_topk_threshold(const void *input, int dtype, int64_t n, int64_t k,
                        void *stream);
 
 /*
+ * The threshold compress() applies (train.py:75-84): thr as for
+ * zen_topk_threshold over the multiset input[sample_index[j]], j < s, the
+ * sample the reference draws with torch.randint and gathers with
+ * tensor[sample_index] before its topk.  sample_index: int64 positions on the
+ * device, each in [0, n) (one outside sets ZEN_STAT_BAD_INDEX and counts as a
+ * zero); 1 <= k <= s.  One gather kernel writes the sample into the workspace,
+ * the radix select of zen_topk_threshold runs on it; nothing is allocated and
+ * nothing waits for the device.
+ */
+size_t zen_sample_threshold_workspace(int64_t s, int dtype);
+int zen_sample_threshold(const void *input, int dtype, int64_t n,
+                         const int64_t *sample_index, int64_t s, int64_t k,
+                         uint32_t *thr, void *workspace,
+                         size_t workspace_bytes, int32_t *status,
+                         void *stream);
+
+/*
  * zen_topk_threshold without a workspace argument and without any allocation.
  * No counterpart in the reference: it is for callers that cannot allocate or
  * carry a workspace (code under HIP graph capture, tight serving loops,
@@ -293,6 +310,23 @@ int zen_merge(const void *idx, int idx64_in, const void *val, int dtype,
               void *out_idx, int idx64_out, float *out_val, int64_t capacity,
               int64_t *out_count, int mode, void *workspace, size_t workspace_bytes,
               int32_t *status, void *stream);
+
+/*
+ * The merged entries on their way to the second exchange: comm.py:125-127
+ * scatters the sums into a dense tensor of the gradient's type and takes its
+ * nonzeros again; here every fp32 sum of zen_merge's output is rounded once to
+ * `dtype` and the entries whose sum rounds to zero are dropped, the rest keep
+ * their ascending order.  idx / out_idx: int32 or int64 (idx64), *count
+ * entries on the device (at most `capacity` are looked at); out_val: `dtype`.
+ * out_idx / out_val need room for `capacity` entries and must not be the
+ * inputs.  Nothing waits for the device.
+ */
+size_t zen_round_compact_workspace(int64_t capacity);
+int zen_round_compact(const void *idx, int idx64, const float *sums,
+                      const int64_t *count, int64_t capacity, int dtype,
+                      void *out_idx, void *out_val, int64_t *out_count,
+                      void *workspace, size_t workspace_bytes,
+                      int32_t *status, void *stream);
 
 /*
  * One step of the path in one call: zen_load_balance of the rank's own gradient and zen_merge of the entries it

@@ -423,3 +423,62 @@ def test_comm_hook_between_four_ranks(zen, method, fused):
         assert out.numel() == n and torch.equal(out != 0, total != 0)
         assert bool(((out.double() - total).abs() <= scale * 1e-6).all())
         assert torch.equal(out, results[0])
+
+
+@pytest.mark.parametrize("fused,headroom", [(True, 1.5), (True, 0.05), (False, 1.5)])
+def test_comm_hook_on_a_bucket_of_training_size(zen, fused, headroom):
+    """The hook between two ranks on a bucket of 64 Mi bf16 elements, the size at which the load balance takes
+    its fast paths (asserted), with the threshold handed to the all-reduce (fused), with far too little room
+    for the selection (the call is declined, falls back, learns the size and starts again), and the reference's
+    way (masked copy first): all three give every rank the same tensor, the sum of the ranks' compressed
+    buckets."""
+    from zen_repro_amd import _lib
+
+    P, n, top_k = 2, 64 << 20, 1
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    grads = [(torch.randn(n, device="cuda", generator=gen) * 1e-3).to(torch.bfloat16) for _ in range(P)]
+    samples = [torch.randint(0, n, ((n + 99) // 100,), device="cuda", generator=gen) for _ in range(P)]
+    L = _lib.lib()
+    m = zen.TensorPartition(P, 1, 3).table_sizes(n)[0]
+    room = int(n * top_k / 100 * 1.5) + 4096
+    assert L.zen_load_balance_path(n, m, _lib.BF16, room, P, 0, _lib.MODE_FAST) >= 2
+    ex = ThreadExchange(P)
+    results, compressed, errors = [None] * P, [None] * P, []
+
+    def run(rank):
+        try:
+            torch.cuda.set_device(0)
+            lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P, rank), None, None)
+            lba.ddp = ex.view(rank)
+            hook = zen.SparseCommHook(lba, top_k=top_k, method=3, tp_group=zen.LocalGroup(1, 0),
+                                      sample_index=lambda numel, r=rank: samples[r], fused=fused, headroom=headroom)
+            hook(None, _StubBucket(grads[rank]))  # the first call is passed through
+            compressed[rank] = zen.compress_with_allgather(top_k, grads[rank], zen.LocalGroup(1, 0),
+                                                           sample_index=samples[rank])
+            results[rank] = hook(None, _StubBucket(grads[rank])).value()
+            torch.cuda.current_stream().synchronize()  # the hook made this stream wait for its own
+        except BaseException as e:  # noqa: BLE001
+            errors.append((rank, repr(e)))
+            ex.barrier.abort()
+
+    threads = [threading.Thread(target=run, args=(r,)) for r in range(P)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=150)
+    assert not errors, errors
+    # two bf16 values per index at most: their fp32 sum rounded once to bf16
+    want = (compressed[0].float() + compressed[1].float()).to(torch.bfloat16)
+    want = torch.where(want == 0, torch.zeros((), dtype=torch.bfloat16, device="cuda"), want)  # no negative zeros
+    for r in range(P):
+        assert results[r].dtype == torch.bfloat16 and results[r].numel() == n
+        assert torch.equal(results[r].view(torch.int16), want.view(torch.int16))
+
+
+def test_comm_hook_needs_a_backend_for_more_than_one_rank(zen):
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(2, 0), None, None)
+    hook = zen.SparseCommHook(lba, top_k=1, method=3, tp_group=zen.LocalGroup(1, 0))
+    grad = torch.zeros(8192, device="cuda")
+    hook(None, _StubBucket(grad))
+    with pytest.raises(RuntimeError):
+        hook(None, _StubBucket(grad))

@@ -248,6 +248,43 @@ def test_topk_threshold(zen, oracle, n, dtype):
         assert count == int((keys >= key).sum())
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("n,s", [(5000, 50), (1 << 20, 10486), (3 * (1 << 20) + 17, 1 << 20), (1 << 16, 1 << 18)])
+def test_sample_threshold(zen, oracle, n, s, dtype):
+    """The threshold over tensor[sample_index] (train.py:78-82) in one call: positions drawn with replacement
+    (more positions than elements in the last case), against the k-th largest key of the gathered sample."""
+    import importlib
+
+    C = importlib.import_module("zen_repro_amd.compress")
+    from zen_repro_amd import _lib
+
+    g = make_grad(oracle, n, 1.0, dtype, seed=n + s)
+    d = to_dev(g)
+    rng = np.random.default_rng(s)
+    at = rng.integers(0, n, s)
+    at[0], at[-1] = 0, n - 1
+    at_dev = torch.from_numpy(at).cuda()
+    keys = (g & 0x7FFF) if dtype == "bf16" else (g.view(np.uint32) & 0x7FFFFFFF)
+    for k in (1, max(1, s // 100), s // 2 + 1, s):
+        thr, status = C.sample_threshold(d, at_dev, k)
+        key, count = (int(x) & 0xFFFFFFFF for x in to_np(thr))
+        assert int(status) == 0
+        assert key == oracle.kth_key(g[at], k), (n, s, dtype, k)
+        assert count == int((keys[at] >= key).sum())
+    # an unaligned view of the tensor, and a position outside it: flagged, counted as a zero
+    thr, status = C.sample_threshold(d[1:], at_dev[: s // 2].clamp(max=n - 2), max(1, s // 200))
+    assert int(status) == 0
+    assert int(to_np(thr)[0]) & 0xFFFFFFFF == oracle.kth_key(g[1:][np.minimum(at[: s // 2], n - 2)], max(1, s // 200))
+    bad = at.copy()
+    bad[s // 3] = n
+    bad[s // 2] = -1
+    thr, status = C.sample_threshold(d, torch.from_numpy(bad).cuda(), max(1, s // 100))
+    assert int(status) == _lib.STAT_BAD_INDEX
+    sample = g[np.clip(bad, 0, n - 1)].copy()
+    sample[[s // 3, s // 2]] = 0
+    assert int(to_np(thr)[0]) & 0xFFFFFFFF == oracle.kth_key(sample, max(1, s // 100))
+
+
 def test_topk_threshold_heavy_ties_and_zeros(zen, oracle):
     n = 1 << 18
     g = np.zeros(n, np.float32)

@@ -75,6 +75,10 @@ def lib():
         "zen_topk_threshold_workspace": (sz, []),
         "zen_topk_threshold": (i32, [vp, i32, i64, i64, vp, vp, sz, vp]),
         "zen_topk_threshold_static": (i32, [vp, i32, i64, i64, vp, vp]),
+        "zen_round_compact_workspace": (sz, [i64]),
+        "zen_round_compact": (i32, [vp, i32, vp, vp, i64, i32, vp, vp, vp, vp, sz, vp, vp]),
+        "zen_sample_threshold_workspace": (sz, [i64, i32]),
+        "zen_sample_threshold": (i32, [vp, i32, i64, vp, i64, i64, vp, vp, sz, vp, vp]),
         "zen_compress": (i32, [vp, i32, i64, vp, vp, vp]),
         "zen_select_workspace": (sz, [i64, i32]),
         "zen_select": (i32, [vp, i32, i64, vp, vp, i32, vp, i64, vp, vp, sz, vp, vp]),

@@ -26,9 +26,10 @@ class LocalGroup:
         return self._rank
 
 
-def _select(tensor, thr, idx64, capacity=None):
-    """Ascending (indices, values, count) of the selected elements of a flat
-    tensor; count is a device int64[1] and may exceed capacity."""
+def _select_raw(tensor, thr, idx64, capacity=None):
+    """(indices, values, count, status bits) of the selected elements of a flat tensor, ascending; the count
+    is that of all elements that pass, also beyond `capacity` (then the bits hold STAT_CAPACITY and the first
+    `capacity` entries are there).  Synchronises."""
     flat = tensor.reshape(-1)
     n = flat.numel()
     dev = flat.device
@@ -46,9 +47,20 @@ def _select(tensor, thr, idx64, capacity=None):
                       _lib.ptr(status), _lib.stream_of(dev))
     _lib.check(rc, "select")
     host = torch.cat([count, status.to(torch.int64)]).tolist()
-    if host[1]:
-        raise RuntimeError("select: " + _lib.describe_status(host[1]))
-    return out_idx[:host[0]], out_val[:host[0]], host[0]
+    kept = min(host[0], capacity)
+    return out_idx[:kept], out_val[:kept], host[0], host[1]
+
+
+def _select(tensor, thr, idx64, capacity=None, grow=False):
+    """Ascending (indices, values, count) of the selected elements of a flat tensor.  With `grow`, a selection
+    that does not fit `capacity` is taken again with room for exactly what passed (the first call counted
+    it); any other trouble raises at once."""
+    idx, val, count, bits = _select_raw(tensor, thr, idx64, capacity)
+    if bits == _lib.STAT_CAPACITY and grow:
+        idx, val, count, bits = _select_raw(tensor, thr, idx64, count)
+    if bits:
+        raise RuntimeError("select: " + _lib.describe_status(bits))
+    return idx, val, count
 
 
 class LoadBalanceAllreduce:
@@ -223,12 +235,48 @@ class LoadBalanceAllreduce:
             m_idx.data_ptr(), 0, m_val.data_ptr(), r, count.data_ptr(),
             _lib.MODE_FAST | self.fast_flags | _lib.MODE_ZEROED, mws.data_ptr(), mws.numel(), m_status.data_ptr(),
             _lib.stream_handle(dev), merge_stream.cuda_stream if merge_stream is not None else None)
+        self.last_encode_merge_args = a  # what the library was called with (its buffers live as long as the results)
         rc = L.zen_encode_merge(ctypes.byref(a))
         if rc != _lib.OK:
             mws[:L.zen_merge_zero_bytes()].zero_()
         _lib.check(rc, "encode_merge")
         partition._after_call(dev, slot, int(k), used)
         return (out_idx, out_val, splits, status), (m_idx, m_val, count, m_status)
+
+    def round_merged_flat(self, indices, sums, count, dtype):
+        """What comm.py:125-127 hands to the second exchange, from merge_sparse_flat's output and without host
+        synchronisation: the fp32 sums rounded once to `dtype`, the entries that round to zero dropped, the rest
+        in their order.  Returns (indices, values, count int64[1], status int32[1])."""
+        _lib.require_gpu(indices, "indices")
+        dev = indices.device
+        L = _lib.lib()
+        cap = indices.numel()
+        out_idx = torch.empty_like(indices)
+        out_val = torch.empty(cap, dtype=dtype, device=dev)
+        kept = _lib.zeros.take(dev, 1, torch.int64)
+        status = _lib.status_word(dev)
+        ws = _lib.scratch.get(dev, "round_compact", L.zen_round_compact_workspace(cap))
+        rc = L.zen_round_compact(_lib.ptr(indices), int(indices.dtype == torch.int64), _lib.ptr(sums), _lib.ptr(count),
+                                 cap, _lib.dtype_code(out_val), _lib.ptr(out_idx), _lib.ptr(out_val), _lib.ptr(kept),
+                                 _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
+        _lib.check(rc, "round_merged")
+        return out_idx, out_val, kept, status
+
+    def merge_rounded(self, indices_tensors, values_tensors, dense_size, dtype):
+        """merge_sparse followed by the rounding of round_merged_flat: (int64 indices, values of `dtype`), with
+        one host synchronisation (the result's size) instead of three."""
+        for mode in self._fast_then_general():
+            idx, val, count, status = self.merge_sparse_flat(indices_tensors, values_tensors, dense_size,
+                                                             idx64=True, mode=mode)
+            r_idx, r_val, kept, r_status = self.round_merged_flat(idx, val, count, dtype)
+            host = torch.cat([kept, status.to(torch.int64), r_status.to(torch.int64)]).tolist()
+            if host[1] & (_lib.STAT_RETRY | _lib.STAT_INTERNAL):
+                self.reset_merge_workspace(idx.device)
+            if not host[1] & _lib.STAT_RETRY:
+                break
+        if host[1] | host[2]:
+            raise RuntimeError("merge_rounded: " + _lib.describe_status(host[1] | host[2]))
+        return r_idx[:host[0]], r_val[:host[0]]
 
     def reset_merge_workspace(self, device, slot=0):
         """After a merge_sparse_flat whose status carried STAT_RETRY or
@@ -422,15 +470,7 @@ class LoadBalanceAllreduce:
                 sparse_indices, sparse_values = self.encode_sparse_tensor(tensor)
             else:
                 _lib.require_gpu(tensor, "input")
-                room = capacity
-                while True:
-                    try:
-                        sparse_indices, sparse_values, _ = _select(tensor, thr, idx64=True, capacity=room)
-                        break
-                    except RuntimeError:
-                        if room is None or room >= numel:
-                            raise
-                        room = min(numel, room * 4)  # more passed the threshold than the estimate allowed for
+                sparse_indices, sparse_values, _ = _select(tensor, thr, idx64=True, capacity=capacity, grow=True)
             indices_tensors = ddp.allgather_padding(sparse_indices)
             values_tensors = ddp.allgather_padding(sparse_values)
             return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
@@ -441,11 +481,7 @@ class LoadBalanceAllreduce:
         values_tensors = ddp.alltoallv(values, gather_splits)
         # decode_sparse_tensors + encode_sparse_tensor (comm.py:125-127) without the dense tensor in between:
         # fp32 sums in payload order, rounded once to the tensor's type, what rounds to zero dropped
-        sparse_indices, sums = self.merge_sparse(indices_tensors, values_tensors, numel)
-        sparse_values = sums.to(tensor.dtype)
-        nonzero = sparse_values != 0
-        if not bool(nonzero.all()):
-            sparse_indices, sparse_values = sparse_indices[nonzero], sparse_values[nonzero]
+        sparse_indices, sparse_values = self.merge_rounded(indices_tensors, values_tensors, numel, tensor.dtype)
         if method == 2:
             indices_tensors = ddp.allgather_padding(sparse_indices)
         else:

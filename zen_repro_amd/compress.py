@@ -24,6 +24,28 @@ def topk_threshold(tensor, k):
     return thr
 
 
+def sample_threshold(tensor, sample_index, k):
+    """(thr, status): thr as topk_threshold returns it for the multiset tensor.reshape(-1)[sample_index] (the
+    sample of train.py:78-80), status int32[1] on the device (STAT_BAD_INDEX: a position outside the tensor).
+    One gather kernel and the radix select, no intermediate tensor, no host sync."""
+    _lib.require_gpu(tensor, "input")
+    _lib.require_gpu(sample_index, "sample_index")
+    flat = tensor.reshape(-1)
+    if sample_index.dtype != torch.int64:
+        raise RuntimeError("sample_index must be int64")
+    L = _lib.lib()
+    dev = flat.device
+    s = sample_index.numel()
+    code = _lib.dtype_code(flat)
+    thr = torch.empty(2, dtype=torch.int32, device=dev)
+    status = _lib.status_word(dev)
+    ws = _lib.scratch.get(dev, "sample_threshold", L.zen_sample_threshold_workspace(s, code))
+    rc = L.zen_sample_threshold(_lib.ptr(flat), code, flat.numel(), _lib.ptr(sample_index.reshape(-1)), s, int(k),
+                                _lib.ptr(thr), _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
+    _lib.check(rc, "sample_threshold")
+    return thr, status
+
+
 def threshold_value(tensor, thr):
     """The threshold as a 0-dim tensor of tensor.dtype (synchronises)."""
     key = int(thr[0].item()) & 0xFFFFFFFF
@@ -55,12 +77,12 @@ def compress(top_k, tensor, sample_index=None):
     flat = tensor.reshape(-1)
     if sample_index is None:
         sample_index = torch.randint(0, numel, (math.ceil(0.01 * numel),), device=tensor.device)
-    sample = flat[sample_index]
-    k = sample.numel() * top_k // 100
+    k = sample_index.numel() * top_k // 100
     if k < 1:
         # torch.min of the empty topk result raises in the reference
         raise RuntimeError("compress: top-k of the sample is empty")
-    thr = topk_threshold(sample, k)
+    # a position outside the tensor counts as a zero and is flagged in the status word (not waited for here)
+    thr, _ = sample_threshold(flat, sample_index, k)
     return mask_below(flat, thr).view_as(tensor)
 
 
@@ -76,15 +98,17 @@ def threshold_with_allgather(top_k, tensor, pg_group, sample_index=None, all_gat
     flat = tensor.reshape(-1)
     if sample_index is None:
         sample_index = torch.randint(0, numel, (math.ceil(0.01 * numel),), device=tensor.device)
-    sample = flat[sample_index]
-    if all_gather is not None:
-        samples = all_gather(sample)
-        if samples.numel() != pg_group.size() * sample.numel():
-            raise RuntimeError("compress_with_allgather: the gathered samples have the wrong size")
-    elif pg_group.size() == 1:
-        samples = sample
-    else:
+    if all_gather is None and pg_group.size() == 1:
+        k = sample_index.numel() * top_k // 100
+        if k < 1:
+            raise RuntimeError("compress_with_allgather: top-k of the samples is empty")
+        return sample_threshold(flat, sample_index, k)[0]  # one rank: its own sample is the whole multiset
+    if all_gather is None:
         raise RuntimeError("compress_with_allgather needs an all_gather callable for more than one rank")
+    sample = flat[sample_index]  # the exchange needs the sample as a tensor of its own
+    samples = all_gather(sample)
+    if samples.numel() != pg_group.size() * sample.numel():
+        raise RuntimeError("compress_with_allgather: the gathered samples have the wrong size")
     k = samples.numel() * top_k // 100
     if k < 1:
         raise RuntimeError("compress_with_allgather: top-k of the samples is empty")

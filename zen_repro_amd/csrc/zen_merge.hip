@@ -681,3 +681,107 @@ int zen_decode_dense(const void *idx, int idx64_in, const void *val, int dtype, 
 }
 
 }  // extern "C"
+
+namespace zen {
+namespace {
+
+// The merged entries on their way to the second exchange (comm.py:125-127 turns the dense fp32 sums into the
+// tensor's type and takes the nonzeros again): every sum is rounded once to the type V, entries whose sum
+// rounds to zero are dropped, the others keep their order.  One pass: a tile of kRcBlock * kRcItems entries per
+// workgroup, the tiles' kept counts chained by look-back.  count sits on the device.
+constexpr int kRcBlock = 256, kRcItems = 8, kRcTile = kRcBlock * kRcItems;
+template <typename I, typename V>
+__global__ __launch_bounds__(kRcBlock) void k_round_compact(const I *__restrict__ idx, const float *__restrict__ sums,
+                                                            const int64_t *__restrict__ count, int64_t capacity,
+                                                            I *__restrict__ out_idx, V *__restrict__ out_val,
+                                                            int64_t *out_count, ScanState st, int32_t *status) {
+  __shared__ uint32_t tile_s;
+  __shared__ uint32_t scan_s[kRcBlock / 64 + 1];
+  __shared__ uint64_t base_s;
+  if (threadIdx.x == 0) tile_s = atomicAdd(st.ticket, 1u);
+  __syncthreads();
+  const uint32_t tile = tile_s;
+  int64_t n = *count;
+  if (n > capacity) n = capacity;
+  const int64_t first = (int64_t)tile * kRcTile + (int64_t)threadIdx.x * kRcItems;
+  I k[kRcItems];
+  V v[kRcItems];
+  uint32_t keep = 0, mine = 0;
+#pragma unroll
+  for (int i = 0; i < kRcItems; ++i) {
+    const int64_t j = first + i;
+    k[i] = 0;
+    v[i] = 0;
+    if (j < n) {
+      k[i] = idx[j];
+      const float f = sums[j];
+      if constexpr (sizeof(V) == 2) {
+        v[i] = f32_to_bf16_rne(f);
+        if (v[i] & 0x7fffu) keep |= 1u << i;
+      } else {
+        v[i] = __float_as_uint(f);
+        if (v[i] & 0x7fffffffu) keep |= 1u << i;
+      }
+    }
+  }
+  mine = __popc(keep);
+  uint32_t total;
+  const uint32_t before = block_exclusive_scan<uint32_t, kRcBlock>(mine, scan_s, &total);
+  const uint64_t base = lookback_exclusive(st, (int)tile, total, status, &base_s);
+  uint64_t at = base + before;
+#pragma unroll
+  for (int i = 0; i < kRcItems; ++i)
+    if (keep & (1u << i)) {
+      out_idx[at] = k[i];
+      out_val[at] = v[i];
+      ++at;
+    }
+  if (tile == gridDim.x - 1 && threadIdx.x == kRcBlock - 1) *out_count = (int64_t)(base + before + mine);
+}
+
+}  // namespace
+}  // namespace zen
+
+extern "C" {
+
+size_t zen_round_compact_workspace(int64_t capacity) {
+  if (capacity < 0) return 0;
+  return zen::scan_words(zen::ceil_div(capacity > 0 ? capacity : 1, (int64_t)zen::kRcTile)) * sizeof(uint64_t);
+}
+
+int zen_round_compact(const void *idx, int idx64, const float *sums, const int64_t *count, int64_t capacity, int dtype,
+                      void *out_idx, void *out_val, int64_t *out_count, void *workspace, size_t workspace_bytes,
+                      int32_t *status, void *stream) {
+  using namespace zen;
+  if (!count || !out_count || !status || capacity < 0) return fail(ZEN_EINVAL, "zen_round_compact: null pointer");
+  if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_round_compact: bad dtype");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (capacity == 0) {
+    launch_fill<int64_t>(out_count, 0, 1, s);
+    ZEN_LAUNCH_CHECK("zen_round_compact: zero count");
+    return ZEN_OK;
+  }
+  if (!idx || !sums || !out_idx || !out_val || !workspace) return fail(ZEN_EINVAL, "zen_round_compact: null pointer");
+  if (workspace_bytes < zen_round_compact_workspace(capacity))
+    return fail(ZEN_EWORKSPACE, "zen_round_compact: workspace too small");
+  const int64_t tiles = ceil_div(capacity, (int64_t)kRcTile);
+  if (tiles > 0x7fffffffll) return fail(ZEN_EINVAL, "zen_round_compact: too many entries");
+  launch_fill<uint64_t>(static_cast<uint64_t *>(workspace), 0ull, scan_words(tiles), s);
+  ZEN_LAUNCH_CHECK("zen_round_compact: clear");
+  const ScanState st = scan_state(workspace, tiles);
+  const dim3 grid((unsigned)tiles), block(kRcBlock);
+#define ZEN_RC(I, V)                                                                                              \
+  k_round_compact<I, V><<<grid, block, 0, s>>>(static_cast<const I *>(idx), sums, count, capacity,              \
+                                               static_cast<I *>(out_idx), static_cast<V *>(out_val), out_count, \
+                                               st, status)
+  if (idx64) {
+    if (dtype == ZEN_BF16) ZEN_RC(int64_t, uint16_t); else ZEN_RC(int64_t, uint32_t);
+  } else {
+    if (dtype == ZEN_BF16) ZEN_RC(int32_t, uint16_t); else ZEN_RC(int32_t, uint32_t);
+  }
+#undef ZEN_RC
+  ZEN_LAUNCH_CHECK("k_round_compact");
+  return ZEN_OK;
+}
+
+}  // extern "C"

@@ -1329,6 +1329,55 @@ __global__ __launch_bounds__(256) void k_stream_read(const u32x4 *__restrict__ i
 }  // namespace
 }  // namespace zen
 
+namespace zen {
+namespace {
+
+// out[j] = in[sample_index[j]] for j < s: the sample compress() draws (train.py:78-80), gathered for the
+// radix select that follows.  Four positions per thread; a position outside [0, n) is flagged and reads as zero.
+constexpr int kGatherBlock = 256, kGatherItems = 4;
+template <typename S>
+__global__ __launch_bounds__(kGatherBlock) void k_sample_gather(const S *__restrict__ in, int64_t n,
+                                                                const int64_t *__restrict__ at, int64_t s,
+                                                                S *__restrict__ out, int32_t *status) {
+  const int64_t base = (int64_t)blockIdx.x * (kGatherBlock * kGatherItems) + threadIdx.x;
+  int64_t pos[kGatherItems];
+  S v[kGatherItems];
+  bool bad = false;
+#pragma unroll
+  for (int i = 0; i < kGatherItems; ++i) {
+    const int64_t j = base + (int64_t)i * kGatherBlock;
+    pos[i] = j < s ? __builtin_nontemporal_load(at + j) : 0;
+    if (pos[i] < 0 || pos[i] >= n) {
+      bad = true;
+      pos[i] = -1;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kGatherItems; ++i) v[i] = pos[i] >= 0 ? in[pos[i]] : S(0);
+#pragma unroll
+  for (int i = 0; i < kGatherItems; ++i) {
+    const int64_t j = base + (int64_t)i * kGatherBlock;
+    if (j < s) out[j] = v[i];
+  }
+  if (bad) atomicOr(status, ZEN_STAT_BAD_INDEX);
+}
+
+size_t sample_gather_bytes(int64_t s, int dtype) { return align_up((size_t)s * (dtype == ZEN_BF16 ? 2 : 4), 256); }
+
+template <typename S>
+int sample_threshold_launch(const S *in, int64_t n, const int64_t *at, int64_t s, int64_t k, uint32_t *thr,
+                            void *workspace, int32_t *status, hipStream_t stream) {
+  S *sample = static_cast<S *>(workspace);
+  void *topk = static_cast<unsigned char *>(workspace) + sample_gather_bytes(s, sizeof(S) == 2 ? ZEN_BF16 : ZEN_F32);
+  const int64_t blocks = ceil_div(s, (int64_t)kGatherBlock * kGatherItems);
+  k_sample_gather<S><<<dim3((unsigned)blocks), dim3(kGatherBlock), 0, stream>>>(in, n, at, s, sample, status);
+  ZEN_LAUNCH_CHECK("k_sample_gather");
+  return topk_launch(sample, s, nullptr, k, thr, topk, nullptr, 0, stream);
+}
+
+}  // namespace
+}  // namespace zen
+
 extern "C" {
 
 int zen_stream_read(const void *input, size_t bytes, uint32_t *sink, void *stream) {
@@ -1370,6 +1419,27 @@ int zen_topk_threshold(const void *input, int dtype, int64_t n, int64_t k, uint3
   if (workspace_bytes < zen_topk_threshold_workspace()) return fail(ZEN_EWORKSPACE, "zen_topk_threshold: workspace too small");
   hipStream_t s = static_cast<hipStream_t>(stream);
   return topk_exact(input, dtype, n, nullptr, k, thr, workspace, nullptr, 0, s);
+}
+
+size_t zen_sample_threshold_workspace(int64_t s, int dtype) {
+  if (s < 0) return 0;
+  return zen::sample_gather_bytes(s, dtype) + zen::topk_scratch_bytes();
+}
+
+int zen_sample_threshold(const void *input, int dtype, int64_t n, const int64_t *sample_index, int64_t s, int64_t k,
+                         uint32_t *thr, void *workspace, size_t workspace_bytes, int32_t *status, void *stream) {
+  using namespace zen;
+  if (!input || !sample_index || !thr || !workspace || !status) return fail(ZEN_EINVAL, "zen_sample_threshold: null pointer");
+  if (dtype != ZEN_F32 && dtype != ZEN_BF16) return fail(ZEN_EINVAL, "zen_sample_threshold: bad dtype");
+  if (n <= 0 || s <= 0 || s > 0x7fffffffll || k < 1 || k > s)
+    return fail(ZEN_EINVAL, "zen_sample_threshold: need n > 0 and 1 <= k <= s < 2^31");
+  if (workspace_bytes < zen_sample_threshold_workspace(s, dtype))
+    return fail(ZEN_EWORKSPACE, "zen_sample_threshold: workspace too small");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t *at = sample_index;
+  if (dtype == ZEN_BF16)
+    return sample_threshold_launch(static_cast<const uint16_t *>(input), n, at, s, k, thr, workspace, status, st);
+  return sample_threshold_launch(static_cast<const uint32_t *>(input), n, at, s, k, thr, workspace, status, st);
 }
 
 int zen_compress(const void *input, int dtype, int64_t n, const uint32_t *thr, void *out, void *stream) {

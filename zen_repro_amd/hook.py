@@ -2,9 +2,18 @@
 (train.py:158-185) as a callable object: same arguments, same return value (a
 completed torch.futures.Future holding the tensor), same steps in the same
 order.  The exchanges belong to the LoadBalanceAllreduce's `ddp` backend, which
-this package does not ship: with a group of one rank (or no backend) the hook
-returns the compressed bucket, as the reference does when dp_group.size() == 1
-(train.py:178)."""
+this package does not ship: with a group of one rank the hook returns the
+compressed bucket, as the reference does when dp_group.size() == 1
+(train.py:178); a larger group without a backend is an error.
+
+Stream order: the reference switches to its side stream and completes the
+future at once (train.py:165-181), leaving it to host time that the gradients
+are written before the hook reads them and that the result is complete before
+it is used.  Here the side stream first waits for the caller's current stream
+(whatever produced the bucket there has finished before the path reads it), and
+the caller's current stream waits for the side stream before the hook returns
+(whatever consumes the future's tensor in that stream's order finds it
+complete).  Neither wait blocks the host."""
 import torch
 
 from .compress import mask_below, threshold_with_allgather
@@ -29,10 +38,15 @@ class SparseCommHook:
                             handed to the all-reduce, which selects while it
                             reads the bucket: same result, two passes over the
                             bucket fewer
+    headroom                fused only: the buffers of the selection are sized for
+                            top_k per cent of the bucket times this factor (the
+                            sampled threshold lets a little more or less than
+                            top_k per cent pass); if more pass, the call repeats
+                            itself with more room
     The first call passes the bucket through untouched (train.py:170-174)."""
 
     def __init__(self, load_balance_allreduce, top_k, method, tp_group, all_gather=None, stream=None,
-                 sample_index=None, fused=True):
+                 sample_index=None, fused=True, headroom=1.5):
         self.lba = load_balance_allreduce
         self.top_k = top_k
         self.method = method
@@ -41,6 +55,7 @@ class SparseCommHook:
         self.stream = stream if stream is not None else torch.cuda.Stream()
         self.sample_index = sample_index  # callable(numel) -> int64 sample positions; None: drawn like the reference
         self.fused = fused
+        self.headroom = headroom
         self.skip = True
 
     def __call__(self, state, bucket):
@@ -50,23 +65,29 @@ class SparseCommHook:
             future.set_result(tensors)
             self.skip = False
             return future
+        exchange = self.lba.process_group.size() > 1
+        if exchange and getattr(self.lba, "ddp", None) is None:
+            raise RuntimeError("SparseCommHook: a group of more than one rank needs a communication backend in "
+                               "load_balance_allreduce.ddp")
+        caller = torch.cuda.current_stream(tensors.device)
+        self.stream.wait_stream(caller)
         with torch.cuda.stream(self.stream):
             index = self.sample_index(tensors.numel()) if self.sample_index is not None else None
             thr = threshold_with_allgather(self.top_k, tensors, self.tp_group, sample_index=index,
                                            all_gather=self.all_gather)
-            exchange = self.lba.process_group.size() > 1 and getattr(self.lba, "ddp", None) is not None
             if thr is None:  # a small bucket: not compressed (train.py:58-59)
                 if exchange:
                     tensors = self.lba.zen_sparse_comm(tensors, self.method)
             elif exchange and self.fused:
                 # about top_k per cent of the bucket pass the sampled threshold; the call grows its buffers if more do
-                room = int(tensors.numel() * self.top_k / 100 * 1.5) + 4096
+                room = int(tensors.numel() * self.top_k / 100 * self.headroom) + 4096
                 tensors = self.lba.zen_sparse_comm(tensors, self.method, thr=thr, capacity=min(room, tensors.numel()))
             else:
                 tensors = mask_below(tensors.reshape(-1), thr).view_as(tensors)
                 if exchange:
                     tensors = self.lba.zen_sparse_comm(tensors, self.method)
-        # like the reference, the future is completed at once: whoever consumes the result does so in the
-        # stream order of `self.stream` (train.py:181)
+        caller.wait_stream(self.stream)
+        # like the reference, the future is completed at once (train.py:181): its tensor is complete in the
+        # order of the caller's stream and of `self.stream`
         future.set_result(tensors)
         return future

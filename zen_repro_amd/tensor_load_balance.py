@@ -91,11 +91,15 @@ class TensorPartition:
         """Room for the selection without guessing `numel` (which would take a
         small selection off the bucket-slab path and size the workspace for the
         whole tensor): from k, from the count the threshold came with, or from
-        a count of the nonzeros.  The last two read a device value."""
+        a count of the nonzeros.  The last two take a pass over the tensor and read a device value."""
         if k > 0:
             return int(k) + int(k) // 4 + 4096  # ties at the threshold
         if thr is not None:
-            return int(thr[1].item()) + 1024
+            # thr[1] counts the multiset the threshold was computed on, which may be a sample of the tensor
+            # (compress): count what passes it in the tensor itself
+            from .comm import _select_raw
+
+            return _select_raw(flat, thr, False, 0)[2] + 1024
         return int(torch.count_nonzero(flat)) + 1024
 
     def _ahead_state(self, device, slot, create=False):
@@ -251,6 +255,8 @@ class TensorPartition:
             _lib.ptr(flat), code, n, m, self.partitions, self.rehash, _lib.ptr(thr), int(k), _lib.ptr(thr_out),
             _lib.ptr(out_idx), _lib.ptr(out_val), capacity, _lib.ptr(splits), _lib.ptr(table), mode | flags,
             _lib.ptr(ws), ws.numel(), _lib.ptr(status), _lib.stream_of(dev))
+        if rc != _lib.OK:
+            table.zero_()  # a call that failed half way may have left entries behind
         _lib.check(rc, "load_balance")
         self._after_call(dev, slot, int(k), used)
         return out_idx, out_val, splits, status
@@ -270,8 +276,9 @@ class TensorPartition:
         if capacity is None:
             capacity = min(n, self._honest_capacity(flat, thr, k))
         fast = _lib.MODE_FAST | self.fast_flags
-        modes = ([fast] + ([_lib.MODE_FAST | _lib.MODE_SLABS] if not fast & _lib.MODE_SLABS else []) +
+        every = ([fast] + ([_lib.MODE_FAST | _lib.MODE_SLABS] if not fast & _lib.MODE_SLABS else []) +
                  [_lib.MODE_GENERAL]) if mode is None else [mode]
+        modes = list(every)
         while modes:
             out_idx, out_val, splits, status = self.load_balance_flat(tensor, thr, capacity, k, modes[0])
             host = torch.cat([splits, status.to(torch.int64)]).tolist()
@@ -283,7 +290,10 @@ class TensorPartition:
             if bits & _lib.STAT_RETRY:
                 modes.pop(0)
             elif bits & _lib.STAT_CAPACITY and grow and capacity < n:
-                capacity = min(n, capacity * 4)  # more ties at the threshold than allowed for
+                # more passed than allowed for (a fast path short of room declines, so this is mostly the general
+                # mode speaking): with more room the fast modes get their turn again
+                capacity = min(n, max(sum(host[:-1]) + 1024, capacity * 4))
+                modes = list(every)
             else:
                 break
         if bits:
