@@ -212,3 +212,21 @@ def test_cpu_baseline_restatement_agrees_with_oracle(oracle):
     assert np.array_equal(m_idx.numpy(), mi)
     assert np.array_equal(m_val.view(torch.int16).numpy().view(np.uint16), mv)
     assert set(times) == {"select", "partition", "merge"}
+
+
+def test_ranges_are_off_by_default_and_cost_nothing():
+    """The named ranges (the reference's nvtx names) are plain null contexts unless switched on."""
+    import contextlib
+
+    from zen_repro_amd import _lib
+
+    was = _lib._ranges_on
+    try:
+        _lib.ranges_enable(False)
+        assert isinstance(_lib.annotate("load_balance"), contextlib.nullcontext)
+        with _lib.annotate("load_balance"), _lib.annotate("decode_sparse_tensors"):
+            pass
+        _lib.ranges_enable(True)
+        assert not isinstance(_lib.annotate("load_balance"), contextlib.nullcontext)
+    finally:
+        _lib.ranges_enable(was)

@@ -298,3 +298,26 @@ def profile_read():
         if cnt.value:
             out[L.zen_profile_name(tag).decode()] = (ms.value, cnt.value)
     return out
+
+
+# ---------------------------------------------------------------- ranges
+# Named ranges around the steps of the path, under the names the reference gives its nvtx ranges (comm.py:66-144,
+# tensor_load_balance.py:25-44, train.py:65-69, 176), so that a rocprofv3 --marker-trace run of a training step
+# reads like an Nsight trace of the reference.  Off unless ZEN_ROCTX=1 is set or ranges_enable(True) is called:
+# the hot calls then pay nothing for them.
+import contextlib
+
+_ranges_on = os.environ.get("ZEN_ROCTX", "") not in ("", "0")
+_no_range = contextlib.nullcontext()
+
+
+def ranges_enable(on=True):
+    global _ranges_on
+    _ranges_on = bool(on)
+
+
+def annotate(name):
+    """Context manager: a roctx range called `name` (torch.cuda.nvtx is roctx on ROCm), or nothing when ranges are off."""
+    if not _ranges_on:
+        return _no_range
+    return torch.cuda.nvtx.range(name)

@@ -465,38 +465,60 @@ class LoadBalanceAllreduce:
         if ddp is None:
             raise RuntimeError("zen_sparse_comm needs a communication backend in self.ddp")
         numel = tensor.numel()
+        ann = _lib.annotate
         if method == 1:
-            if thr is None:
-                sparse_indices, sparse_values = self.encode_sparse_tensor(tensor)
-            else:
-                _lib.require_gpu(tensor, "input")
-                sparse_indices, sparse_values, _ = _select(tensor, thr, idx64=True, capacity=capacity, grow=True)
-            indices_tensors = ddp.allgather_padding(sparse_indices)
-            values_tensors = ddp.allgather_padding(sparse_values)
-            return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
-        indices, values, splits = self.tensor_partition.load_balance(tensor, thr=thr, capacity=capacity,
-                                                                     grow=True if thr is not None else None)
-        gather_splits = ddp.allgather(splits)
-        indices_tensors = ddp.alltoallv(indices, gather_splits)
-        values_tensors = ddp.alltoallv(values, gather_splits)
+            with ann("encode_sparse_tensor"):
+                if thr is None:
+                    sparse_indices, sparse_values = self.encode_sparse_tensor(tensor)
+                else:
+                    _lib.require_gpu(tensor, "input")
+                    sparse_indices, sparse_values, _ = _select(tensor, thr, idx64=True, capacity=capacity, grow=True)
+            with ann("allgatherv indices"):
+                indices_tensors = ddp.allgather_padding(sparse_indices)
+            with ann("allgatherv values"):
+                values_tensors = ddp.allgather_padding(sparse_values)
+            with ann("decode_sparse_tensors"):
+                return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
+        with ann("load_balance"):
+            indices, values, splits = self.tensor_partition.load_balance(tensor, thr=thr, capacity=capacity,
+                                                                         grow=True if thr is not None else None)
+        with ann("allgather"):
+            gather_splits = ddp.allgather(splits)
+        with ann("alltoallv indices"):
+            indices_tensors = ddp.alltoallv(indices, gather_splits)
+        with ann("alltoallv values"):
+            values_tensors = ddp.alltoallv(values, gather_splits)
         # decode_sparse_tensors + encode_sparse_tensor (comm.py:125-127) without the dense tensor in between:
-        # fp32 sums in payload order, rounded once to the tensor's type, what rounds to zero dropped
-        sparse_indices, sparse_values = self.merge_rounded(indices_tensors, values_tensors, numel, tensor.dtype)
+        # fp32 sums in payload order, rounded once to the tensor's type, what rounds to zero dropped (the two
+        # ranges of the reference are one step here and carry both names)
+        with ann("decode_sparse_tensors"), ann("encode_sparse_tensor"):
+            sparse_indices, sparse_values = self.merge_rounded(indices_tensors, values_tensors, numel, tensor.dtype)
         if method == 2:
-            indices_tensors = ddp.allgather_padding(sparse_indices)
+            with ann("allgather indices"):
+                indices_tensors = ddp.allgather_padding(sparse_indices)
         else:
             if numel not in self.mapping:
-                self.mapping[numel] = self.calculate_mapping(numel)
-            bitmap_indices = self.encode_bitmap(sparse_indices, numel)
-            bitmap_indices_gather = ddp.allgather_padding(bitmap_indices)
-            values_tensors = ddp.allgather_padding(sparse_values)
+                with ann("calculate_mapping"):
+                    self.mapping[numel] = self.calculate_mapping(numel)
+            with ann("allgather_bitmap"):
+                with ann("encode_bitmap"):
+                    bitmap_indices = self.encode_bitmap(sparse_indices, numel)
+                with ann("allgatherv"):
+                    bitmap_indices_gather = ddp.allgather_padding(bitmap_indices)
+            with ann("allgather indices"):
+                values_tensors = ddp.allgather_padding(sparse_values)
             if self.partitions <= 64:
                 # decode_bitmap + decode_sparse_tensors (comm.py:140-145) in one pass, without the indices
-                return self.decode_bitmaps_dense(bitmap_indices_gather, values_tensors, numel)
-            indices_tensors = self.decode_bitmap(bitmap_indices_gather, numel)
+                with ann("decode_bitmap"), ann("decode_sparse_tensors"):
+                    return self.decode_bitmaps_dense(bitmap_indices_gather, values_tensors, numel)
+            with ann("decode_bitmap"):
+                indices_tensors = self.decode_bitmap(bitmap_indices_gather, numel)
+            with ann("decode_sparse_tensors"):
+                return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
+        with ann("allgather indices"):
+            values_tensors = ddp.allgather_padding(sparse_values)
+        with ann("decode_sparse_tensors"):
             return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
-        values_tensors = ddp.allgather_padding(sparse_values)
-        return self.decode_sparse_tensors(indices_tensors, values_tensors, numel, ascending=True)
 
 
 def _as_one_buffer(tensors):

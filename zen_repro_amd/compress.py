@@ -122,7 +122,9 @@ def compress_with_allgather(top_k, tensor, pg_group, sample_index=None, all_gath
     the samples of all ranks as one tensor (the reference calls
     dist.all_gather_into_tensor there); this build ships no exchange, so it
     has to be passed in for groups of more than one rank."""
-    thr = threshold_with_allgather(top_k, tensor, pg_group, sample_index, all_gather)
+    with _lib.annotate("topk"), _lib.annotate("min"):  # train.py:65-68: one radix select here
+        thr = threshold_with_allgather(top_k, tensor, pg_group, sample_index, all_gather)
     if thr is None:
         return tensor
-    return mask_below(tensor.reshape(-1), thr).view_as(tensor)
+    with _lib.annotate("where"):  # train.py:69
+        return mask_below(tensor.reshape(-1), thr).view_as(tensor)

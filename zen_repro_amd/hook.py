@@ -16,6 +16,7 @@ the caller's current stream waits for the side stream before the hook returns
 complete).  Neither wait blocks the host."""
 import torch
 
+from ._lib import annotate
 from .compress import mask_below, threshold_with_allgather
 
 
@@ -73,8 +74,9 @@ class SparseCommHook:
         self.stream.wait_stream(caller)
         with torch.cuda.stream(self.stream):
             index = self.sample_index(tensors.numel()) if self.sample_index is not None else None
-            thr = threshold_with_allgather(self.top_k, tensors, self.tp_group, sample_index=index,
-                                           all_gather=self.all_gather)
+            with annotate("compress"):  # train.py:176 (the masked copy, if one is made, comes below)
+                thr = threshold_with_allgather(self.top_k, tensors, self.tp_group, sample_index=index,
+                                               all_gather=self.all_gather)
             if thr is None:  # a small bucket: not compressed (train.py:58-59)
                 if exchange:
                     tensors = self.lba.zen_sparse_comm(tensors, self.method)

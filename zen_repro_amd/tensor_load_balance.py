@@ -35,12 +35,13 @@ class TensorPartition:
     # ------------------------------------------- reference-shaped pieces
     def balance_sparse_tensor(self, tensor):
         """Allocates and fills the two tables (tensor_load_balance.py:13-21)."""
-        memory_size, serial_memory_size = self.table_sizes(tensor.numel())
-        memory = torch.zeros(memory_size, dtype=torch.int32, device=tensor.device)
-        serial_memory = torch.zeros(serial_memory_size, dtype=torch.int32, device=tensor.device)
-        sparse_balance(tensor, memory, serial_memory, self.partitions, rehash=self.rehash)
-        last_status().check()
-        return memory, serial_memory
+        with _lib.annotate("balance_sparse_tensor"):  # tensor_load_balance.py:44
+            memory_size, serial_memory_size = self.table_sizes(tensor.numel())
+            memory = torch.zeros(memory_size, dtype=torch.int32, device=tensor.device)
+            serial_memory = torch.zeros(serial_memory_size, dtype=torch.int32, device=tensor.device)
+            sparse_balance(tensor, memory, serial_memory, self.partitions, rehash=self.rehash)
+            last_status().check()
+            return memory, serial_memory
 
     def get_sub_sparse_tensors(self, tensor, memory):
         """Per-partition nonzero entries of a table and the values they point
