@@ -90,6 +90,9 @@ def parse():
                     help="one library call for the encode and one for the merge instead of one per bucket for both "
                          "(zen_encode_merge); the kernels and streams are the same")
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
+    ap.add_argument("--prepare-on", choices=["own", "main"], default="own",
+                    help="where the next step's sample is taken ahead: on a stream of its own, or on the step's "
+                         "stream right behind the step")
     ap.add_argument("--no-prepare", action="store_true",
                     help="do not take the next step's sample ahead on a stream of its own")
     ap.add_argument("--merge-beside", action="store_true",
@@ -594,7 +597,7 @@ def main():
                 if ms_ is None:
                     merge()  # behind the encode, on its stream
         if prep_stream is not None and more and depth == 1:
-            with torch.cuda.stream(prep_stream):
+            with torch.cuda.stream(es if args.prepare_on == "main" else prep_stream):
                 for j, b in enumerate(buckets):
                     tp.prepare(grad_sets[j][(i + 1) % len(grad_sets[j])], b.k, caps[j], slot=slot)
         if ms_ is not None and not fused:

@@ -15,7 +15,8 @@ constexpr int kRefineBlock = 512;
 // The candidates' histogram resolves the 15 leading bits of an fp32 key: after the select kernel thr[0] is
 // the lowest key of the bin the k-th largest lies in, thr[1] the number of candidates at or above it and
 // *above the number in the bins above.  This kernel histograms the low 16 key bits of the candidates of that
-// bin (they sit in word plane `val_plane` of the coarse slabs or wide buckets; element 0, which is never handed on, is looked at in the tensor), and the
+// bin (they sit in word plane `val_plane` of the coarse slabs, or with val_plane < 0 in the second word of the
+// wide buckets' two-word records; element 0, which is never handed on, is looked at in the tensor), and the
 // workgroup that finishes last replaces thr[0..1] by the exact key and the number of elements at or above it.
 // Grid: any number of workgroups, which take the parts of the coarse slabs in turn.  hist: kRefineBins + 1 zeroed words.
 __global__ __launch_bounds__(kRefineBlock) void k_refine_threshold(CoarseGeom cg, int val_plane,
@@ -34,9 +35,11 @@ __global__ __launch_bounds__(kRefineBlock) void k_refine_threshold(CoarseGeom cg
   for (uint32_t part = blockIdx.x; part < parts; part += gridDim.x) {
     uint32_t count = coarse_cursor[part * kCoarsePad];
     if (count > cg.cap) count = cg.cap;
-    const uint32_t *vals = coarse_words + (size_t)val_plane * plane + (size_t)part * cg.cap;
+    const uint32_t *vals = val_plane < 0 ? coarse_words + (size_t)part * cg.cap * 2 + 1
+                                         : coarse_words + (size_t)val_plane * plane + (size_t)part * cg.cap;
+    const uint32_t stride = val_plane < 0 ? 2u : 1u;
     for (uint32_t e = threadIdx.x; e < count; e += kRefineBlock) {
-      const uint32_t d = (vals[e] & KeyOf<uint32_t>::kMask) - base;
+      const uint32_t d = (vals[e * stride] & KeyOf<uint32_t>::kMask) - base;
       if (d < (uint32_t)kRefineBins) atomicAdd(&hist[d], 1u);
     }
   }

@@ -108,8 +108,8 @@ struct StageArgs {
   uint32_t *coarse_cursor = nullptr;
   uint32_t *coarse_words = nullptr;  // plane 0: indices; plane 1: values in the tensor's type
   bool wide = false;                // the destinations are wide buckets (zen_wide.h): cg.groups of them (at most
-                                    // 256), cg.per = 1, cg.cap entries per part; plane 1 holds the level-1 hash slots,
-                                    // plane 2 the values
+                                    // 256), cg.per = 1, cg.cap entries per part; coarse_words holds records of two
+                                    // words (index, value bits) instead of planes
   uint32_t *ticket = nullptr;       // select_stage_ticket_words() words
   uint32_t *cand_hist = nullptr;
   int64_t pick_k = 0;

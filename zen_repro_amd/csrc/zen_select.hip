@@ -736,7 +736,7 @@ __device__ inline uint32_t pick_elem<uint32_t>(const uint4 (&q)[kSelVecs], int o
 }
 
 // Where the candidates go: the coarse slabs of zen_slab_feed.h (two word planes: index, value), or straight to
-// wide buckets (zen_wide.h; three planes: index, level-1 slot, value).  Either way a destination is kept in
+// wide buckets (zen_wide.h; records of two words: index, value bits).  Either way a destination is kept in
 // kCoarseSplit parts with a cursor each.
 struct StageSlabs {
   SlabGeom geo;
@@ -817,16 +817,23 @@ __device__ inline void stage_flush(uint32_t count, int32_t *st_idx, S *st_val, S
   __syncthreads();
   const uint32_t total = fl.pref[ndst];
   const size_t plane = (size_t)ndst * kCoarseSplit * out.cg.cap;
-  S *val_plane = reinterpret_cast<S *>(out.words + (out.wide ? 2 : 1) * plane);
+  S *val_plane = reinterpret_cast<S *>(out.words + plane);
+  uint2 *records = reinterpret_cast<uint2 *>(out.words);
   for (uint32_t p = threadIdx.x; p < total; p += kSelBlock) {
     const uint32_t g = fl.dst[p];
     const uint32_t at = fl.gbase[g] + (p - fl.pref[g]);
     if (at < out.cg.cap) {
       const size_t o = (size_t)(g * kCoarseSplit + part) * out.cg.cap + at;
       const uint32_t idx = (uint32_t)st_idx[p];
-      out.words[o] = idx;
-      if (out.wide) out.words[plane + o] = out.geo.mod_m(poly(idx) + kSeed1);  // hashed again: cheaper than staging it
-      val_plane[o] = st_val[p];
+      if (out.wide) {
+        // one 8-byte record per candidate: a run of eight fills two 32-byte sectors (three planes of their
+        // own cost three partly filled ones per run, and the scattered stores are what a flush spends its
+        // time on)
+        records[o] = make_uint2(idx, (uint32_t)st_val[p]);
+      } else {
+        out.words[o] = idx;
+        val_plane[o] = st_val[p];
+      }
     } else {
       atomicOr(status, ZEN_STAT_RETRY);  // a slab is full: another path answers
     }

@@ -116,7 +116,7 @@ struct WideTables {
   uint32_t *done;              // [1] workgroups that have finished
   Counters *ctr;               // [P] (the claims of the partition's map)
   // workspace
-  uint32_t *words;             // [3][B * kWideSplit * part_cap] raw candidates: index, level-1 slot, value
+  uint32_t *words;             // [B * kWideSplit * part_cap] raw candidates, two words each: index, value bits
   uint32_t *slab_idx;          // [B * kWideCap] sorted indices (| kRemovedBit: lost level 1)
   uint32_t *sub_index;         // [B * kWideIndexLen] first sorted place of narrow range 4 j, and of 4 j + 4 in the high half
   uint32_t *log_t, *log_cell;  // [P * log_cap] losers; the map cell each ends in (kNone: none)
@@ -272,10 +272,8 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
     longest = 0;
   }
   const uint32_t thr_key = filter ? filter[0] : 0u;
-  const size_t plane = (size_t)B * kWideSplit * tb.part_cap;
-  const uint32_t *idx_plane = tb.words + (size_t)b * kWideSplit * tb.part_cap;
-  const uint32_t *slot_plane = idx_plane + plane;
-  const S *val_plane = reinterpret_cast<const S *>(tb.words + 2 * plane) + (size_t)b * kWideSplit * tb.part_cap;
+  // the bucket's records: (index, value bits), kWideSplit parts of part_cap records
+  const uint2 *records = reinterpret_cast<const uint2 *>(tb.words) + (size_t)b * kWideSplit * tb.part_cap;
   __syncthreads();
   const uint32_t lo = sh.lo;
   const int shift = geo.sub_shift;
@@ -293,9 +291,9 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
       for (int q = 0; q < kWideSplit; ++q) {
         const uint32_t e = tid + (uint32_t)r * kWideBlock;
         const size_t at = (size_t)q * tb.part_cap + (e < pcount[q] ? e : 0u);
-        const uint32_t slot = slot_plane[at];
-        const S v = val_plane[at];
-        const bool keep = e < pcount[q] && (v & KeyOf<S>::kMask) >= thr_key;
+        const uint2 rec = records[at];
+        const uint32_t slot = geo.mod_m(poly(rec.x) + kSeed1);  // the level-1 slot: a dozen instructions, not a plane of its own
+        const bool keep = e < pcount[q] && (rec.y & KeyOf<S>::kMask) >= thr_key;
         off[r * kWideSplit + q] = keep ? slot - lo : kInvalid;
       }
     }
@@ -438,10 +436,10 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
       }
       uint32_t lost = 0;
       if (twins) {
-        const uint32_t mine = idx_plane[raw_at(my & 0x7fffu)];
+        const uint32_t mine = records[raw_at(my & 0x7fffu)].x;
         for (uint32_t u = g0; u < g1; ++u) {
           const uint32_t w = sh.word[u];
-          if ((w >> 15) == key && w != my) lost += idx_plane[raw_at(w & 0x7fffu)] < mine;
+          if ((w >> 15) == key && w != my) lost += records[raw_at(w & 0x7fffu)].x < mine;
         }
       }
       sh.q_word[e] = (g0 + less + lost) | (lost ? kRemovedBit : 0u);  // the entry's thread is its only reader
@@ -474,8 +472,9 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
       for (int q = 0; q < kWideSplit; ++q) {
         const uint32_t e = tid + (uint32_t)r * kWideBlock;
         const size_t at = (size_t)q * tb.part_cap + (rk[r * kWideSplit + q] != kInvalid ? e : 0u);
-        t[q] = idx_plane[at];
-        v[q] = val_plane[at];
+        const uint2 rec = records[at];
+        t[q] = rec.x;
+        v[q] = (S)rec.y;
       }
 #pragma unroll
       for (int q = 0; q < kWideSplit; ++q) {
@@ -828,7 +827,7 @@ WidePlan plan_wide(void *workspace, void *state, const SlabGeom &geo, int partit
   p.cg.per = 1;
   p.cg.cap = p.tb.part_cap;
   p.cg.inv_per = slab_inverse_below(1);
-  p.tb.words = cv.take<uint32_t>((size_t)3 * B * kWideSplit * p.tb.part_cap);
+  p.tb.words = cv.take<uint32_t>((size_t)2 * B * kWideSplit * p.tb.part_cap);
   p.tb.slab_idx = cv.take<uint32_t>(B * kWideCap);
   p.tb.sub_index = cv.take<uint32_t>(B * kWideIndexLen);
   p.tb.log_cap = (uint32_t)(list_cap / 4 / (int64_t)P + 1024);
@@ -915,7 +914,7 @@ int wide_load_balance(const SlabBalanceArgs &a, size_t state_offset, hipStream_t
   if (refine) {
     const uint32_t refine_parts = p.cg.groups * (uint32_t)kCoarseSplit;
     k_refine_threshold<<<dim3(refine_parts < 128u ? refine_parts : 128u), dim3(kRefineBlock), 0, s>>>(
-        p.cg, 2, p.tb.cursor, p.tb.words, static_cast<const uint32_t *>(a.input), p.thr, p.thr + 4, (uint32_t)a.k,
+        p.cg, -1, p.tb.cursor, p.tb.words, static_cast<const uint32_t *>(a.input), p.thr, p.thr + 4, (uint32_t)a.k,
         p.refine_hist, a.thr_out, a.status);
     ZEN_LAUNCH_CHECK("k_refine_threshold");
   }
