@@ -90,9 +90,9 @@ def parse():
                     help="one library call for the encode and one for the merge instead of one per bucket for both "
                          "(zen_encode_merge); the kernels and streams are the same")
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
-    ap.add_argument("--prepare-on", choices=["own", "main"], default="own",
-                    help="where the next step's sample is taken ahead: on a stream of its own, or on the step's "
-                         "stream right behind the step")
+    ap.add_argument("--prepare-on", choices=["own", "main"], default="main",
+                    help="where the next step's sample is taken ahead: on the step's stream right behind the step "
+                         "(no event between the kernels: about 10 us per step less), or on a stream of its own")
     ap.add_argument("--no-prepare", action="store_true",
                     help="do not take the next step's sample ahead on a stream of its own")
     ap.add_argument("--merge-beside", action="store_true",
@@ -405,11 +405,11 @@ def reference_bucket(dev, steps, warmup):
     tp = TensorPartition(P, 1, 3)
     lba = LoadBalanceAllreduce(LocalGroup(P), None, None)
     main = torch.cuda.current_stream(dev)
-    second, beside, ahead = (torch.cuda.Stream(device=dev) for _ in range(3))
+    second, beside = (torch.cuda.Stream(device=dev) for _ in range(2))
 
     def run(count, depth, marks=None):
         outs = []
-        for s_ in (second, beside, ahead):
+        for s_ in (second, beside):
             s_.wait_stream(main)
         for i in range(count):
             es = second if (depth == 2 and i % 2) else main
@@ -417,12 +417,11 @@ def reference_bucket(dev, steps, warmup):
                 outs.append(lba.encode_merge_flat(tp, grads[i % copies], cap, b.k, fi, fv, b.n, slot=i % depth,
                                                   merge_stream=beside if depth == 1 else None))
             if depth == 1 and i + 1 < count:
-                with torch.cuda.stream(ahead):
-                    tp.prepare(grads[(i + 1) % copies], b.k, cap, slot=0)
-            if marks is not None:
+                tp.prepare(grads[(i + 1) % copies], b.k, cap, slot=0)  # behind the step, on its stream
+            if marks is not None and i % (2 * depth) == 2 * depth - 1:
                 marks.append(torch.cuda.Event(enable_timing=True))
                 marks[-1].record(es)
-        for s_ in (second, beside, ahead):
+        for s_ in (second, beside):
             main.wait_stream(s_)
         return outs
 
@@ -441,9 +440,9 @@ def reference_bucket(dev, steps, warmup):
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) * 1e3 / steps
         marks = []
-        run(max(21, min(steps, 60)) + depth, depth, marks)
+        run(2 * depth * 22, depth, marks)
         torch.cuda.synchronize()
-        per = sorted(marks[i].elapsed_time(marks[i + depth]) / depth for i in range(len(marks) - depth))
+        per = sorted(marks[i].elapsed_time(marks[i + 1]) / (2 * depth) for i in range(len(marks) - 1))
         call_us = None
         if depth == 1:
             # what the one call of the library costs the host: the last step's call again, a hundred times, timed
@@ -613,7 +612,9 @@ def main():
             s_.wait_stream(main)  # the inputs were produced on the main stream
         for i in range(count):
             outs.append(step(i, more=i + 1 < count))
-            if marks is not None:  # where the step's encode stream stands once the step is enqueued
+            if marks is not None and i % (2 * depth) == 2 * depth - 1:
+                # where the step's stream stands once the step is enqueued; behind every second step per
+                # stream only: an event between two kernels of a stream holds the second one up for microseconds
                 marks.append(torch.cuda.Event(enable_timing=True))
                 marks[-1].record(enc_streams[i % depth])
         for s_ in side:
@@ -713,12 +714,13 @@ def main():
     device_ms = None
     if not args.graph:
         marks = []
-        run(max(21, min(args.steps, 60)) + depth, marks)
+        run(2 * depth * 22, marks)
         torch.cuda.synchronize()
-        per = sorted(marks[i].elapsed_time(marks[i + depth]) / depth for i in range(len(marks) - depth))
+        per = sorted(marks[i].elapsed_time(marks[i + 1]) / (2 * depth) for i in range(len(marks) - 1))
         device_ms = {"median": round(per[len(per) // 2], 4), "min": round(per[0], 4), "max": round(per[-1], 4),
-                     "steps": len(per),
-                     "what": "time between the ends of consecutive steps' encodes on the device, back to back, untimed pass"}
+                     "samples": len(per), "steps_per_sample": 2 * depth,
+                     "what": "device time per step between events recorded behind every second step of a stream, "
+                             "back to back, in an untimed pass of its own"}
 
     last = outs[-1]
     nnz = [int(enc[2].sum()) for enc, _ in last]

@@ -9,6 +9,26 @@ from . import _lib
 from .functions import last_status, sparse_balance
 
 
+class _Mark:
+    """A point in a stream's order that work on other streams may have to wait for.  The event is recorded
+    only when another stream asks, at the tail the stream has then (further on in its order than the mark:
+    waiting for more is safe, and since every dependency points back in host time no cycle can form), so a
+    sequence of calls that stays on one stream puts no event between its kernels: on the device an event
+    between two kernels of a stream costs about ten microseconds."""
+
+    def __init__(self, stream):
+        self.stream = stream
+        self.event = None
+
+    def wait(self, consumer):
+        if consumer == self.stream:
+            return
+        if self.event is None:
+            self.event = torch.cuda.Event()
+            self.event.record(self.stream)
+        consumer.wait_event(self.event)
+
+
 class TensorPartition:
     """Same constructor and methods as the reference class
     (tensor_load_balance.py:5-51)."""
@@ -104,8 +124,8 @@ class TensorPartition:
         return int(torch.count_nonzero(flat)) + 1024
 
     def _ahead_state(self, device, slot, create=False):
-        # "free": per set of sampling memory, the event after the last call that used it; "pending": samples
-        # taken and not yet picked up by their calls (tensor, size, k, capacity, workspace, set, event, type,
+        # "free": per set of sampling memory, the mark behind the last call that used it; "pending": samples
+        # taken and not yet picked up by their calls (tensor, size, k, capacity, workspace, set, mark, type,
         # workspace bytes)
         key = (_lib.device_index(device), slot)
         state = self._ahead.get(key)
@@ -143,7 +163,7 @@ class TensorPartition:
         which = 1 if 1 not in busy else 0  # the second first: a call that samples for itself prefers the first
         stream = torch.cuda.current_stream(dev)
         if state["free"][which] is not None:
-            stream.wait_event(state["free"][which])  # the call that used this set last has finished
+            state["free"][which].wait(stream)  # the call that used this set last has finished
         nbytes = L.zen_load_balance_workspace(n, m, code, capacity, self.partitions)
         ws = _lib.scratch.get(dev, f"load_balance/{slot}", nbytes)
         table = self._table(dev, m, slot)
@@ -152,9 +172,8 @@ class TensorPartition:
                                         _lib.ptr(ws), ws.numel(),
                                         _lib.stream_of(dev))
         _lib.check(rc, "load_balance prepare")
-        done = torch.cuda.Event()
-        done.record(stream)
-        state["pending"].append((flat.data_ptr(), n, int(k), capacity, ws.data_ptr(), which, done, code, ws.numel()))
+        state["pending"].append((flat.data_ptr(), n, int(k), capacity, ws.data_ptr(), which, _Mark(stream), code,
+                                 ws.numel()))
 
     def _take_ahead(self, flat, n, k, capacity, ws, slot, mode, thr, near):
         """The sample taken ahead for the call that is about to be made, if there is one: (mode flags that tell
@@ -178,7 +197,7 @@ class TensorPartition:
             self._discard(ahead, slot, dev)
             ahead = None
         if ahead is not None:
-            cur.wait_event(ahead[6])
+            ahead[6].wait(cur)
             return _lib.MODE_PREPARED | (_lib.MODE_SECOND if ahead[5] else 0), ahead[5]
         # the call samples for itself, in a set no pending sample sits in (and whose last user has finished)
         busy = {entry[5] for entry in state["pending"]}
@@ -189,14 +208,14 @@ class TensorPartition:
             self._discard(old, slot, dev)
             which = old[5]
         if state["free"][which] is not None:
-            cur.wait_event(state["free"][which])
+            state["free"][which].wait(cur)
         return (_lib.MODE_SECOND if which else 0), which
 
     def _discard(self, entry, slot, dev):
         """Clears the sampling memory of a sample nobody will pick up (with the arguments it was taken with)."""
         L = _lib.lib()
         a_ptr, a_n, a_k, a_cap, a_ws, a_which, a_done, a_code, a_bytes = entry
-        torch.cuda.current_stream(dev).wait_event(a_done)
+        a_done.wait(torch.cuda.current_stream(dev))
         a_m, _ = self.table_sizes(a_n)
         _lib.check(L.zen_load_balance_prepare(
             ctypes.c_void_p(a_ptr), a_code, a_n, a_m, self.partitions, a_k, a_cap,
@@ -208,9 +227,7 @@ class TensorPartition:
         """The set of sampling memory a top-k call used is free again once the call has finished."""
         state = self._ahead_state(dev, slot)
         if k > 0 and state is not None:
-            free = torch.cuda.Event()
-            free.record(torch.cuda.current_stream(dev))
-            state["free"][used] = free
+            state["free"][used] = _Mark(torch.cuda.current_stream(dev))
 
     def load_balance_flat(self, tensor, thr=None, capacity=None, k=0, mode=_lib.MODE_FAST, thr_out=None, slot=0,
                           near=None):
