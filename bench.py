@@ -419,8 +419,12 @@ def reference_bucket(dev, steps, warmup):
             if depth == 1 and i + 1 < count:
                 tp.prepare(grads[(i + 1) % copies], b.k, cap, slot=0)  # behind the step, on its stream
             if marks is not None and i % (2 * depth) == 2 * depth - 1:
-                marks.append(torch.cuda.Event(enable_timing=True))
-                marks[-1].record(es)
+                pair = [torch.cuda.Event(enable_timing=True)]
+                pair[0].record(es)
+                if depth == 1:
+                    pair.append(torch.cuda.Event(enable_timing=True))
+                    pair[1].record(beside)
+                marks.append(pair)
         for s_ in (second, beside):
             main.wait_stream(s_)
         return outs
@@ -440,9 +444,12 @@ def reference_bucket(dev, steps, warmup):
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) * 1e3 / steps
         marks = []
+        ref = torch.cuda.Event(enable_timing=True)
+        ref.record(main)
         run(2 * depth * 22, depth, marks)
         torch.cuda.synchronize()
-        per = sorted(marks[i].elapsed_time(marks[i + 1]) / (2 * depth) for i in range(len(marks) - 1))
+        ends = [max(ref.elapsed_time(e) for e in pair) for pair in marks]
+        per = sorted((ends[i + 1] - ends[i]) / (2 * depth) for i in range(len(ends) - 1))
         call_us = None
         if depth == 1:
             # what the one call of the library costs the host: the last step's call again, a hundred times, timed
@@ -613,10 +620,15 @@ def main():
         for i in range(count):
             outs.append(step(i, more=i + 1 < count))
             if marks is not None and i % (2 * depth) == 2 * depth - 1:
-                # where the step's stream stands once the step is enqueued; behind every second step per
-                # stream only: an event between two kernels of a stream holds the second one up for microseconds
-                marks.append(torch.cuda.Event(enable_timing=True))
-                marks[-1].record(enc_streams[i % depth])
+                # where the step's streams stand once the step is enqueued (the later of the two is the step's
+                # end); behind every second step per stream only: an event between two kernels of a stream holds
+                # the second one up for microseconds
+                pair = [torch.cuda.Event(enable_timing=True)]
+                pair[0].record(enc_streams[i % depth])
+                if mrg_streams[i % depth] is not None:
+                    pair.append(torch.cuda.Event(enable_timing=True))
+                    pair[1].record(mrg_streams[i % depth])
+                marks.append(pair)
         for s_ in side:
             main.wait_stream(s_)
         return outs
@@ -714,13 +726,16 @@ def main():
     device_ms = None
     if not args.graph:
         marks = []
+        ref = torch.cuda.Event(enable_timing=True)
+        ref.record(main)
         run(2 * depth * 22, marks)
         torch.cuda.synchronize()
-        per = sorted(marks[i].elapsed_time(marks[i + 1]) / (2 * depth) for i in range(len(marks) - 1))
+        ends = [max(ref.elapsed_time(e) for e in pair) for pair in marks]
+        per = sorted((ends[i + 1] - ends[i]) / (2 * depth) for i in range(len(ends) - 1))
         device_ms = {"median": round(per[len(per) // 2], 4), "min": round(per[0], 4), "max": round(per[-1], 4),
                      "samples": len(per), "steps_per_sample": 2 * depth,
-                     "what": "device time per step between events recorded behind every second step of a stream, "
-                             "back to back, in an untimed pass of its own"}
+                     "what": "device time per step between events recorded behind every second step on the step's "
+                             "streams (the later one counts), back to back, in an untimed pass of its own"}
 
     last = outs[-1]
     nnz = [int(enc[2].sum()) for enc, _ in last]
