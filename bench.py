@@ -90,9 +90,10 @@ def parse():
                     help="one library call for the encode and one for the merge instead of one per bucket for both "
                          "(zen_encode_merge); the kernels and streams are the same")
     ap.add_argument("--one-stream", action="store_true", help="run encode and merge back to back on one stream")
-    ap.add_argument("--prepare-on", choices=["own", "main"], default="main",
-                    help="where the next step's sample is taken ahead: on the step's stream right behind the step "
-                         "(no event between the kernels: about 10 us per step less), or on a stream of its own")
+    ap.add_argument("--prepare-on", choices=["call", "main", "own"], default="call",
+                    help="how the next step's sample is taken ahead: by the current step's pass over its tensor (no "
+                         "kernel of its own), by a kernel on the step's stream right behind the step, or by one on a "
+                         "stream of its own")
     ap.add_argument("--no-prepare", action="store_true",
                     help="do not take the next step's sample ahead on a stream of its own")
     ap.add_argument("--merge-beside", action="store_true",
@@ -415,9 +416,9 @@ def reference_bucket(dev, steps, warmup):
             es = second if (depth == 2 and i % 2) else main
             with torch.cuda.stream(es):
                 outs.append(lba.encode_merge_flat(tp, grads[i % copies], cap, b.k, fi, fv, b.n, slot=i % depth,
-                                                  merge_stream=beside if depth == 1 else None))
-            if depth == 1 and i + 1 < count:
-                tp.prepare(grads[(i + 1) % copies], b.k, cap, slot=0)  # behind the step, on its stream
+                                                  merge_stream=beside if depth == 1 else None,
+                                                  next_tensor=grads[(i + 1) % copies] if depth == 1 and i + 1 < count
+                                                  else None))
             if marks is not None and i % (2 * depth) == 2 * depth - 1:
                 pair = [torch.cuda.Event(enable_timing=True)]
                 pair[0].record(es)
@@ -586,12 +587,17 @@ def main():
                 mrg.append(lba.merge_sparse_flat(fi, fv, b.n, capacity=fi.numel(), slot=slot))
 
         def both():
+            along = prep_stream is not None and more and depth == 1 and args.prepare_on == "call"
             for j, b in enumerate(buckets):
                 g = grad_sets[j][i % len(grad_sets[j])]
                 fi, fv = flat_sets[j][i % len(flat_sets[j])]
+                # the bucket that follows this one on the slot: the next bucket of the step, or the next step's first
+                nj, ni = (j + 1, i) if j + 1 < len(buckets) else (0, i + 1)
                 e_, m_ = lba.encode_merge_flat(tp, g, caps[j], b.k, fi, fv, b.n, slot=slot,
                                                thr_out=warm_thr[j] if warm else None, near=near_keys[j],
-                                               merge_stream=ms_)
+                                               merge_stream=ms_,
+                                               next_tensor=grad_sets[nj][ni % len(grad_sets[nj])] if along else None,
+                                               next_k=buckets[nj].k)
                 enc.append(e_)
                 mrg.append(m_)
 
@@ -602,8 +608,8 @@ def main():
                 encode()
                 if ms_ is None:
                     merge()  # behind the encode, on its stream
-        if prep_stream is not None and more and depth == 1:
-            with torch.cuda.stream(es if args.prepare_on == "main" else prep_stream):
+        if prep_stream is not None and more and depth == 1 and not (fused and args.prepare_on == "call"):
+            with torch.cuda.stream(prep_stream if args.prepare_on == "own" else es):
                 for j, b in enumerate(buckets):
                     tp.prepare(grad_sets[j][(i + 1) % len(grad_sets[j])], b.k, caps[j], slot=slot)
         if ms_ is not None and not fused:

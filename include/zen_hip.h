@@ -371,7 +371,19 @@ typedef struct zen_encode_merge_args {
   size_t merge_workspace_bytes;
   int32_t *merge_status;
   void *stream, *merge_stream;
+  /* Optional (NULL / 0: none): the gradient of the NEXT call on this table and workspace, of this one's type,
+     n, m, partitions and capacity, and that call's k.  On the fast paths the pass over `input` then also takes
+     the sample that gives the next call's selection its floor (its workgroups do it when they are through with
+     their own tensor: no kernel of its own, nothing that waits), in the set of sampling memory this call does
+     not use.  The next call says so like after zen_load_balance_prepare: ZEN_MODE_PREPARED, with
+     ZEN_MODE_SECOND unless THIS call's mode has ZEN_MODE_SECOND.  zen_encode_merge_samples_next tells whether
+     a call with these sizes does it (the other paths ignore the fields).  next_input must be readable in the
+     order of `stream`. */
+  const void *next_input;
+  int64_t next_k;
 } zen_encode_merge_args;
+int zen_encode_merge_samples_next(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions, int64_t k,
+                                  int mode);
 int zen_encode_merge(const zen_encode_merge_args *args);
 
 /*

@@ -37,6 +37,7 @@ class EncodeMergeArgs(ctypes.Structure):
         ("merged_count", _vp), ("merge_mode", _i32), ("merge_workspace", _vp), ("merge_workspace_bytes", _sz),
         ("merge_status", _vp),
         ("stream", _vp), ("merge_stream", _vp),
+        ("next_input", _vp), ("next_k", _i64),
     ]
 
 
@@ -72,6 +73,7 @@ def lib():
         "zen_bitmap_decode_workspace": (sz, [i64]),
         "zen_bitmap_decode": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, sz, vp, vp]),
         "zen_sparse_balance": (i32, [vp, i32, i64, vp, i64, vp, i64, vp, i32, i32, vp, vp]),
+        "zen_encode_merge_samples_next": (i32, [i64, i64, i32, i64, i32, i64, i32]),
         "zen_topk_threshold_workspace": (sz, []),
         "zen_topk_threshold": (i32, [vp, i32, i64, i64, vp, vp, sz, vp]),
         "zen_topk_threshold_static": (i32, [vp, i32, i64, i64, vp, vp]),

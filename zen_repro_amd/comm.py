@@ -189,13 +189,16 @@ class LoadBalanceAllreduce:
         return out_idx, out_val, count, status
 
     def encode_merge_flat(self, partition, tensor, capacity, k, recv_indices, recv_values, dense_size, slot=0,
-                          thr_out=None, near=None, merge_stream=None):
+                          thr_out=None, near=None, merge_stream=None, next_tensor=None, next_k=None):
         """One bucket's step in one call of the library: partition.load_balance_flat(tensor, None, capacity,
         k=k, slot=slot, thr_out=thr_out, near=near) of the rank's own gradient and merge_sparse_flat(recv_indices,
         recv_values, dense_size, slot=slot) of the entries it received, whose values have the gradient's type.
         Returns the two calls' tuples.  Everything is enqueued on the current stream unless `merge_stream` (a
         torch stream in whose order the received entries are ready) takes the merge.  A sample taken ahead with
-        partition.prepare() is picked up as load_balance_flat would."""
+        partition.prepare() is picked up as load_balance_flat would.  `next_tensor` (ready in the current stream's
+        order) is the gradient of the call that follows on this slot, `next_k` its k (default: this call's): if
+        it has this tensor's size and type, the pass over this tensor takes the sample of that call along (no
+        kernel of its own), as if partition.prepare(next_tensor, next_k, capacity, slot) had been called."""
         from .tensor_load_balance import TensorPartition  # noqa: F401 (the type of `partition`)
 
         _lib.require_gpu(tensor, "input")
@@ -227,6 +230,9 @@ class LoadBalanceAllreduce:
         thr = None
         if near is not None and k > 0:
             thr, flags = near, flags | _lib.MODE_FLOOR
+        if next_k is None:
+            next_k = k
+        nxt = partition._next_sample(flat, next_tensor, int(next_k), capacity, ws, slot, mode | flags, used)
         a = _lib.EncodeMergeArgs(
             flat.data_ptr(), code, n, m, P, partition.rehash, thr.data_ptr() if thr is not None else None, int(k),
             thr_out.data_ptr() if thr_out is not None else None, out_idx.data_ptr(), out_val.data_ptr(), capacity,
@@ -234,13 +240,16 @@ class LoadBalanceAllreduce:
             indices.data_ptr(), int(indices.dtype == torch.int64), values.data_ptr(), r, dense_size,
             m_idx.data_ptr(), 0, m_val.data_ptr(), r, count.data_ptr(),
             _lib.MODE_FAST | self.fast_flags | _lib.MODE_ZEROED, mws.data_ptr(), mws.numel(), m_status.data_ptr(),
-            _lib.stream_handle(dev), merge_stream.cuda_stream if merge_stream is not None else None)
+            _lib.stream_handle(dev), merge_stream.cuda_stream if merge_stream is not None else None,
+            nxt.data_ptr() if nxt is not None else None, int(next_k) if nxt is not None else 0)
         self.last_encode_merge_args = a  # what the library was called with (its buffers live as long as the results)
         rc = L.zen_encode_merge(ctypes.byref(a))
         if rc != _lib.OK:
             mws[:L.zen_merge_zero_bytes()].zero_()
         _lib.check(rc, "encode_merge")
         partition._after_call(dev, slot, int(k), used)
+        if nxt is not None:
+            partition._sample_taken(nxt, int(next_k), capacity, ws, slot, 1 - used)
         return (out_idx, out_val, splits, status), (m_idx, m_val, count, m_status)
 
     def round_merged_flat(self, indices, sums, count, dtype):

@@ -432,10 +432,15 @@ int zen_load_balance_prepare(const void *input, int dtype, int64_t n, int64_t m,
   return slab_prepare(sa, static_cast<hipStream_t>(stream));
 }
 
-int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
-                     const uint32_t *thr, int64_t k, uint32_t *thr_out, int32_t *out_idx, void *out_val,
-                     int64_t capacity, int64_t *splits, int32_t *table, int mode, void *workspace,
-                     size_t workspace_bytes, int32_t *status, void *stream) {
+}  // extern "C"
+
+namespace {
+
+// zen_load_balance, and for zen_encode_merge the same with the next call's tensor handed along.
+int load_balance_call(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
+                      const uint32_t *thr, int64_t k, uint32_t *thr_out, int32_t *out_idx, void *out_val,
+                      int64_t capacity, int64_t *splits, int32_t *table, int mode, void *workspace,
+                      size_t workspace_bytes, int32_t *status, void *stream, const void *next_input, int64_t next_k) {
   using namespace zen;
   const int prepared = (mode & ZEN_MODE_PREPARED) ? ((mode & ZEN_MODE_SECOND) ? 2 : 1) : 0;
   const bool second_set = (mode & ZEN_MODE_SECOND) != 0;
@@ -490,6 +495,8 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
     sa.prepared = near_key ? 0 : prepared;
     sa.second = second_set;
     sa.near_key = near_key;
+    sa.next_input = next_input;
+    sa.next_k = next_k;
     if (wide) return wide_load_balance(sa, slab_state_offset(sa.hash_log2), s);
     return slab_load_balance(sa, s);
   }
@@ -584,12 +591,30 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
   return ZEN_OK;
 }
 
+}  // namespace
+
+extern "C" {
+
+int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
+                     const uint32_t *thr, int64_t k, uint32_t *thr_out, int32_t *out_idx, void *out_val,
+                     int64_t capacity, int64_t *splits, int32_t *table, int mode, void *workspace,
+                     size_t workspace_bytes, int32_t *status, void *stream) {
+  return load_balance_call(input, dtype, n, m, partitions, rehash, thr, k, thr_out, out_idx, out_val, capacity, splits,
+                           table, mode, workspace, workspace_bytes, status, stream, nullptr, 0);
+}
+
+int zen_encode_merge_samples_next(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions, int64_t k,
+                                  int mode) {
+  const int path = zen_load_balance_path(n, m, dtype, capacity, partitions, k, mode);
+  return path == 2 || path == 3;
+}
+
 int zen_encode_merge(const zen_encode_merge_args *a) {
   using namespace zen;
   if (!a) return fail(ZEN_EINVAL, "zen_encode_merge: null pointer");
-  const int rc = zen_load_balance(a->input, a->dtype, a->n, a->m, a->partitions, a->rehash, a->thr, a->k, a->thr_out,
-                                  a->out_idx, a->out_val, a->capacity, a->splits, a->table, a->mode, a->workspace,
-                                  a->workspace_bytes, a->status, a->stream);
+  const int rc = load_balance_call(a->input, a->dtype, a->n, a->m, a->partitions, a->rehash, a->thr, a->k, a->thr_out,
+                                   a->out_idx, a->out_val, a->capacity, a->splits, a->table, a->mode, a->workspace,
+                                   a->workspace_bytes, a->status, a->stream, a->next_input, a->next_k);
   if (rc != ZEN_OK) return rc;
   return zen_merge(a->recv_idx, a->recv_idx64, a->recv_val, a->dtype, a->r, a->dense_n, a->merged_idx, a->merged_idx64,
                    a->merged_val, a->merged_capacity, a->merged_count, a->merge_mode, a->merge_workspace,

@@ -97,6 +97,17 @@ constexpr int kCandHistWords = kCandRows * kCandBins + 1;
 // cand_hist / pick_k / pick_thr the k-th largest key is read off the candidates' histogram (element 0
 // included) as in SelectArgs (and copied to thr_copy if that is not null): exactly for bf16, for fp32 the
 // lowest key of its bin of 65536 keys.
+// What the selecting kernel needs to take the next call's sample (see StageArgs::next_in).
+struct StageSample {
+  const void *in = nullptr;
+  int64_t n = 0;
+  uint32_t *hist = nullptr;
+  uint32_t rank = 0;
+  int block_log2 = 0;
+  int64_t nblocks = 0;
+  uint32_t *floor_out = nullptr;
+};
+
 struct StageArgs {
   const void *in = nullptr;
   int dtype = ZEN_F32;
@@ -118,6 +129,13 @@ struct StageArgs {
   uint32_t *thr_copy = nullptr;
   uint32_t *clear = nullptr;        // optional: clear_words words the kernel sets to zero (memory of an earlier
   uint32_t clear_words = 0;         // kernel that nobody needs any more)
+  // The sample of the NEXT call on the same table and workspace (a tensor of this one's size and type, next_k
+  // its k) is taken by this kernel's workgroups when they are through with their own tensor: next_hist = that
+  // call's sampling memory (zero, left as k_sample_hist leaves it), next_floor receives its floor key.
+  const void *next_in = nullptr;
+  int64_t next_k = 0;
+  uint32_t *next_hist = nullptr;
+  uint32_t *next_floor = nullptr;
   int32_t *status = nullptr;
 };
 int select_stage_slabs(const StageArgs &a, hipStream_t stream);

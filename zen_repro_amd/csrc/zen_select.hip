@@ -18,6 +18,30 @@ constexpr int kHistBlock = 256;
 constexpr int kSampleLog2Min = 6, kSampleLog2Max = 10;  // the sample is one 16-byte vector in 64 ... 1024
 constexpr int64_t kSampleHits = 7000;  // sample elements wanted at or above the threshold
 
+// How thin the sample is (one vector of V elements in 2^log2) and the rank looked for in it.
+struct SamplePlan {
+  int log2;
+  int64_t nblocks;
+  uint32_t rank;
+};
+inline SamplePlan sample_plan(int64_t n, int64_t k, int V) {
+  SamplePlan sp;
+  const int64_t nvec = ceil_div(n, V);
+  // The sample is as thin as leaves about kSampleHits of its elements above the threshold (their count then
+  // scatters by 1.2 %, and the six deviations allowed for below cost 7 % more candidates): a thicker one
+  // lengthens the load and histogram phases and buys nothing.
+  sp.log2 = kSampleLog2Max;
+  while (sp.log2 > kSampleLog2Min && (k >> sp.log2) < kSampleHits) --sp.log2;
+  sp.nblocks = ceil_div(nvec, 1ll << sp.log2);
+  // rank to look for in the sample: the expected one plus six standard
+  // deviations of a binomial count, so that the full tensor almost surely holds
+  // at least k elements at or above the bin found (callers verify and retry)
+  const double expect = (double)k * ((double)sp.nblocks * V) / (double)n;
+  const double want = expect + 6.0 * sqrt(expect) + 16.0;
+  sp.rank = want > 4.0e9 ? 0xffffffffu : (uint32_t)want;
+  return sp;
+}
+
 struct TopkState {
   uint32_t prefix;    // key bits fixed so far (right aligned)
   uint32_t k_rem;     // rank still to find among elements matching the prefix
@@ -143,22 +167,28 @@ __device__ inline uint32_t fine_place(uint32_t bin) { return ((bin & 63u) << 9) 
 // Walks down from the highest populated bin (hist[kFineBins + 1]) in windows of one bin per thread, with
 // consecutive lanes on consecutive words (one workgroup fetching 32768 scattered words past the caches would
 // take tens of microseconds), until `rank` sample elements lie at or above a bin.
+template <int BLOCK>
 __device__ inline void sample_pick_block(const uint32_t *hist, uint32_t rank, int key_shift, uint32_t *floor_out,
                                          uint32_t *smem) {
   int base = (int)load_fresh(&hist[kFineBins + 1]);
   if (base > kFineBins - 1) base = kFineBins - 1;
   uint32_t cum = 0;
-  for (;; base -= kSampleBlock) {
+  for (;; base -= BLOCK) {
     const int bin = base - (int)threadIdx.x;
     const uint32_t c = bin >= 0 ? load_fresh(&hist[fine_place((uint32_t)bin)]) : 0u;
     uint32_t total;
-    const uint32_t above = cum + block_exclusive_scan<uint32_t, kSampleBlock>(c, smem, &total);
+    const uint32_t above = cum + block_exclusive_scan<uint32_t, BLOCK>(c, smem, &total);
     if (above < rank && rank <= above + c) floor_out[0] = (uint32_t)bin << key_shift;
     cum += total;
     if (cum >= rank) return;
-    if (base < kSampleBlock) break;
+    if (base < BLOCK) break;
   }
   if (threadIdx.x == 0) floor_out[0] = 0;  // the sample is too small
+}
+
+// The sample: vector number sample_vec(b) for b = 0 .. nblocks - 1, one out of every 2^block_log2.
+__device__ inline int64_t sample_vec(int64_t b, int block_log2) {
+  return (b << block_log2) + (poly((uint32_t)b) >> 7 & ((1u << block_log2) - 1u));
 }
 
 template <typename S, bool ALIGNED>
@@ -178,7 +208,7 @@ __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restric
   const int64_t nblocks = (nvec + (1ll << block_log2) - 1) >> block_log2;
   for (int64_t b = blockIdx.x * (int64_t)kSampleBlock + threadIdx.x; b < nblocks;
        b += (int64_t)gridDim.x * kSampleBlock) {
-    const int64_t v = (b << block_log2) + (poly((uint32_t)b) >> 7 & ((1u << block_log2) - 1u));
+    const int64_t v = sample_vec(b, block_log2);
     if (v >= nvec) continue;
     S e[V];
     const int live = load_vec<S, ALIGNED>(in, v * V, n, e);
@@ -240,7 +270,7 @@ __global__ __launch_bounds__(kSampleBlock) void k_sample_hist(const S *__restric
   if (threadIdx.x == 0) s_last = atomicAdd(&hist[kFineBins], 1u) == gridDim.x - 1;
   __syncthreads();
   if (!s_last) return;
-  sample_pick_block(hist, rank, kShift, floor_out, smem);
+  sample_pick_block<kSampleBlock>(hist, rank, kShift, floor_out, smem);
 }
 
 // Run by one whole block (BLOCK threads) over the complete candidate
@@ -858,11 +888,122 @@ struct StageSched {
   uint32_t ticket_tiles; // tiles of kStageSmall sub-tiles after that
 };
 
+// LDS of a selecting workgroup that changes hands: the stage with what a flush needs, and after the last
+// flush the window of the next call's sample (16-bit counters, two to a word, a pad word per 32).
+constexpr int kSampleWindow = 8192;  // bins below a workgroup's largest sample element that it counts
+template <typename S>
+struct StageRun {
+  union {
+    struct {
+      int32_t idx[kScatStage];
+      S val[kScatStage];
+      StageFlushShared flush;
+    } run;
+    uint32_t window[kSampleWindow / 2 + kSampleWindow / 64];
+  };
+};
+static_assert(sizeof(StageRun<uint16_t>) == sizeof(int32_t) * kScatStage + 2 * kScatStage + sizeof(StageFlushShared),
+              "the window fits where the stage is");
+
+// The sample of the NEXT call's tensor, taken by the workgroups of this call's selecting kernel when they are
+// through with their own tensor: no launch of its own, and nothing that waits.  Every workgroup histograms its
+// share of the sample (the vectors k_sample_hist would read) in a window of kSampleWindow exact bins below
+// its own largest element (a factor 2^64 in magnitude; what lies further down cannot matter unless the
+// workgroup's largest element towers that far above the threshold, and leaving it out only lowers the floor)
+// and adds the top of it to the device-wide histogram; the workgroup that finishes last reads the floor off
+// the complete histogram, as k_sample_hist's last workgroup does.  The histogram is left as k_sample_hist
+// leaves it: the call that picks the sample up clears it.
+template <typename S>
+__device__ inline void stage_sample_next(const StageSample &smp, uint32_t *window, uint32_t *smem) {
+  constexpr int V = VecOf<S>::kN;
+  constexpr int kShift = KeyOf<S>::kBits - 15;
+  constexpr int kWords = kSampleWindow / 2 / kSelBlock;  // window words per thread (16)
+  __shared__ uint32_t s_top;
+  __shared__ bool s_last;
+  const S *in = static_cast<const S *>(smp.in);
+  const int64_t n = smp.n;
+  const int64_t nvec = (n + V - 1) / V;
+  const int64_t first = (int64_t)blockIdx.x * kSelBlock + threadIdx.x, step = (int64_t)gridDim.x * kSelBlock;
+  if (threadIdx.x == 0) s_top = 0;
+  for (int i = threadIdx.x; i < kSampleWindow / 2 + kSampleWindow / 64; i += kSelBlock) window[i] = 0;
+  __syncthreads();
+  uint32_t top = 0;
+  for (int64_t b = first; b < smp.nblocks; b += step) {
+    const int64_t v = sample_vec(b, smp.block_log2);
+    if (v >= nvec) continue;
+    S e[V];
+    const int live = load_vec<S, false>(in, v * V, n, e);
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+      if (i < live) {
+        const uint32_t bin = (e[i] & KeyOf<S>::kMask) >> kShift;
+        top = bin > top ? bin : top;
+      }
+  }
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) {
+    const uint32_t o = __shfl_xor(top, d, 64);
+    top = o > top ? o : top;
+  }
+  if ((threadIdx.x & 63) == 0 && top) atomicMax(&s_top, top);
+  __syncthreads();
+  const uint32_t hi_bin = s_top;
+  const uint32_t lo_bin = hi_bin >= (uint32_t)kSampleWindow - 1u ? hi_bin - ((uint32_t)kSampleWindow - 1u) : 0u;
+  for (int64_t b = first; b < smp.nblocks; b += step) {  // the same vectors again (they are in the caches now)
+    const int64_t v = sample_vec(b, smp.block_log2);
+    if (v >= nvec) continue;
+    S e[V];
+    const int live = load_vec<S, false>(in, v * V, n, e);
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+      if (i < live) {
+        const uint32_t bin = (e[i] & KeyOf<S>::kMask) >> kShift;
+        if (bin >= lo_bin) {
+          const uint32_t w = bin - lo_bin;
+          atomicAdd(&window[(w >> 1) + (w >> 6)], 1u << (16 * (w & 1u)));
+        }
+      }
+  }
+  __syncthreads();
+  {
+    // from the top down, until the workgroup has added a few times its share of the rank (see k_sample_hist)
+    const uint64_t lim64 = 4ull * smp.rank / gridDim.x + 256ull;
+    const uint32_t limit = lim64 > 0xffffffffull ? 0xffffffffu : (uint32_t)lim64;
+    uint32_t c[kWords];
+    uint32_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < kWords; ++j) {
+      const int w = kSampleWindow / 2 - 1 - (threadIdx.x * kWords + j);
+      c[j] = window[w + (w >> 5)];
+      mine += (c[j] & 0xffffu) + (c[j] >> 16);
+    }
+    uint32_t total;
+    uint32_t above = block_exclusive_scan<uint32_t, kSelBlock>(mine, smem, &total);
+    if (threadIdx.x == 0 && total) atomicMax(&smp.hist[kFineBins + 1], hi_bin);
+#pragma unroll
+    for (int j = 0; j < kWords; ++j) {
+      const int w = kSampleWindow / 2 - 1 - (threadIdx.x * kWords + j);
+      const uint32_t hi = c[j] >> 16, lo = c[j] & 0xffffu;
+      if (hi && above < limit) atomicAdd(&smp.hist[fine_place(lo_bin + 2 * w + 1)], hi);
+      above += hi;
+      if (lo && above < limit) atomicAdd(&smp.hist[fine_place(lo_bin + 2 * w)], lo);
+      above += lo;
+    }
+  }
+  // the adds are carried out before the workgroup counts itself as finished (see k_sample_hist)
+  wait_global_acks();
+  __syncthreads();
+  if (threadIdx.x == 0) s_last = atomicAdd(&smp.hist[kFineBins], 1u) == gridDim.x - 1;
+  __syncthreads();
+  if (s_last) sample_pick_block<kSelBlock>(smp.hist, smp.rank, kShift, smp.floor_out, smem);
+}
+
 template <typename S, bool ALIGNED>
 __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
     const S *__restrict__ in, int64_t n, const uint32_t *__restrict__ thr, StageSlabs out, uint32_t *ticket,
     StageSched sch, uint32_t *cand_hist, uint32_t pick_k, uint32_t *pick_thr, uint32_t *pick_above,
-    uint32_t *thr_copy, uint32_t *clear, uint32_t clear_words, uint32_t floor_margin, int32_t *status) {
+    uint32_t *thr_copy, uint32_t *clear, uint32_t clear_words, uint32_t floor_margin, StageSample next,
+    int32_t *status) {
   constexpr int V = VecOf<S>::kN;
   constexpr int kSub = kSelBlock * kSelVecs * V;
   constexpr int kWaves = kSelBlock / 64;
@@ -871,9 +1012,11 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
   for (uint32_t i = blockIdx.x * kSelBlock + threadIdx.x; i < clear_words; i += gridDim.x * kSelBlock) clear[i] = 0;
   __shared__ uint32_t s_wave[2][kWaves];
   __shared__ uint32_t s_next[2];
-  __shared__ int32_t st_idx[kScatStage];
-  __shared__ S st_val[kScatStage];
-  __shared__ StageFlushShared s_flush;
+  // the stage and what a flush needs; after the last flush, the window of the next call's sample
+  __shared__ StageRun<S> s_run;
+  int32_t (&st_idx)[kScatStage] = s_run.run.idx;
+  S (&st_val)[kScatStage] = s_run.run.val;
+  StageFlushShared &s_flush = s_run.run.flush;
   __shared__ uint32_t s_tail;
   __shared__ uint32_t s_pick[kSelBlock / 64 + 1];
   __shared__ uint32_t s_hist[kCandBins];
@@ -1072,6 +1215,10 @@ __global__ __launch_bounds__(kSelBlock, 3) void k_select_stage(
     const uint32_t c = s_tail;
     if (c) stage_flush<S>(c, st_idx, st_val, s_flush, hist, floor_key, out, status);
   }
+  if (next.hist) {
+    __syncthreads();  // the stage is no longer needed
+    stage_sample_next<S>(next, s_run.window, s_pick);
+  }
   if (hist) {
     __syncthreads();
     uint32_t *row = cand_hist + (size_t)(blockIdx.x % kCandRows) * kCandBins;
@@ -1135,15 +1282,26 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   const S *in = static_cast<const S *>(a.in);
   const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15u) == 0 && a.n >= V;
   const StageSlabs out{a.geo, a.cg, a.coarse_cursor, a.coarse_words, a.wide ? 1u : 0u};
+  StageSample next;
+  if (a.next_in && a.next_hist && a.next_k > 0) {
+    const SamplePlan sp = sample_plan(a.n, a.next_k, V);  // the next tensor has this one's size and type
+    next.in = a.next_in;
+    next.n = a.n;
+    next.hist = a.next_hist;
+    next.rank = sp.rank;
+    next.block_log2 = sp.log2;
+    next.nblocks = sp.nblocks;
+    next.floor_out = a.next_floor;
+  }
   ProfScope prof(kProfSelectStage, stream);
   if (aligned)
     k_select_stage<S, true><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
         in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.pick_above, a.thr_copy,
-        a.clear, a.clear_words, a.floor_margin, a.status);
+        a.clear, a.clear_words, a.floor_margin, next, a.status);
   else
     k_select_stage<S, false><<<dim3((unsigned)blocks), dim3(kSelBlock), 0, stream>>>(
         in, a.n, a.thr, out, a.ticket, sch, a.cand_hist, (uint32_t)a.pick_k, a.pick_thr, a.pick_above, a.thr_copy,
-        a.clear, a.clear_words, a.floor_margin, a.status);
+        a.clear, a.clear_words, a.floor_margin, next, a.status);
   ZEN_LAUNCH_CHECK("k_select_stage");
   return ZEN_OK;
 }
@@ -1200,19 +1358,10 @@ int sample_launch(const S *in, int64_t n, int64_t k, uint32_t *thr_lo, void *wor
                   bool is_zero) {
   constexpr int V = VecOf<S>::kN;
   uint32_t *hist = static_cast<uint32_t *>(workspace);
-  const int64_t nvec = ceil_div(n, V);
-  // The sample is as thin as leaves about kSampleHits of its elements above the threshold (their count then
-  // scatters by 1.2 %, and the six deviations allowed for below cost 7 % more candidates): a thicker one
-  // lengthens the kernel's load and histogram phases and buys nothing.
-  int sample_log2 = kSampleLog2Max;
-  while (sample_log2 > kSampleLog2Min && (k >> sample_log2) < kSampleHits) --sample_log2;
-  const int64_t nblocks = ceil_div(nvec, 1ll << sample_log2);
-  // rank to look for in the sample: the expected one plus six standard
-  // deviations of a binomial count, so that the full tensor almost surely holds
-  // at least k elements at or above the bin found (callers verify and retry)
-  const double expect = (double)k * ((double)nblocks * V) / (double)n;
-  const double want = expect + 6.0 * sqrt(expect) + 16.0;
-  const uint32_t rank = want > 4.0e9 ? 0xffffffffu : (uint32_t)want;
+  const SamplePlan sp = sample_plan(n, k, V);
+  const int sample_log2 = sp.log2;
+  const int64_t nblocks = sp.nblocks;
+  const uint32_t rank = sp.rank;
   if (!is_zero) {
     launch_fill<uint32_t>(hist, 0u, kFineBins + 2, stream);
     ZEN_LAUNCH_CHECK("sample: clear histogram");

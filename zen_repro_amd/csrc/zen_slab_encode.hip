@@ -817,6 +817,12 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
     sc.clear = p.sample_hist[set];  // the sample kernel is through with its histogram
     sc.clear_words = (uint32_t)(sampled_floor_zero_bytes() / sizeof(uint32_t));
   }
+  if (a.next_input && a.next_k > 0) {
+    sc.next_in = a.next_input;
+    sc.next_k = a.next_k;
+    sc.next_hist = p.sample_hist[1 - set];
+    sc.next_floor = p.thr + 2 + 4 * (1 - set);
+  }
   if ((rc = select_stage_slabs(sc, s)) != ZEN_OK) return rc;
   if (refine) {
     const uint32_t refine_parts = p.cg.groups * (uint32_t)kCoarseSplit;

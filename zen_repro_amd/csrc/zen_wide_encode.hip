@@ -908,6 +908,12 @@ int wide_load_balance(const SlabBalanceArgs &a, size_t state_offset, hipStream_t
     sc.clear = p.sample_hist[set];
     sc.clear_words = (uint32_t)(sampled_floor_zero_bytes() / sizeof(uint32_t));
   }
+  if (a.next_input && a.next_k > 0) {
+    sc.next_in = a.next_input;
+    sc.next_k = a.next_k;
+    sc.next_hist = p.sample_hist[1 - set];
+    sc.next_floor = p.thr + 2 + 4 * (1 - set);
+  }
   if ((rc = select_stage_slabs(sc, s)) != ZEN_OK) return rc;
   uint32_t *clear = p.cand_hist;  // the candidates' histogram and the select kernel's tickets lie side by side
   uint32_t clear_words = (uint32_t)(reinterpret_cast<char *>(p.tb.cursor) - reinterpret_cast<char *>(p.cand_hist)) / 4u;

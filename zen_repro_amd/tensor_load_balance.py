@@ -175,6 +175,34 @@ class TensorPartition:
         state["pending"].append((flat.data_ptr(), n, int(k), capacity, ws.data_ptr(), which, _Mark(stream), code,
                                  ws.numel()))
 
+    def _next_sample(self, flat, next_tensor, next_k, capacity, ws, slot, mode, used):
+        """The flat view of `next_tensor` if the call that is about to be made can take that tensor's sample
+        along (same size and type, a path that samples, the other set of sampling memory free), else None."""
+        if next_tensor is None or next_k <= 0:
+            return None
+        nxt = next_tensor.reshape(-1)
+        if (nxt.numel() != flat.numel() or nxt.dtype != flat.dtype or nxt.device != flat.device
+                or not nxt.is_contiguous() or (mode & 0xff) != _lib.MODE_FAST):
+            return None
+        n = flat.numel()
+        m, _ = self.table_sizes(n)
+        if not _lib.lib().zen_encode_merge_samples_next(n, m, _lib.dtype_code(flat), capacity, self.partitions, next_k,
+                                                        mode & (0xff | _lib.MODE_SLABS)):
+            return None
+        state = self._ahead_state(flat.device, slot, create=True)
+        if any(entry[5] == 1 - used for entry in state["pending"]):
+            return None  # the other set holds a sample that is still to be picked up
+        if state["free"][1 - used] is not None:
+            state["free"][1 - used].wait(torch.cuda.current_stream(flat.device))
+        return nxt
+
+    def _sample_taken(self, nxt, next_k, capacity, ws, slot, which):
+        """Books the sample the last call took along for the call that follows (see _next_sample)."""
+        dev = nxt.device
+        state = self._ahead_state(dev, slot, create=True)
+        state["pending"].append((nxt.data_ptr(), nxt.numel(), next_k, capacity, ws.data_ptr(), which,
+                                 _Mark(torch.cuda.current_stream(dev)), _lib.dtype_code(nxt), ws.numel()))
+
     def _take_ahead(self, flat, n, k, capacity, ws, slot, mode, thr, near):
         """The sample taken ahead for the call that is about to be made, if there is one: (mode flags that tell
         the library, the set of sampling memory the call will use).  Samples taken for other calls stay where
