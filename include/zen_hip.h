@@ -284,8 +284,9 @@ int zen_load_balance_prepare(const void *input, int dtype, int64_t n, int64_t m,
 /*
  * Which implementation a zen_load_balance call with these sizes takes: 0 = owner table (the general
  * mode), 1 = sort-based owner resolution, 2 = bucket slabs (large inputs whose expected output is a small
- * fraction of the table: one streaming pass, then per-bucket sorts inside LDS).  No counterpart in the
- * reference; tests and benchmarks use it to know what they measured.
+ * fraction of the table: one streaming pass, then per-bucket sorts inside LDS), 3 = wide buckets (the same
+ * for an expected output of up to a few million entries: at most 256 buckets, one resident workgroup each,
+ * two launches).  No counterpart in the reference; tests and benchmarks use it to know what they measured.
  */
 int zen_load_balance_path(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions, int64_t k, int mode);
 
@@ -303,7 +304,8 @@ int zen_load_balance_path(int64_t n, int64_t m, int dtype, int64_t capacity, int
  */
 size_t zen_merge_workspace(int64_t r, int64_t dense_n);
 size_t zen_merge_zero_bytes(void); /* see ZEN_MODE_ZEROED; the same for every r and dense_n */
-/* 0 = radix sort (general mode), 1 = one bucket pass + per-range sorts, 2 = bucket slabs; see zen_load_balance_path */
+/* 0 = radix sort (general mode), 1 = one bucket pass + per-range sorts, 2 = bucket slabs, 3 = wide buckets; see
+   zen_load_balance_path */
 int zen_merge_path(int64_t r, int64_t dense_n, int mode);
 int zen_merge(const void *idx, int idx64_in, const void *val, int dtype,
               int64_t r, int64_t dense_n,
