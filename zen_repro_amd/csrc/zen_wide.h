@@ -35,6 +35,9 @@ inline bool wide_geometry(int64_t m, int partitions, int64_t expected, int cus, 
       expected < 1)
     return false;
   int64_t most = cus < kWideMaxBuckets ? cus : kWideMaxBuckets;
+  // half the chip where that holds the records: a bucket's workgroup wants a compute unit to itself, and the
+  // encode's and the merge's workgroups of one step then find room side by side instead of one after the other
+  if (most >= 2 * partitions && expected <= most / 2 * (int64_t)kWideTarget) most /= 2;
   int64_t bpp = most / partitions;
   const int64_t npp = m / partitions;
   if (bpp > npp / (4 * (int64_t)kWideSubs)) bpp = npp / (4 * (int64_t)kWideSubs);  // buckets wider than their sub-ranges
