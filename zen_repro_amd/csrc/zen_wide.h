@@ -31,7 +31,8 @@ constexpr uint32_t kWideCursorWords = kWideMaxBuckets * kWideSplit * kWidePad;
 // a chip of `cus` compute units; false if the layout does not suit these sizes.  The result is a SlabGeom
 // whose sub_shift refers to kWideSubs narrow ranges.
 inline bool wide_geometry(int64_t m, int partitions, int64_t expected, int cus, SlabGeom *out) {
-  if (m < (1ll << 22) || m > 0x7fffffffll || partitions < 1 || partitions > kWideMaxBuckets || m % partitions != 0 ||
+  // a table of 4 MB or more: the map at its head takes at most half, the counters behind it less than 1 MB
+  if (m < (1ll << 20) || m > 0x7fffffffll || partitions < 1 || partitions > kWideMaxBuckets || m % partitions != 0 ||
       expected < 1)
     return false;
   int64_t most = cus < kWideMaxBuckets ? cus : kWideMaxBuckets;

@@ -856,9 +856,16 @@ bool wide_balance_fits(int64_t m, int partitions, int64_t capacity, int64_t k, i
 
 // Whatever k a call comes with: the layout only depends on the table and the partitions.
 size_t wide_balance_bytes(int64_t m, int partitions, int dtype, int64_t capacity, int cus) {
-  SlabGeom geo;
-  if (capacity > 0x1fffffffll || cus <= 0 || !wide_geometry(m, partitions, 1, cus, &geo)) return 0;
-  return plan_wide(nullptr, nullptr, geo, partitions, dtype, list_capacity(capacity)).bytes;
+  // with few expected records the buckets take half the chip, else all of it: room for either
+  SlabGeom half, full;
+  if (capacity > 0x1fffffffll || cus <= 0 || !wide_geometry(m, partitions, 1, cus, &half)) return 0;
+  size_t bytes = plan_wide(nullptr, nullptr, half, partitions, dtype, list_capacity(capacity)).bytes;
+  const int64_t most = cus < kWideMaxBuckets ? cus : kWideMaxBuckets;
+  if (wide_geometry(m, partitions, most * (int64_t)kWideTarget, cus, &full)) {
+    const size_t other = plan_wide(nullptr, nullptr, full, partitions, dtype, list_capacity(capacity)).bytes;
+    if (other > bytes) bytes = other;
+  }
+  return bytes;
 }
 
 int wide_load_balance(const SlabBalanceArgs &a, size_t state_offset, hipStream_t s) {

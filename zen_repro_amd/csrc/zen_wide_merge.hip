@@ -374,7 +374,7 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_merge(SlabGeom geo, WideSla
 
 bool wide_merge_fits(int64_t r, int64_t dense_n, int cus, SlabGeom *geo) {
   SlabGeom g;
-  if (r < (1 << 15) || r > 0x7ffffffell || cus <= 0 || !wide_geometry(dense_n, 1, r, cus, &g)) return false;
+  if (r < (1 << 12) || r > 0x7ffffffell || cus <= 0 || !wide_geometry(dense_n, 1, r, cus, &g)) return false;
   if (g.sub_shift + ceil_log2_u64((uint64_t)r) > 32) return false;  // (index inside a narrow range, arrival number) must fit a word
   // a slab record carries the index's offset inside its bucket and the arrival number in fixed fields
   if ((uint64_t)g.sub_shift + 14 > kWmOffBits || (uint64_t)r >= (1ull << kWmArrBits)) return false;
