@@ -414,11 +414,18 @@ def reference_bucket(dev, steps, warmup):
             s_.wait_stream(main)
         for i in range(count):
             es = second if (depth == 2 and i % 2) else main
-            with torch.cuda.stream(es):
+
+            def call():
                 outs.append(lba.encode_merge_flat(tp, grads[i % copies], cap, b.k, fi, fv, b.n, slot=i % depth,
                                                   merge_stream=beside if depth == 1 else None,
                                                   next_tensor=grads[(i + 1) % copies] if depth == 1 and i + 1 < count
                                                   else None))
+
+            if es is main:
+                call()
+            else:
+                with torch.cuda.stream(es):
+                    call()
             if marks is not None and i % (2 * depth) == 2 * depth - 1:
                 pair = [torch.cuda.Event(enable_timing=True)]
                 pair[0].record(es)
@@ -601,13 +608,19 @@ def main():
                 enc.append(e_)
                 mrg.append(m_)
 
-        with torch.cuda.stream(es):
+        def on_stream():
             if fused:
                 both()
             else:
                 encode()
                 if ms_ is None:
                     merge()  # behind the encode, on its stream
+
+        if es is main:
+            on_stream()  # already the current stream: entering it again costs the host 10 us a step
+        else:
+            with torch.cuda.stream(es):
+                on_stream()
         if prep_stream is not None and more and depth == 1 and not (fused and args.prepare_on == "call"):
             with torch.cuda.stream(prep_stream if args.prepare_on == "own" else es):
                 for j, b in enumerate(buckets):

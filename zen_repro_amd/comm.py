@@ -76,6 +76,7 @@ class LoadBalanceAllreduce:
         self.tensor_partition = self.get_tensor_partition_obj(memory_scale, rehash)
         self.logger = logger
         self.mapping = {}
+        self._step_sizes = {}    # shape of an encode_merge_flat call -> (table size, workspace bytes, merge workspace bytes)
         self._bitmap_ranks = {}  # numel -> (mapping list of this rank, its rank table)
         self._dense_dicts = {}   # numel -> dictionary of decode_bitmaps_dense
 
@@ -212,8 +213,15 @@ class LoadBalanceAllreduce:
         L = _lib.lib()
         n, r = flat.numel(), indices.numel()
         code = _lib.dtype_code(flat)
-        m, _ = partition.table_sizes(n)
         P = partition.partitions
+        # sizes that only depend on the call's shape are worked out once (three crossings into the library less)
+        shape = (n, code, capacity, P, partition.memory_scale, r, dense_size)
+        sizes = self._step_sizes.get(shape)
+        if sizes is None:
+            m = partition.table_sizes(n)[0]
+            sizes = self._step_sizes[shape] = (m, L.zen_load_balance_workspace(n, m, code, capacity, P),
+                                               L.zen_merge_workspace(r, dense_size))
+        m, ws_bytes, mws_bytes = sizes
         mode = _lib.MODE_FAST | partition.fast_flags
         out_idx = torch.empty(capacity, dtype=torch.int32, device=dev)
         out_val = torch.empty(capacity, dtype=flat.dtype, device=dev)
@@ -223,8 +231,8 @@ class LoadBalanceAllreduce:
         splits, count = small[:P], small[P:P + 1]
         status2 = small[P + 1:P + 2].view(torch.int32)
         status, m_status = status2[0:1], status2[1:2]
-        ws = _lib.scratch.get(dev, f"load_balance/{slot}", L.zen_load_balance_workspace(n, m, code, capacity, P))
-        mws = _lib.scratch.get(dev, f"merge/{slot}", L.zen_merge_workspace(r, dense_size), zero=True)
+        ws = _lib.scratch.get(dev, f"load_balance/{slot}", ws_bytes)
+        mws = _lib.scratch.get(dev, f"merge/{slot}", mws_bytes, zero=True)
         table = partition._table(dev, m, slot)
         flags, used = partition._take_ahead(flat, n, int(k), capacity, ws, slot, mode, None, near)
         thr = None

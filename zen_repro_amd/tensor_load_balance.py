@@ -43,6 +43,7 @@ class TensorPartition:
         self.device = torch.cuda.current_device()
         self._tables = {}
         self._ahead = {}  # (device, slot) -> samples taken ahead of their calls (prepare)
+        self._samples_next = {}  # shape of a call -> whether its pass over the tensor can take the next sample along
 
     # ------------------------------------------------------------ sizes
     def table_sizes(self, numel):
@@ -185,9 +186,13 @@ class TensorPartition:
                 or not nxt.is_contiguous() or (mode & 0xff) != _lib.MODE_FAST):
             return None
         n = flat.numel()
-        m, _ = self.table_sizes(n)
-        if not _lib.lib().zen_encode_merge_samples_next(n, m, _lib.dtype_code(flat), capacity, self.partitions, next_k,
-                                                        mode & (0xff | _lib.MODE_SLABS)):
+        key = (n, flat.dtype, capacity, next_k, mode & (0xff | _lib.MODE_SLABS))
+        able = self._samples_next.get(key)
+        if able is None:
+            m, _ = self.table_sizes(n)
+            able = self._samples_next[key] = bool(_lib.lib().zen_encode_merge_samples_next(
+                n, m, _lib.dtype_code(flat), capacity, self.partitions, next_k, key[4]))
+        if not able:
             return None
         state = self._ahead_state(flat.device, slot, create=True)
         if any(entry[5] == 1 - used for entry in state["pending"]):
