@@ -778,3 +778,37 @@ def test_profile_every_nth_launch(zen, oracle):
     finally:
         _lib.profile_enable(False)
         _lib.check(_lib.lib().zen_profile_every(1), "profile_every")
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("idx64", [False, True])
+@pytest.mark.parametrize("count", [0, 1, 2047, 2049, 300000])
+def test_round_merged_sums(zen, oracle, dtype, idx64, count):
+    """zen_round_compact: what comm.py:125-127 makes of the merged sums (a dense tensor of the gradient's type,
+    then its nonzeros): every fp32 sum rounded once to the type, entries that round to zero dropped, order
+    kept; only the first `count` entries (a device value) are looked at.  Sums that are tiny, negative zeros,
+    NaN and infinities included."""
+    cap = count + 100
+    rng = np.random.default_rng(count + 7)
+    sums = (rng.standard_normal(cap) * 1e-3).astype(np.float32)
+    sums[rng.integers(0, cap, cap // 5)] = 0.0
+    sums[rng.integers(0, cap, cap // 7)] = -0.0
+    sums[rng.integers(0, cap, cap // 9)] = 1e-41 if dtype == "bf16" else 1e-45  # bf16: rounds to zero
+    sums[rng.integers(0, cap, 3)] = np.nan
+    sums[rng.integers(0, cap, 3)] = -np.inf
+    idx = np.sort(rng.choice(1 << 30, cap, replace=False)).astype(np.int64 if idx64 else np.int32)
+    lba = zen.LoadBalanceAllreduce(zen.LocalGroup(4), None, None)
+    tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
+    cnt = torch.tensor([count], dtype=torch.int64, device="cuda")
+    o_idx, o_val, kept, status = lba.round_merged_flat(to_dev(idx), to_dev(sums), cnt, tdt)
+    assert int(status) == 0
+    rounded = torch.from_numpy(sums[:count]).to(tdt)
+    keep = (rounded != 0).numpy()  # NaN != 0 is true, -0.0 != 0 false: what torch.nonzero keeps
+    u = int(kept)
+    assert u == int(keep.sum())
+    assert np.array_equal(to_np(o_idx)[:u], idx[:count][keep])
+    bits = torch.int16 if dtype == "bf16" else torch.int32
+    got, want = o_val[:u].cpu(), rounded[torch.from_numpy(keep)]
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan)  # a NaN stays a NaN (which of the NaN patterns is the converter's business)
+    assert torch.equal(got[~nan].view(bits), want[~nan].view(bits))
