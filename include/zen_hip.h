@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define ZEN_ABI_VERSION 1
+#define ZEN_ABI_VERSION 2 /* 2: zen_encode_merge (its argument struct), zen_sample_threshold, zen_round_compact, path code 3 */
 
 #define ZEN_F32 0
 #define ZEN_BF16 1

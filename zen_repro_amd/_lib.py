@@ -117,7 +117,7 @@ def lib():
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
         fn.restype, fn.argtypes = res, args
-    if L.zen_abi_version() != 1:
+    if L.zen_abi_version() != 2:
         raise RuntimeError("libzen_hip.so: unexpected ABI version")
     _lib = L
     return L
