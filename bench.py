@@ -826,6 +826,19 @@ def main():
                "path_frac_of_hbm_peak": round(b_alg / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                "what": "the same steps with two in flight on two streams, a step's merge behind its encode (--depth 2)"}
 
+    # the roofline kernel with the chip to itself: the encodes alone on the main stream (no merge beside them,
+    # nothing left over from a step before), events around every launch of that kernel
+    alone = None
+    if dom and not args.graph:
+        torch.cuda.synchronize()
+        _lib.profile_enable(True, only=dom, every=1)
+        for i in range(12):
+            for j, b in enumerate(buckets):
+                tp.load_balance_flat(grad_sets[j][i % len(grad_sets[j])], None, caps[j], k=b.k, slot=0, near=near_keys[j])
+        torch.cuda.synchronize()
+        alone = _lib.profile_read().get(dom)
+        _lib.profile_enable(False)
+
     # dominant kernel: the one with the largest summed duration among the
     # kernels that stream the dense gradient; its algorithmic bytes per launch
     # (several buckets: the mean over the buckets' launches, all of which are timed)
@@ -846,6 +859,16 @@ def main():
                     "algorithmic_bytes_per_launch": int(per_launch[dom]),
                     "measured_read_ceiling_GBps": round(ceiling, 1) if ceiling else None,
                     "frac_of_read_ceiling": round(achieved / ceiling, 4) if ceiling else None}
+        if alone:
+            a_ms = alone[0] / alone[1]
+            a_rate = per_launch[dom] / (a_ms * 1e-3) / 1e9
+            roofline["alone"] = {"avg_launch_ms": round(a_ms, 4), "achieved": round(a_rate, 1),
+                                 "frac": round(a_rate / HBM_PEAK_GBS, 4),
+                                 "frac_of_read_ceiling": round(a_rate / ceiling, 4) if ceiling else None,
+                                 "launches": alone[1],
+                                 "what": "the same kernel with the chip to itself (encodes alone on one stream, untimed "
+                                         "pass): in a step its launches wait for compute units the merge before them "
+                                         "still holds and share the memory system with the merge's scatter"}
 
     if roofline and args.graph:
         roofline["timed_in"] = "the untimed pass with every stage's events on (graph replays carry no events)"
