@@ -30,7 +30,10 @@ def test_every_declared_symbol_is_exported(L):
     raw = ctypes.CDLL(os.path.join(ROOT, "zen_repro_amd", "csrc", "libzen_hip.so"))
     for n in sorted(names):
         assert hasattr(raw, n), f"{n} declared in zen_hip.h but not exported"
-    assert L.zen_abi_version() == 2
+    from zen_repro_amd import _lib
+
+    declared = int(re.search(r"#define\s+ZEN_ABI_VERSION\s+(\d+)", header).group(1))
+    assert L.zen_abi_version() == declared == _lib.ABI_VERSION
 
 
 def test_workspace_queries_are_host_only(L):

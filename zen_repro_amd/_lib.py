@@ -21,6 +21,9 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # ZEN_HIP_LIB names another build of the library (a debug build, a build with other compile-time settings)
 LIB_PATH = os.environ.get("ZEN_HIP_LIB") or os.path.join(_HERE, "csrc", "libzen_hip.so")
 
+# ZEN_ABI_VERSION of include/zen_hip.h this loader's signatures and structs are written for
+ABI_VERSION = 2
+
 _lib = None
 
 
@@ -117,7 +120,7 @@ def lib():
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
         fn.restype, fn.argtypes = res, args
-    if L.zen_abi_version() != 2:
+    if L.zen_abi_version() != ABI_VERSION:
         raise RuntimeError("libzen_hip.so: unexpected ABI version")
     _lib = L
     return L
