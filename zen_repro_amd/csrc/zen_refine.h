@@ -77,21 +77,29 @@ __global__ __launch_bounds__(kRefineBlock) void k_refine_threshold(CoarseGeom cg
     if (threadIdx.x == 0) atomicOr(status, ZEN_STAT_RETRY);  // the two histograms disagree: let the general mode answer
     return;
   }
+  // the thread whose bins hold the rank hands them to the first wave: a lane takes two bins, from the top down
+  __shared__ uint32_t s_hi, s_before;
   if (before < need && need <= before + mine) {
-    const uint4 *own = reinterpret_cast<const uint4 *>(hist + (hi - (uint32_t)kPer));
-    for (int j = 1; j <= kPer; ++j) {
-      const uint4 q = own[(kPer - j) >> 2];  // the bin hi - j, in the lines read above
-      const uint32_t w = (uint32_t)(kPer - j) & 3u;
-      const uint32_t c = w == 0 ? q.x : w == 1 ? q.y : w == 2 ? q.z : q.w;
-      if (before < need && need <= before + c) {
-        thr[0] = base + hi - (uint32_t)j;
-        thr[1] = over + before + c;
-        if (thr_copy) {
-          thr_copy[0] = base + hi - (uint32_t)j;
-          thr_copy[1] = over + before + c;
-        }
-      }
-      before += c;
+    s_hi = hi;
+    s_before = before;
+  }
+  __syncthreads();
+  if (threadIdx.x >= 64) return;
+  static_assert(kPer == 128, "two bins per lane of one wave");
+  const uint32_t top = s_hi;  // the bins top - 1, top - 2, ... top - kPer
+  const uint2 two = *reinterpret_cast<const uint2 *>(hist + (top - 2u * (threadIdx.x + 1u)));  // .y is the upper bin
+  const uint32_t pair = two.x + two.y;
+  const uint32_t incl = wave_inclusive_scan(pair);
+  const uint32_t ahead = s_before + incl - pair;  // elements above the lane's two bins
+  if (ahead < need && need <= ahead + pair) {
+    const bool upper = need <= ahead + two.y;
+    const uint32_t bin = top - 2u * threadIdx.x - (upper ? 1u : 2u);
+    const uint32_t at_or_above = over + ahead + two.y + (upper ? 0u : two.x);
+    thr[0] = base + bin;
+    thr[1] = at_or_above;
+    if (thr_copy) {
+      thr_copy[0] = base + bin;
+      thr_copy[1] = at_or_above;
     }
   }
 }

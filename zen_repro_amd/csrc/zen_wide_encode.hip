@@ -241,7 +241,8 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
                                                           const S *__restrict__ dense, int32_t *__restrict__ out_idx,
                                                           S *__restrict__ out_val, uint32_t capacity,
                                                           int64_t *__restrict__ splits, uint32_t *clear,
-                                                          uint32_t clear_words, int32_t *status) {
+                                                          uint32_t clear_words, uint32_t *clear_too,
+                                                          uint32_t clear_too_words, int32_t *status) {
   __shared__ WideShared<S> sh;
   const uint32_t b = blockIdx.x, B = geo.nbuckets, bpp = geo.bpp;
   const uint32_t part = b / bpp;
@@ -249,6 +250,7 @@ __global__ __launch_bounds__(kWideBlock) void k_wide_tail(SlabGeom geo, Probe g,
   WIDE_MARK(0);
   // counters of the kernels before this one that nobody needs any more: back to zero, a slice per workgroup
   for (uint32_t i = b * kWideBlock + tid; i < clear_words; i += B * kWideBlock) clear[i] = 0;
+  for (uint32_t i = b * kWideBlock + tid; i < clear_too_words; i += B * kWideBlock) clear_too[i] = 0;  // fp32: the refinement's histogram
   if (tid == 0) {
     sh.lo = geo.first_key(b);
     sh.lost_n = sh.nrm = sh.mv_n = sh.ser_n = sh.big = 0;
@@ -932,23 +934,22 @@ int wide_load_balance(const SlabBalanceArgs &a, size_t state_offset, hipStream_t
     ZEN_LAUNCH_CHECK("k_refine_threshold");
   }
   const uint32_t *filter = a.k > 0 ? p.thr : nullptr;
+  uint32_t *clear_too = refine ? p.refine_hist : nullptr;
+  const uint32_t clear_too_words = refine ? (uint32_t)kRefineBins + 1u : 0u;
   if ((rc = wide_line_enter(s)) != ZEN_OK) return rc;
   {
     ProfScope prof(kProfWideTail, s);
     if (a.dtype == ZEN_BF16)
       k_wide_tail<uint16_t><<<dim3(geo.nbuckets), dim3(kWideBlock), 0, s>>>(
           geo, a.g, p.tb, filter, a.hash, a.spp, static_cast<const uint16_t *>(a.input), a.out_idx,
-          static_cast<uint16_t *>(a.out_val), (uint32_t)a.capacity, a.splits, clear, clear_words, a.status);
+          static_cast<uint16_t *>(a.out_val), (uint32_t)a.capacity, a.splits, clear, clear_words, clear_too,
+          clear_too_words, a.status);
     else
       k_wide_tail<uint32_t><<<dim3(geo.nbuckets), dim3(kWideBlock), 0, s>>>(
           geo, a.g, p.tb, filter, a.hash, a.spp, static_cast<const uint32_t *>(a.input), a.out_idx,
-          static_cast<uint32_t *>(a.out_val), (uint32_t)a.capacity, a.splits, clear, clear_words, a.status);
+          static_cast<uint32_t *>(a.out_val), (uint32_t)a.capacity, a.splits, clear, clear_words, clear_too,
+          clear_too_words, a.status);
     ZEN_LAUNCH_CHECK("k_wide_tail");
-  }
-  if (refine) {
-    // the refinement histogram is the tail kernel's to clear on the other path; here a fill does it
-    launch_fill<uint32_t>(p.refine_hist, 0u, (size_t)kRefineBins + 1, s);
-    ZEN_LAUNCH_CHECK("wide: clear the refinement histogram");
   }
   return wide_line_leave(s);
 }
