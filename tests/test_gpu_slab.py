@@ -198,6 +198,39 @@ def test_slab_load_balance_fused_topk_fp32(zen, oracle):
         assert np.array_equal(to_np(ov)[:total], val_o)
 
 
+def test_fused_topk_fp32_wherever_the_kth_key_lies_in_its_bin(zen, oracle, fast_path):
+    """The fp32 threshold's last 16 bits for a k-th key at the top, the bottom and the middle of the threshold's
+    bin of 65536 keys, at even and odd keys and either side of a multiple of 128 (the refinement's last
+    workgroup gives a thread 128 keys and a lane of its first wave two of them)."""
+    n, P = (1 << 20) if fast_path == "wide" else (1 << 24), 4
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(n) * 0.2).astype(np.float32)
+    base = 0x3F000000  # 0.5: the bin is [0.5, 0.50390625)
+    keys = x.view(np.uint32) & 0x7FFFFFFF
+    x[(keys >> 16) == (base >> 16)] = 0.3  # nobody else in that bin
+    x[0] = 0.25
+    lows = [65535, 65534, 65409, 65408, 65407, 32769, 32768, 129, 128, 127, 1, 0]
+    at = rng.choice(np.arange(1, n), 3 * len(lows), replace=False)
+    sign = np.where(rng.random(len(at)) < 0.5, 0x80000000, 0).astype(np.uint32)
+    x.view(np.uint32)[at] = (np.repeat(np.array(lows, np.uint32), 3) + np.uint32(base)) | sign  # three of each
+    ordered = np.sort(x.view(np.uint32) & 0x7FFFFFFF)
+    above = n - int(np.searchsorted(ordered, base + 65536, "left"))
+    assert int(oracle.kth_key(x, above + 4)) == base + lows[1]
+    capacity = int(1.5 * above) + 4096
+    tp = zen.TensorPartition(P, 1, 3)
+    d = to_dev(x)
+    thr_out = torch.zeros(2, dtype=torch.int32, device="cuda")
+    for j in range(1, 3 * len(lows) + 1):
+        k = above + j
+        key = base + lows[(j - 1) // 3]  # the k-th largest key: the ((j - 1) // 3)-th of the planted ones
+        kept = n - int(np.searchsorted(ordered, key, "left"))
+        assert on_fast_path(lb_path(zen, n, P, "f32", capacity, k=k))
+        _, _, splits, status = tp.load_balance_flat(d, capacity=capacity, k=k, thr_out=thr_out)
+        assert status.item() == 0, (j, status.item())
+        assert to_np(thr_out).tolist() == [key, kept], j
+        assert int(to_np(splits).sum()) == kept - int((x.view(np.uint32)[0] & 0x7FFFFFFF) >= key)  # index 0 is never handed on
+
+
 def test_slab_load_balance_threshold_given(zen, oracle):
     """Selection by a threshold the caller computed (topk_threshold) instead of k."""
     from zen_repro_amd import _lib
