@@ -604,7 +604,7 @@ def main():
                                                thr_out=warm_thr[j] if warm else None, near=near_keys[j],
                                                merge_stream=ms_,
                                                next_tensor=grad_sets[nj][ni % len(grad_sets[nj])] if along else None,
-                                               next_k=buckets[nj].k)
+                                               next_k=buckets[nj].k, next_capacity=caps[nj])
                 enc.append(e_)
                 mrg.append(m_)
 

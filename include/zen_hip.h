@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define ZEN_ABI_VERSION 2 /* 2: zen_encode_merge (its argument struct), zen_sample_threshold, zen_round_compact, path code 3 */
+#define ZEN_ABI_VERSION 3 /* 2: zen_encode_merge (its argument struct), zen_sample_threshold, zen_round_compact, path code 3; 3: next_n .. next_table */
 
 #define ZEN_F32 0
 #define ZEN_BF16 1
@@ -373,16 +373,21 @@ typedef struct zen_encode_merge_args {
   size_t merge_workspace_bytes;
   int32_t *merge_status;
   void *stream, *merge_stream;
-  /* Optional (NULL / 0: none): the gradient of the NEXT call on this table and workspace, of this one's type,
-     n, m, partitions and capacity, and that call's k.  On the fast paths the pass over `input` then also takes
-     the sample that gives the next call's selection its floor (its workgroups do it when they are through with
-     their own tensor: no kernel of its own, nothing that waits), in the set of sampling memory this call does
-     not use.  The next call says so like after zen_load_balance_prepare: ZEN_MODE_PREPARED, with
-     ZEN_MODE_SECOND unless THIS call's mode has ZEN_MODE_SECOND.  zen_encode_merge_samples_next tells whether
-     a call with these sizes does it (the other paths ignore the fields).  next_input must be readable in the
-     order of `stream`. */
+  /* Optional (NULL / 0: none): the gradient of the NEXT call on this workspace, of this one's type and
+     partitions, and that call's k.  On the fast paths the pass over `input` then also takes the sample that
+     gives the next call's selection its floor (its workgroups do it when they are through with their own
+     tensor: no kernel of its own, nothing that waits), in the set of sampling memory this call does not use.
+     The next call says so like after zen_load_balance_prepare: ZEN_MODE_PREPARED, with ZEN_MODE_SECOND unless
+     THIS call's mode has ZEN_MODE_SECOND.  zen_encode_merge_samples_next tells whether a call with these sizes
+     does it (the other paths ignore the fields).  next_input must be readable in the order of `stream`.
+       A next call of another size (gradient buckets differ in length) names its own n, m, capacity and table
+     in next_n, next_m, next_capacity and next_table (0 / NULL: this call's); its sizes must take path 2 or 3
+     (zen_load_balance_path), or the call is refused with ZEN_EINVAL: only those paths keep sampling memory in
+     their table.  The workspace must be large enough for either call. */
   const void *next_input;
   int64_t next_k;
+  int64_t next_n, next_m, next_capacity;
+  int32_t *next_table;
 } zen_encode_merge_args;
 int zen_encode_merge_samples_next(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions, int64_t k,
                                   int mode);

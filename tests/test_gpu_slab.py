@@ -682,41 +682,45 @@ def test_encode_and_merge_in_one_call(zen, oracle, dtype):
 
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
 def test_sample_taken_along_by_the_call_before(zen, oracle, dtype):
-    """encode_merge_flat(..., next_tensor=): the pass over one bucket takes the next bucket's sample along.  Three
-    different gradients in a row on one slot, each call handed its successor; every result equals the oracle's
-    (so the floor the call before left behind selected nothing wrong), every call after the first picks its
-    sample up (no sample kernel of its own is launched: counted), and a successor of another size is simply not
-    sampled."""
+    """encode_merge_flat(..., next_tensor=): the pass over one bucket takes the next bucket's sample along.  Four
+    different gradients in a row on one slot, the third of another size (with its own k, capacity and table),
+    each call handed its successor; every result equals the oracle's (so the floor the call before left behind
+    selected nothing wrong), and every call after the first picks its sample up (no sample kernel of its own is
+    launched: counted)."""
     from zen_repro_amd import _lib
 
     n, P = 1 << 24, 16
-    k = n // 200
-    grads = [make_grad(oracle, n, 1.0, dtype, seed=41 + i) for i in range(3)]
+    sizes = [n, n, n // 4 * 3, n]
+    ks = [s // 200 for s in sizes]
+    caps = [int(k * 1.25) + 4096 for k in ks]
+    grads = [make_grad(oracle, s, 1.0, dtype, seed=41 + i) for i, s in enumerate(sizes)]
     rng = np.random.default_rng(9)
     ci, cv = payloads(oracle, rng, n, P, 9000, 0.25, dtype)
     ci = ci.astype(np.int32)
-    cap = int(k * 1.25) + 4096
     ds = [to_dev(g) for g in grads]
     di, dv = to_dev(ci), to_dev(cv)
     tp = zen.TensorPartition(P, 1, 3)
     lba = zen.LoadBalanceAllreduce(zen.LocalGroup(P), None, None)
-    m, _ = oracle.table_sizes(n, P, 1)
-    assert on_fast_path(_lib.lib().zen_load_balance_path(n, m, _lib.dtype_code(ds[0]), cap, P, k, _lib.MODE_FAST | FLAGS))
+    for s_, k_, c_ in zip(sizes, ks, caps):
+        m, _ = oracle.table_sizes(s_, P, 1)
+        assert on_fast_path(_lib.lib().zen_load_balance_path(s_, m, _lib.dtype_code(ds[0]), c_, P, k_, _lib.MODE_FAST | FLAGS))
     want_m = oracle.merge_sparse(ci, cv, n)
     _lib.profile_enable(True)
     outs = []
-    for i in range(3):
-        nxt = ds[i + 1] if i + 1 < 3 else ds[0][: n // 2]  # the last successor has another size: not sampled
-        outs.append(lba.encode_merge_flat(tp, ds[i], cap, k, di, dv, n, next_tensor=nxt))
+    for i in range(4):
+        more = i + 1 < 4
+        outs.append(lba.encode_merge_flat(tp, ds[i], caps[i], ks[i], di, dv, n, next_tensor=ds[i + 1] if more else None,
+                                          next_k=ks[i + 1] if more else None,
+                                          next_capacity=caps[i + 1] if more else None))
     torch.cuda.synchronize()
     launched = _lib.profile_read()
     _lib.profile_enable(False)
-    assert launched["k_sample_hist"][1] == 1 and launched["k_select_stage"][1] == 3  # only the first call sampled for itself
+    assert launched["k_sample_hist"][1] == 1 and launched["k_select_stage"][1] == 4  # only the first call sampled for itself
     state = tp._ahead_state(ds[0].device, 0)
     assert state is not None and not state["pending"]
     for i, (e, mg) in enumerate(outs):
         assert e[3].item() == 0 and mg[3].item() == 0
-        key = oracle.kth_key(grads[i], k)
+        key = oracle.kth_key(grads[i], ks[i])
         sel, _ = oracle.mask_dense(grads[i], key)
         idx_o, val_o, splits_o, st_o = oracle.load_balance(sel, P, 1, 3)
         total = int(splits_o.sum())
@@ -725,4 +729,9 @@ def test_sample_taken_along_by_the_call_before(zen, oracle, dtype):
         cnt = int(mg[2])
         assert cnt == len(want_m[0]) and np.array_equal(to_np(mg[0])[:cnt], want_m[0].astype(np.int32))
         assert np.array_equal(to_np(mg[1])[:cnt].view(np.uint32), want_m[1].view(np.uint32))
-    assert not tp._table(ds[0].device, m).any()
+    for s_ in set(sizes):
+        assert not tp._table(ds[0].device, oracle.table_sizes(s_, P, 1)[0]).any()
+    # a successor whose sizes take no path that keeps a sample is refused by the library, and not offered by the wrapper
+    small = ds[0][: 1 << 12]
+    e, _ = lba.encode_merge_flat(tp, ds[0], caps[0], ks[0], di, dv, n, next_tensor=small, next_k=20, next_capacity=64)
+    assert e[3].item() == 0 and not tp._ahead_state(ds[0].device, 0)["pending"]

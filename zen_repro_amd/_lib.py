@@ -22,7 +22,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("ZEN_HIP_LIB") or os.path.join(_HERE, "csrc", "libzen_hip.so")
 
 # ZEN_ABI_VERSION of include/zen_hip.h this loader's signatures and structs are written for
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 
@@ -40,7 +40,8 @@ class EncodeMergeArgs(ctypes.Structure):
         ("merged_count", _vp), ("merge_mode", _i32), ("merge_workspace", _vp), ("merge_workspace_bytes", _sz),
         ("merge_status", _vp),
         ("stream", _vp), ("merge_stream", _vp),
-        ("next_input", _vp), ("next_k", _i64),
+        ("next_input", _vp), ("next_k", _i64), ("next_n", _i64), ("next_m", _i64), ("next_capacity", _i64),
+        ("next_table", _vp),
     ]
 
 

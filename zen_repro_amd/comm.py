@@ -190,7 +190,8 @@ class LoadBalanceAllreduce:
         return out_idx, out_val, count, status
 
     def encode_merge_flat(self, partition, tensor, capacity, k, recv_indices, recv_values, dense_size, slot=0,
-                          thr_out=None, near=None, merge_stream=None, next_tensor=None, next_k=None):
+                          thr_out=None, near=None, merge_stream=None, next_tensor=None, next_k=None,
+                          next_capacity=None):
         """One bucket's step in one call of the library: partition.load_balance_flat(tensor, None, capacity,
         k=k, slot=slot, thr_out=thr_out, near=near) of the rank's own gradient and merge_sparse_flat(recv_indices,
         recv_values, dense_size, slot=slot) of the entries it received, whose values have the gradient's type.
@@ -198,8 +199,9 @@ class LoadBalanceAllreduce:
         torch stream in whose order the received entries are ready) takes the merge.  A sample taken ahead with
         partition.prepare() is picked up as load_balance_flat would.  `next_tensor` (ready in the current stream's
         order) is the gradient of the call that follows on this slot, `next_k` its k (default: this call's): if
-        it has this tensor's size and type, the pass over this tensor takes the sample of that call along (no
-        kernel of its own), as if partition.prepare(next_tensor, next_k, capacity, slot) had been called."""
+        it has this tensor's type, the pass over this tensor takes the sample of that call along (no kernel of
+        its own), as if partition.prepare(next_tensor, next_k, next_capacity, slot) had been called
+        (`next_capacity`: that call's capacity, default this call's; gradient buckets differ in size)."""
         from .tensor_load_balance import TensorPartition  # noqa: F401 (the type of `partition`)
 
         _lib.require_gpu(tensor, "input")
@@ -231,6 +233,19 @@ class LoadBalanceAllreduce:
         splits, count = small[:P], small[P:P + 1]
         status2 = small[P + 1:P + 2].view(torch.int32)
         status, m_status = status2[0:1], status2[1:2]
+        if next_k is None:
+            next_k = k
+        if next_capacity is None:
+            next_capacity = capacity
+        if next_tensor is not None and next_k > 0 and (next_tensor.numel() != n or next_capacity != capacity):
+            # the next call shares the slot's workspace: it must not move between the two calls
+            n2 = next_tensor.numel()
+            shape2 = (n2, code, next_capacity, P, partition.memory_scale)
+            bytes2 = self._step_sizes.get(shape2)
+            if bytes2 is None:
+                bytes2 = self._step_sizes[shape2] = L.zen_load_balance_workspace(
+                    n2, partition.table_sizes(n2)[0], code, next_capacity, P)
+            ws_bytes = max(ws_bytes, bytes2)
         ws = _lib.scratch.get(dev, f"load_balance/{slot}", ws_bytes)
         mws = _lib.scratch.get(dev, f"merge/{slot}", mws_bytes, zero=True)
         table = partition._table(dev, m, slot)
@@ -238,9 +253,9 @@ class LoadBalanceAllreduce:
         thr = None
         if near is not None and k > 0:
             thr, flags = near, flags | _lib.MODE_FLOOR
-        if next_k is None:
-            next_k = k
-        nxt = partition._next_sample(flat, next_tensor, int(next_k), capacity, ws, slot, mode | flags, used)
+        nxt, nxt_table = partition._next_sample(flat, next_tensor, int(next_k), capacity, next_capacity, slot,
+                                                mode | flags, used)
+        other = nxt is not None and nxt_table is not None
         a = _lib.EncodeMergeArgs(
             flat.data_ptr(), code, n, m, P, partition.rehash, thr.data_ptr() if thr is not None else None, int(k),
             thr_out.data_ptr() if thr_out is not None else None, out_idx.data_ptr(), out_val.data_ptr(), capacity,
@@ -249,7 +264,9 @@ class LoadBalanceAllreduce:
             m_idx.data_ptr(), 0, m_val.data_ptr(), r, count.data_ptr(),
             _lib.MODE_FAST | self.fast_flags | _lib.MODE_ZEROED, mws.data_ptr(), mws.numel(), m_status.data_ptr(),
             _lib.stream_handle(dev), merge_stream.cuda_stream if merge_stream is not None else None,
-            nxt.data_ptr() if nxt is not None else None, int(next_k) if nxt is not None else 0)
+            nxt.data_ptr() if nxt is not None else None, int(next_k) if nxt is not None else 0,
+            nxt.numel() if other else 0, nxt_table.numel() if other else 0, next_capacity if other else 0,
+            nxt_table.data_ptr() if other else None)
         self.last_encode_merge_args = a  # what the library was called with (its buffers live as long as the results)
         rc = L.zen_encode_merge(ctypes.byref(a))
         if rc != _lib.OK:
@@ -257,7 +274,7 @@ class LoadBalanceAllreduce:
         _lib.check(rc, "encode_merge")
         partition._after_call(dev, slot, int(k), used)
         if nxt is not None:
-            partition._sample_taken(nxt, int(next_k), capacity, ws, slot, 1 - used)
+            partition._sample_taken(nxt, int(next_k), next_capacity, ws, slot, 1 - used)
         return (out_idx, out_val, splits, status), (m_idx, m_val, count, m_status)
 
     def round_merged_flat(self, indices, sums, count, dtype):

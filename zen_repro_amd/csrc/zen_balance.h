@@ -142,8 +142,10 @@ struct SlabBalanceArgs {
   int32_t *status;
   const uint32_t *near_key = nullptr;  // optional, k > 0: a key close to the k-th largest (no sample is taken)
   int prepared = 0;           // 1 / 2: the sampled floor of the first / second set is there already (zen_load_balance_prepare)
-  const void *next_input = nullptr;  // the next call's tensor (this one's size and type): its sample is taken
+  const void *next_input = nullptr;  // the next call's tensor (this one's type): its sample is taken
   int64_t next_k = 0;                // by this call's pass over the tensor, in the other set of sampling memory
+  int64_t next_n = 0;                // its length (0: this call's)
+  void *next_state = nullptr;        // the zero-between-calls memory in the next call's table (null: this call's)
   bool second = false;        // the call's sample uses the second set of sampling memory (always so with prepared == 2)
   bool only_prepare = false;  // take the sample for that set and nothing else
   bool discard = false;       // with only_prepare: clear the set's sampling memory instead (a sample nobody picks up)

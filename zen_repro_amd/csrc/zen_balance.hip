@@ -440,7 +440,8 @@ namespace {
 int load_balance_call(const void *input, int dtype, int64_t n, int64_t m, int partitions, int rehash,
                       const uint32_t *thr, int64_t k, uint32_t *thr_out, int32_t *out_idx, void *out_val,
                       int64_t capacity, int64_t *splits, int32_t *table, int mode, void *workspace,
-                      size_t workspace_bytes, int32_t *status, void *stream, const void *next_input, int64_t next_k) {
+                      size_t workspace_bytes, int32_t *status, void *stream, const void *next_input, int64_t next_k,
+                      int64_t next_n, int64_t next_m, int64_t next_capacity, int32_t *next_table) {
   using namespace zen;
   const int prepared = (mode & ZEN_MODE_PREPARED) ? ((mode & ZEN_MODE_SECOND) ? 2 : 1) : 0;
   const bool second_set = (mode & ZEN_MODE_SECOND) != 0;
@@ -495,8 +496,24 @@ int load_balance_call(const void *input, int dtype, int64_t n, int64_t m, int pa
     sa.prepared = near_key ? 0 : prepared;
     sa.second = second_set;
     sa.near_key = near_key;
-    sa.next_input = next_input;
-    sa.next_k = next_k;
+    if (next_input && next_k > 0) {
+      sa.next_input = next_input;
+      sa.next_k = next_k;
+      if (next_n > 0 || next_m > 0 || next_capacity > 0 || next_table) {  // a next call of its own size
+        const int64_t n2 = next_n > 0 ? next_n : n, m2 = next_m > 0 ? next_m : m;
+        const int64_t cap2 = next_capacity > 0 ? next_capacity : capacity;
+        int32_t *table2 = next_table ? next_table : table;
+        if (n2 > 0x7fffffffll || m2 > 0x7fffffffll || m2 % partitions != 0 || cap2 > 0x1fffffffll || next_k > n2 ||
+            (reinterpret_cast<uintptr_t>(table2) & 7u) != 0 ||
+            (!wide_balance_fits(m2, partitions, cap2, next_k, wide_device_cus(), nullptr) &&
+             !slab_balance_fits(n2, m2, partitions, dtype, cap2, next_k, nullptr)))
+          return fail(ZEN_EINVAL, "zen_encode_merge: the next call's sizes do not take a path that keeps a sample");
+        if (workspace_bytes < zen_load_balance_workspace(n2, m2, dtype, cap2, partitions))
+          return fail(ZEN_EWORKSPACE, "zen_encode_merge: workspace too small for the next call");
+        sa.next_n = n2;
+        sa.next_state = reinterpret_cast<char *>(table2) + slab_state_offset(slab_hash_log2(m2));
+      }
+    }
     if (wide) return wide_load_balance(sa, slab_state_offset(sa.hash_log2), s);
     return slab_load_balance(sa, s);
   }
@@ -600,7 +617,7 @@ int zen_load_balance(const void *input, int dtype, int64_t n, int64_t m, int par
                      int64_t capacity, int64_t *splits, int32_t *table, int mode, void *workspace,
                      size_t workspace_bytes, int32_t *status, void *stream) {
   return load_balance_call(input, dtype, n, m, partitions, rehash, thr, k, thr_out, out_idx, out_val, capacity, splits,
-                           table, mode, workspace, workspace_bytes, status, stream, nullptr, 0);
+                           table, mode, workspace, workspace_bytes, status, stream, nullptr, 0, 0, 0, 0, nullptr);
 }
 
 int zen_encode_merge_samples_next(int64_t n, int64_t m, int dtype, int64_t capacity, int partitions, int64_t k,
@@ -614,7 +631,8 @@ int zen_encode_merge(const zen_encode_merge_args *a) {
   if (!a) return fail(ZEN_EINVAL, "zen_encode_merge: null pointer");
   const int rc = load_balance_call(a->input, a->dtype, a->n, a->m, a->partitions, a->rehash, a->thr, a->k, a->thr_out,
                                    a->out_idx, a->out_val, a->capacity, a->splits, a->table, a->mode, a->workspace,
-                                   a->workspace_bytes, a->status, a->stream, a->next_input, a->next_k);
+                                   a->workspace_bytes, a->status, a->stream, a->next_input, a->next_k, a->next_n,
+                                   a->next_m, a->next_capacity, a->next_table);
   if (rc != ZEN_OK) return rc;
   return zen_merge(a->recv_idx, a->recv_idx64, a->recv_val, a->dtype, a->r, a->dense_n, a->merged_idx, a->merged_idx64,
                    a->merged_val, a->merged_capacity, a->merged_count, a->merge_mode, a->merge_workspace,

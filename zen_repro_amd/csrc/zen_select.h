@@ -129,11 +129,13 @@ struct StageArgs {
   uint32_t *thr_copy = nullptr;
   uint32_t *clear = nullptr;        // optional: clear_words words the kernel sets to zero (memory of an earlier
   uint32_t clear_words = 0;         // kernel that nobody needs any more)
-  // The sample of the NEXT call on the same table and workspace (a tensor of this one's size and type, next_k
-  // its k) is taken by this kernel's workgroups when they are through with their own tensor: next_hist = that
-  // call's sampling memory (zero, left as k_sample_hist leaves it), next_floor receives its floor key.
+  // The sample of the NEXT call on the same workspace (a tensor of this one's type and of next_n elements, 0:
+  // this one's length; next_k its k) is taken by this kernel's workgroups when they are through with their own
+  // tensor: next_hist = that call's sampling memory (zero, left as k_sample_hist leaves it), next_floor
+  // receives its floor key.
   const void *next_in = nullptr;
   int64_t next_k = 0;
+  int64_t next_n = 0;
   uint32_t *next_hist = nullptr;
   uint32_t *next_floor = nullptr;
   int32_t *status = nullptr;

@@ -1284,9 +1284,10 @@ static int stage_launch(const StageArgs &a, hipStream_t stream) {
   const StageSlabs out{a.geo, a.cg, a.coarse_cursor, a.coarse_words, a.wide ? 1u : 0u};
   StageSample next;
   if (a.next_in && a.next_hist && a.next_k > 0) {
-    const SamplePlan sp = sample_plan(a.n, a.next_k, V);  // the next tensor has this one's size and type
+    const int64_t next_n = a.next_n > 0 ? a.next_n : a.n;  // the next tensor has this one's type
+    const SamplePlan sp = sample_plan(next_n, a.next_k, V);
     next.in = a.next_in;
-    next.n = a.n;
+    next.n = next_n;
     next.hist = a.next_hist;
     next.rank = sp.rank;
     next.block_log2 = sp.log2;

@@ -820,7 +820,14 @@ int slab_load_balance(const SlabBalanceArgs &a, hipStream_t s) {
   if (a.next_input && a.next_k > 0) {
     sc.next_in = a.next_input;
     sc.next_k = a.next_k;
+    sc.next_n = a.next_n;
     sc.next_hist = p.sample_hist[1 - set];
+    if (a.next_state) {  // the sampling memory sits at the head of that table's zero-between-calls memory
+      Carver cn(a.next_state);
+      uint32_t *first = cn.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
+      uint32_t *second = cn.take<uint32_t>(sampled_floor_zero_bytes() / sizeof(uint32_t));
+      sc.next_hist = set ? first : second;
+    }
     sc.next_floor = p.thr + 2 + 4 * (1 - set);
   }
   if ((rc = select_stage_slabs(sc, s)) != ZEN_OK) return rc;

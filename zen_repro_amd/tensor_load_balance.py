@@ -176,30 +176,39 @@ class TensorPartition:
         state["pending"].append((flat.data_ptr(), n, int(k), capacity, ws.data_ptr(), which, _Mark(stream), code,
                                  ws.numel()))
 
-    def _next_sample(self, flat, next_tensor, next_k, capacity, ws, slot, mode, used):
-        """The flat view of `next_tensor` if the call that is about to be made can take that tensor's sample
-        along (same size and type, a path that samples, the other set of sampling memory free), else None."""
+    def _next_sample(self, flat, next_tensor, next_k, capacity, next_capacity, slot, mode, used):
+        """(flat view of `next_tensor`, its table or None if it has this call's size) if the call that is about
+        to be made can take that tensor's sample along (same type, paths that sample, the other set of sampling
+        memory free), else (None, None)."""
         if next_tensor is None or next_k <= 0:
-            return None
+            return None, None
         nxt = next_tensor.reshape(-1)
-        if (nxt.numel() != flat.numel() or nxt.dtype != flat.dtype or nxt.device != flat.device
-                or not nxt.is_contiguous() or (mode & 0xff) != _lib.MODE_FAST):
-            return None
-        n = flat.numel()
-        key = (n, flat.dtype, capacity, next_k, mode & (0xff | _lib.MODE_SLABS))
+        if (nxt.dtype != flat.dtype or nxt.device != flat.device or not nxt.is_contiguous()
+                or (mode & 0xff) != _lib.MODE_FAST):
+            return None, None
+        n, n2 = flat.numel(), nxt.numel()
+        key = (n, n2, flat.dtype, capacity, next_capacity, next_k, mode & (0xff | _lib.MODE_SLABS))
         able = self._samples_next.get(key)
         if able is None:
+            L = _lib.lib()
             m, _ = self.table_sizes(n)
-            able = self._samples_next[key] = bool(_lib.lib().zen_encode_merge_samples_next(
-                n, m, _lib.dtype_code(flat), capacity, self.partitions, next_k, key[4]))
+            m2, _ = self.table_sizes(n2)
+            code = _lib.dtype_code(flat)
+            # this call must be on a path whose pass over the tensor samples, the next one on a path that picks
+            # a sample up from its table
+            able = self._samples_next[key] = bool(
+                L.zen_encode_merge_samples_next(n, m, code, capacity, self.partitions, next_k, key[6])
+                and L.zen_load_balance_path(n2, m2, code, next_capacity, self.partitions, next_k, key[6]) in (2, 3))
         if not able:
-            return None
+            return None, None
         state = self._ahead_state(flat.device, slot, create=True)
         if any(entry[5] == 1 - used for entry in state["pending"]):
-            return None  # the other set holds a sample that is still to be picked up
+            return None, None  # the other set holds a sample that is still to be picked up
         if state["free"][1 - used] is not None:
             state["free"][1 - used].wait(torch.cuda.current_stream(flat.device))
-        return nxt
+        if n2 == n and next_capacity == capacity:
+            return nxt, None
+        return nxt, self._table(flat.device, self.table_sizes(n2)[0], slot)
 
     def _sample_taken(self, nxt, next_k, capacity, ws, slot, which):
         """Books the sample the last call took along for the call that follows (see _next_sample)."""
