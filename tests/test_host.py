@@ -89,6 +89,14 @@ def test_bad_arguments_are_rejected_on_the_host(L):
     assert L.zen_merge(one, 0, one, 0, 10, 100, one, 0, one, 10, one, 7, one, 1 << 20, one, None) == _lib.EINVAL  # mode
     assert L.zen_merge(one, 0, one, 0, 10, 100, one, 0, one, 10, one, 0, one, 16, one, None) == _lib.EWORKSPACE
     assert L.zen_sort_pairs(one, one, 100, None, 33, one, 1 << 20, one, None) == _lib.EINVAL
+    # zen_encode_merge: a next call of its own size must take a path that keeps a sample in its table
+    n = 1 << 24
+    a = _lib.EncodeMergeArgs(
+        256, 1, n, n, 16, 3, None, n // 200, None, 256, 256, n // 100, 256, 256, _lib.MODE_FAST | _lib.MODE_SLABS, 256,
+        1 << 40, 256, 256, 0, 256, 1000, n, 256, 0, 256, 1000, 256, _lib.MODE_FAST, 256, 1 << 40, 256, None, None,
+        256, 20, 4096, 4096, 64, 256)
+    assert L.zen_encode_merge(ctypes.byref(a)) == _lib.EINVAL and b"next call" in L.zen_last_error()
+    assert L.zen_encode_merge(None) == _lib.EINVAL
     with pytest.raises(ValueError):
         _lib.check(_lib.EINVAL, "x")
     with pytest.raises(RuntimeError):

@@ -505,8 +505,8 @@ int load_balance_call(const void *input, int dtype, int64_t n, int64_t m, int pa
         int32_t *table2 = next_table ? next_table : table;
         if (n2 > 0x7fffffffll || m2 > 0x7fffffffll || m2 % partitions != 0 || cap2 > 0x1fffffffll || next_k > n2 ||
             (reinterpret_cast<uintptr_t>(table2) & 7u) != 0 ||
-            (!wide_balance_fits(m2, partitions, cap2, next_k, wide_device_cus(), nullptr) &&
-             !slab_balance_fits(n2, m2, partitions, dtype, cap2, next_k, nullptr)))
+            (!(!slabs_only && wide_balance_fits(m2, partitions, cap2, next_k, wide_device_cus(), nullptr)) &&
+             !slab_balance_fits(n2, m2, partitions, dtype, cap2, next_k, nullptr)))  // (with this call's ZEN_MODE_SLABS)
           return fail(ZEN_EINVAL, "zen_encode_merge: the next call's sizes do not take a path that keeps a sample");
         if (workspace_bytes < zen_load_balance_workspace(n2, m2, dtype, cap2, partitions))
           return fail(ZEN_EWORKSPACE, "zen_encode_merge: workspace too small for the next call");
